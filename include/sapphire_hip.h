@@ -1,0 +1,188 @@
+/*
+ * sapphire_hip.h -- C ABI of the MI355X (gfx950) backend for Sapphire's
+ * matrix-multiplication path.
+ *
+ * Everything the reference's device leaf needs is reachable through these
+ * entry points: plain pointers and sizes, no C++ or framework types.  Every
+ * function returns 0 on success and a non-zero SphStatus otherwise; the text
+ * of the last failure on the calling thread is available from
+ * sph_last_error().  Nothing throws across this boundary.
+ *
+ * All device work is enqueued on one HIP stream per (device, host thread),
+ * the slot the reference fills with a cuBLAS handle per (device, thread)
+ * (Sources/Sapphire/compute/dense/cuda/Gemm.cu:24-30,
+ *  Includes/Sapphire/util/ResourceManager.hpp:152-157).  Calls from one thread
+ * execute in call order; copies to the host wait for preceding work, as the
+ * reference's blocking cudaMemcpy did.
+ *
+ * Citations are relative to the reference tree.
+ */
+#ifndef SAPPHIRE_HIP_H
+#define SAPPHIRE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum
+{
+    SPH_OK = 0,
+    SPH_ERR_INVALID = 1,  /* bad argument (null pointer, zero M*N, size overflow) */
+    SPH_ERR_DEVICE = 2,   /* a HIP runtime call failed */
+    SPH_ERR_UNSUPPORTED = 3
+} SphStatus;
+
+/* IEEE binary16 bit pattern */
+typedef uint16_t sph_f16;
+
+/* Text of the last non-zero status on this thread ("" if none). */
+const char* sph_last_error(void);
+
+/* ---- device / memory / stream ------------------------------------------- *
+ * Replace Sapphire::Compute::Cuda::{CudaSetDevice,CudaMalloc,CudaFree,
+ * CopyHostToDevice,CopyDeviceToHost,CopyDeviceToDevice,CopyDeviceToDeviceAsync}
+ * (Includes/Sapphire/compute/cudaUtil/Memory.hpp:14-30,
+ *  Sources/Sapphire/compute/cudaUtil/Memory.cpp:14-98).  Sizes are size_t: the
+ * reference's unsigned-int byte counts (4 GiB cap) are not inherited. */
+
+typedef struct
+{
+    char name[128];
+    char arch[32];            /* e.g. "gfx950:sramecc+:xnack-" */
+    int computeUnits;
+    int clockMHz;             /* peak engine clock */
+    int memoryClockMHz;
+    int memoryBusWidthBits;
+    int ldsBytesPerBlock;
+    int l2Bytes;
+    uint64_t totalMemoryBytes;
+    int wavefrontSize;
+} SphDeviceInfo;
+
+int sph_device_count(int* count);
+/* replaces CudaSetDevice (Memory.cpp:14-28); SPH_ERR_INVALID when deviceId is
+ * not below the device count */
+int sph_set_device(int deviceId);
+int sph_get_device(int* deviceId);
+int sph_device_info(int deviceId, SphDeviceInfo* info);
+
+int sph_malloc(void** ptr, size_t bytes);              /* Memory.cpp:30-36 */
+int sph_free(void* ptr);                               /* Memory.cpp:38-44 */
+int sph_memcpy_h2d(void* dev, const void* host, size_t bytes); /* :46-53 */
+int sph_memcpy_d2h(void* host, const void* dev, size_t bytes); /* :55-63 */
+int sph_memcpy_d2d(void* dst, const void* src, size_t bytes);  /* :65-72 */
+/* enqueue only, no wait (Memory.cpp:74-82) */
+int sph_memcpy_d2d_async(void* dst, const void* src, size_t bytes);
+/* pinned host staging memory for callers that want asynchronous transfers */
+int sph_host_malloc(void** ptr, size_t bytes);
+int sph_host_free(void* ptr);
+
+/* Wait for everything this thread enqueued on the current device. */
+int sph_stream_sync(void);
+/* The hipStream_t this thread's calls run on (created on first use). */
+int sph_get_stream(void** hipStream);
+/* Run this thread's later calls on a caller-owned hipStream_t; NULL returns
+ * to the library's own stream. */
+int sph_set_stream(void* hipStream);
+
+/* Events on this thread's stream, for timing launches from a host language
+ * that has no HIP binding. */
+int sph_event_create(void** event);
+int sph_event_record(void* event);
+int sph_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for stop */
+int sph_event_destroy(void* event);
+
+/* ---- fills and element-wise neighbours ----------------------------------- */
+
+/* dst[i] = value.  Replaces Dense::Cuda::Scalar
+ * (Sources/Sapphire/compute/dense/cuda/Initialize.cu:46-59), which zero-fills
+ * every fresh device buffer (Sources/Sapphire/tensor/TensorData.cpp:354) and
+ * backs Initialize::Ones/Zeros in Linear (Linear.cpp:118,133). */
+int sph_fill_f32(float* dst, float value, size_t count);
+
+/* out[i] = in[i] > 0 ? in[i] : 0.  Replaces Dense::Cuda::ReLU
+ * (Sources/Sapphire/compute/dense/cuda/kernels/ActivationKernel.cu:11-22);
+ * CPU counterpart NaiveBasic.cpp:159-165. */
+int sph_relu_f32(float* out, const float* in, size_t count);
+
+/* Batched 2-D transpose, out[b][j][i] = in[b][i][j]; with broadcast != 0 the
+ * one input matrix is used for every batch.  Replaces Dense::Cuda::Transpose
+ * (Sources/Sapphire/compute/dense/cuda/Basic.cu:85-102,
+ *  kernels/BasicKernel.cu:78-113). */
+int sph_transpose_f32(float* out, const float* in, uint32_t rows, uint32_t cols,
+                      uint32_t batch, int broadcast);
+
+/* dst[i] = (binary16, round-to-nearest-even) src[i] */
+int sph_convert_f32_to_f16(sph_f16* dst, const float* src, size_t count);
+
+/* ---- dense GEMM ---------------------------------------------------------- */
+
+/* out[b] += A[b] * B[b] for b < batch; row-major; A is M x K, B is K x N,
+ * out is M x N; fp32 storage, fp32 MFMA products and accumulation.
+ * Strides are in elements between consecutive matrices; 0 repeats the
+ * operand for every b (batch broadcast).
+ *
+ * Replaces Dense::Cuda::Gemm (Includes/Sapphire/compute/dense/cuda/Gemm.cuh:15-18,
+ * Sources/Sapphire/compute/dense/cuda/Gemm.cu:19-51): batch = totalSize/(M*N),
+ * strideOut = M*N, strideA = M*K, strideB = K*N; and
+ * Dense::Cuda::GemmMatrixWiseBroadcast (Gemm.cuh:20-25, Gemm.cu:55-85):
+ * strideA = 0 when broadcastA, strideB = 0 when broadcastB.
+ * K == 0 leaves out untouched; M*N == 0 or batch == 0 is SPH_ERR_INVALID. */
+int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M,
+                 uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,
+                 int64_t strideA, int64_t strideB);
+
+/* One M x N unit product per entry, out[outOff] += A[aOff] * B[bOff], offsets
+ * in elements from the three bases.  Entries are read from host memory.  This
+ * is the whole leaf list of BroadcastWith2Inputs
+ * (Includes/Sapphire/compute/Broadcast.hpp:83-133) issued as one launch in
+ * place of one cuBLAS call per leaf.  Entries whose outOff coincide are
+ * applied in entry order. */
+typedef struct
+{
+    uint64_t outOff;
+    uint64_t aOff;
+    uint64_t bOff;
+} SphGemmEntry;
+
+int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out,
+                         const float* A, const float* B, uint32_t M, uint32_t N,
+                         uint32_t K);
+
+/* Half-precision inputs, fp32 accumulation, fp32 output: the tensor-core path
+ * the reference declares as WmmaGemm
+ * (Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50) and
+ * never defines.  Same layout, stride and += contract as sph_gemm_f32.
+ * flags: SPH_GEMM_OVERWRITE stores A*B without reading out (for callers that
+ * know out holds zeros); default accumulates like the reference. */
+#define SPH_GEMM_ACCUMULATE 0u
+#define SPH_GEMM_OVERWRITE 1u
+
+int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M,
+                    uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,
+                    int64_t strideA, int64_t strideB, uint32_t flags);
+
+/* ---- CSR sparse x dense -------------------------------------------------- */
+
+/* out[m][n] (+)= sum over p in [ROW[m], ROW[m+1]) of V[p] * B[COL[p]][n],
+ * entries taken in storage order, products and sums rounded separately in
+ * fp32 (no fused multiply-add), so the result equals the reference's dense
+ * leaf on the densified matrix bit for bit.
+ * V/COL/ROW are the device arrays of a SparseMatrix
+ * (Includes/Sapphire/compute/sparse/SparseMatrix.hpp:28-38); ROW holds M+1
+ * offsets.  Kdim is the sparse matrix's column count (= rows of B); N is the
+ * dense column count.  accumulate == 0 stores (rows without entries become
+ * 0), otherwise adds into out.
+ * The reference declares no sparse x dense product (Sparse.hpp:20-162 holds
+ * sparse x sparse declarations only); this entry fills that slot. */
+int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL,
+                     const uint32_t* ROW, uint32_t M, uint32_t Kdim, uint32_t N,
+                     const float* B, int accumulate);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,432 @@
+// fp32 GEMM  out[u] += A[u] * B[u]  on the CDNA4 matrix cores.
+//
+// Storage, products and accumulation are all fp32 (v_mfma_f32_32x32x2_f32), so
+// the only difference from the reference's scalar CPU loop
+// (Sources/Sapphire/compute/dense/naive/NaiveGemm.cpp:12-38) is the order in
+// which the K products are summed.
+//
+// Work decomposition
+//   * one workgroup (4 wavefronts of 64 lanes, arranged 2 x 2) owns a
+//     BM x BN tile of one M x N unit; BM = BN = 128 when that still gives at
+//     least one tile per compute unit, 64 otherwise;
+//   * the K loop advances 16 columns at a time: the A slab (BM x 16) is stored
+//     k-major in LDS and the B slab (16 x BN) row-major, so that both MFMA
+//     operands are read with lane-consecutive addresses (no bank conflicts);
+//   * the slab for step i+1 is fetched from HBM into registers while the MFMAs
+//     of step i run, and written to the other LDS buffer afterwards;
+//   * units come either from (batch, stride) arithmetic -- stride 0 repeats an
+//     operand -- or from a table of element offsets in device memory.
+//
+// Loads are 16 bytes wide when K, N and every base/stride allow it; otherwise
+// a scalar, fully predicated path handles arbitrary shapes such as the
+// reference's random test sizes (Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:26-33).
+#include "sph_internal.h"
+
+#include <cstring>
+#include <mutex>
+#include <unordered_set>
+
+namespace
+{
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kBK = 16;
+
+struct GemmF32Args
+{
+    float* out;
+    const float* A;
+    const float* B;
+    const SphGemmEntry* entries;  // device table, or null for stride arithmetic
+    uint32_t M, N, K;
+    uint32_t tilesM, tilesN;
+    int64_t strideOut, strideA, strideB;
+};
+
+template <int BM, int BN, bool VEC>
+__global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args)
+{
+    constexpr int WM = BM / 2;   // rows per wavefront
+    constexpr int WN = BN / 2;   // columns per wavefront
+    constexpr int TM = WM / 32;  // MFMA tiles per wavefront, vertically
+    constexpr int TN = WN / 32;
+    constexpr int LDA = BM + 4;  // k-major A slab: As[k][m]
+    constexpr int LDB = BN + 4;  // Bs[k][n]
+    constexpr int A_QUADS = BM * kBK / 4 / kThreads;  // 4-element groups per lane
+    constexpr int B_QUADS = BN * kBK / 4 / kThreads;
+
+    __shared__ float As[2][kBK * LDA];
+    __shared__ float Bs[2][kBK * LDB];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t waveM = wave >> 1;
+    const uint32_t waveN = wave & 1;
+
+    uint32_t id = blockIdx.x;
+    const uint32_t tn = id % args.tilesN;
+    id /= args.tilesN;
+    const uint32_t tm = id % args.tilesM;
+    const uint32_t unit = id / args.tilesM;
+
+    const float* __restrict__ A;
+    const float* __restrict__ B;
+    float* __restrict__ out;
+    if (args.entries != nullptr)
+    {
+        const SphGemmEntry e = args.entries[unit];
+        A = args.A + e.aOff;
+        B = args.B + e.bOff;
+        out = args.out + e.outOff;
+    }
+    else
+    {
+        A = args.A + args.strideA * static_cast<int64_t>(unit);
+        B = args.B + args.strideB * static_cast<int64_t>(unit);
+        out = args.out + args.strideOut * static_cast<int64_t>(unit);
+    }
+
+    const uint32_t M = args.M, N = args.N, K = args.K;
+    const uint32_t rowBase = tm * BM;
+    const uint32_t colBase = tn * BN;
+
+    // ---- which 4-element groups this lane moves from HBM to LDS ------------
+    // A slab: BM rows x 4 groups; group g covers k = 4g..4g+3 of one row.
+    // B slab: 16 rows x BN/4 groups.
+    float4 stageA[A_QUADS];
+    float4 stageB[B_QUADS];
+
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < A_QUADS; ++i)
+        {
+            const uint32_t q = tid + i * kThreads;
+            const uint32_t r = q >> 2;
+            const uint32_t kq = (q & 3) * 4;
+            const uint32_t gr = rowBase + r;
+            const uint32_t gk = k0 + kq;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (gr < M)
+            {
+                const float* p = A + static_cast<size_t>(gr) * K + gk;
+                if (VEC)
+                {
+                    if (gk < K)
+                        v = *reinterpret_cast<const float4*>(p);
+                }
+                else
+                {
+                    if (gk + 0 < K) v.x = p[0];
+                    if (gk + 1 < K) v.y = p[1];
+                    if (gk + 2 < K) v.z = p[2];
+                    if (gk + 3 < K) v.w = p[3];
+                }
+            }
+            stageA[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < B_QUADS; ++i)
+        {
+            const uint32_t q = tid + i * kThreads;
+            const uint32_t kr = q / (BN / 4);
+            const uint32_t nq = (q % (BN / 4)) * 4;
+            const uint32_t gk = k0 + kr;
+            const uint32_t gc = colBase + nq;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (gk < K)
+            {
+                const float* p = B + static_cast<size_t>(gk) * N + gc;
+                if (VEC)
+                {
+                    if (gc < N)
+                        v = *reinterpret_cast<const float4*>(p);
+                }
+                else
+                {
+                    if (gc + 0 < N) v.x = p[0];
+                    if (gc + 1 < N) v.y = p[1];
+                    if (gc + 2 < N) v.z = p[2];
+                    if (gc + 3 < N) v.w = p[3];
+                }
+            }
+            stageB[i] = v;
+        }
+    };
+
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_QUADS; ++i)
+        {
+            const uint32_t q = tid + i * kThreads;
+            const uint32_t r = q >> 2;
+            const uint32_t kq = (q & 3) * 4;
+            float* dst = &As[buf][kq * LDA + r];
+            dst[0 * LDA] = stageA[i].x;
+            dst[1 * LDA] = stageA[i].y;
+            dst[2 * LDA] = stageA[i].z;
+            dst[3 * LDA] = stageA[i].w;
+        }
+#pragma unroll
+        for (int i = 0; i < B_QUADS; ++i)
+        {
+            const uint32_t q = tid + i * kThreads;
+            const uint32_t kr = q / (BN / 4);
+            const uint32_t nq = (q % (BN / 4)) * 4;
+            *reinterpret_cast<float4*>(&Bs[buf][kr * LDB + nq]) = stageB[i];
+        }
+    };
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                acc[i][j][v] = 0.f;
+
+    const uint32_t steps = (K + kBK - 1) / kBK;
+    if (steps > 0)
+    {
+        fetch(0);
+        stash(0);
+    }
+    __syncthreads();
+
+    // MFMA 32x32x2 operand layout: lane l supplies A[l % 32][l / 32] and
+    // B[l / 32][l % 32]; two k values per instruction.
+    const uint32_t l32 = lane & 31;
+    const uint32_t khalf = lane >> 5;
+
+    for (uint32_t s = 0; s < steps; ++s)
+    {
+        const int cur = s & 1;
+        if (s + 1 < steps)
+            fetch((s + 1) * kBK);
+
+        const float* as = &As[cur][waveM * WM + l32];
+        const float* bs = &Bs[cur][waveN * WN + l32];
+#pragma unroll
+        for (int kk = 0; kk < kBK; kk += 2)
+        {
+            float a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                a[i] = as[(kk + khalf) * LDA + i * 32];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                b[j] = bs[(kk + khalf) * LDB + j * 32];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] =
+                        __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+
+        if (s + 1 < steps)
+            stash(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- out += acc ---------------------------------------------------------
+    // 32x32 accumulator layout: register v of lane l holds
+    // row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+        {
+            const uint32_t c = colBase + waveN * WN + j * 32 + l32;
+            if (c >= N)
+                continue;
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+            {
+                const uint32_t r =
+                    rowBase + waveM * WM + i * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
+                if (r < M)
+                {
+                    float* p = out + static_cast<size_t>(r) * N + c;
+                    *p = *p + acc[i][j][v];
+                }
+            }
+        }
+}
+
+// Device table for grouped launches: one growing buffer per device with a
+// pinned staging copy.  The table is shared by every caller, so its use is
+// serialised by a mutex and, across streams, by waiting for the stream that
+// used it last.
+struct EntryTable
+{
+    SphGemmEntry* dev = nullptr;
+    SphGemmEntry* staging = nullptr;  // pinned
+    size_t capacity = 0;
+    hipEvent_t uploaded = nullptr;    // staging may be overwritten after this
+    bool uploadPending = false;
+    hipStream_t lastStream = nullptr;
+};
+std::mutex gTableMutex;
+EntryTable gTables[16];
+
+int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, hipStream_t stream)
+{
+    GemmF32Args args = base;
+    const bool aligned =
+        allowVector && (args.K % 4 == 0) && (args.N % 4 == 0) &&
+        ((reinterpret_cast<uintptr_t>(args.A) | reinterpret_cast<uintptr_t>(args.B)) & 15u) == 0;
+
+    const uint64_t tiles128 =
+        static_cast<uint64_t>((args.M + 127) / 128) * ((args.N + 127) / 128) * units;
+    const bool big = tiles128 >= static_cast<uint64_t>(sph::ComputeUnits());
+    const uint32_t bm = big ? 128 : 64;
+    args.tilesM = (args.M + bm - 1) / bm;
+    args.tilesN = (args.N + bm - 1) / bm;
+    const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
+    if (blocks >= (1ull << 31))
+        return sph::Fail(SPH_ERR_INVALID, "sph_gemm_f32 - too many tiles for one launch");
+
+    const dim3 grid(static_cast<uint32_t>(blocks));
+    const dim3 block(kThreads);
+    if (big)
+    {
+        if (aligned)
+            hipLaunchKernelGGL((GemmF32Kernel<128, 128, true>), grid, block, 0, stream, args);
+        else
+            hipLaunchKernelGGL((GemmF32Kernel<128, 128, false>), grid, block, 0, stream, args);
+    }
+    else
+    {
+        if (aligned)
+            hipLaunchKernelGGL((GemmF32Kernel<64, 64, true>), grid, block, 0, stream, args);
+        else
+            hipLaunchKernelGGL((GemmF32Kernel<64, 64, false>), grid, block, 0, stream, args);
+    }
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int GrowTable(EntryTable& t, size_t count)
+{
+    if (t.capacity >= count)
+        return SPH_OK;
+    // nothing may still be reading the old buffers
+    if (t.lastStream != nullptr)
+        SPH_HIP_TRY(hipStreamSynchronize(t.lastStream));
+    if (t.dev != nullptr)
+        SPH_HIP_TRY(hipFree(t.dev));
+    if (t.staging != nullptr)
+        SPH_HIP_TRY(hipHostFree(t.staging));
+    t.dev = nullptr;
+    t.staging = nullptr;
+    t.capacity = 0;
+    t.uploadPending = false;
+    size_t cap = 1024;
+    while (cap < count)
+        cap *= 2;
+    SPH_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&t.dev), cap * sizeof(SphGemmEntry)));
+    SPH_HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&t.staging), cap * sizeof(SphGemmEntry),
+                              hipHostMallocDefault));
+    if (t.uploaded == nullptr)
+        SPH_HIP_TRY(hipEventCreateWithFlags(&t.uploaded, hipEventDisableTiming));
+    t.capacity = cap;
+    return SPH_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M, uint32_t N, uint32_t K,
+                 uint32_t batch, int64_t strideOut, int64_t strideA, int64_t strideB)
+{
+    SPH_REQUIRE(M != 0 && N != 0 && batch != 0, "M, N and batch must be non-zero");
+    if (K == 0)
+        return SPH_OK;
+    SPH_REQUIRE(out != nullptr && A != nullptr && B != nullptr, "null pointer");
+    SPH_REQUIRE(strideOut >= 0 && strideA >= 0 && strideB >= 0, "negative stride");
+    SPH_REQUIRE(batch == 1 || strideOut >= static_cast<int64_t>(M) * N,
+                "output matrices of a batch must not overlap");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+
+    GemmF32Args args{};
+    args.out = out;
+    args.A = A;
+    args.B = B;
+    args.entries = nullptr;
+    args.M = M;
+    args.N = N;
+    args.K = K;
+    args.strideOut = strideOut;
+    args.strideA = strideA;
+    args.strideB = strideB;
+    const bool stridesAligned = (strideA % 4 == 0) && (strideB % 4 == 0);
+    return Launch(args, batch, stridesAligned, stream);
+}
+
+int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out, const float* A,
+                         const float* B, uint32_t M, uint32_t N, uint32_t K)
+{
+    SPH_REQUIRE(M != 0 && N != 0, "M and N must be non-zero");
+    if (count == 0 || K == 0)
+        return SPH_OK;
+    SPH_REQUIRE(entries != nullptr && out != nullptr && A != nullptr && B != nullptr,
+                "null pointer");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+
+    bool offsetsAligned = true;
+    for (uint32_t i = 0; i < count && offsetsAligned; ++i)
+        offsetsAligned = ((entries[i].aOff | entries[i].bOff) % 4) == 0;
+
+    std::lock_guard<std::mutex> lock(gTableMutex);
+    EntryTable& t = gTables[sph::CurrentDevice()];
+    {
+        const int rc = GrowTable(t, count);
+        if (rc != SPH_OK)
+            return rc;
+    }
+    if (t.lastStream != nullptr && t.lastStream != stream)
+        SPH_HIP_TRY(hipStreamSynchronize(t.lastStream));
+    if (t.uploadPending)
+        SPH_HIP_TRY(hipEventSynchronize(t.uploaded));
+    std::memcpy(t.staging, entries, count * sizeof(SphGemmEntry));
+    SPH_HIP_TRY(hipMemcpyAsync(t.dev, t.staging, count * sizeof(SphGemmEntry),
+                               hipMemcpyHostToDevice, stream));
+    SPH_HIP_TRY(hipEventRecord(t.uploaded, stream));
+    t.uploadPending = true;
+    t.lastStream = stream;
+
+    // Entries that add into the same output unit must be applied in order:
+    // cut the list into launches inside which every outOff is distinct.
+    uint32_t begin = 0;
+    std::unordered_set<uint64_t> seen;
+    while (begin < count)
+    {
+        seen.clear();
+        uint32_t end = begin;
+        while (end < count && seen.insert(entries[end].outOff).second)
+            ++end;
+
+        GemmF32Args args{};
+        args.out = out;
+        args.A = A;
+        args.B = B;
+        args.entries = t.dev + begin;
+        args.M = M;
+        args.N = N;
+        args.K = K;
+        const int rc = Launch(args, end - begin, offsetsAligned, stream);
+        if (rc != SPH_OK)
+            return rc;
+        begin = end;
+    }
+    return SPH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,57 @@
+// Internal helpers shared by the translation units of libsapphire_hip.so.
+#ifndef SPH_INTERNAL_H
+#define SPH_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <string>
+
+#include "sapphire_hip.h"
+
+namespace sph
+{
+// Records `msg` as this thread's last error and returns `status`.
+int Fail(int status, const std::string& msg);
+
+// Stream that this thread's work on the current device is enqueued on.
+// Returns nullptr (and records the error) when it cannot be created.
+hipStream_t CurrentStream();
+
+// Device the calling thread last selected through sph_set_device (0 at start).
+int CurrentDevice();
+
+// Number of compute units of the current device (cached).
+int ComputeUnits();
+}  // namespace sph
+
+#define SPH_HIP_TRY(expr)                                                      \
+    do                                                                         \
+    {                                                                          \
+        const hipError_t sphErr__ = (expr);                                    \
+        if (sphErr__ != hipSuccess)                                            \
+            return ::sph::Fail(SPH_ERR_DEVICE, std::string(#expr) +            \
+                                                   " failed with " +           \
+                                                   hipGetErrorString(sphErr__)); \
+    } while (0)
+
+#define SPH_REQUIRE(cond, what)                                                \
+    do                                                                         \
+    {                                                                          \
+        if (!(cond))                                                           \
+            return ::sph::Fail(SPH_ERR_INVALID, std::string(__func__) +        \
+                                                    " - " + (what));           \
+    } while (0)
+
+// Checks the launch that was just issued.
+#define SPH_CHECK_LAUNCH()                                                     \
+    do                                                                         \
+    {                                                                          \
+        const hipError_t sphErr__ = hipGetLastError();                         \
+        if (sphErr__ != hipSuccess)                                            \
+            return ::sph::Fail(SPH_ERR_DEVICE, std::string(__func__) +         \
+                                                   " launch failed with " +    \
+                                                   hipGetErrorString(sphErr__)); \
+    } while (0)
+
+#endif

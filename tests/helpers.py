@@ -1,0 +1,79 @@
+"""Shared pieces of the parity tests: error metrics and device round trips."""
+import sys
+
+import numpy as np
+
+from sapphire_amd import capi
+
+
+def announce(*what):
+    """Name the case on stdout before the GPU step runs."""
+    print("[case]", *what)
+    sys.stdout.flush()
+
+
+def normalised_error(got, ref, absA, absB_or_denominator, is_denominator=False):
+    """max_ij |got - ref| / sum_k |a_ik * b_kj|   (the K-length normalisation)."""
+    if is_denominator:
+        den = absB_or_denominator
+    else:
+        den = absA.astype(np.float64) @ absB_or_denominator.astype(np.float64)
+    den = np.maximum(den, np.finfo(np.float32).tiny)
+    return float(np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)) / den))
+
+
+def gpu_gemm_f32(C, A, B, M, N, K, batch=1, stride_out=None, stride_a=None, stride_b=None):
+    """C (numpy, any shape, float32) += A*B through sph_gemm_f32; returns the new C."""
+    so = M * N if stride_out is None else stride_out
+    sa = M * K if stride_a is None else stride_a
+    sb = K * N if stride_b is None else stride_b
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    capi.call("sph_gemm_f32", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, so, sa, sb)
+    out = dC.download(np.float32, C.shape)
+    for d in (dA, dB, dC):
+        d.release()
+    return out
+
+
+def gpu_gemm_f16(C, A16, B16, M, N, K, batch=1, stride_out=None, stride_a=None, stride_b=None,
+                 flags=0):
+    so = M * N if stride_out is None else stride_out
+    sa = M * K if stride_a is None else stride_a
+    sb = K * N if stride_b is None else stride_b
+    assert A16.dtype == np.float16 and B16.dtype == np.float16
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A16, B16, C))
+    capi.call("sph_gemm_f16f32", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, so, sa, sb, flags)
+    out = dC.download(np.float32, C.shape)
+    for d in (dA, dB, dC):
+        d.release()
+    return out
+
+
+def gpu_gemm_grouped(C, A, B, M, N, K, triples):
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    entries = capi.make_entries(triples)
+    capi.call("sph_gemm_f32_grouped", entries, len(triples), dC.ptr, dA.ptr, dB.ptr, M, N, K)
+    out = dC.download(np.float32, C.shape)
+    for d in (dA, dB, dC):
+        d.release()
+    return out
+
+
+def gpu_spmm(C, V, COL, ROW, M, Kdim, N, B, accumulate, canary=0):
+    """Runs sph_spmm_csr_f32 with `canary` guard floats on both sides of out."""
+    guard = np.full(canary, np.float32(-12345.5), dtype=np.float32)
+    padded = np.concatenate([guard, C.ravel(), guard]).astype(np.float32)
+    dC = capi.DeviceBuffer.from_array(padded)
+    dV = capi.DeviceBuffer.from_array(V if V.size else np.zeros(1, np.float32))
+    dCol = capi.DeviceBuffer.from_array(COL if COL.size else np.zeros(1, np.uint32))
+    dRow = capi.DeviceBuffer.from_array(ROW)
+    dB = capi.DeviceBuffer.from_array(B)
+    capi.call("sph_spmm_csr_f32", dC.at(4 * canary), dV.ptr, dCol.ptr, dRow.ptr, M, Kdim, N,
+              dB.ptr, 1 if accumulate else 0)
+    back = dC.download(np.float32, padded.shape)
+    for d in (dC, dV, dCol, dRow, dB):
+        d.release()
+    if canary:
+        assert np.array_equal(back[:canary], guard), "write before the start of out"
+        assert np.array_equal(back[-canary:], guard), "write past the end of out"
+    return back[canary:canary + C.size].reshape(C.shape)

@@ -1,0 +1,114 @@
+"""fp16-input / fp32-accumulate GEMM through the C ABI.
+
+Oracle: the reference's fp32 CPU loop run on the fp16 inputs exactly widened to fp32, so only
+the summation order differs.  Tolerance (fp16-in path): max_ij |gpu - cpu| / sum_k|a_ik b_kj|
+<= 1e-2.  Integer-valued inputs make every product and partial sum exact, so tiling and
+indexing are additionally checked bit for bit.
+"""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from sapphire_amd import capi, synth
+from tests import helpers as h
+
+pytestmark = pytest.mark.gpu
+TOL_F16 = 1e-2
+
+
+def _oracle(C, A16, B16, M, N, K, batch=1, sa=None, sb=None):
+    A = A16.astype(np.float32)
+    B = B16.astype(np.float32)
+    return po.gemm_rows(C.copy(), A, B, M, N, K, batch=batch, stride_a=sa, stride_b=sb, threads=8)
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 64), (256, 512, 128), (512, 256, 192),
+                                   (768, 1024, 256)])
+def test_tile256_exact_on_integers(dev, shape):
+    M, N, K = shape
+    h.announce("sph_gemm_f16f32 tile256 integer exactness", shape)
+    A = synth.small_integers(1, (M, K)).astype(np.float16)
+    B = synth.small_integers(2, (K, N)).astype(np.float16)
+    C = synth.small_integers(3, (M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K)
+    assert np.array_equal(got, ref)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, flags=capi.SPH_GEMM_OVERWRITE)
+    assert np.array_equal(got, ref - C)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 2), (31, 33, 17), (64, 64, 32), (100, 72, 40),
+                                   (128, 128, 64), (130, 254, 96), (200, 8, 1000), (257, 255, 63)])
+def test_general_exact_on_integers(dev, shape):
+    M, N, K = shape
+    h.announce("sph_gemm_f16f32 general integer exactness", shape)
+    A = synth.small_integers(4, (M, K), span=3).astype(np.float16)
+    B = synth.small_integers(5, (K, N), span=3).astype(np.float16)
+    C = synth.small_integers(6, (M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K)
+    assert np.array_equal(got, ref)
+
+
+def test_batched_and_broadcast(dev):
+    h.announce("sph_gemm_f16f32 batch 3, strideB = 0, tile256 path")
+    M, N, K, batch = 256, 256, 128, 3
+    A = synth.normal(7, (batch, M, K), 0.1).astype(np.float16)
+    B = synth.normal(8, (1, K, N), 0.1).astype(np.float16)
+    C = synth.uniform(9, (batch, M, N))
+    ref = _oracle(C, A, B, M, N, K, batch=batch, sb=0)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, stride_b=0)
+    for b in range(batch):
+        err = h.normalised_error(got[b], ref[b], np.abs(A[b]).astype(np.float32),
+                                 np.abs(B[0]).astype(np.float32))
+        assert err <= TOL_F16
+    h.announce("sph_gemm_f16f32 batch 4 general path, strideA = 0")
+    M, N, K, batch = 70, 90, 50, 4
+    A = synth.normal(10, (1, M, K), 0.1).astype(np.float16)
+    B = synth.normal(11, (batch, K, N), 0.1).astype(np.float16)
+    C = synth.uniform(12, (batch, M, N))
+    ref = _oracle(C, A, B, M, N, K, batch=batch, sa=0)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, stride_a=0)
+    for b in range(batch):
+        err = h.normalised_error(got[b], ref[b], np.abs(A[0]).astype(np.float32),
+                                 np.abs(B[b]).astype(np.float32))
+        assert err <= TOL_F16
+
+
+def test_config3_4096_cubed(dev):
+    """The headline shape: M = N = K = 4096, N(0, 1/sqrt(K)) fp16 inputs, C zeros."""
+    h.announce("sph_gemm_f16f32 config3 4096^3")
+    d = synth.config3()
+    n = 4096
+    ref = _oracle(d["C"], d["A"], d["B"], n, n, n)
+    got = h.gpu_gemm_f16(d["C"], d["A"], d["B"], n, n, n)
+    den = np.abs(d["A"]).astype(np.float32) @ np.abs(d["B"]).astype(np.float32)
+    err = h.normalised_error(got, ref, None, den.astype(np.float64), True)
+    assert np.isfinite(got).all()
+    assert err <= TOL_F16, err
+    # the same data with the overwrite flag must give the same bits (C is zero)
+    got2 = h.gpu_gemm_f16(d["C"], d["A"], d["B"], n, n, n, flags=capi.SPH_GEMM_OVERWRITE)
+    assert np.array_equal(got, got2)
+    # linearity in the accumulator, size-independent: run again on top of the result
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (d["A"], d["B"], got))
+    capi.call("sph_gemm_f16f32", dC.ptr, dA.ptr, dB.ptr, n, n, n, 1, n * n, n * n, n * n, 0)
+    twice = dC.download(np.float32, got.shape)
+    for x in (dA, dB, dC):
+        x.release()
+    assert np.array_equal(twice, got + got)
+
+
+def test_convert_f32_to_f16_matches_numpy_rounding(dev):
+    h.announce("sph_convert_f32_to_f16")
+    x = np.concatenate([synth.normal(13, (100003,), 3.0),
+                        np.array([0.0, -0.0, 65504.0, 65520.0, 1e-8, 6e-8, -7e4, np.inf],
+                                 np.float32)])
+    dX = capi.DeviceBuffer.from_array(x)
+    dY = capi.DeviceBuffer(2 * x.size)
+    capi.call("sph_convert_f32_to_f16", dY.ptr, dX.ptr, x.size)
+    got = dY.download(np.uint16, x.shape)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+    dX.release()
+    dY.release()

@@ -1,0 +1,178 @@
+"""fp32 GEMM through the C ABI against the CPU checker on identical seeded inputs.
+
+Tolerance (fp32 path): max_ij |gpu - cpu| / sum_k |a_ik * b_kj| <= 1e-4.
+"""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from sapphire_amd import capi, synth
+from tests import helpers as h
+
+pytestmark = pytest.mark.gpu
+TOL_F32 = 1e-4
+
+
+def _check(got, ref, A2, B2, what):
+    err = h.normalised_error(got, ref, np.abs(A2), np.abs(B2))
+    assert np.isfinite(got).all(), what
+    assert err <= TOL_F32, "%s: normalised error %.3e" % (what, err)
+    return err
+
+
+def test_config1_256_cubed(dev):
+    h.announce("sph_gemm_f32 config1 256^3")
+    d = synth.config1()
+    ref = po.naive_gemm(d["C"].copy(), d["A"], d["B"], 256, 256, 256)
+    got = h.gpu_gemm_f32(d["C"], d["A"], d["B"], 256, 256, 256)
+    _check(got, ref, d["A"], d["B"], "config1")
+    # C really takes part: result minus product of a zero-C run equals C up to rounding
+    got0 = h.gpu_gemm_f32(np.zeros_like(d["C"]), d["A"], d["B"], 256, 256, 256)
+    assert np.max(np.abs((got - got0) - d["C"])) < 1e-4
+
+
+def test_config2_batch_broadcast_B(dev):
+    h.announce("sph_gemm_f32 config2 A[16,512,512] B[1,512,512] strideB=0")
+    d = synth.config2()
+    ref = po.compute_gemm(d["C"].copy(), d["A"], d["B"], threads=8)
+    got = h.gpu_gemm_f32(d["C"], d["A"], d["B"], 512, 512, 512, batch=16, stride_b=0)
+    for b in range(16):
+        _check(got[b], ref[b], d["A"][b], d["B"][0], "config2 unit %d" % b)
+
+
+def test_broadcast_A(dev):
+    h.announce("sph_gemm_f32 strideA=0")
+    A = synth.uniform(11, (1, 96, 40))
+    B = synth.uniform(12, (5, 40, 72))
+    C = synth.uniform(13, (5, 96, 72))
+    ref = po.compute_gemm(C.copy(), A, B)
+    got = h.gpu_gemm_f32(C, A, B, 96, 72, 40, batch=5, stride_a=0)
+    for b in range(5):
+        _check(got[b], ref[b], A[0], B[b], "unit %d" % b)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_reference_recipe_gemm1(dev, seed):
+    """Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:20-84: M, N, K in [1,100], batch in
+    [1,30], shapes {b,M,K} x {b,K,N} -> {b,M,N}, out zero.  Also meets that test's own bound
+    (absolute difference <= 2.0 with inputs N(10,5))."""
+    r = synth.bits64(0xC0FFEE + seed, 4)
+    M, N, K = (int(x % 100) + 1 for x in r[:3])
+    batch = int(r[3] % 100 + 1) % 30 + 1
+    h.announce("Gemm1 recipe seed", seed, "M N K batch =", M, N, K, batch)
+    A = (synth.normal(100 + seed, (batch, M, K), 5.0) + 10).astype(np.float32)
+    B = (synth.normal(200 + seed, (batch, K, N), 5.0) + 10).astype(np.float32)
+    C = np.zeros((batch, M, N), np.float32)
+    ref = po.compute_gemm(C.copy(), A, B)
+    got = h.gpu_gemm_f32(C, A, B, M, N, K, batch=batch)
+    assert np.max(np.abs(got - ref)) <= 2.0
+    assert np.any(got != 0)
+    for b in range(batch):
+        _check(got[b], ref[b], A[b], B[b], "unit %d" % b)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (1, 7, 3), (33, 1, 5), (64, 64, 16), (65, 63, 17),
+                                   (128, 128, 15), (129, 257, 31), (300, 40, 1), (4, 4, 1000)])
+def test_edges(dev, shape):
+    M, N, K = shape
+    h.announce("sph_gemm_f32 edge", shape)
+    A = synth.uniform(21, (M, K))
+    B = synth.uniform(22, (K, N))
+    C = synth.uniform(23, (M, N))
+    ref = po.naive_gemm(C.copy(), A, B, M, N, K)
+    got = h.gpu_gemm_f32(C, A, B, M, N, K)
+    _check(got, ref, A, B, str(shape))
+
+
+def test_closed_forms(dev):
+    h.announce("sph_gemm_f32 closed forms")
+    n = 200
+    B = synth.uniform(31, (n, n))
+    C = synth.uniform(32, (n, n))
+    eye = np.eye(n, dtype=np.float32)
+    got = h.gpu_gemm_f32(C, eye, B, n, n, n)
+    assert np.array_equal(got, C + B)          # identity: out = B + C exactly
+    ones = np.ones((n, n), np.float32)
+    got = h.gpu_gemm_f32(np.zeros((n, n), np.float32), ones, ones, n, n, n)
+    assert np.array_equal(got, np.full((n, n), float(n), np.float32))
+    # K = 1 outer product: how Linear adds its bias (Linear.cpp:134)
+    col = np.ones((n, 1), np.float32)
+    bias = synth.uniform(33, (1, n))
+    got = h.gpu_gemm_f32(np.zeros((n, n), np.float32), col, bias, n, n, 1)
+    assert np.array_equal(got, np.broadcast_to(bias, (n, n)))
+
+
+def test_k_zero_leaves_out_untouched(dev):
+    C = synth.uniform(41, (8, 8))
+    got = h.gpu_gemm_f32(C, np.zeros(1, np.float32), np.zeros(1, np.float32), 8, 8, 0)
+    assert np.array_equal(got, C)
+
+
+def test_unaligned_bases(dev):
+    """Operands that start 4 bytes into an allocation take the scalar load path."""
+    h.announce("sph_gemm_f32 unaligned bases")
+    M, N, K = 72, 64, 48
+    A = synth.uniform(51, (M * K + 1,))
+    B = synth.uniform(52, (K * N + 1,))
+    C = synth.uniform(53, (M * N + 1,))
+    ref = po.naive_gemm(C[1:].copy(), A[1:].copy(), B[1:].copy(), M, N, K)
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    capi.call("sph_gemm_f32", dC.at(4), dA.at(4), dB.at(4), M, N, K, 1, M * N, M * K, K * N)
+    got = dC.download(np.float32, C.shape)
+    assert got[0] == C[0]
+    _check(got[1:].reshape(M, N), ref.reshape(M, N), A[1:].reshape(M, K), B[1:].reshape(K, N),
+           "unaligned")
+
+
+def test_grouped_plan_with_modulo_quirk(dev):
+    """{b,1,M,K} x {b,M,K,N} -> {b,M,M,N} (BroadcastTest.cpp:32-34): the walk picks
+    A matrix i % b, which is not NumPy broadcasting; the leaves go out as one launch."""
+    b, M, K, N = 2, 3, 2, 2
+    ys, as_, bs = [b, M, M, N], [b, 1, M, K], [b, M, K, N]
+    dims, leaves = po.gemm_plan(ys, as_, bs)
+    assert [(o // (M * N), a // (M * K), bb // (K * N)) for o, a, bb, _ in leaves] == \
+        [(0, 0, 0), (1, 1, 1), (2, 0, 2), (3, 1, 3), (4, 0, 4), (5, 1, 5)]
+    h.announce("sph_gemm_f32_grouped modulo quirk")
+    A = synth.uniform(61, as_)
+    B = synth.uniform(62, bs)
+    C = synth.uniform(63, ys)
+    ref = po.compute_gemm(C.copy(), A, B)
+    triples = []
+    for o, a, bb, total in leaves:
+        for u in range(total // (M * N)):
+            triples.append((o + u * M * N, a + u * M * K, bb + u * K * N))
+    got = h.gpu_gemm_grouped(C, A, B, M, N, K, triples)
+    den = np.full(C.shape, 1e-30)
+    flatA, flatB = A.reshape(-1, M, K), B.reshape(-1, K, N)
+    den = den.reshape(-1, M, N)
+    for i, (o, a, bb) in enumerate(triples):
+        den[o // (M * N)] = np.abs(flatA[a // (M * K)]).astype(np.float64) @ np.abs(flatB[bb // (K * N)])
+    err = h.normalised_error(got.reshape(-1, M, N), ref.reshape(-1, M, N), None, den, True)
+    assert err <= TOL_F32
+
+
+def test_grouped_repeated_output_is_applied_in_order(dev):
+    """Two entries adding into one output unit are serialised, as the host walk would."""
+    h.announce("sph_gemm_f32_grouped repeated outOff")
+    M, N, K = 40, 24, 16
+    A = synth.uniform(71, (3, M, K))
+    B = synth.uniform(72, (3, K, N))
+    C = synth.uniform(73, (2, M, N))
+    triples = [(0, 0, 0), (M * N, M * K, K * N), (0, 2 * M * K, 2 * K * N)]
+    ref = C.copy()
+    for o, a, bb in triples:
+        po.naive_gemm(ref.reshape(-1)[o:o + M * N], A.reshape(-1)[a:a + M * K].copy(),
+                      B.reshape(-1)[bb:bb + K * N].copy(), M, N, K)
+    got = h.gpu_gemm_grouped(C, A, B, M, N, K, triples)
+    assert np.max(np.abs(got - ref)) < 1e-4
+
+
+def test_errors_are_statuses_not_crashes(dev):
+    with pytest.raises(capi.SphError) as e:
+        capi.call("sph_gemm_f32", None, None, None, 4, 4, 4, 1, 16, 16, 16)
+    assert e.value.status == 1 and "null" in str(e.value)
+    with pytest.raises(capi.SphError):
+        capi.call("sph_gemm_f32", 1, 1, 1, 0, 4, 4, 1, 0, 0, 0)
+    with pytest.raises(capi.SphError) as e:
+        capi.call("sph_set_device", 99)
+    assert "exceeds number of available devices" in str(e.value)
