@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the matrix-multiplication path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+
+A step is one pass of the hot path over one batch of synthetic input: one launch of the
+fp16-input / fp32-accumulate GEMM at M = N = K = 4096 (configuration 3), out += A*B with the
+inputs already resident in HBM.  The script does W untimed steps, then times exactly K steps
+between two synchronisation points and prints ONE JSON line.  `value` is TFLOP/s of those K
+steps (2*4096^3 flop each).  The same line carries
+
+  roofline      the GEMM kernel against the dense fp16 MFMA peak, from HIP events recorded on
+                the stream the kernel runs on;
+  spmm          the CSR x dense product of configuration 5 (8192 x 8192 at 1 % times
+                8192 x 256), timed the same way, against the HBM peak on algorithmic bytes;
+  cpu_baseline  the reference's own scalar CPU GEMM (built into oracle/_ref from the
+                reference's NaiveGemm.cpp; the plain-C port when that build is absent) timed
+                on a bounded slice of the same workload on this machine's host cores.
+
+Everything runs on one GPU; --gpus above 1 is refused.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA, vendor figure
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=10)
+    p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    p.add_argument("--all", action="store_true",
+                   help="also time configurations 1, 2 and 4 (reported under 'others')")
+    p.add_argument("--only", choices=["gemm", "spmm"], default=None,
+                   help="run a single kernel (for profiler runs); the JSON line is reduced")
+    return p.parse_args()
+
+
+def timed_launches(capi, launch, steps, warmup):
+    """Average milliseconds per launch from HIP events on the launch stream, and the wall-clock
+    milliseconds per step between two stream synchronisations."""
+    for _ in range(warmup):
+        launch()
+    capi.sync()
+    start, stop = capi.Event(), capi.Event()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        launch()
+    stop.record()
+    capi.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    event_ms = stop.elapsed_ms_since(start) / steps
+    start.destroy()
+    stop.destroy()
+    return event_ms, wall_ms
+
+
+def bench_gemm_f16(capi, synth, steps, warmup, flags=0):
+    n = 4096
+    d = synth.config3(n)
+    dA = capi.DeviceBuffer.from_array(d["A"])
+    dB = capi.DeviceBuffer.from_array(d["B"])
+    dC = capi.DeviceBuffer.from_array(d["C"])
+
+    def launch():
+        capi.call("sph_gemm_f16f32", dC.ptr, dA.ptr, dB.ptr, n, n, n, 1, n * n, n * n, n * n, flags)
+
+    event_ms, wall_ms = timed_launches(capi, launch, steps, warmup)
+    for b in (dA, dB, dC):
+        b.release()
+    return event_ms, wall_ms, d
+
+
+def bench_spmm(capi, synth, steps, warmup):
+    d = synth.config5()
+    M, K, N = d["M"], d["K"], d["N"]
+    dV = capi.DeviceBuffer.from_array(d["V"])
+    dCol = capi.DeviceBuffer.from_array(d["COL"])
+    dRow = capi.DeviceBuffer.from_array(d["ROW"])
+    dB = capi.DeviceBuffer.from_array(d["B"])
+    dC = capi.DeviceBuffer.from_array(d["C"])
+
+    def launch():
+        capi.call("sph_spmm_csr_f32", dC.ptr, dV.ptr, dCol.ptr, dRow.ptr, M, K, N, dB.ptr, 0)
+
+    event_ms, wall_ms = timed_launches(capi, launch, steps, warmup)
+    for b in (dV, dCol, dRow, dB, dC):
+        b.release()
+    nnz = int(d["V"].size)
+    # store mode: V + COL, ROW, B once, out written once
+    alg_bytes = nnz * 8 + (M + 1) * 4 + K * N * 4 + M * N * 4
+    return event_ms, wall_ms, d, nnz, alg_bytes
+
+
+def bench_f32(capi, A, B, C, M, N, K, batch, sb, steps, warmup):
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+
+    def launch():
+        capi.call("sph_gemm_f32", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, M * N, M * K, sb)
+
+    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    for b in (dA, dB, dC):
+        b.release()
+    return event_ms
+
+
+def cpu_gemm_baseline(d, rows=96):
+    """The reference's scalar loop on rows [0, rows) of configuration 3 (inputs widened to fp32
+    exactly), one thread, as the reference runs it."""
+    from oracle import pyoracle as po
+    n = d["A"].shape[0]
+    A = np.ascontiguousarray(d["A"][:rows].astype(np.float32))
+    B = d["B"].astype(np.float32)
+    out = np.zeros((rows, n), np.float32)
+    if po.have_ref():
+        fn, kind = po.ref().ref_naive_gemm, "reference"
+    else:
+        fn, kind = po.oracle().orc_naive_gemm, "port"
+    t0 = time.perf_counter()
+    fn(out.size, po._f(out), po._f(A), po._f(B), rows, n, n)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * rows * n * n
+    return {
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
+        "sample": "rows 0..%d of configuration 3 (%dx%dx%d fp32 after exact widening), "
+                  "Dense::Naive::Gemm scalar loop, %.1f s" % (rows - 1, rows, n, n, dt),
+        "host_cores_available": os.cpu_count(),
+    }
+
+
+def cpu_spmm_baseline(d):
+    from oracle import pyoracle as po
+    out = np.zeros((d["M"], d["N"]), np.float32)
+    t0 = time.perf_counter()
+    po.spmm_csr(out, d["V"], d["COL"], d["ROW"], d["M"], d["N"], d["B"], threads=1)
+    dt = time.perf_counter() - t0
+    return dt
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; --gpus %d is not supported (the path shards without "
+              "collectives and every box here has one GPU)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from sapphire_amd import capi, synth
+    capi.call("sph_set_device", 0)
+    info = capi.device_info(0)
+    device_peak = info.computeUnits * 4096 * info.clockMHz * 1e6 / 1e12  # fp16 flop/clk/CU = 4096
+
+    result = {}
+    n = 4096
+    flops = 2.0 * n ** 3
+    if args.only in (None, "gemm"):
+        event_ms, wall_ms, d3 = bench_gemm_f16(capi, synth, args.steps, args.warmup)
+        tflops = flops / (wall_ms * 1e-3) / 1e12
+        kernel_tflops = flops / (event_ms * 1e-3) / 1e12
+        result.update({
+            "metric": "GEMM TFLOP/s + % MFMA peak (4096^3 fp16->fp32); SpMM GB/s + % HBM peak",
+            "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": wall_ms, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f16 in / f32 accumulate",
+            "data": "synthetic",
+            "config": {"workload": "configuration 3: out[4096,4096] f32 += A[4096,4096] f16 * "
+                                   "B[4096,4096] f16, N(0,1/sqrt(K)) inputs, row-major, one launch "
+                                   "per step, inputs resident in HBM",
+                       "entry_point": "sph_gemm_f16f32 (accumulate)"},
+            "roofline": {"bound": "mfma", "kernel": "GemmF16Tile256",
+                         "achieved": kernel_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": kernel_tflops / PEAK_FP16_TFLOPS, "traffic": None,
+                         "launch_ms": event_ms, "flop_per_launch": flops,
+                         "peak_from_device": device_peak,
+                         "peak_from_device_note": "%d CUs x 4096 flop/clk x %d MHz"
+                                                  % (info.computeUnits, info.clockMHz)},
+            "device": {"name": info.name.decode(), "arch": info.arch.decode(),
+                       "compute_units": info.computeUnits, "clock_mhz": info.clockMHz},
+        })
+        if args.only is None:
+            ev_over, _, _ = bench_gemm_f16(capi, synth, args.steps, args.warmup,
+                                           flags=capi.SPH_GEMM_OVERWRITE)
+            result["gemm_overwrite_variant"] = {
+                "note": "same launch with SPH_GEMM_OVERWRITE (out is not read)",
+                "launch_ms": ev_over, "tflops": flops / (ev_over * 1e-3) / 1e12}
+
+    if args.only in (None, "spmm"):
+        sp_steps = max(args.steps * 4, 100)
+        sp_event, sp_wall, d5, nnz, alg_bytes = bench_spmm(capi, synth, sp_steps, args.warmup)
+        gbs = alg_bytes / (sp_event * 1e-3) / 1e9
+        spmm = {
+            "workload": "configuration 5: CSR 8192x8192 at 1 %% (nnz %d) x dense 8192x256 f32, "
+                        "store mode" % nnz,
+            "entry_point": "sph_spmm_csr_f32", "steps": sp_steps, "launch_ms": sp_event,
+            "value": gbs, "unit": "GB/s", "gflops": 2.0 * nnz * 256 / (sp_event * 1e-3) / 1e9,
+            "roofline": {"bound": "hbm", "kernel": "SpmmRowVec4", "achieved": gbs,
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                         "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                         "gather_bytes_per_launch": nnz * 256 * 4},
+        }
+        if not args.no_cpu and args.only is None:
+            dt = cpu_spmm_baseline(d5)
+            spmm["cpu_baseline"] = {"value": alg_bytes / dt / 1e9, "unit": "GB/s", "cores": 1,
+                                    "kind": "port",
+                                    "sample": "whole configuration 5, storage-order CSR loop "
+                                              "(the reference has no sparse x dense code), %.2f s" % dt}
+        result["spmm"] = spmm
+
+    if args.all and args.only is None:
+        others = {}
+        c1 = synth.config1()
+        ms = bench_f32(capi, c1["A"], c1["B"], c1["C"], 256, 256, 256, 1, 256 * 256, 1000, 50)
+        others["config1_f32_256"] = {"launch_ms": ms, "tflops": 2 * 256 ** 3 / (ms * 1e-3) / 1e12}
+        c2 = synth.config2()
+        ms = bench_f32(capi, c2["A"], c2["B"], c2["C"], 512, 512, 512, 16, 0, 200, 20)
+        tf = 16 * 2 * 512 ** 3 / (ms * 1e-3) / 1e12
+        others["config2_f32_batched"] = {"launch_ms": ms, "tflops": tf,
+                                         "frac_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
+        result["others"] = others
+
+    if not args.no_cpu and args.only is None:
+        result["cpu_baseline"] = cpu_gemm_baseline(d3)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -31,6 +31,13 @@
 //     loads when K, N and the bases allow), padded LDS rows.
 #include "sph_internal.h"
 
+#include <cstdlib>
+#include <type_traits>
+
+#ifndef SPH_ABLATE
+#define SPH_ABLATE 0
+#endif
+
 namespace
 {
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
@@ -50,6 +57,9 @@ struct GemmF16Args
     uint32_t totalTiles;  // tilesM * tilesN * batch
     int64_t strideOut, strideA, strideB;
     uint32_t overwrite;
+#if SPH_ABLATE & 16
+    long long* trace;
+#endif
 };
 
 // Transposing LDS read: within each group of 16 lanes, lane s supplies the
@@ -58,6 +68,34 @@ struct GemmF16Args
 __device__ __forceinline__ halfx4 LdsReadTr(const _Float16* p)
 {
     return __builtin_bit_cast(halfx4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsShortx4Ptr)(p)));
+}
+
+// Asynchronous 16-byte-per-lane copy from global memory straight into LDS
+// (global_load_lds_dwordx4): lane i reads 16 bytes at uniformBase + laneByteOffset +
+// OFFSET and they land at ldsByteAddr + OFFSET + 16*i.  ldsByteAddr must be uniform
+// across the wavefront (it travels in M0) and so must uniformBase (an SGPR pair).
+// The copy is counted by vmcnt like any vector memory load; the caller waits with
+// WaitVmem() before the data is read.  Issued through inline assembly so that the
+// compiler does not serialise it against unrelated LDS reads.
+template <int OFFSET>
+__device__ __forceinline__ void DmaToLds16(uint32_t laneByteOffset, const void* uniformBase,
+                                           uint32_t ldsByteAddr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+                 :
+                 : "s"(ldsByteAddr), "v"(laneByteOffset), "s"(uniformBase), "n"(OFFSET)
+                 : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void WaitVmem()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+__device__ __forceinline__ uint32_t LdsAddress(const void* p)
+{
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsPtr)(p)));
 }
 
 __device__ __forceinline__ halfx8 Join(halfx4 lo, halfx4 hi)
@@ -91,17 +129,31 @@ __device__ __forceinline__ bool MapTile(uint32_t id, uint32_t tilesM, uint32_t t
 }
 
 // ---------------------------------------------------------------------------
-// 256 x 256 x 64 tile kernel
+// 256 x 256 tile kernel, K step 32, four LDS stages
 // ---------------------------------------------------------------------------
 constexpr int kT = 256;         // tile edge
-constexpr int kTK = 64;         // K step
-constexpr int kTThreads = 512;  // 8 wavefronts
-constexpr int kStageHalfs = kT * kTK;  // per operand per stage (32 KiB)
+constexpr int kTK = 32;         // K step
+constexpr int kTStages = 4;
+constexpr int kStageBytes = kT * kTK * 2;  // per operand per stage (16 KiB)
+constexpr int kStageHalfs = kT * kTK;
 
-__global__ __launch_bounds__(kTThreads) void GemmF16Tile256(const GemmF16Args args)
+// WAVES wavefronts arranged 2 x (WAVES/2): each owns 128 rows and 512/WAVES columns of
+// the tile, i.e. 4 x TJ MFMA tiles with TJ = 16/WAVES.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args args)
 {
-    __shared__ __attribute__((aligned(1024))) _Float16 As[2][kStageHalfs];  // [row][64], swizzled
-    __shared__ __attribute__((aligned(1024))) _Float16 Bs[2][kStageHalfs];  // [k][256], swizzled
+    constexpr int WN = WAVES / 2;          // wavefront columns
+    constexpr int TJ = 8 / WN;             // 32-column MFMA blocks per wavefront
+    constexpr int ROUNDS = 16 / WAVES;     // copies per lane per operand per stage
+    constexpr int WAVE_LDS = ROUNDS * 1024;  // bytes of a stage one wavefront fills
+    constexpr int COPIES_PER_STAGE = 2 * ROUNDS;
+    constexpr uint32_t kBias = 4096;       // keeps every lane offset non-negative
+
+    // A stage: 128 LDS rows of 128 bytes; LDS row R holds A[R][k0..k0+31] in its first 64
+    // bytes and A[R+128][k0..k0+31] in the last 64, 16-byte chunks XOR-swizzled with R%8.
+    // B stage: 32 k-rows of 512 bytes, 32-byte chunks XOR-swizzled with 2*(k%4).
+    __shared__ __attribute__((aligned(1024))) _Float16 As[kTStages][kStageHalfs];
+    __shared__ __attribute__((aligned(1024))) _Float16 Bs[kTStages][kStageHalfs];
 
     uint32_t unit, tm, tn;
     if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
@@ -110,8 +162,8 @@ __global__ __launch_bounds__(kTThreads) void GemmF16Tile256(const GemmF16Args ar
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = tid >> 6;
-    const uint32_t waveM = wave >> 2;  // 0..1 -> 128 rows each
-    const uint32_t waveN = wave & 3;   // 0..3 -> 64 columns each
+    const uint32_t waveM = wave / WN;  // 0..1 -> 128 rows each
+    const uint32_t waveN = wave % WN;
 
     const uint32_t K = args.K, N = args.N;
     const _Float16* __restrict__ A =
@@ -122,129 +174,253 @@ __global__ __launch_bounds__(kTThreads) void GemmF16Tile256(const GemmF16Args ar
                               static_cast<size_t>(tm) * kT * N + static_cast<size_t>(tn) * kT;
 
     // ---- global -> LDS copy plan --------------------------------------------
-    // Each pass moves 8 KiB per operand: wavefront w writes the 1 KiB at
-    // pass*8192 + w*1024, lane i its 16 bytes at + i*16.
-    //   A stage [256 rows][128 B]: that is row pass*64 + w*8 + i/8, physical
-    //     chunk i%8, which must hold logical chunk (i%8) ^ (row%8) = (i%8)^(i/8).
-    //   B stage [64 k][512 B]: k = pass*16 + w*2 + i/32, physical 16-byte chunk
-    //     i%32; 32-byte chunks are swizzled with 2*(k%4).
-    const uint32_t aRow = wave * 8 + (lane >> 3);                  // + pass*64
-    const uint32_t aChunk = (lane & 7) ^ (lane >> 3);              // logical
-    const _Float16* aSrc = A + static_cast<size_t>(aRow) * K + aChunk * 8;
-    const size_t aPassStride = static_cast<size_t>(64) * K;
-
-    const uint32_t bK = wave * 2 + (lane >> 5);                    // + pass*16
-    const uint32_t bPhys16 = lane & 31;
-    const uint32_t bLogical16 = (((bPhys16 >> 1) ^ (2 * (bK & 3))) << 1) | (bPhys16 & 1);
-    const _Float16* bSrc = B + static_cast<size_t>(bK) * N + bLogical16 * 8;
-    const size_t bPassStride = static_cast<size_t>(16) * N;
-
-    auto copyStage = [&](int stage, uint32_t kt) {
-        const _Float16* a = aSrc + static_cast<size_t>(kt) * kTK;
-        const _Float16* b = bSrc + static_cast<size_t>(kt) * kTK * N;
+    // A copy instruction moves 1 KiB per wavefront.  Wavefront w fills the WAVE_LDS bytes
+    // at w*WAVE_LDS of a stage in ROUNDS copies; copy r puts lane i's 16 bytes at
+    // w*WAVE_LDS + r*1024 + i*16.
+    //   A: that is LDS row R = w*8*ROUNDS + r*8 + i/8, physical chunk i%8, which must hold
+    //      logical chunk L = (i%8) ^ (R%8) = (i%8) ^ (i/8): matrix row R (L < 4) or R+128
+    //      (L >= 4), k offset (L%4)*8.
+    //   B: k = w*2*ROUNDS + r*2 + i/32, physical 16-byte chunk i%32, 32-byte chunks
+    //      swizzled with 2*(k%4).
+    // The global address of a copy is a uniform base that advances with the K step plus a
+    // per-lane byte offset that never changes.  The instruction offset r*1024 is added to
+    // both the LDS and the global address, so the lane offsets subtract it again.
+    uint32_t aLane[ROUNDS], bLane[ROUNDS];
+    {
+        const uint32_t aL = (lane & 7) ^ (lane >> 3);
+        const uint32_t aRow0 = wave * (8 * ROUNDS) + (lane >> 3) + ((aL & 4) ? 128u : 0u);
 #pragma unroll
-        for (int pass = 0; pass < 4; ++pass)
-        {
-            __builtin_amdgcn_global_load_lds(
-                a + pass * aPassStride,
-                (LdsPtr)(&As[stage][pass * 4096 + wave * 512]), 16, 0, 0);
-        }
+        for (int r = 0; r < ROUNDS; ++r)
+            aLane[r] = ((aRow0 + 8 * r) * K + (aL & 3) * 8) * 2 + kBias - r * 1024;
+        const uint32_t phys16 = lane & 31;
 #pragma unroll
-        for (int pass = 0; pass < 4; ++pass)
+        for (int r = 0; r < ROUNDS; ++r)
         {
-            __builtin_amdgcn_global_load_lds(
-                b + pass * bPassStride,
-                (LdsPtr)(&Bs[stage][pass * 4096 + wave * 512]), 16, 0, 0);
+            const uint32_t k = wave * (2 * ROUNDS) + r * 2 + (lane >> 5);
+            const uint32_t logical16 = (((phys16 >> 1) ^ (2 * (k & 3))) << 1) | (phys16 & 1);
+            bLane[r] = (k * N + logical16 * 8) * 2 + kBias - r * 1024;
         }
+    }
+    const uint32_t waveU = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t aLds = LdsAddress(&As[0][0]) + waveU * WAVE_LDS;
+    const uint32_t bLds = LdsAddress(&Bs[0][0]) + waveU * WAVE_LDS;
+    const char* aGlobal = reinterpret_cast<const char*>(A) - kBias;
+    const char* bGlobal = reinterpret_cast<const char*>(B) - kBias;
+    const size_t bStepBytes = static_cast<size_t>(kTK) * N * 2;
+
+    // K steps beyond the last are clamped to it: those copies land in buffers that are no
+    // longer read, which keeps the number of copies in flight constant.
+    const uint32_t steps = K / kTK;
+    auto copyA = [&](uint32_t kt, int stage, auto round) {
+        constexpr int r = decltype(round)::value;
+        const uint32_t src = min(kt, steps - 1);
+        DmaToLds16<r * 1024>(aLane[r], aGlobal + static_cast<size_t>(src) * (kTK * 2),
+                             aLds + stage * kStageBytes);
+    };
+    auto copyB = [&](uint32_t kt, int stage, auto round) {
+        constexpr int r = decltype(round)::value;
+        const uint32_t src = min(kt, steps - 1);
+        DmaToLds16<r * 1024>(bLane[r], bGlobal + static_cast<size_t>(src) * bStepBytes,
+                             bLds + stage * kStageBytes);
     };
 
     // ---- LDS -> fragment read plan ------------------------------------------
-    // A fragment (MFMA tile row block i, k sub-step ks): lane l reads row
-    //   waveM*128 + i*32 + l%32, logical chunk ks*2 + l/32.
+    // A fragment (row block i, k sub-step ks): lane l reads matrix row
+    //   waveM*128 + i*32 + l%32 = half waveM of LDS row R = i*32 + l%32,
+    //   logical chunk waveM*4 + ks*2 + l/32.
     const uint32_t l32 = lane & 31;
     const uint32_t khalf = lane >> 5;
-    const uint32_t aFragRow = waveM * 128 + l32;  // + i*32 (row%8 unchanged)
-    const uint32_t aRowSwz = aFragRow & 7;
-    // B fragment (tile column block j, sub-step ks): 16-lane group g = l/16,
-    //   s = l%16; columns waveN*64 + j*32 + 16*(g%2) + 4*(s%4)..+3,
+    const uint32_t aSwz = l32 & 7;
+    const uint32_t aChunkBase = waveM * 4 + khalf;  // + ks*2
+    // B fragment (column block j, sub-step ks): 16-lane group g = l/16, s = l%16;
+    //   columns waveN*(32*TJ) + j*32 + 16*(g%2) + 4*(s%4)..+3,
     //   k = ks*16 + 8*(g/2) + 4*h + s/4 for the two reads h = 0, 1.
     const uint32_t g = lane >> 4;
     const uint32_t s = lane & 15;
-    const uint32_t bKLocal = 8 * (g >> 1) + (s >> 2);               // + ks*16 + 4*h
-    const uint32_t bCol32 = (waveN * 64 + 16 * (g & 1)) / 16;       // + j*2, logical 32B chunk
-    const uint32_t bSwz = 2 * ((s >> 2) & 3);                       // 2*(k%4)
-    const uint32_t bInChunk = (s & 3) * 4;                          // halves inside the 32B chunk
+    const uint32_t bKLocal = 8 * (g >> 1) + (s >> 2);          // + ks*16 + 4*h
+    const uint32_t bCol32 = waveN * (2 * TJ) + (g & 1);         // + j*2, logical 32-byte chunk
+    const uint32_t bSwz = 2 * ((s >> 2) & 3);                   // 2*(k%4)
+    const uint32_t bInChunk = (s & 3) * 4;                      // halves inside the chunk
 
-    floatx16 acc[4][2];
+    // element offsets inside a stage, fixed for the whole kernel
+    uint32_t aOff[2], bOff[2][TJ];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+    {
+        aOff[ks] = l32 * 64 + (((aChunkBase + ks * 2) ^ aSwz) * 8);  // + i*32*64
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+            bOff[ks][j] =
+                (ks * 16 + bKLocal) * kT + (((bCol32 + j * 2) ^ bSwz) * 16) + bInChunk;
+    }
+
+    auto loadA = [&](int stage, int ks, int i) {
+        return *reinterpret_cast<const halfx8*>(&As[stage][aOff[ks] + i * 32 * 64]);
+    };
+    auto loadB = [&](int stage, int ks, int j) {
+        const _Float16* p = &Bs[stage][bOff[ks][j]];
+        return Join(LdsReadTr(p), LdsReadTr(p + 4 * kT));
+    };
+
+    floatx16 acc[4][TJ];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TJ; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v)
                 acc[i][j][v] = 0.f;
 
-    const uint32_t steps = K / kTK;
-    copyStage(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // ---- pipeline ---------------------------------------------------------------
+    // LDS holds four K steps.  While step kt is multiplied, the B copies of step kt+3
+    // and the A copies of step kt+4 are issued, spread between the MFMAs so that the
+    // memory pipe sees a steady stream; a copy has three steps to land.  Copies
+    // complete in issue order and exactly 2*COPIES_PER_STAGE are issued between the
+    // last copy of step kt+1 and the synchronisation point of step kt, so
+    // vmcnt <= 2*COPIES_PER_STAGE there means step kt+1 is in LDS.  The barrier sits
+    // in the middle of a step: the MFMAs of the second half need no LDS access of
+    // their own and cover the latency of the first fragment reads of the next step.
+    // The loop body is written out for the four stages so that every LDS address is a
+    // register plus an immediate; sched_barrier fences pin the interleaving of MFMAs,
+    // LDS reads and copies written here (a few non-MFMA instructions after each MFMA).
+#define SPH_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+    // One half step: the 4*TJ MFMAs of fragments (AF, BF), with the reads that fill
+    // (AFN, BFN) from stage `stageN`, sub-step `ksN`, and one operand's copies of K step
+    // ktCopy into stage `stageCopy` slotted between them.
+    auto halfStep = [&](const halfx8 (&AF)[4], const halfx8 (&BF)[TJ], halfx8 (&AFN)[4],
+                        halfx8 (&BFN)[TJ], int stageN, int ksN, uint32_t ktCopy, int stageCopy,
+                        bool copyIsA) {
+        auto copy = [&](auto round) {
+            if (SPH_ABLATE & 1)
+                return;
+            if (copyIsA)
+                copyA(ktCopy, stageCopy, round);
+            else
+                copyB(ktCopy, stageCopy, round);
+        };
+        auto group = [&](auto iC) {
+            constexpr int i = decltype(iC)::value;
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+            {
+                if (!(SPH_ABLATE & 2))
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(BF[j], AF[i], acc[i][j],
+                                                                       0, 0, 0);
+                SPH_FENCE();
+                if (!(SPH_ABLATE & 4))
+                {
+                    if (j == 0)
+                        AFN[i] = loadA(stageN, ksN, i);
+                    if constexpr (i < TJ)
+                    {
+                        if (j == 1)
+                            BFN[i] = loadB(stageN, ksN, i);
+                    }
+                }
+                SPH_FENCE();
+            }
+            // copies of this group: rounds [i*ROUNDS/4, (i+1)*ROUNDS/4)
+            if constexpr (ROUNDS == 4)
+                copy(std::integral_constant<int, i>{});
+            else if constexpr (i == 1)
+                copy(std::integral_constant<int, 0>{});
+            else if constexpr (i == 3)
+                copy(std::integral_constant<int, 1>{});
+            SPH_FENCE();
+        };
+        group(std::integral_constant<int, 0>{});
+        group(std::integral_constant<int, 1>{});
+        group(std::integral_constant<int, 2>{});
+        group(std::integral_constant<int, 3>{});
+    };
+
+    auto copyAllA = [&](uint32_t kt, int stage) {
+        copyA(kt, stage, std::integral_constant<int, 0>{});
+        copyA(kt, stage, std::integral_constant<int, 1>{});
+        if constexpr (ROUNDS == 4)
+        {
+            copyA(kt, stage, std::integral_constant<int, 2>{});
+            copyA(kt, stage, std::integral_constant<int, 3>{});
+        }
+    };
+    auto copyAllB = [&](uint32_t kt, int stage) {
+        copyB(kt, stage, std::integral_constant<int, 0>{});
+        copyB(kt, stage, std::integral_constant<int, 1>{});
+        if constexpr (ROUNDS == 4)
+        {
+            copyB(kt, stage, std::integral_constant<int, 2>{});
+            copyB(kt, stage, std::integral_constant<int, 3>{});
+        }
+    };
+
+#pragma unroll
+    for (int st = 0; st < 3; ++st)
+    {
+        copyAllA(st, st);
+        copyAllB(st, st);
+    }
+    copyAllA(3, 3);
+    // stage 0 is followed by 2.5 stages' worth of copies
+    WaitVmem<(5 * COPIES_PER_STAGE) / 2>();
     __syncthreads();
 
-    for (uint32_t kt = 0; kt < steps; ++kt)
-    {
-        const int cur = kt & 1;
-        if (kt + 1 < steps)
-            copyStage(cur ^ 1, kt + 1);
+    halfx8 af0[4], bf0[TJ], af1[4], bf1[TJ];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        af0[i] = loadA(0, 0, i);
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+        bf0[j] = loadB(0, 0, j);
 
-        const _Float16* as = As[cur];
-        const _Float16* bs = Bs[cur];
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-        {
-            halfx8 af[4];
-            halfx8 bf[2];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-            {
-                const uint32_t chunk = (ks * 2 + khalf) ^ aRowSwz;
-                af[i] = *reinterpret_cast<const halfx8*>(as + (aFragRow + i * 32) * kTK +
-                                                         chunk * 8);
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-            {
-                const uint32_t chunk32 = (bCol32 + j * 2) ^ bSwz;
-                const _Float16* p = bs + (ks * 16 + bKLocal) * kT + chunk32 * 16 + bInChunk;
-                const halfx4 lo = LdsReadTr(p);
-                const halfx4 hi = LdsReadTr(p + 4 * kT);
-                bf[j] = Join(lo, hi);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j],
-                                                                       0, 0, 0);
-        }
-
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // one K step with its stage index known at compile time
+    auto step = [&](auto stageC, uint32_t kt) {
+        constexpr int cur = decltype(stageC)::value;
+        constexpr int nxt = (cur + 1) % kTStages;
+        // first half: multiply sub-step 0, fetch sub-step 1, request B of step kt+3
+        halfStep(af0, bf0, af1, bf1, cur, 1, kt + 3, (cur + 3) % kTStages, false);
+        // step kt+1 has landed for every wavefront, and every wavefront is done reading
+        // step kt, whose buffer now takes step kt+4
+        WaitVmem<(SPH_ABLATE & 1) ? 0 : 2 * COPIES_PER_STAGE>();
         __syncthreads();
+        // second half: multiply sub-step 1, fetch sub-step 0 of step kt+1, request A of kt+4
+        halfStep(af1, bf1, af0, bf0, nxt, 0, kt + 4, cur, true);
+    };
+
+    for (uint32_t kt = 0;; kt += 4)
+    {
+        step(std::integral_constant<int, 0>{}, kt);
+        if (kt + 1 >= steps)
+            break;
+        step(std::integral_constant<int, 1>{}, kt + 1);
+        if (kt + 2 >= steps)
+            break;
+        step(std::integral_constant<int, 2>{}, kt + 2);
+        if (kt + 3 >= steps)
+            break;
+        step(std::integral_constant<int, 3>{}, kt + 3);
+        if (kt + 4 >= steps)
+            break;
     }
+#undef SPH_FENCE
 
     // ---- epilogue -------------------------------------------------------------
     // With the operands swapped the 32x32 result block is indexed [n][m]:
     // register v of lane l holds column 8*(v/4) + 4*(l/32) + v%4 of row l%32,
     // i.e. registers 4q..4q+3 are 4 consecutive columns.
+    if ((SPH_ABLATE & 8) && args.M != 1)
+        return;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
     {
         const uint32_t r = waveM * 128 + i * 32 + l32;
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TJ; ++j)
         {
 #pragma unroll
             for (int q = 0; q < 4; ++q)
             {
-                const uint32_t c = waveN * 64 + j * 32 + 8 * q + 4 * khalf;
+                const uint32_t c = waveN * (32 * TJ) + j * 32 + 8 * q + 4 * khalf;
                 float4* p = reinterpret_cast<float4*>(out + static_cast<size_t>(r) * N + c);
                 float4 v = make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
                                        acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
@@ -509,6 +685,12 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.strideA = strideA;
     args.strideB = strideB;
     args.overwrite = (flags & SPH_GEMM_OVERWRITE) ? 1u : 0u;
+#if SPH_ABLATE & 16
+    {
+        const char* t = getenv("SPH_TRACE_PTR");
+        args.trace = t ? reinterpret_cast<long long*>(strtoull(t, nullptr, 0)) : nullptr;
+    }
+#endif
 
     const bool aligned16 =
         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
@@ -526,7 +708,7 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
 
     if (tile256)
     {
-        hipLaunchKernelGGL(GemmF16Tile256, dim3(grid), dim3(kTThreads), 0, stream, args);
+        hipLaunchKernelGGL(GemmF16Tile256<8>, dim3(grid), dim3(512), 0, stream, args);
     }
     else
     {

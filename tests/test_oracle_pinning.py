@@ -1,0 +1,260 @@
+"""Pins the CPU checker before anything is compared against it.
+
+Three independent anchors:
+  1. the reference's own objects (oracle/_ref, built from the reference's NaiveGemm.cpp,
+     NaiveBasic.cpp, shape.cpp and Broadcast.hpp where they lie) -- bit for bit, when built;
+  2. fixtures recorded from those objects (tests/golden/*.json, *.npz) -- always;
+  3. what the arithmetic fixes on its own: identity / ones / K = 1 closed forms, a float64
+     brute force bound, an order-sensitivity probe that a reordered or fused sum fails.
+"""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from sapphire_amd import synth
+from tests.golden.cases import KAT_GEMM_CASES, KAT_OP_CASES, PLAN_CASES, SHAPE_CASES
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+needs_ref = pytest.mark.skipif(not po.have_ref(), reason="oracle/_ref not built on this machine")
+
+
+def bits(x):
+    return np.ascontiguousarray(x).view(np.uint32)
+
+
+# ---- shapes ---------------------------------------------------------------------------------
+
+def test_shape_ops_match_recorded_reference_answers():
+    o = po.oracle()
+    for entry in json.load(open(os.path.join(GOLDEN, "shape_ops.json"))):
+        dims = entry["dims"]
+        s = po.make_shape(dims)
+        assert o.orc_shape_rows(ctypes.byref(s)) == entry["rows"]
+        assert o.orc_shape_cols(ctypes.byref(s)) == entry["cols"]
+        assert o.orc_shape_size(ctypes.byref(s)) == entry["size"]
+        assert [o.orc_shape_num_units(ctypes.byref(s), k) for k in range(5)] == entry["units"]
+        for k, want in enumerate(entry["expand"]):
+            t = po.make_shape(dims)
+            assert o.orc_shape_expand(ctypes.byref(t), k) == 0
+            assert po.shape_list(t) == want
+        for k, want in zip(range(1, 7), entry["shrink"]):
+            t = po.make_shape(dims)
+            assert o.orc_shape_shrink(ctypes.byref(t), k) == 0
+            assert po.shape_list(t) == want
+
+
+def test_shape_hand_table():
+    o = po.oracle()
+    s = po.make_shape([5])
+    o.orc_shape_expand(ctypes.byref(s), 2)
+    assert po.shape_list(s) == [1, 5]                     # 1-D [n] -> [1, n]
+    s = po.make_shape([2, 3, 4, 5])
+    o.orc_shape_shrink(ctypes.byref(s), 2)
+    assert po.shape_list(s) == [24, 5]                    # Linear's 2-D view of x
+    assert o.orc_shape_num_units(ctypes.byref(po.make_shape([2, 3, 4, 5])), 1) == 24
+    assert o.orc_shape_num_units(ctypes.byref(po.make_shape([4, 5])), 2) == 1   # the dead fast path
+
+
+# ---- broadcast walk -------------------------------------------------------------------------
+
+def test_plans_match_recorded_reference_walks():
+    recorded = json.load(open(os.path.join(GOLDEN, "gemm_plans.json")))
+    assert len(recorded) == len(PLAN_CASES)
+    for rec in recorded:
+        dims, leaves = po.gemm_plan(rec["y"], rec["a"], rec["b"])
+        assert dims == rec["dims"], rec
+        assert [list(l) for l in leaves] == rec["leaves"], rec
+
+
+def test_modulo_offset_rule_six_leaf_fixture():
+    """{2,1,3,2} x {2,3,2,2} -> {2,3,3,2}: A matrix index is i % 2, not i // 3."""
+    _, leaves = po.gemm_plan([2, 3, 3, 2], [2, 1, 3, 2], [2, 3, 2, 2])
+    assert [(o // 6, a // 6, b // 4) for o, a, b, _ in leaves] == \
+        [(0, 0, 0), (1, 1, 1), (2, 0, 2), (3, 1, 3), (4, 0, 4), (5, 1, 5)]
+
+
+def test_worked_examples():
+    d, leaves = po.gemm_plan([256, 256], [256, 256], [256, 256])
+    assert (d["M"], d["N"], d["K"]) == (256, 256, 256) and len(leaves) == 1
+    d, leaves = po.gemm_plan([16, 512, 512], [16, 512, 512], [1, 512, 512])
+    assert len(leaves) == 16 and all(b == 0 for _, _, b, _ in leaves)
+    assert [o for o, _, _, _ in leaves] == [i * 512 * 512 for i in range(16)]
+    d, leaves = po.gemm_plan([7, 5, 3], [7, 5, 4], [7, 4, 3])
+    assert leaves == [(0, 0, 0, 105)]                     # one strided-batched leaf, batch 7
+    d, leaves = po.gemm_plan([1024, 1024], [1024, 1], [1, 1024])
+    assert (d["M"], d["N"], d["K"]) == (1024, 1024, 1)    # Linear's bias step
+
+
+@needs_ref
+def test_plans_match_reference_on_random_shapes():
+    rng = synth.bits64(0xABCD, 4000)
+    pos = 0
+    for case in range(300):
+        nd = int(rng[pos] % 4) + 2
+        pos += 1
+        M, N, K = (int(rng[pos + i] % 5) + 1 for i in range(3))
+        pos += 3
+        lead = [int(rng[pos + i] % 3) + 1 for i in range(nd - 2)]
+        pos += nd - 2
+        ys = lead + [M, N]
+        # operands keep, drop to 1, or lose leading dims
+        def variant(tail):
+            nonlocal pos
+            keep = [(d if rng[pos + i] % 3 else 1) for i, d in enumerate(lead)]
+            pos += len(lead)
+            cut = int(rng[pos] % (len(keep) + 1))
+            pos += 1
+            return keep[cut:] + tail
+        as_ = variant([M, K])
+        bs = variant([K, N])
+        got = po.gemm_plan(ys, as_, bs)
+        want = po.gemm_plan(ys, as_, bs, lib="ref")
+        assert got == want, (ys, as_, bs)
+
+
+# ---- dense leaf -----------------------------------------------------------------------------
+
+def test_leaf_and_operator_match_recorded_reference_outputs():
+    kat = np.load(os.path.join(GOLDEN, "naive_gemm_kat.npz"))
+    for name, batch, M, N, K, seed in KAT_GEMM_CASES:
+        A = synth.uniform(seed + 1, (batch, M, K))
+        B = synth.uniform(seed + 2, (batch, K, N))
+        C = synth.uniform(seed + 3, (batch, M, N))
+        want = kat["leaf_" + name]
+        assert np.array_equal(bits(po.naive_gemm(C.copy(), A, B, M, N, K)), bits(want)), name
+        assert np.array_equal(bits(po.gemm_rows(C.copy(), A, B, M, N, K, batch=batch, threads=3)),
+                              bits(want)), name
+    for name, ys, as_, bs, seed in KAT_OP_CASES:
+        A = synth.uniform(seed + 1, as_)
+        B = synth.uniform(seed + 2, bs)
+        C = synth.uniform(seed + 3, ys)
+        want = kat["op_" + name]
+        assert np.array_equal(bits(po.compute_gemm(C.copy(), A, B)), bits(want)), name
+        assert np.array_equal(bits(po.compute_gemm(C.copy(), A, B, threads=4)), bits(want)), name
+    x = synth.uniform(900, (1000,))
+    assert np.array_equal(bits(po.relu(x)), bits(kat["relu"]))
+    t = synth.uniform(901, (3, 5, 7))
+    assert np.array_equal(bits(po.transpose(t, 5, 7, 3)), bits(kat["transpose"]))
+
+
+@needs_ref
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (2, 3, 5, 7), (4, 33, 17, 65), (1, 128, 96, 200)])
+def test_leaf_bit_exact_against_reference_object(shape):
+    batch, M, N, K = shape
+    A = synth.normal(1, (batch, M, K), 5.0) + 10
+    B = synth.normal(2, (batch, K, N), 5.0) + 10
+    C = synth.uniform(3, (batch, M, N))
+    want = C.copy()
+    po.ref().ref_naive_gemm(want.size, po._f(want), po._f(A), po._f(B), M, N, K)
+    assert np.array_equal(bits(po.naive_gemm(C.copy(), A, B, M, N, K)), bits(want))
+    assert np.array_equal(bits(po.gemm_rows(C.copy(), A, B, M, N, K, batch=batch, threads=5)),
+                          bits(want))
+
+
+def test_leaf_closed_forms():
+    n = 37
+    B = synth.uniform(5, (n, n))
+    C = synth.uniform(6, (n, n))
+    eye = np.eye(n, dtype=np.float32)
+    assert np.array_equal(po.naive_gemm(C.copy(), eye, B, n, n, n), C + B)
+    ones = np.ones((n, n), np.float32)
+    assert np.array_equal(po.naive_gemm(np.zeros((n, n), np.float32), ones, ones, n, n, n),
+                          np.full((n, n), float(n), np.float32))
+    col = np.ones((n, 1), np.float32)
+    bias = synth.uniform(7, (1, n))
+    assert np.array_equal(po.naive_gemm(np.zeros((n, n), np.float32), col, bias, n, n, 1),
+                          np.broadcast_to(bias, (n, n)))
+    # transposed operands would fail this: A is not symmetric
+    A = synth.uniform(8, (3, 4))
+    Bm = synth.uniform(9, (4, 2))
+    want = (A.astype(np.float64) @ Bm.astype(np.float64))
+    got = po.naive_gemm(np.zeros((3, 2), np.float32), A, Bm, 3, 2, 4)
+    assert np.max(np.abs(got - want)) < 1e-6
+
+
+def test_leaf_rounding_order_is_k_ascending_unfused():
+    """Catastrophic-cancellation probe: 1e8 + 1 - 1e8 summed left to right in fp32 is 0, any
+    other order or a fused multiply-add gives something else."""
+    A = np.array([[1e8, 1.0, -1e8]], np.float32)
+    B = np.array([[1.0], [1.0], [1.0]], np.float32)
+    assert po.naive_gemm(np.zeros((1, 1), np.float32), A, B, 1, 1, 3)[0, 0] == 0.0
+    A = np.array([[1.0, 1e8, -1e8]], np.float32)
+    assert po.naive_gemm(np.zeros((1, 1), np.float32), A, B, 1, 1, 3)[0, 0] == 0.0
+    A = np.array([[1e8, -1e8, 1.0]], np.float32)
+    assert po.naive_gemm(np.zeros((1, 1), np.float32), A, B, 1, 1, 3)[0, 0] == 1.0
+    # separate rounding of the product: (1+2^-12)^2 rounds to 1+2^-11 in fp32 before the add
+    a = np.float32(1 + 2.0 ** -12)
+    A = np.array([[a, -1.0]], np.float32)
+    B = np.array([[a], [np.float32(1 + 2.0 ** -11)]], np.float32)
+    assert po.naive_gemm(np.zeros((1, 1), np.float32), A, B, 1, 1, 2)[0, 0] == 0.0
+    # the local sum starts at 0 and is added to out once: out + (a + b), not (out + a) + b
+    A = np.array([[1.0, 1.0]], np.float32)
+    B = np.array([[2.0 ** -24], [2.0 ** -24]], np.float32)
+    out = np.ones((1, 1), np.float32)
+    assert po.naive_gemm(out, A, B, 1, 1, 2)[0, 0] == np.float32(1 + 2.0 ** -23)
+
+
+def test_leaf_float64_brute_force_bound():
+    M, N, K = 9, 8, 300
+    A = synth.uniform(11, (M, K))
+    B = synth.uniform(12, (K, N))
+    want = np.zeros((M, N))
+    for m in range(M):
+        for n in range(N):
+            want[m, n] = sum(float(A[m, k]) * float(B[k, n]) for k in range(K))
+    got = po.naive_gemm(np.zeros((M, N), np.float32), A, B, M, N, K)
+    bound = K * 2.0 ** -24 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert np.all(np.abs(got - want) <= bound)
+
+
+def test_batch_independence_and_padding_invariance():
+    A = synth.uniform(13, (3, 5, 6))
+    B = synth.uniform(14, (3, 6, 4))
+    whole = po.naive_gemm(np.zeros((3, 5, 4), np.float32), A, B, 5, 4, 6)
+    for b in range(3):
+        one = po.naive_gemm(np.zeros((5, 4), np.float32), A[b].copy(), B[b].copy(), 5, 4, 6)
+        assert np.array_equal(bits(one), bits(whole[b]))
+    # zero K-columns appended to A (and rows to B) change nothing
+    Ap = np.concatenate([A[0], np.zeros((5, 3), np.float32)], axis=1)
+    Bp = np.concatenate([B[0], synth.uniform(15, (3, 4))], axis=0)
+    padded = po.naive_gemm(np.zeros((5, 4), np.float32), Ap, Bp, 5, 4, 9)
+    assert np.array_equal(bits(padded), bits(whole[0]))
+
+
+# ---- Linear and CSR -------------------------------------------------------------------------
+
+def test_linear_forward_is_bias_plus_product():
+    x = synth.uniform(21, (6, 5), 0.0, 1.0)
+    W = synth.uniform(22, (5, 4))
+    b = synth.uniform(23, (4,))
+    y = po.linear_forward(x, W, b)
+    want = np.broadcast_to(b, (6, 4)).copy()
+    po.naive_gemm(want, x, W, 6, 4, 5)
+    assert np.array_equal(bits(y), bits(want))
+    eye = np.eye(5, dtype=np.float32)
+    assert np.array_equal(po.linear_forward(x, eye, np.zeros(5, np.float32)), x)
+
+
+def test_csr_equals_dense_leaf_on_densified_matrix():
+    for seed, (M, K, N) in enumerate([(1, 1, 1), (7, 9, 5), (40, 300, 33), (64, 2048, 16)]):
+        forced = {0: 0} if M > 1 else None
+        v, col, row = synth.csr_matrix(50 + seed, M, K, min(K, 12.0), forced=forced)
+        B = synth.uniform(60 + seed, (K, N))
+        C = synth.uniform(70 + seed, (M, N))
+        dense = synth.densify(v, col, row, M, K)
+        want = po.naive_gemm(C.copy(), dense, B, M, N, K)
+        assert np.array_equal(bits(po.spmm_csr(C.copy(), v, col, row, M, N, B)), bits(want))
+        assert np.array_equal(bits(po.spmm_csr(C.copy(), v, col, row, M, N, B, threads=3)), bits(want))
+
+
+def test_csr_brute_force_tiny():
+    V = np.array([2.0, -1.0, 0.5, 4.0], np.float32)
+    COL = np.array([0, 2, 1, 2], np.uint32)
+    ROW = np.array([0, 2, 2, 3, 4], np.uint32)      # row 1 empty, row 3 hits the last column
+    B = np.array([[1, 2], [3, 4], [5, 6]], np.float32)
+    out = po.spmm_csr(np.zeros((4, 2), np.float32), V, COL, ROW, 4, 2, B)
+    assert out.tolist() == [[2 * 1 - 5, 2 * 2 - 6], [0, 0], [1.5, 2.0], [20, 24]]
