@@ -44,7 +44,7 @@ def parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     p.add_argument("--all", action="store_true",
                    help="also time configurations 1, 2 and 4 (reported under 'others')")
-    p.add_argument("--only", choices=["gemm", "spmm"], default=None,
+    p.add_argument("--only", choices=["gemm", "spmm", "copy"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
     return p.parse_args()
 
@@ -116,6 +116,22 @@ def bench_f32(capi, A, B, C, M, N, K, batch, sb, steps, warmup):
     for b in (dA, dB, dC):
         b.release()
     return event_ms
+
+
+def bench_copy(capi, steps, warmup, mib=64):
+    """A plain one-pass kernel of known size (ReLU over `mib` MiB: reads it once, writes it
+    once), used to calibrate the profiler's FETCH_SIZE / WRITE_SIZE counters."""
+    n = mib * (1 << 20) // 4
+    src = capi.DeviceBuffer.from_array(np.ones(n, np.float32))
+    dst = capi.DeviceBuffer(4 * n)
+
+    def launch():
+        capi.call("sph_relu_f32", dst.ptr, src.ptr, n)
+
+    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    src.release()
+    dst.release()
+    return event_ms, 4 * n
 
 
 def cpu_gemm_baseline(d, rows=96):
@@ -196,6 +212,11 @@ def main():
             result["gemm_overwrite_variant"] = {
                 "note": "same launch with SPH_GEMM_OVERWRITE (out is not read)",
                 "launch_ms": ev_over, "tflops": flops / (ev_over * 1e-3) / 1e12}
+
+    if args.only == "copy":
+        ms, nbytes = bench_copy(capi, args.steps, args.warmup)
+        result["copy"] = {"kernel": "ReluKernel", "bytes_read": nbytes, "bytes_written": nbytes,
+                          "launch_ms": ms, "gbs": 2 * nbytes / (ms * 1e-3) / 1e9}
 
     if args.only in (None, "spmm"):
         sp_steps = max(args.steps * 4, 100)

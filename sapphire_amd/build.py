@@ -6,6 +6,7 @@
 Outputs (git-ignored, next to the package so that they travel with the tree):
     sapphire_amd/libsapphire_hip.so    C ABI of include/sapphire_hip.h
     sapphire_amd/libsapphire_host.so   C++ operator layer (Sapphire:: namespace)
+    tests/host_harness/libhost_harness.so   C view of that layer for the Python tests
 """
 import concurrent.futures
 import os
@@ -89,6 +90,20 @@ def build_host():
     return HOST_LIB
 
 
+HARNESS_DIR = os.path.join(ROOT, "tests", "host_harness")
+HARNESS_LIB = os.path.join(HARNESS_DIR, "libhost_harness.so")
+
+
+def build_harness():
+    """C entry points over the C++ layer for the Python parity tests."""
+    flags = ["-O2", "-std=c++17", "-fPIC", "-x", "c++",
+             "-I" + os.path.join(ROOT, "include"), "-I" + HOST]
+    objs = _compile_all(_sources(HARNESS_DIR, {".cpp"}), flags, "harness")
+    _run([_hipcc(), "-shared", "-fPIC", "-o", HARNESS_LIB] + objs +
+         ["-L" + PKG, "-lsapphire_host", "-lsapphire_hip", "-Wl,-rpath,$ORIGIN/../../sapphire_amd"])
+    return HARNESS_LIB
+
+
 def build_oracle():
     """The CPU checker (test infrastructure): oracle/liboracle.so and, when the
     reference tree is present, oracle/_ref/libsapphire_ref.so."""
@@ -97,14 +112,14 @@ def build_oracle():
 
 def build_all():
     build_hip()
-    if os.path.isdir(HOST) and _sources(HOST, {".cpp"}):
-        build_host()
+    build_host()
+    build_harness()
     build_oracle()
 
 
 if __name__ == "__main__":
     parts = sys.argv[1:] or ["all"]
     for part in parts:
-        {"hip": build_hip, "host": build_host, "oracle": build_oracle,
-         "all": build_all}[part]()
+        {"hip": build_hip, "host": build_host, "harness": build_harness,
+         "oracle": build_oracle, "all": build_all}[part]()
         print("built", part)

@@ -1,0 +1,95 @@
+#include <Sapphire/compute/BasicOps.hpp>
+
+#include <Sapphire/compute/BroadcastPlan.hpp>
+#include <Sapphire/compute/dense/cuda/Gemm.hpp>
+
+#include <stdexcept>
+#include <string>
+
+namespace Sapphire::Compute
+{
+namespace
+{
+void RequireSameMode(const TensorData& y, const TensorData& x, const char* op)
+{
+    if (y.Mode() != x.Mode())
+        throw std::invalid_argument(std::string("Compute::") + op + " - Device mode inequality");
+}
+
+void RequireDeviceMode(const TensorData& y, const char* op)
+{
+    if (y.Mode() != ComputeMode::Cuda)
+        throw std::runtime_error(std::string("Compute::") + op +
+                                 " - Host mode is not provided by the device backend");
+}
+}  // namespace
+
+void Gemm(TensorData& y, const TensorData& a, const TensorData& b)
+{
+    RequireSameMode(y, a, "Gemm");
+    RequireSameMode(y, b, "Gemm");
+    RequireDeviceMode(y, "Gemm");
+
+    const GemmPlan plan = PlanGemm(y.GetShape(), a.GetShape(), b.GetShape());
+    const int deviceId = y.GetCudaDevice().GetID();
+    float* out = y.CudaMutableRawPtr();
+    const float* A = a.CudaRawPtr();
+    const float* B = b.CudaRawPtr();
+
+    // the whole walk as one strided-batched launch when its offsets are affine (all the
+    // common cases: no batch, equal batches, one operand shared by the batch) ...
+    std::uint32_t count = 0;
+    std::int64_t strideOut = 0, strideA = 0, strideB = 0;
+    if (AsStridedBatch(plan, count, strideOut, strideA, strideB))
+    {
+        if (strideOut == static_cast<std::int64_t>(plan.M) * plan.N &&
+            strideA == static_cast<std::int64_t>(plan.M) * plan.K &&
+            strideB == static_cast<std::int64_t>(plan.K) * plan.N)
+        {
+            Dense::Cuda::Gemm(count * plan.M * plan.N, out, A, B, plan.M, plan.N, plan.K, deviceId);
+            return;
+        }
+        if ((strideA == 0 || strideA == static_cast<std::int64_t>(plan.M) * plan.K) &&
+            (strideB == 0 || strideB == static_cast<std::int64_t>(plan.K) * plan.N) &&
+            strideOut == static_cast<std::int64_t>(plan.M) * plan.N)
+        {
+            Dense::Cuda::GemmMatrixWiseBroadcast(out, A, B, plan.M, plan.N, plan.K, count,
+                                                 strideA == 0, strideB == 0, deviceId);
+            return;
+        }
+    }
+
+    // ... otherwise as one grouped launch over the list of unit products
+    const std::uint64_t mn = static_cast<std::uint64_t>(plan.M) * plan.N;
+    const std::uint64_t mk = static_cast<std::uint64_t>(plan.M) * plan.K;
+    const std::uint64_t kn = static_cast<std::uint64_t>(plan.K) * plan.N;
+    std::vector<Dense::Cuda::GemmUnit> units;
+    for (const BroadcastLeaf& leaf : plan.leaves)
+    {
+        const std::uint64_t run = mn ? leaf.totalSizeOut / mn : 0;
+        for (std::uint64_t u = 0; u < run; ++u)
+            units.push_back({ leaf.outOff + u * mn, leaf.aOff + u * mk, leaf.bOff + u * kn });
+    }
+    Dense::Cuda::GemmGrouped(units, out, A, B, plan.M, plan.N, plan.K, deviceId);
+}
+
+void Transpose(TensorData& y, const TensorData& x)
+{
+    RequireSameMode(y, x, "Transpose");
+    RequireDeviceMode(y, "Transpose");
+    const int rows = x.Rows();
+    const int cols = x.Cols();
+    const bool broadcast = x.GetNumUnits(2) == 1;
+    const int matrices = y.GetShape().Size() / (rows * cols);
+    Dense::Cuda::Transpose(y.CudaMutableRawPtr(), x.CudaRawPtr(), static_cast<unsigned int>(rows),
+                           static_cast<unsigned int>(cols), static_cast<unsigned int>(matrices),
+                           broadcast);
+}
+
+void ReLU(TensorData& y, const TensorData& x)
+{
+    RequireSameMode(y, x, "ReLU");
+    RequireDeviceMode(y, "ReLU");
+    Dense::Cuda::ReLU(y.CudaMutableRawPtr(), x.CudaRawPtr(), static_cast<unsigned int>(y.Size()));
+}
+}  // namespace Sapphire::Compute

@@ -1,0 +1,29 @@
+// Operator-level entry points on TensorData, with the reference's signatures
+// (Includes/Sapphire/compute/BasicOps.hpp:16-31, Includes/Sapphire/compute/ActivationOps.hpp).
+//
+// Only the device branch lives here.  The reference's Host branch (its scalar CPU loops)
+// stays where it is in the reference; calling these with tensors in ComputeMode::Host throws
+// std::runtime_error, there is no CPU fallback in this library.
+#ifndef SAPPHIRE_AMD_COMPUTE_BASICOPS_HPP
+#define SAPPHIRE_AMD_COMPUTE_BASICOPS_HPP
+
+#include <Sapphire/tensor/TensorData.hpp>
+
+namespace Sapphire::Compute
+{
+using TensorUtil::TensorData;
+
+//! y += a * b over the trailing two dimensions, leading dimensions broadcast by the walk of
+//! BroadcastWith2Inputs.  No shape validation, as documented for the reference
+//! (Includes/Sapphire/compute/BasicOps.hpp:16-19).  All three must be in the same mode.
+void Gemm(TensorData& y, const TensorData& a, const TensorData& b);
+
+//! y = transpose of the trailing two dimensions of x; a 2-D x is repeated for every matrix
+//! of y (Sources/Sapphire/compute/BasicOps.cpp:269-290).
+void Transpose(TensorData& y, const TensorData& x);
+
+//! y = x > 0 ? x : 0 (Sources/Sapphire/compute/ActivationOps.cpp:52-67).
+void ReLU(TensorData& y, const TensorData& x);
+}  // namespace Sapphire::Compute
+
+#endif

@@ -1,0 +1,52 @@
+// Device leaves of the dense matrix product, with the reference's signatures
+// (Includes/Sapphire/compute/dense/cuda/Gemm.cuh:15-25).  Where the reference calls
+// cublasGemmStridedBatchedEx (Sources/Sapphire/compute/dense/cuda/Gemm.cu:19-85) these
+// forward to the MFMA kernels behind the C ABI.  A failing call throws std::runtime_error.
+#ifndef SAPPHIRE_AMD_COMPUTE_DENSE_CUDA_GEMM_HPP
+#define SAPPHIRE_AMD_COMPUTE_DENSE_CUDA_GEMM_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <vector>
+
+namespace Sapphire::Compute::Dense::Cuda
+{
+//! out[c] += A[c] * B[c] for c < totalSize / (M*N); matrices packed back to back.
+void Gemm(unsigned int totalSize, float* out, const float* A, const float* B, unsigned int M,
+          unsigned int N, unsigned int K, int deviceId);
+
+//! Same with one shared A and/or B for the whole batch.
+void GemmMatrixWiseBroadcast(float* out, const float* A, const float* B, unsigned int M,
+                             unsigned int N, unsigned int K, unsigned int batchSize,
+                             bool broadcastA, bool broadcastB, int deviceId);
+
+//! Element offsets of one M x N unit product.
+struct GemmUnit
+{
+    std::uint64_t outOff, aOff, bOff;
+};
+
+//! All units in one launch: out[outOff] += A[aOff] * B[bOff] for every unit, units that share
+//! an output applied in list order.  This is how a whole broadcast walk is issued.
+void GemmGrouped(const std::vector<GemmUnit>& units, float* out, const float* A, const float* B,
+                 unsigned int M, unsigned int N, unsigned int K, int deviceId);
+
+//! Half-precision inputs, fp32 accumulation (the path the reference declares as WmmaGemm,
+//! Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50).  A and B hold IEEE
+//! binary16 bit patterns; strides in elements, 0 repeats the operand.
+void GemmHalf(float* out, const std::uint16_t* A, const std::uint16_t* B, unsigned int M,
+              unsigned int N, unsigned int K, unsigned int batchSize, std::size_t strideOut,
+              std::size_t strideA, std::size_t strideB, bool overwrite, int deviceId);
+
+//! dst[i] = binary16(src[i]), round to nearest even.
+void ConvertToHalf(std::uint16_t* dst, const float* src, std::size_t size);
+
+//! y = x > 0 ? x : 0 (Sources/Sapphire/compute/dense/cuda/Activation.cu, ReLU).
+void ReLU(float* y, const float* x, unsigned int totalSize);
+
+//! Batched 2-D transpose (Sources/Sapphire/compute/dense/cuda/Basic.cu:85-102).
+void Transpose(float* y, const float* x, unsigned int inputNumRows, unsigned int inputNumCols,
+               unsigned int batchSize, bool broadcastInput);
+}  // namespace Sapphire::Compute::Dense::Cuda
+
+#endif

@@ -1,0 +1,29 @@
+// Forward pass of the fully connected layer on TensorData, i.e. the compute part of
+// NN::Linear::operator() (Sources/Sapphire/operations/Forward/Linear.cpp:113-136) without the
+// autograd bookkeeping around it:
+//
+//     ones = [batch, 1] filled with 1            (Linear.cpp:113-118)
+//     x, y, bias viewed as 2-D                   (Linear.cpp:121, Util::ChangeTensorDataDimension)
+//     Gemm(y, ones, bias)    K = 1, adds the bias to every row   (Linear.cpp:134)
+//     Gemm(y, x, weight)     weight stored [in, out]             (Linear.cpp:136)
+//
+// y is expected to hold zeros on entry (a fresh TensorData does).
+#ifndef SAPPHIRE_AMD_OPERATIONS_FORWARD_LINEARFORWARD_HPP
+#define SAPPHIRE_AMD_OPERATIONS_FORWARD_LINEARFORWARD_HPP
+
+#include <Sapphire/tensor/TensorData.hpp>
+
+namespace Sapphire::Util
+{
+//! Views `data` with exactly `dimension` extents: Expand then Shrink of its shape
+//! (Includes/Sapphire/util/UnitUtils.hpp:18-36).
+void ChangeTensorDataDimension(int dimension, TensorUtil::TensorData& data);
+}  // namespace Sapphire::Util
+
+namespace Sapphire::NN
+{
+void LinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
+                   const TensorUtil::TensorData& weight, const TensorUtil::TensorData& bias);
+}  // namespace Sapphire::NN
+
+#endif

@@ -1,0 +1,408 @@
+// C entry points over the C++ operator layer so that the Python parity tests can drive it the
+// way the reference's own tests drive Compute::Gemm and friends: build TensorData objects,
+// move them to the device, call the operator, bring the result back
+// (Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:20-84, BroadcastTest.cpp:20-202).
+// Every function returns 0 on success and -1 after catching an exception, whose text
+// sphh_last_error() returns.
+#include <Sapphire/compute/BasicOps.hpp>
+#include <Sapphire/compute/BroadcastPlan.hpp>
+#include <Sapphire/compute/Initialize.hpp>
+#include <Sapphire/compute/cudaUtil/Memory.hpp>
+#include <Sapphire/compute/sparse/SparseGemm.hpp>
+#include <Sapphire/operations/Forward/LinearForward.hpp>
+#include <Sapphire/util/ResourceManager.hpp>
+
+#include <cstring>
+#include <exception>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+using namespace Sapphire;
+using TensorUtil::TensorData;
+
+namespace
+{
+thread_local std::string lastError;
+
+Shape MakeShape(const int* dims, int n)
+{
+    return Shape(std::vector<int>(dims, dims + n));
+}
+
+template <typename F>
+int Guard(F&& body)
+{
+    try
+    {
+        body();
+        return 0;
+    }
+    catch (const std::exception& e)
+    {
+        lastError = e.what();
+        return -1;
+    }
+}
+
+// A device tensor holding `values`: built in Host mode, filled, then sent with ToCuda(), the
+// sequence the reference's tests use.
+TensorData Upload(const Shape& shape, const float* values, const CudaDevice& device)
+{
+    TensorData t(shape, Type::Dense, device);
+    t.SetMode(ComputeMode::Host);
+    t.SetData(std::vector<float>(values, values + shape.Size()));
+    t.ToCuda();
+    return t;
+}
+
+void Download(TensorData& t, float* out)
+{
+    t.ToHost();
+    std::memcpy(out, t.HostRawPtr(), t.HostTotalSize * sizeof(float));
+}
+}  // namespace
+
+extern "C" {
+
+const char* sphh_last_error()
+{
+    return lastError.c_str();
+}
+
+// op 0: Expand(arg), 1: Shrink(arg), 2: Squeeze(), 3: GetTranspose; returns the new Dim
+int sphh_shape_op(const int* dims, int n, int op, int arg, int* outDims)
+{
+    int result = -1;
+    Guard([&] {
+        Shape s = MakeShape(dims, n);
+        if (op == 0)
+            s.Expand(arg);
+        else if (op == 1)
+            s.Shrink(arg);
+        else if (op == 2)
+            s.Squeeze();
+        else
+            s = s.GetTranspose();
+        for (int i = 0; i < s.Dim(); ++i)
+            outDims[i] = s.At(i);
+        result = s.Dim();
+    });
+    return result;
+}
+
+// what 0: Rows, 1: Cols, 2: Size, 3: GetNumUnits(arg), 4: GetUnitSize(arg)
+int sphh_shape_query(const int* dims, int n, int what, int arg)
+{
+    int result = -1;
+    Guard([&] {
+        const Shape s = MakeShape(dims, n);
+        switch (what)
+        {
+            case 0: result = s.Rows(); break;
+            case 1: result = s.Cols(); break;
+            case 2: result = s.Size(); break;
+            case 3: result = s.GetNumUnits(arg); break;
+            default: result = s.GetUnitSize(arg); break;
+        }
+    });
+    return result;
+}
+
+// leaves: 4 x uint64 per leaf (outOff, aOff, bOff, totalSizeOut); dims7: M N K maxDim sizes;
+// strided4: [isStrided, count, strideOut, strideA, strideB]
+long sphh_gemm_plan(const int* y, int yn, const int* a, int an, const int* b, int bn, int* dims7,
+                    unsigned long long* leaves, long cap, long long* strided5)
+{
+    long count = -1;
+    Guard([&] {
+        const Compute::GemmPlan plan = Compute::PlanGemm(MakeShape(y, yn), MakeShape(a, an),
+                                                         MakeShape(b, bn));
+        dims7[0] = static_cast<int>(plan.M);
+        dims7[1] = static_cast<int>(plan.N);
+        dims7[2] = static_cast<int>(plan.K);
+        dims7[3] = plan.maxDim;
+        dims7[4] = plan.sizeOut;
+        dims7[5] = plan.sizeA;
+        dims7[6] = plan.sizeB;
+        long i = 0;
+        for (const auto& leaf : plan.leaves)
+        {
+            if (i < cap)
+            {
+                leaves[4 * i + 0] = leaf.outOff;
+                leaves[4 * i + 1] = leaf.aOff;
+                leaves[4 * i + 2] = leaf.bOff;
+                leaves[4 * i + 3] = leaf.totalSizeOut;
+            }
+            ++i;
+        }
+        std::uint32_t n = 0;
+        std::int64_t so = 0, sa = 0, sb = 0;
+        strided5[0] = Compute::AsStridedBatch(plan, n, so, sa, sb) ? 1 : 0;
+        strided5[1] = n;
+        strided5[2] = so;
+        strided5[3] = sa;
+        strided5[4] = sb;
+        count = i;
+    });
+    return count;
+}
+
+// y (holding yData on entry) += a * b through Compute::Gemm in Cuda mode
+int sphh_compute_gemm(float* yData, const int* y, int yn, const float* aData, const int* a, int an,
+                      const float* bData, const int* b, int bn)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData A = Upload(MakeShape(a, an), aData, cuda);
+        TensorData B = Upload(MakeShape(b, bn), bData, cuda);
+        TensorData Out = Upload(MakeShape(y, yn), yData, cuda);
+        Compute::Gemm(Out, A, B);
+        Download(Out, yData);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// Compute::Gemm on Host-mode tensors must throw: returns 1 when it does
+int sphh_gemm_in_host_mode_throws()
+{
+    TensorData A(Shape({ 2, 2 }), Type::Dense), B(Shape({ 2, 2 }), Type::Dense),
+        Y(Shape({ 2, 2 }), Type::Dense);
+    const int rc = Guard([&] { Compute::Gemm(Y, A, B); });
+    Util::ResourceManager::Clean();
+    return rc == -1 ? 1 : 0;
+}
+
+// layers Linear -> ReLU -> ... -> Linear (no ReLU after the last), sizes has layers + 1 entries
+int sphh_mlp_forward(const float* x, int batch, const int* sizes, int layers,
+                     const float* const* weights, const float* const* biases, float* out)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData cur = Upload(Shape({ batch, sizes[0] }), x, cuda);
+        for (int l = 0; l < layers; ++l)
+        {
+            TensorData W = Upload(Shape({ sizes[l], sizes[l + 1] }), weights[l], cuda);
+            TensorData bias = Upload(Shape({ sizes[l + 1] }), biases[l], cuda);
+            TensorData y(Shape({ batch, sizes[l + 1] }), Type::Dense, cuda);  // zero-filled
+            NN::LinearForward(y, cur, W, bias);
+            if (l + 1 < layers)
+            {
+                TensorData act(y.GetShape(), Type::Dense, cuda);
+                Compute::ReLU(act, y);
+                cur = act;
+            }
+            else
+                cur = y;
+        }
+        Download(cur, out);
+        Util::ResourceManager::Clean();
+    });
+}
+
+int sphh_transpose(float* yData, const int* y, int yn, const float* xData, const int* x, int xn)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData X = Upload(MakeShape(x, xn), xData, cuda);
+        TensorData Y(MakeShape(y, yn), Type::Dense, cuda);
+        Compute::Transpose(Y, X);
+        Download(Y, yData);
+        Util::ResourceManager::Clean();
+    });
+}
+
+int sphh_sparse_gemm(float* yData, int M, int K, int N, const float* V, const unsigned* COL,
+                     const unsigned* ROW, const float* bData, int accumulate)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        const unsigned nnz = ROW[M];
+        SparseMatrix m = Compute::Sparse::Cuda::CreateSparseMatrix(
+            std::vector<float>(V, V + nnz), std::vector<uint32_t>(COL, COL + nnz),
+            std::vector<uint32_t>(ROW, ROW + M + 1), static_cast<uint32_t>(M),
+            static_cast<uint32_t>(K), 0);
+        TensorData A;
+        A.SparseMatCuda = &m;
+        TensorData B = Upload(Shape({ K, N }), bData, cuda);
+        TensorData Y = Upload(Shape({ M, N }), yData, cuda);
+        Compute::SparseGemm(Y, A, B, accumulate != 0);
+        Download(Y, yData);
+        Compute::Sparse::Cuda::FreeSparseMatrix(m);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// Life cycle checks of TensorData / ResourceManager on the device; returns 0 when all hold,
+// otherwise the number of the first failed check (text in sphh_last_error()).
+int sphh_tensor_lifecycle()
+{
+    int failed = 0;
+    const int rc = Guard([&] {
+        auto check = [&](bool ok, int id, const char* what) {
+            if (!ok && failed == 0)
+            {
+                failed = id;
+                lastError = what;
+            }
+        };
+        Util::ResourceManager::ClearAll();
+        const CudaDevice cuda(0, "device0");
+        {
+            TensorData t(Shape({ 3, 5 }), Type::Dense, cuda);
+            check(t.Mode() == ComputeMode::Cuda, 1, "device tensor starts in Cuda mode");
+            std::vector<float> v = t.GetDataCopy();
+            bool zero = true;
+            for (float f : v)
+                zero = zero && f == 0.0f;
+            check(v.size() == 15 && zero, 2, "fresh device buffer is zero");
+            std::vector<float> data(15);
+            for (int i = 0; i < 15; ++i)
+                data[i] = static_cast<float>(i) - 7.f;
+            t.SetData(data);
+            TensorData view = t;  // shallow
+            check(view.CudaRawPtr() == t.CudaRawPtr(), 3, "copies alias the buffer");
+            view.Reshape(Shape({ 15 }));
+            check(view.GetDataCopy() == data, 4, "reshaped view sees the same values");
+            t.ToHost();
+            check(t.Mode() == ComputeMode::Host && t.HostRawPtr()[14] == 7.f, 5, "ToHost copies");
+            t.HostMutableRawPtr()[0] = 42.f;
+            t.ToCuda();
+            check(t.GetDataCopy()[0] == 42.f, 6, "ToCuda copies");
+            TensorData copy = t.CreateCopy();
+            check(copy.CudaRawPtr() != t.CudaRawPtr() && copy.GetDataCopy() == t.GetDataCopy(), 7,
+                  "CreateCopy is deep");
+            bool threw = false;
+            try
+            {
+                t.SetData(std::vector<float>(3));
+            }
+            catch (const std::invalid_argument&)
+            {
+                threw = true;
+            }
+            check(threw, 8, "SetData with a wrong size throws");
+            threw = false;
+            try
+            {
+                t.Reshape(Shape({ 4, 4 }));
+            }
+            catch (const std::runtime_error&)
+            {
+                threw = true;
+            }
+            check(threw, 9, "Reshape to another size throws");
+        }
+        const auto before = Util::ResourceManager::Statistics();
+        check(before.cudaVolatile >= 2 && before.cudaFree == 0, 10, "blocks are volatile while in use");
+        Util::ResourceManager::Clean();
+        const auto cleaned = Util::ResourceManager::Statistics();
+        check(cleaned.cudaVolatile == 0 && cleaned.cudaFree == before.cudaVolatile, 11,
+              "Clean moves volatile blocks to the free pool");
+        {
+            TensorData again(Shape({ 3, 5 }), Type::Dense, cuda);
+            const auto reused = Util::ResourceManager::Statistics();
+            check(reused.cudaFree == cleaned.cudaFree - 1, 12, "an equal-size request reuses a free block");
+            std::vector<float> v = again.GetDataCopy();
+            bool zero = true;
+            for (float f : v)
+                zero = zero && f == 0.0f;
+            check(zero, 13, "a reused block is zero-filled again");
+        }
+        {
+            TensorData hostOnly(Shape({ 4 }), Type::Dense);
+            bool threw = false;
+            try
+            {
+                hostOnly.SetMode(ComputeMode::Cuda);
+            }
+            catch (const std::runtime_error&)
+            {
+                threw = true;
+            }
+            check(threw, 14, "SetMode(Cuda) without a device throws");
+        }
+        {
+            bool threw = false;
+            try
+            {
+                Compute::Cuda::CudaSetDevice(99);
+            }
+            catch (const std::runtime_error& e)
+            {
+                threw = std::string(e.what()).find("exceeds number of available devices") !=
+                        std::string::npos;
+            }
+            check(threw, 15, "CudaSetDevice out of range throws");
+        }
+        Util::ResourceManager::ClearAll();
+        const auto end = Util::ResourceManager::Statistics();
+        check(end.cudaVolatile + end.cudaFree + end.cudaPreserved == 0, 16, "ClearAll releases everything");
+    });
+    if (rc != 0)
+        return -1;
+    return failed;
+}
+
+// Host-only checks (no device): pools, TensorData in Host mode, error paths.
+int sphh_host_only_lifecycle()
+{
+    int failed = 0;
+    const int rc = Guard([&] {
+        auto check = [&](bool ok, int id, const char* what) {
+            if (!ok && failed == 0)
+            {
+                failed = id;
+                lastError = what;
+            }
+        };
+        {
+            TensorData t(Shape({ 2, 3 }), Type::Dense);
+            check(t.Mode() == ComputeMode::Host && t.HostTotalSize == 6, 1, "host tensor");
+            check(t.GetDataCopy() == std::vector<float>(6, 0.f), 2, "host buffer zeroed");
+            t.SetData({ 1, 2, 3, 4, 5, 6 });
+            TensorData wide(Shape({ 2, 2, 3 }), Type::Dense);
+            TensorData::DeepCopy(wide, t);
+            const std::vector<float> twice = { 1, 2, 3, 4, 5, 6, 1, 2, 3, 4, 5, 6 };
+            check(wide.GetDataCopy() == twice, 3, "DeepCopy repeats src");
+            Compute::Initialize::Ones(t);
+            check(t.GetDataCopy() == std::vector<float>(6, 1.f), 4, "Ones on host");
+            bool threw = false;
+            try
+            {
+                TensorData sparse(Shape({ 2, 2 }), Type::Sparse);
+            }
+            catch (const std::runtime_error&)
+            {
+                threw = true;
+            }
+            check(threw, 5, "sparse storage is not implemented, as in the reference");
+        }
+        const auto s = Util::ResourceManager::Statistics();
+        check(s.hostVolatile == 2, 6, "two volatile host blocks");
+        Util::ResourceManager::Clean();
+        check(Util::ResourceManager::Statistics().hostFree == 2, 7, "Clean keeps them for reuse");
+        void* p = Util::ResourceManager::GetMemoryHost(100, true);
+        Util::ResourceManager::MoveToVolatileHost(p);
+        Util::ResourceManager::MoveToPreservedHost(p);
+        Util::ResourceManager::FreePreservedHost(p);
+        bool threw = false;
+        try
+        {
+            Util::ResourceManager::FreePreservedHost(p);
+        }
+        catch (const std::runtime_error&)
+        {
+            threw = true;
+        }
+        check(threw, 8, "freeing an unknown pointer throws");
+        Util::ResourceManager::ClearFreePool();
+        check(Util::ResourceManager::Statistics().hostFree == 0, 9, "ClearFreePool");
+    });
+    if (rc != 0)
+        return -1;
+    return failed;
+}
+
+}  // extern "C"

@@ -1,0 +1,113 @@
+"""ctypes view of tests/host_harness/libhost_harness.so (the C++ operator layer)."""
+import ctypes
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "host_harness", "libhost_harness.so")
+
+_ip = ctypes.POINTER(ctypes.c_int)
+_fp = ctypes.POINTER(ctypes.c_float)
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s missing: python -m sapphire_amd.build host harness" % LIB_PATH)
+        h = ctypes.CDLL(LIB_PATH)
+        h.sphh_last_error.restype = ctypes.c_char_p
+        h.sphh_gemm_plan.restype = ctypes.c_long
+        h.sphh_gemm_plan.argtypes = [_ip, ctypes.c_int, _ip, ctypes.c_int, _ip, ctypes.c_int, _ip,
+                                     ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_long,
+                                     ctypes.POINTER(ctypes.c_longlong)]
+        h.sphh_compute_gemm.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int, _fp, _ip,
+                                        ctypes.c_int]
+        h.sphh_transpose.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int]
+        h.sphh_mlp_forward.argtypes = [_fp, ctypes.c_int, _ip, ctypes.c_int,
+                                       ctypes.POINTER(_fp), ctypes.POINTER(_fp), _fp]
+        h.sphh_sparse_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _fp,
+                                       ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint),
+                                       _fp, ctypes.c_int]
+        h.sphh_shape_op.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip]
+        h.sphh_shape_query.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        _lib = h
+    return _lib
+
+
+def _ints(v):
+    return (ctypes.c_int * max(len(v), 1))(*[int(x) for x in v])
+
+
+def _f(a):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_fp)
+
+
+def _ok(rc):
+    if rc != 0:
+        raise RuntimeError(lib().sphh_last_error().decode())
+
+
+def shape_op(dims, op, arg=0):
+    out = (ctypes.c_int * 32)()
+    n = lib().sphh_shape_op(_ints(dims), len(dims), op, arg, out)
+    if n < 0:
+        raise RuntimeError(lib().sphh_last_error().decode())
+    return [out[i] for i in range(n)]
+
+
+def shape_query(dims, what, arg=0):
+    return lib().sphh_shape_query(_ints(dims), len(dims), what, arg)
+
+
+def gemm_plan(ys, as_, bs):
+    cap = 1 << 16
+    leaves = (ctypes.c_ulonglong * (4 * cap))()
+    dims = (ctypes.c_int * 7)()
+    strided = (ctypes.c_longlong * 5)()
+    n = lib().sphh_gemm_plan(_ints(ys), len(ys), _ints(as_), len(as_), _ints(bs), len(bs), dims,
+                             leaves, cap, strided)
+    if n < 0:
+        raise RuntimeError(lib().sphh_last_error().decode())
+    d = dict(M=dims[0], N=dims[1], K=dims[2], maxDim=dims[3], sizeOut=dims[4], sizeA=dims[5],
+             sizeB=dims[6])
+    out = [tuple(int(leaves[4 * i + j]) for j in range(4)) for i in range(n)]
+    return d, out, [int(x) for x in strided]
+
+
+def compute_gemm(y, a, b):
+    """Compute::Gemm(y, a, b) in Cuda mode on numpy arrays; returns the new y."""
+    out = np.ascontiguousarray(y.copy())
+    _ok(lib().sphh_compute_gemm(_f(out), _ints(y.shape), y.ndim, _f(np.ascontiguousarray(a)),
+                                _ints(a.shape), a.ndim, _f(np.ascontiguousarray(b)),
+                                _ints(b.shape), b.ndim))
+    return out
+
+
+def transpose(x, y_shape):
+    out = np.zeros(y_shape, np.float32)
+    _ok(lib().sphh_transpose(_f(out), _ints(y_shape), len(y_shape), _f(np.ascontiguousarray(x)),
+                             _ints(x.shape), x.ndim))
+    return out
+
+
+def mlp_forward(x, weights, biases):
+    sizes = [x.shape[1]] + [w.shape[1] for w in weights]
+    out = np.zeros((x.shape[0], sizes[-1]), np.float32)
+    wp = (_fp * len(weights))(*[_f(w) for w in weights])
+    bp = (_fp * len(biases))(*[_f(b) for b in biases])
+    _ok(lib().sphh_mlp_forward(_f(x), x.shape[0], _ints(sizes), len(weights), wp, bp, _f(out)))
+    return out
+
+
+def sparse_gemm(y, V, COL, ROW, M, K, N, B, accumulate):
+    out = np.ascontiguousarray(y.copy())
+    up = ctypes.POINTER(ctypes.c_uint)
+    Vp = V if V.size else np.zeros(1, np.float32)
+    Cp = COL if COL.size else np.zeros(1, np.uint32)
+    _ok(lib().sphh_sparse_gemm(_f(out), M, K, N, _f(Vp), Cp.ctypes.data_as(up),
+                               ROW.ctypes.data_as(up), _f(B), 1 if accumulate else 0))
+    return out

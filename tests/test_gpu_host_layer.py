@@ -1,0 +1,159 @@
+"""The C++ operator layer on the device, driven like the reference's own tests: build
+TensorData, ToCuda, Compute::Gemm, ToHost, compare with the CPU result on the same data.
+
+Tolerance (fp32 path): max |gpu - cpu| / sum_k |a b| <= 1e-4; the reference's own absolute
+bounds (2.0 for Gemm1, 1.5 for the broadcast tests, inputs N(10, 5)) are asserted as well.
+"""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from sapphire_amd import synth
+from tests import helpers as h
+from tests import host_layer as hl
+
+pytestmark = pytest.mark.gpu
+TOL_F32 = 1e-4
+
+
+def _n10_5(seed, shape):
+    return (synth.normal(seed, shape, 5.0) + 10).astype(np.float32)
+
+
+def _dims(seed, count, hi):
+    return [int(x % hi) + 1 for x in synth.bits64(seed, count)]
+
+
+def _assert_close_to_cpu(got, y0, a, b, abs_bound):
+    ref = po.compute_gemm(y0.copy(), a, b)
+    assert np.max(np.abs(got - ref)) <= abs_bound
+    assert np.any(got != 0)
+    # normalise by what the same walk gives for |a| |b|
+    den = po.compute_gemm(np.zeros_like(y0), np.abs(a), np.abs(b))
+    err = float(np.max(np.abs(got.astype(np.float64) - ref) / np.maximum(den, 1e-30)))
+    assert err <= TOL_F32, err
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_gemm1_recipe(dev, seed):
+    """GemmTest.cpp:20-84: {b,M,K} x {b,K,N} -> {b,M,N}, dims in [1,100], batch in [1,30]."""
+    M, N, K, braw = _dims(0x100 + seed, 4, 100)
+    batch = braw % 30 + 1
+    h.announce("Compute::Gemm Gemm1 recipe", M, N, K, batch)
+    a, b = _n10_5(1 + seed, (batch, M, K)), _n10_5(50 + seed, (batch, K, N))
+    y0 = np.zeros((batch, M, N), np.float32)
+    _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 2.0)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_broadcast_with_one_dimension(dev, seed):
+    """BroadcastTest.cpp:20-80: A{b,1,M,K} x B{b,M,K,N} -> {b,M,M,N}, dims in [1,10]."""
+    M, N, K, braw = _dims(0x200 + seed, 4, 10)
+    batch = braw % 3 + 1
+    h.announce("Compute::Gemm BroadcastWithOneDimension", M, N, K, batch)
+    a, b = _n10_5(2 + seed, (batch, 1, M, K)), _n10_5(60 + seed, (batch, M, K, N))
+    y0 = np.zeros((batch, M, M, N), np.float32)
+    _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 1.5)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_broadcast_with_missing_dimension(dev, seed):
+    """BroadcastTest.cpp:82-141: A{M,K} x B{M,K,N} -> {M,M,N}."""
+    M, N, K = _dims(0x300 + seed, 3, 10)
+    h.announce("Compute::Gemm BroadcastWithMissingDimension", M, N, K)
+    a, b = _n10_5(3 + seed, (M, K)), _n10_5(70 + seed, (M, K, N))
+    y0 = np.zeros((M, M, N), np.float32)
+    _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 1.5)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_broadcast_mixed(dev, seed):
+    """BroadcastTest.cpp:143-202: A{M,K} x B{N,M,K,N} -> {N,M,M,N}."""
+    M, N, K = _dims(0x400 + seed, 3, 10)
+    h.announce("Compute::Gemm BroadcastMixed", M, N, K)
+    a, b = _n10_5(4 + seed, (M, K)), _n10_5(80 + seed, (N, M, K, N))
+    y0 = np.zeros((N, M, M, N), np.float32)
+    _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 1.5)
+
+
+def test_conv_style_broadcast_of_A_and_accumulation(dev):
+    """Filter {1,C,K} shared by the batch (how the naive Conv2D calls Gemm), y not zero."""
+    h.announce("Compute::Gemm A broadcast {1,6,9} x {5,9,8}")
+    a, b = synth.uniform(5, (1, 6, 9)), synth.uniform(6, (5, 9, 8))
+    y0 = synth.uniform(7, (5, 6, 8))
+    _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 1e-3)
+
+
+def test_repeated_outputs_accumulate_in_walk_order(dev):
+    """y smaller than the operands: several leaves add into the same output unit."""
+    h.announce("Compute::Gemm repeated outputs {2,4,5} <- {6,4,2} x {3,2,5}")
+    a, b = synth.uniform(8, (6, 4, 2)), synth.uniform(9, (3, 2, 5))
+    y0 = synth.uniform(10, (2, 4, 5))
+    _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 1e-3)
+
+
+def test_one_dimensional_operands(dev):
+    h.announce("Compute::Gemm 1-D operands [4] x [4,3] -> [3]")
+    a, b, y0 = synth.uniform(11, (4,)), synth.uniform(12, (4, 3)), synth.uniform(13, (3,))
+    _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 1e-3)
+
+
+def test_config2_through_the_operator(dev):
+    h.announce("Compute::Gemm config2 through TensorData")
+    d = synth.config2()
+    got = hl.compute_gemm(d["C"], d["A"], d["B"])
+    ref = po.compute_gemm(d["C"].copy(), d["A"], d["B"], threads=8)
+    for b in range(16):
+        err = h.normalised_error(got[b], ref[b], np.abs(d["A"][b]), np.abs(d["B"][0]))
+        assert err <= TOL_F32
+
+
+def test_config4_mlp_forward(dev):
+    """3-layer MLP 784 -> 1024 -> 1024 -> 10, batch 1024, Linear = bias GEMM (K = 1) + GEMM,
+    ReLU between layers; compared with the CPU composition layer by layer."""
+    h.announce("config4 MLP forward through NN::LinearForward + Compute::ReLU")
+    d = synth.config4()
+    got = hl.mlp_forward(d["x"], d["W"], d["b"])
+    act = d["x"]
+    bound = np.abs(d["x"]).astype(np.float64)       # propagated sum_k |a b| bound
+    for l in range(3):
+        ref = po.linear_forward(act, d["W"][l], d["b"][l], threads=8)
+        bound = bound @ np.abs(d["W"][l]).astype(np.float64) + np.abs(d["b"][l])
+        act = po.relu(ref) if l < 2 else ref
+    assert got.shape == (1024, 10) and np.isfinite(got).all()
+    err = float(np.max(np.abs(got.astype(np.float64) - act) / bound))
+    assert err <= TOL_F32, err
+    # also against the plain magnitude of the output
+    assert np.max(np.abs(got - act)) <= 1e-4 * max(1.0, float(np.max(np.abs(act))))
+
+
+def test_transpose(dev):
+    h.announce("Compute::Transpose batched and broadcast")
+    x = synth.uniform(14, (3, 37, 65))
+    got = hl.transpose(x, (3, 65, 37))
+    assert np.array_equal(got, np.transpose(x, (0, 2, 1)))
+    assert np.array_equal(got.ravel(), po.transpose(x, 37, 65, 3))
+    x2 = synth.uniform(15, (5, 9))
+    got = hl.transpose(x2, (4, 9, 5))          # 2-D input repeated for every matrix of y
+    assert np.array_equal(got, np.broadcast_to(x2.T, (4, 9, 5)))
+
+
+def test_sparse_gemm_through_tensor_data(dev):
+    h.announce("Compute::SparseGemm through SparseMatrix + TensorData")
+    M, K, N = 200, 333, 48
+    v, col, row = synth.csr_matrix(16, M, K, 9.0, forced={0: 0, 3: 200})
+    B = synth.uniform(17, (K, N))
+    y0 = synth.uniform(18, (M, N))
+    ref = po.spmm_csr(y0.copy(), v, col, row, M, N, B)
+    got = hl.sparse_gemm(y0, v, col, row, M, K, N, B, True)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    ref0 = po.spmm_csr(np.zeros((M, N), np.float32), v, col, row, M, N, B)
+    got0 = hl.sparse_gemm(y0, v, col, row, M, K, N, B, False)
+    assert np.array_equal(got0.view(np.uint32), ref0.view(np.uint32))
+
+
+def test_tensor_data_life_cycle_on_device(dev):
+    h.announce("TensorData / ResourceManager life cycle")
+    lib = hl.lib()
+    rc = lib.sphh_tensor_lifecycle()
+    assert rc == 0, (rc, lib.sphh_last_error())
