@@ -152,8 +152,9 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     // A stage: 128 LDS rows of 128 bytes; LDS row R holds A[R][k0..k0+31] in its first 64
     // bytes and A[R+128][k0..k0+31] in the last 64, 16-byte chunks XOR-swizzled with R%8.
     // B stage: 32 k-rows of 512 bytes, 32-byte chunks XOR-swizzled with 2*(k%4).
-    __shared__ __attribute__((aligned(1024))) _Float16 As[kTStages][kStageHalfs];
-    __shared__ __attribute__((aligned(1024))) _Float16 Bs[kTStages][kStageHalfs];
+    __shared__ __attribute__((aligned(1024))) _Float16 Lds[2][kTStages][kStageHalfs];
+    auto& As = Lds[0];
+    auto& Bs = Lds[1];
 
     uint32_t unit, tm, tn;
     if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
@@ -405,25 +406,54 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
 #undef SPH_FENCE
 
     // ---- epilogue -------------------------------------------------------------
-    // With the operands swapped the 32x32 result block is indexed [n][m]:
-    // register v of lane l holds column 8*(v/4) + 4*(l/32) + v%4 of row l%32,
-    // i.e. registers 4q..4q+3 are 4 consecutive columns.
+    // With the operands swapped the 32x32 result block is indexed [n][m]: register v of
+    // lane l holds column 8*(v/4) + 4*(l/32) + v%4 of row l%32, i.e. registers 4q..4q+3 are
+    // 4 consecutive columns of one row, and one store instruction would touch 32 rows with
+    // 32 bytes each.  To write (and, when accumulating, read) whole 256-byte row segments
+    // instead, each wavefront turns its 128 x (32*TJ) block round through a private 16 KiB
+    // piece of LDS, 64 rows at a time: after that a lane holds 4 consecutive columns and 16
+    // consecutive lanes cover one row of the block.
     if ((SPH_ABLATE & 8) && args.M != 1)
         return;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
+    static_assert(TJ == 2, "the staged epilogue is written for 64-column wavefront blocks");
+    WaitVmem<0>();      // clamped copies of the last steps still target LDS
+    __syncthreads();    // ... and every wavefront is done with the stage buffers
     {
-        const uint32_t r = waveM * 128 + i * 32 + l32;
+        // 64 rows x 64 floats per wavefront, 16-byte chunks XOR-swizzled with row % 16 so
+        // that neither the column-wise writes nor the row-wise reads pile up on one bank
+        float* stage = reinterpret_cast<float*>(&Lds[0][0][0]) + wave * (64 * 64);
+        static_assert(WAVES * 64 * 64 * 4 <= static_cast<int>(sizeof(Lds)), "staging fits");
+        const uint32_t rdRow = lane >> 4;        // + 4*t
+        const uint32_t rdChunk = lane & 15;
 #pragma unroll
-        for (int j = 0; j < TJ; ++j)
+        for (int half = 0; half < 2; ++half)
         {
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
+            for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                    {
+                        const int i = half * 2 + ii;
+                        const uint32_t row = ii * 32 + l32;
+                        const uint32_t chunk = (j * 8 + 2 * q + khalf) ^ (row & 15);
+                        *reinterpret_cast<float4*>(&stage[row * 64 + chunk * 4]) =
+                            make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
+                                        acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+                    }
+            // the block is private to the wavefront: its own LDS writes are visible to it
+            // once they have completed
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            float* outBlock = out + static_cast<size_t>(waveM * 128 + half * 64) * N +
+                              waveN * (32 * TJ) + rdChunk * 4;
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
             {
-                const uint32_t c = waveN * (32 * TJ) + j * 32 + 8 * q + 4 * khalf;
-                float4* p = reinterpret_cast<float4*>(out + static_cast<size_t>(r) * N + c);
-                float4 v = make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
-                                       acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+                const uint32_t r = rdRow + 4 * t;
+                float4 v = *reinterpret_cast<const float4*>(
+                    &stage[r * 64 + ((rdChunk ^ (r & 15)) * 4)]);
+                float4* p = reinterpret_cast<float4*>(outBlock + static_cast<size_t>(r) * N);
                 if (!args.overwrite)
                 {
                     const float4 old = *p;
@@ -434,6 +464,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
                 }
                 *p = v;
             }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
     }
 }
