@@ -227,7 +227,7 @@ def main():
                         "store mode" % nnz,
             "entry_point": "sph_spmm_csr_f32", "steps": sp_steps, "launch_ms": sp_event,
             "value": gbs, "unit": "GB/s", "gflops": 2.0 * nnz * 256 / (sp_event * 1e-3) / 1e9,
-            "roofline": {"bound": "hbm", "kernel": "SpmmRowVec4", "achieved": gbs,
+            "roofline": {"bound": "hbm", "kernel": "SpmmSlabVec4<16>", "achieved": gbs,
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                          "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
                          "gather_bytes_per_launch": nnz * 256 * 4},
