@@ -36,6 +36,19 @@ PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 
+def recorded_traffic(profile_name):
+    """HBM-side bytes per launch from the committed rocprofv3 summary (FETCH_SIZE and
+    WRITE_SIZE counter runs, scaled by the copy-kernel calibration); None when absent."""
+    path = os.path.join(ROOT, "profiles", profile_name)
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -198,7 +211,10 @@ def main():
                        "entry_point": "sph_gemm_f16f32 (accumulate)"},
             "roofline": {"bound": "mfma", "kernel": "GemmF16Tile256",
                          "achieved": kernel_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": kernel_tflops / PEAK_FP16_TFLOPS, "traffic": None,
+                         "frac": kernel_tflops / PEAK_FP16_TFLOPS,
+                         "traffic": recorded_traffic("gemm_f16_tile256_config3.txt"),
+                         "traffic_unit": "bytes per launch (profiles/gemm_f16_tile256_config3.txt)",
+                         "algorithmic_bytes_per_launch": 3 * 64 * (1 << 20),
                          "launch_ms": event_ms, "flop_per_launch": flops,
                          "peak_from_device": device_peak,
                          "peak_from_device_note": "%d CUs x 4096 flop/clk x %d MHz"
@@ -229,7 +245,9 @@ def main():
             "value": gbs, "unit": "GB/s", "gflops": 2.0 * nnz * 256 / (sp_event * 1e-3) / 1e9,
             "roofline": {"bound": "hbm", "kernel": "SpmmSlabVec4<16>", "achieved": gbs,
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                         "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+                         "traffic": recorded_traffic("spmm_slab_config5.txt"),
+                         "traffic_unit": "bytes per launch (profiles/spmm_slab_config5.txt)",
+                         "algorithmic_bytes_per_launch": alg_bytes,
                          "gather_bytes_per_launch": nnz * 256 * 4},
         }
         if not args.no_cpu and args.only is None:
