@@ -425,9 +425,11 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         static_assert(WAVES * 64 * 64 * 4 <= static_cast<int>(sizeof(Lds)), "staging fits");
         const uint32_t rdRow = lane >> 4;        // + 4*t
         const uint32_t rdChunk = lane & 15;
-#pragma unroll
-        for (int half = 0; half < 2; ++half)
-        {
+        float* outBlock = out + static_cast<size_t>(waveM * 128 + rdRow) * N +
+                          waveN * (32 * TJ) + rdChunk * 4;
+        const size_t rowStep = static_cast<size_t>(4) * N;  // between consecutive t
+
+        auto stageHalf = [&](int half) {
 #pragma unroll
             for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
@@ -445,26 +447,49 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
             // the block is private to the wavefront: its own LDS writes are visible to it
             // once they have completed
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            float* outBlock = out + static_cast<size_t>(waveM * 128 + half * 64) * N +
-                              waveN * (32 * TJ) + rdChunk * 4;
+        };
+        auto loadOld = [&](int half, float4 (&old)[16]) {
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
+                old[t] = *reinterpret_cast<const float4*>(outBlock + (half * 16 + t) * rowStep);
+        };
+        auto storeHalf = [&](int half, const float4 (&old)[16], auto accumulate) {
 #pragma unroll
             for (int t = 0; t < 16; ++t)
             {
                 const uint32_t r = rdRow + 4 * t;
                 float4 v = *reinterpret_cast<const float4*>(
                     &stage[r * 64 + ((rdChunk ^ (r & 15)) * 4)]);
-                float4* p = reinterpret_cast<float4*>(outBlock + static_cast<size_t>(r) * N);
-                if (!args.overwrite)
+                if constexpr (decltype(accumulate)::value)
                 {
-                    const float4 old = *p;
-                    v.x += old.x;
-                    v.y += old.y;
-                    v.z += old.z;
-                    v.w += old.w;
+                    v.x += old[t].x;
+                    v.y += old[t].y;
+                    v.z += old[t].z;
+                    v.w += old[t].w;
                 }
-                *p = v;
+                *reinterpret_cast<float4*>(outBlock + (half * 16 + t) * rowStep) = v;
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        };
+
+        float4 old[16];
+        if (args.overwrite)
+        {
+            stageHalf(0);
+            storeHalf(0, old, std::false_type{});
+            stageHalf(1);
+            storeHalf(1, old, std::false_type{});
+        }
+        else
+        {
+            // the old contents of a half are requested in one batch, in flight while its
+            // accumulators are staged
+            loadOld(0, old);
+            stageHalf(0);
+            storeHalf(0, old, std::true_type{});
+            loadOld(1, old);
+            stageHalf(1);
+            storeHalf(1, old, std::true_type{});
         }
     }
 }
