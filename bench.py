@@ -131,6 +131,39 @@ def bench_f32(capi, A, B, C, M, N, K, batch, sb, steps, warmup):
     return event_ms
 
 
+def bench_mlp(capi, synth, steps, warmup):
+    """Configuration 4 through the C ABI: per layer ones[batch,1] x bias (K = 1 GEMM), x x W,
+    ReLU between layers -- the call sequence of Linear's forward pass."""
+    d = synth.config4()
+    batch = d["x"].shape[0]
+    sizes = [d["x"].shape[1]] + [w.shape[1] for w in d["W"]]
+    x = capi.DeviceBuffer.from_array(d["x"])
+    W = [capi.DeviceBuffer.from_array(w) for w in d["W"]]
+    b = [capi.DeviceBuffer.from_array(v) for v in d["b"]]
+    ones = capi.DeviceBuffer.from_array(np.ones(batch, np.float32))
+    y = [capi.DeviceBuffer(4 * batch * n) for n in sizes[1:]]
+    act = [capi.DeviceBuffer(4 * batch * n) for n in sizes[1:-1]]
+
+    def launch():
+        cur = x
+        for l in range(3):
+            n_in, n_out = sizes[l], sizes[l + 1]
+            capi.call("sph_fill_f32", y[l].ptr, 0.0, batch * n_out)
+            capi.call("sph_gemm_f32", y[l].ptr, ones.ptr, b[l].ptr, batch, n_out, 1, 1,
+                      batch * n_out, batch, n_out)
+            capi.call("sph_gemm_f32", y[l].ptr, cur.ptr, W[l].ptr, batch, n_out, n_in, 1,
+                      batch * n_out, batch * n_in, n_in * n_out)
+            if l < 2:
+                capi.call("sph_relu_f32", act[l].ptr, y[l].ptr, batch * n_out)
+                cur = act[l]
+
+    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    for buf in [x, ones] + W + b + y + act:
+        buf.release()
+    flops = 2.0 * batch * sum(sizes[l] * sizes[l + 1] for l in range(3))
+    return event_ms, flops
+
+
 def bench_copy(capi, steps, warmup, mib=64):
     """A plain one-pass kernel of known size (ReLU over `mib` MiB: reads it once, writes it
     once), used to calibrate the profiler's FETCH_SIZE / WRITE_SIZE counters."""
@@ -268,6 +301,9 @@ def main():
         tf = 16 * 2 * 512 ** 3 / (ms * 1e-3) / 1e12
         others["config2_f32_batched"] = {"launch_ms": ms, "tflops": tf,
                                          "frac_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
+        ms, fl = bench_mlp(capi, synth, 100, 10)
+        others["config4_mlp_forward"] = {"forward_ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
+                                         "kernels_per_forward": 11}
         result["others"] = others
 
     if not args.no_cpu and args.only is None:

@@ -41,6 +41,7 @@ struct GemmF32Args
     const SphGemmEntry* entries;  // device table, or null for stride arithmetic
     uint32_t M, N, K;
     uint32_t tilesM, tilesN;
+    uint32_t outVec;  // 16-byte accesses to out are possible
     int64_t strideOut, strideA, strideB;
 };
 
@@ -208,22 +209,34 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
 
         const float* as = &As[cur][waveM * WM + l32];
         const float* bs = &Bs[cur][waveN * WN + l32];
+        // fragments of k pair kk+2 are read while the MFMAs of pair kk run; the fences keep
+        // the compiler from sinking the reads back to their first use
+        float a[2][TM], b[2][TN];
+        auto readPair = [&](int slot, int kk) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                a[slot][i] = as[(kk + khalf) * LDA + i * 32];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                b[slot][j] = bs[(kk + khalf) * LDB + j * 32];
+        };
+        readPair(0, 0);
 #pragma unroll
         for (int kk = 0; kk < kBK; kk += 2)
         {
-            float a[TM], b[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                a[i] = as[(kk + khalf) * LDA + i * 32];
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                b[j] = bs[(kk + khalf) * LDB + j * 32];
+            const int slot = (kk / 2) & 1;
+            if (kk + 2 < kBK)
+                readPair(slot ^ 1, kk + 2);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] =
-                        __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+                    // operands swapped: the 32x32 result block comes out indexed
+                    // [column][row], which leaves 4 consecutive columns in a lane
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[slot][j], a[slot][i],
+                                                                     acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
 
         if (s + 1 < steps)
@@ -232,28 +245,66 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
     }
 
     // ---- out += acc ---------------------------------------------------------
-    // 32x32 accumulator layout: register v of lane l holds
-    // row 8*(v/4) + 4*(l/32) + v%4, column l%32.
+    // With the operands swapped, register v of lane l holds row l%32 and column
+    // 8*(v/4) + 4*(l/32) + v%4 of its 32x32 block: registers 4q..4q+3 are 4
+    // consecutive columns.  The old values of the whole wavefront block are requested
+    // in one batch, then added and stored.
+    constexpr int kQuads = TM * TN * 4;
+    float4 old[kQuads];
+    const bool wide = args.outVec != 0;  // N % 4 == 0 and 16-byte aligned output rows
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-        {
-            const uint32_t c = colBase + waveN * WN + j * 32 + l32;
-            if (c >= N)
-                continue;
 #pragma unroll
-            for (int v = 0; v < 16; ++v)
+            for (int q = 0; q < 4; ++q)
             {
-                const uint32_t r =
-                    rowBase + waveM * WM + i * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
-                if (r < M)
+                const uint32_t r = rowBase + waveM * WM + i * 32 + l32;
+                const uint32_t c = colBase + waveN * WN + j * 32 + 8 * q + 4 * khalf;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (r < M && c < N)
                 {
+                    const float* p = out + static_cast<size_t>(r) * N + c;
+                    if (wide)
+                        v = *reinterpret_cast<const float4*>(p);
+                    else
+                    {
+                        v.x = p[0];
+                        if (c + 1 < N) v.y = p[1];
+                        if (c + 2 < N) v.z = p[2];
+                        if (c + 3 < N) v.w = p[3];
+                    }
+                }
+                old[(i * TN + j) * 4 + q] = v;
+            }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const uint32_t r = rowBase + waveM * WM + i * 32 + l32;
+                const uint32_t c = colBase + waveN * WN + j * 32 + 8 * q + 4 * khalf;
+                if (r < M && c < N)
+                {
+                    float4 v = old[(i * TN + j) * 4 + q];
+                    v.x += acc[i][j][4 * q + 0];
+                    v.y += acc[i][j][4 * q + 1];
+                    v.z += acc[i][j][4 * q + 2];
+                    v.w += acc[i][j][4 * q + 3];
                     float* p = out + static_cast<size_t>(r) * N + c;
-                    *p = *p + acc[i][j][v];
+                    if (wide)
+                        *reinterpret_cast<float4*>(p) = v;
+                    else
+                    {
+                        p[0] = v.x;
+                        if (c + 1 < N) p[1] = v.y;
+                        if (c + 2 < N) p[2] = v.z;
+                        if (c + 3 < N) p[3] = v.w;
+                    }
                 }
             }
-        }
 }
 
 // Device table for grouped launches: one growing buffer per device with a
@@ -272,9 +323,14 @@ struct EntryTable
 std::mutex gTableMutex;
 EntryTable gTables[16];
 
-int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, hipStream_t stream)
+int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOffsetsAligned,
+           hipStream_t stream)
 {
     GemmF32Args args = base;
+    args.outVec = (outOffsetsAligned && (args.N % 4 == 0) &&
+                   (reinterpret_cast<uintptr_t>(args.out) & 15u) == 0)
+                      ? 1u
+                      : 0u;
     const bool aligned =
         allowVector && (args.K % 4 == 0) && (args.N % 4 == 0) &&
         ((reinterpret_cast<uintptr_t>(args.A) | reinterpret_cast<uintptr_t>(args.B)) & 15u) == 0;
@@ -365,7 +421,7 @@ int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M, uint32_
     args.strideA = strideA;
     args.strideB = strideB;
     const bool stridesAligned = (strideA % 4 == 0) && (strideB % 4 == 0);
-    return Launch(args, batch, stridesAligned, stream);
+    return Launch(args, batch, stridesAligned, strideOut % 4 == 0 || batch == 1, stream);
 }
 
 int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out, const float* A,
@@ -380,9 +436,12 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
 
-    bool offsetsAligned = true;
-    for (uint32_t i = 0; i < count && offsetsAligned; ++i)
-        offsetsAligned = ((entries[i].aOff | entries[i].bOff) % 4) == 0;
+    bool offsetsAligned = true, outAligned = true;
+    for (uint32_t i = 0; i < count; ++i)
+    {
+        offsetsAligned = offsetsAligned && ((entries[i].aOff | entries[i].bOff) % 4) == 0;
+        outAligned = outAligned && (entries[i].outOff % 4) == 0;
+    }
 
     std::lock_guard<std::mutex> lock(gTableMutex);
     EntryTable& t = gTables[sph::CurrentDevice()];
@@ -421,7 +480,7 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
         args.M = M;
         args.N = N;
         args.K = K;
-        const int rc = Launch(args, end - begin, offsetsAligned, stream);
+        const int rc = Launch(args, end - begin, offsetsAligned, outAligned, stream);
         if (rc != SPH_OK)
             return rc;
         begin = end;
