@@ -307,6 +307,186 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
             }
 }
 
+// ---------------------------------------------------------------------------
+// Few-tile shapes (small M x N, long K): 32 x 32 output tile per workgroup, K split four
+// ways across its wavefronts.
+//
+// With few output tiles the tiled kernel above leaves most compute units idle and is bound by
+// the latency of one load -> LDS -> MFMA chain per K step.  Here every wavefront reads its
+// operands straight from global memory in MFMA layout (A: 16 bytes per lane along K, lines
+// reused from L1 over the next steps; B: one row segment per lane half), keeps several loads
+// in flight, and accumulates a private 32 x 32 partial over its quarter of K.  The four
+// partials are then added in wavefront order through LDS, so the result does not depend on
+// timing.  The two k values of one MFMA come from lanes 0-31 and 32-63; which k each half
+// holds is free as long as A and B agree, and is chosen so that A is read with float4.
+// ---------------------------------------------------------------------------
+constexpr int kSkinnyThreads = 256;
+
+template <bool VEC>
+__global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const GemmF32Args args)
+{
+    __shared__ float partial[3][32 * 32];
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t l32 = lane & 31;
+    const uint32_t khalf = lane >> 5;
+
+    uint32_t id = blockIdx.x;
+    const uint32_t tn = id % args.tilesN;
+    id /= args.tilesN;
+    const uint32_t tm = id % args.tilesM;
+    const uint32_t unit = id / args.tilesM;
+
+    const float* __restrict__ A;
+    const float* __restrict__ B;
+    float* __restrict__ out;
+    if (args.entries != nullptr)
+    {
+        const SphGemmEntry e = args.entries[unit];
+        A = args.A + e.aOff;
+        B = args.B + e.bOff;
+        out = args.out + e.outOff;
+    }
+    else
+    {
+        A = args.A + args.strideA * static_cast<int64_t>(unit);
+        B = args.B + args.strideB * static_cast<int64_t>(unit);
+        out = args.out + args.strideOut * static_cast<int64_t>(unit);
+    }
+    const uint32_t M = args.M, N = args.N, K = args.K;
+    const uint32_t row = tm * 32 + l32;
+    const uint32_t col = tn * 32 + l32;
+
+    // this wavefront's K range, in groups of 8 (one float4 of A per lane half)
+    const uint32_t groups = (K + 7) / 8;
+    const uint32_t perWave = (groups + 3) / 4;
+    const uint32_t gBegin = min(wave * perWave, groups);
+    const uint32_t gEnd = min(gBegin + perWave, groups);
+
+    const float* aRow = A + static_cast<size_t>(min(row, M - 1)) * K;
+    const bool rowOk = row < M;
+    const bool colOk = col < N;
+
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+        acc[v] = 0.f;
+
+    // lane half h holds k = 8*g + 4*h + e for e = 0..3
+    auto loadA = [&](uint32_t g) {
+        const uint32_t k = g * 8 + khalf * 4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (rowOk)
+        {
+            if (VEC)
+            {
+                if (k < K)
+                    v = *reinterpret_cast<const float4*>(aRow + k);
+            }
+            else
+            {
+                if (k + 0 < K) v.x = aRow[k + 0];
+                if (k + 1 < K) v.y = aRow[k + 1];
+                if (k + 2 < K) v.z = aRow[k + 2];
+                if (k + 3 < K) v.w = aRow[k + 3];
+            }
+        }
+        return v;
+    };
+    auto loadB = [&](uint32_t g) {
+        const uint32_t k = g * 8 + khalf * 4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (colOk)
+        {
+            const float* p = B + static_cast<size_t>(k) * N + col;
+            if (k + 0 < K) v.x = p[0];
+            if (k + 1 < K) v.y = p[static_cast<size_t>(N)];
+            if (k + 2 < K) v.z = p[2 * static_cast<size_t>(N)];
+            if (k + 3 < K) v.w = p[3 * static_cast<size_t>(N)];
+        }
+        return v;
+    };
+
+    constexpr int kDepth = 4;  // groups in flight
+    float4 fa[kDepth], fb[kDepth];
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d)
+    {
+        fa[d] = gBegin + d < gEnd ? loadA(gBegin + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+        fb[d] = gBegin + d < gEnd ? loadB(gBegin + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (uint32_t g = gBegin; g < gEnd; g += kDepth)
+    {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d)
+        {
+            const float4 a = fa[d];
+            const float4 b = fb[d];
+            const uint32_t next = g + kDepth + d;
+            fa[d] = next < gEnd ? loadA(next) : make_float4(0.f, 0.f, 0.f, 0.f);
+            fb[d] = next < gEnd ? loadB(next) : make_float4(0.f, 0.f, 0.f, 0.f);
+            // groups past gEnd carry zeros and add nothing
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.x, a.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.y, a.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.z, a.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.w, a.w, acc, 0, 0, 0);
+        }
+    }
+
+    // partial sums of wavefronts 1..3 go through LDS; wavefront 0 adds them in order
+    if (wave != 0)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<float4*>(&partial[wave - 1][l32 * 32 + 8 * q + 4 * khalf]) =
+                make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+    }
+    __syncthreads();
+    if (wave != 0)
+        return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const float4 p =
+                *reinterpret_cast<const float4*>(&partial[w][l32 * 32 + 8 * q + 4 * khalf]);
+            acc[4 * q + 0] += p.x;
+            acc[4 * q + 1] += p.y;
+            acc[4 * q + 2] += p.z;
+            acc[4 * q + 3] += p.w;
+        }
+    // operands were swapped: lane l holds row l%32, columns 8q + 4*(l/32) + 0..3
+    if (!rowOk)
+        return;
+    const bool wide = args.outVec != 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+    {
+        const uint32_t c = tn * 32 + 8 * q + 4 * khalf;
+        if (c >= N)
+            continue;
+        float* p = out + static_cast<size_t>(row) * N + c;
+        if (wide)
+        {
+            float4 v = *reinterpret_cast<const float4*>(p);
+            v.x += acc[4 * q + 0];
+            v.y += acc[4 * q + 1];
+            v.z += acc[4 * q + 2];
+            v.w += acc[4 * q + 3];
+            *reinterpret_cast<float4*>(p) = v;
+        }
+        else
+        {
+            p[0] += acc[4 * q + 0];
+            if (c + 1 < N) p[1] += acc[4 * q + 1];
+            if (c + 2 < N) p[2] += acc[4 * q + 2];
+            if (c + 3 < N) p[3] += acc[4 * q + 3];
+        }
+    }
+}
+
 // Device table for grouped launches: one growing buffer per device with a
 // pinned staging copy.  The table is shared by every caller, so its use is
 // serialised by a mutex and, across streams, by waiting for the stream that
@@ -334,6 +514,27 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const bool aligned =
         allowVector && (args.K % 4 == 0) && (args.N % 4 == 0) &&
         ((reinterpret_cast<uintptr_t>(args.A) | reinterpret_cast<uintptr_t>(args.B)) & 15u) == 0;
+
+    // few 64 x 64 tiles and a long K: split K inside the workgroup instead
+    const uint64_t tiles64 =
+        static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
+    if (tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) && args.K >= 64)
+    {
+        args.tilesM = (args.M + 31) / 32;
+        args.tilesN = (args.N + 31) / 32;
+        const uint64_t blocks32 = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
+        const dim3 grid32(static_cast<uint32_t>(blocks32));
+        const bool aVec = allowVector && (args.K % 4 == 0) &&
+                          (reinterpret_cast<uintptr_t>(args.A) & 15u) == 0;
+        if (aVec)
+            hipLaunchKernelGGL(GemmF32SkinnyKernel<true>, grid32, dim3(kSkinnyThreads), 0, stream,
+                               args);
+        else
+            hipLaunchKernelGGL(GemmF32SkinnyKernel<false>, grid32, dim3(kSkinnyThreads), 0, stream,
+                               args);
+        SPH_CHECK_LAUNCH();
+        return SPH_OK;
+    }
 
     const uint64_t tiles128 =
         static_cast<uint64_t>((args.M + 127) / 128) * ((args.N + 127) / 128) * units;
