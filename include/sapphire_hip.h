@@ -118,7 +118,37 @@ int sph_transpose_f32(float* out, const float* in, uint32_t rows, uint32_t cols,
 /* dst[i] = (binary16, round-to-nearest-even) src[i] */
 int sph_convert_f32_to_f16(sph_f16* dst, const float* src, size_t count);
 
+/* out[i] = in[i] * factor.  Replaces Dense::Cuda::Scale (called from
+ * Sources/Sapphire/compute/BasicOps.cpp Compute::Scale); CPU counterpart
+ * NaiveBasic.cpp:54-61.  out may alias in. */
+int sph_scale_f32(float* out, const float* in, float factor, size_t count);
+
+/* out[i] = a[i % la] - b[i % lb] with la = broadcastA ? inputStride : count,
+ * lb likewise: the leaf Compute::Sub hands to BroadcastWith2Inputs
+ * (Sources/Sapphire/compute/BasicOps.cpp:70-103).  Replaces Dense::Cuda::Sub;
+ * CPU counterpart NaiveBasic.cpp:28-39.  out may alias a or b when neither is
+ * broadcast.  inputStride must be non-zero when a broadcast flag is set. */
+int sph_sub_f32(float* out, const float* a, const float* b, size_t count,
+                size_t inputStride, int broadcastA, int broadcastB);
+
+/* dx[i] += x[i] > 0 ? dy[i] : 0.  Replaces Dense::Cuda::ReLUBackward
+ * (Sources/Sapphire/compute/ActivationOps.cpp:69-85); CPU counterpart
+ * NaiveBasic.cpp:167-174. */
+int sph_relu_backward_f32(float* dx, const float* dy, const float* x, size_t count);
+
+/* z[i] = z[i] - dz[i] * learningRate, the product rounded to fp32 before the
+ * subtraction: one pass with the result of the Scale-into-temporary followed
+ * by Sub that Optimizer::SGD performs (Sources/Sapphire/operations/optimizers/SGD.cpp:22-28),
+ * bit for bit, without the temporary. */
+int sph_sgd_step_f32(float* z, const float* dz, float learningRate, size_t count);
+
 /* ---- dense GEMM ---------------------------------------------------------- */
+
+/* flags of the GEMM entry points that take them */
+#define SPH_GEMM_ACCUMULATE 0u /* out += A*B, like the reference            */
+#define SPH_GEMM_OVERWRITE 1u  /* out  = A*B, out is not read               */
+#define SPH_GEMM_TRANS_A 2u    /* A is stored K x M (the transpose of M x K) */
+#define SPH_GEMM_TRANS_B 4u    /* B is stored N x K (the transpose of K x N) */
 
 /* out[b] += A[b] * B[b] for b < batch; row-major; A is M x K, B is K x N,
  * out is M x N; fp32 storage, fp32 MFMA products and accumulation.
@@ -134,6 +164,19 @@ int sph_convert_f32_to_f16(sph_f16* dst, const float* src, size_t count);
 int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M,
                  uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,
                  int64_t strideA, int64_t strideB);
+
+/* sph_gemm_f32 with flags.  SPH_GEMM_TRANS_A / SPH_GEMM_TRANS_B read an
+ * operand that is stored transposed, so that the products of the backward
+ * pass, dx += dy * W^T and dw = x^T * dy, need no materialised transpose:
+ * they replace the Compute::Transpose + Compute::Gemm pairs of
+ * Sources/Sapphire/operations/Backward/LinearBackward.cpp:49-50,70-73 and
+ * MathBackward.cpp:46-51.  The K products of an output element are added in
+ * the same order with or without the flags, so the result is bit-identical
+ * to sph_transpose_f32 followed by sph_gemm_f32.  SPH_GEMM_OVERWRITE stores
+ * the product without reading out (K == 0 then stores zeros). */
+int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M,
+                    uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,
+                    int64_t strideA, int64_t strideB, uint32_t flags);
 
 /* One M x N unit product per entry, out[outOff] += A[aOff] * B[bOff], offsets
  * in elements from the three bases.  Entries are read from host memory.  This
@@ -157,9 +200,8 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
  * (Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50) and
  * never defines.  Same layout, stride and += contract as sph_gemm_f32.
  * flags: SPH_GEMM_OVERWRITE stores A*B without reading out (for callers that
- * know out holds zeros); default accumulates like the reference. */
-#define SPH_GEMM_ACCUMULATE 0u
-#define SPH_GEMM_OVERWRITE 1u
+ * know out holds zeros); default accumulates like the reference.  The
+ * transpose flags are not supported here (SPH_ERR_UNSUPPORTED). */
 
 int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M,
                     uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,

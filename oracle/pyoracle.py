@@ -71,6 +71,22 @@ def oracle():
         o.orc_relu.restype = None
         o.orc_transpose.argtypes = [_fp, _fp, _u, _u, _u, ctypes.c_int]
         o.orc_transpose.restype = None
+        o.orc_scale.argtypes = [_fp, _fp, ctypes.c_float, _u]
+        o.orc_scale.restype = None
+        o.orc_sub.argtypes = [_u, _fp, _fp, _fp, _u, ctypes.c_int, ctypes.c_int]
+        o.orc_sub.restype = None
+        o.orc_relu_backward.argtypes = [_fp, _fp, _fp, _u]
+        o.orc_relu_backward.restype = None
+        o.orc_get_matching_dim.argtypes = [ctypes.POINTER(OrcShape), ctypes.c_int]
+        o.orc_get_matching_dim.restype = ctypes.c_int
+        o.orc_compute_sub.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int, _fp, _ip,
+                                      ctypes.c_int]
+        o.orc_compute_sub.restype = ctypes.c_int
+        o.orc_sgd.argtypes = [_fp, _fp, ctypes.c_float, _u]
+        o.orc_sgd.restype = None
+        o.orc_linear_backward.argtypes = [_fp, _fp, _fp, _fp, _fp, _u, _u, _u, ctypes.c_float,
+                                          ctypes.c_int]
+        o.orc_linear_backward.restype = None
         o.orc_linear_forward.argtypes = [_fp, _fp, _fp, _fp, _u, _u, _u, ctypes.c_int]
         o.orc_linear_forward.restype = None
         o.orc_spmm_csr.argtypes = [_fp, _fp, _up, _up, ctypes.c_uint32, ctypes.c_uint32, _fp,
@@ -103,6 +119,15 @@ def ref():
         r.ref_relu.restype = None
         r.ref_transpose.argtypes = [_fp, _fp, _u, _u, _u, ctypes.c_int]
         r.ref_transpose.restype = None
+        r.ref_scale.argtypes = [_fp, _fp, ctypes.c_float, _u]
+        r.ref_scale.restype = None
+        r.ref_sub.argtypes = [_u, _fp, _fp, _fp, _u, ctypes.c_int, ctypes.c_int]
+        r.ref_sub.restype = None
+        r.ref_relu_backward.argtypes = [_fp, _fp, _fp, _u]
+        r.ref_relu_backward.restype = None
+        r.ref_compute_sub.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int, _fp, _ip,
+                                      ctypes.c_int, ctypes.c_int]
+        r.ref_compute_sub.restype = None
         r.ref_shape_op.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip]
         r.ref_shape_op.restype = ctypes.c_int
         r.ref_shape_query.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int]
@@ -192,6 +217,64 @@ def transpose(x, rows, cols, batch, broadcast=False):
     out = np.zeros(batch * rows * cols, dtype=np.float32)
     oracle().orc_transpose(_f(out), _f(x), rows, cols, batch, 1 if broadcast else 0)
     return out
+
+
+def scale(x, factor):
+    out = np.empty_like(x)
+    oracle().orc_scale(_f(out), _f(x), factor, x.size)
+    return out
+
+
+def sub_leaf(a, b, count, input_stride=0, broadcast_a=False, broadcast_b=False):
+    out = np.empty(count, dtype=np.float32)
+    oracle().orc_sub(count, _f(out), _f(a), _f(b), input_stride, int(broadcast_a),
+                     int(broadcast_b))
+    return out
+
+
+def relu_backward(dx, dy, x):
+    out = np.ascontiguousarray(dx.copy())
+    oracle().orc_relu_backward(_f(out), _f(dy), _f(x), x.size)
+    return out
+
+
+def matching_dim(shapes):
+    arr = (OrcShape * max(len(shapes), 1))()
+    for i, dims in enumerate(shapes):
+        arr[i] = make_shape(dims)
+    return oracle().orc_get_matching_dim(arr, len(shapes))
+
+
+def compute_sub(y_shape, a, b, lib=None):
+    """Compute::Sub host branch; returns y (zeros where the walk writes nothing)."""
+    y = np.zeros(y_shape, dtype=np.float32)
+    ys, as_, bs = list(y_shape), list(a.shape), list(b.shape)
+    if lib == "ref":
+        dim = max(len(ys), len(as_), len(bs))
+        pad = lambda v: [1] * (dim - len(v)) + v
+        leaf_dim = matching_dim([pad(ys), pad(as_), pad(bs)])
+        ref().ref_compute_sub(_f(y), _ints(ys), len(ys), _f(a), _ints(as_), len(as_), _f(b),
+                              _ints(bs), len(bs), leaf_dim)
+    else:
+        rc = oracle().orc_compute_sub(_f(y), _ints(ys), len(ys), _f(a), _ints(as_), len(as_),
+                                      _f(b), _ints(bs), len(bs))
+        assert rc == 0
+    return y
+
+
+def sgd(z, dz, lr):
+    out = np.ascontiguousarray(z.copy())
+    oracle().orc_sgd(_f(out), _f(dz), lr, z.size)
+    return out
+
+
+def linear_backward(dx, W, bias, dy, x, lr, threads=1):
+    """Returns the updated (dx, W, bias)."""
+    dx, W, bias = (np.ascontiguousarray(v.copy()) for v in (dx, W, bias))
+    batch, fin = x.shape
+    oracle().orc_linear_backward(_f(dx), _f(W), _f(bias), _f(dy), _f(x), batch, fin, W.shape[1],
+                                 lr, threads)
+    return dx, W, bias
 
 
 def linear_forward(x, W, bias, threads=1):

@@ -103,6 +103,43 @@ void ref_transpose(float* out, const float* in, unsigned int rows,
                                                broadcast != 0);
 }
 
+void ref_scale(float* out, const float* in, float factor, unsigned int totalSize)
+{
+    Sapphire::Compute::Dense::Naive::Scale(out, in, factor, totalSize);
+}
+
+void ref_sub(unsigned int totalSize, float* out, const float* A, const float* B,
+             unsigned int inputStride, int broadcastA, int broadcastB)
+{
+    Sapphire::Compute::Dense::Naive::Sub(totalSize, out, A, B, inputStride,
+                                         broadcastA != 0, broadcastB != 0);
+}
+
+void ref_relu_backward(float* dx, const float* dy, const float* x,
+                       unsigned int totalSize)
+{
+    Sapphire::Compute::Dense::Naive::ReLUBackward(dx, dy, x, totalSize);
+}
+
+// Host branch of Compute::Sub, BasicOps.cpp:70-103, with the matching
+// dimension passed in (Util::GetMatchingDim lives in a header that pulls in
+// the model classes and cannot be compiled here).
+void ref_compute_sub(float* y, const int* yShape, int yDim, const float* a,
+                     const int* aShape, int aDim, const float* b,
+                     const int* bShape, int bDim, int minRequiredDim)
+{
+    auto so = MakeShape(yShape, yDim);
+    auto sa = MakeShape(aShape, aDim);
+    auto sb = MakeShape(bShape, bDim);
+    const int maxDim = std::max({ yDim, aDim, bDim });
+    so.Expand(maxDim);
+    sa.Expand(maxDim);
+    sb.Expand(maxDim);
+    Sapphire::Compute::BroadcastWith2Inputs(
+        so, sa, sb, so.Size(), sa.Size(), sb.Size(), y, a, b, 0, minRequiredDim,
+        Sapphire::Compute::Dense::Naive::Sub, 0, false, false);
+}
+
 // op: 0 Expand(arg), 1 Shrink(arg); writes the resulting dims, returns Dim
 int ref_shape_op(const int* v, int dim, int op, int arg, int* outDims)
 {

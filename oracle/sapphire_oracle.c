@@ -400,6 +400,159 @@ void orc_transpose(float* out, const float* in, unsigned int inputRows,
     }
 }
 
+void orc_scale(float* out, const float* in, float factor,
+               unsigned int totalSize)
+{
+    /* NaiveBasic.cpp:54-61 */
+    for (unsigned int i = 0; i < totalSize; i++)
+        out[i] = in[i] * factor;
+}
+
+void orc_sub(unsigned int totalSize, float* out, const float* A, const float* B,
+             unsigned int inputStride, int broadcastA, int broadcastB)
+{
+    /* NaiveBasic.cpp:28-39 */
+    const unsigned int leftOverA = broadcastA ? inputStride : totalSize;
+    const unsigned int leftOverB = broadcastB ? inputStride : totalSize;
+    for (unsigned int i = 0; i < totalSize; i++)
+        out[i] = A[i % leftOverA] - B[i % leftOverB];
+}
+
+void orc_relu_backward(float* dx, const float* dy, const float* x,
+                       unsigned int totalSize)
+{
+    /* NaiveBasic.cpp:167-174 */
+    for (unsigned int i = 0; i < totalSize; ++i)
+        dx[i] += x[i] > 0.0f ? dy[i] : 0.0f;
+}
+
+int orc_get_matching_dim(const orc_shape* shapes, int count)
+{
+    /* UnitUtils.hpp:38-73: curDimFromLast runs -1, -2, ... while every shape
+     * still has that position and holds shapes[0]'s extent there. */
+    if (count <= 0)
+        return -1;
+    int curDimFromLast = -1;
+    for (;;)
+    {
+        if (shapes[0].dim + curDimFromLast < 0)
+            break;
+        const int want = shapes[0].d[shapes[0].dim + curDimFromLast];
+        int match = 1;
+        for (int s = 0; s < count; ++s)
+        {
+            if (shapes[s].dim + curDimFromLast < 0 ||
+                shapes[s].d[shapes[s].dim + curDimFromLast] != want)
+            {
+                match = 0;
+                break;
+            }
+        }
+        if (!match)
+            break;
+        curDimFromLast -= 1;
+    }
+    return -(curDimFromLast + 1);
+}
+
+static void fill_shape(orc_shape* s, const int* v, int dim)
+{
+    s->dim = dim;
+    for (int i = 0; i < dim; ++i)
+        s->d[i] = v[i];
+}
+
+int orc_compute_sub(float* y, const int* yShape, int yDim, const float* a,
+                    const int* aShape, int aDim, const float* b,
+                    const int* bShape, int bDim)
+{
+    /* BasicOps.cpp:63-103 */
+    orc_shape sh[3];
+    fill_shape(&sh[0], yShape, yDim);
+    fill_shape(&sh[1], aShape, aDim);
+    fill_shape(&sh[2], bShape, bDim);
+    int maxDim = yDim;
+    if (aDim > maxDim) maxDim = aDim;
+    if (bDim > maxDim) maxDim = bDim;
+    for (int i = 0; i < 3; ++i)
+        if (orc_shape_expand(&sh[i], maxDim) != 0)
+            return -1;
+    const int minRequiredDim = orc_get_matching_dim(sh, 3);
+    size_t cap = 1024;
+    orc_leaf* leaves = (orc_leaf*)malloc(cap * sizeof(orc_leaf));
+    size_t n = orc_broadcast_with_2_inputs(
+        &sh[0], &sh[1], &sh[2], (unsigned int)orc_shape_size(&sh[0]),
+        (unsigned int)orc_shape_size(&sh[1]), (unsigned int)orc_shape_size(&sh[2]),
+        0, (unsigned int)minRequiredDim, leaves, cap);
+    if (n > cap)
+    {
+        free(leaves);
+        cap = n;
+        leaves = (orc_leaf*)malloc(cap * sizeof(orc_leaf));
+        if (!leaves)
+            return -1;
+        n = orc_broadcast_with_2_inputs(
+            &sh[0], &sh[1], &sh[2], (unsigned int)orc_shape_size(&sh[0]),
+            (unsigned int)orc_shape_size(&sh[1]),
+            (unsigned int)orc_shape_size(&sh[2]), 0,
+            (unsigned int)minRequiredDim, leaves, cap);
+    }
+    for (size_t i = 0; i < n; ++i)
+        orc_sub(leaves[i].totalSizeOut, y + leaves[i].outOff,
+                a + leaves[i].aOff, b + leaves[i].bOff, 0, 0, 0);
+    free(leaves);
+    return 0;
+}
+
+void orc_sgd(float* z, const float* dz, float learningRate, unsigned int size)
+{
+    /* SGD.cpp:22-28 */
+    float* temp = (float*)malloc((size ? size : 1) * sizeof(float));
+    const int shape[1] = { (int)size };
+    orc_scale(temp, dz, learningRate, size);
+    orc_compute_sub(z, shape, 1, z, shape, 1, temp, shape, 1);
+    free(temp);
+}
+
+void orc_linear_backward(float* dx, float* W, float* bias, const float* dy,
+                         const float* x, unsigned int batch, unsigned int in,
+                         unsigned int outF, float learningRate, int threads)
+{
+    const int dxs[2] = { (int)batch, (int)in };
+    const int dys[2] = { (int)batch, (int)outF };
+    const int ws[2] = { (int)in, (int)outF };
+    const int wts[2] = { (int)outF, (int)in };
+    const int xts[2] = { (int)in, (int)batch };
+    const int os[2] = { 1, (int)batch };
+    const int bs[1] = { (int)outF };
+
+    /* LinearBackward.cpp:37-51 */
+    float* wt = (float*)calloc((size_t)in * outF + 1, sizeof(float));
+    orc_transpose(wt, W, in, outF, 1, 1);
+    orc_compute_gemm(dx, dxs, 2, dy, dys, 2, wt, wts, 2, threads);
+    free(wt);
+
+    /* LinearBackward.cpp:53-77 */
+    float* xt = (float*)calloc((size_t)batch * in + 1, sizeof(float));
+    float* dw = (float*)calloc((size_t)in * outF + 1, sizeof(float));
+    orc_transpose(xt, x, batch, in, 1, 1);
+    orc_compute_gemm(dw, ws, 2, xt, xts, 2, dy, dys, 2, threads);
+    orc_sgd(W, dw, learningRate, in * outF);
+    free(xt);
+    free(dw);
+
+    /* LinearBackward.cpp:79-99 */
+    float* ones = (float*)malloc((batch ? batch : 1) * sizeof(float));
+    float* dB = (float*)calloc(outF + 1, sizeof(float));
+    for (unsigned int i = 0; i < batch; ++i)
+        ones[i] = 1.0f;
+    orc_compute_gemm(dB, bs, 1, ones, os, 2, dy, dys, 2, 1);
+    orc_scale(dB, dB, 1.0f / (float)batch, outF);
+    orc_sgd(bias, dB, learningRate, outF);
+    free(ones);
+    free(dB);
+}
+
 void orc_linear_forward(float* y, const float* x, const float* W,
                         const float* bias, unsigned int batch, unsigned int in,
                         unsigned int outF, int threads)

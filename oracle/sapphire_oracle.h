@@ -131,6 +131,57 @@ void orc_transpose(float* out, const float* in, unsigned int inputRows,
                    unsigned int inputCols, unsigned int batchSize,
                    int broadcast);
 
+/* NaiveBasic.cpp:54-61  out = in * factor.
+ * pinned: oracle/_ref bit-exact. */
+void orc_scale(float* out, const float* in, float factor,
+               unsigned int totalSize);
+
+/* NaiveBasic.cpp:28-39  out[i] = A[i % la] - B[i % lb], la = broadcastA ?
+ * inputStride : totalSize (lb likewise).
+ * pinned: oracle/_ref bit-exact, with and without the broadcast flags. */
+void orc_sub(unsigned int totalSize, float* out, const float* A, const float* B,
+             unsigned int inputStride, int broadcastA, int broadcastB);
+
+/* NaiveBasic.cpp:167-174  dx += x > 0 ? dy : 0.
+ * pinned: oracle/_ref bit-exact. */
+void orc_relu_backward(float* dx, const float* dy, const float* x,
+                       unsigned int totalSize);
+
+/* Includes/Sapphire/util/UnitUtils.hpp:38-73: number of trailing dimensions on
+ * which all `count` shapes agree (a shape that runs out stops the count).
+ * -1 when count == 0 (the reference throws).
+ * The header cannot be compiled here (it includes the model classes), so this
+ * is pinned by a hand-derived table: equal shapes, differing last dimension,
+ * shorter shapes, single shape. */
+int orc_get_matching_dim(const orc_shape* shapes, int count);
+
+/* Sources/Sapphire/compute/BasicOps.cpp:63-103 host branch: shapes expanded to
+ * the longest, leaf dims = orc_get_matching_dim, walk from shapeIdx 0, each
+ * leaf orc_sub(totalSizeOut, ..., 0, false, false).
+ * pinned: oracle/_ref running the reference walk with the reference leaf (the
+ * matching dimension supplied by orc_get_matching_dim); y = a - b closed form
+ * for equal shapes. */
+int orc_compute_sub(float* y, const int* yShape, int yDim, const float* a,
+                    const int* aShape, int aDim, const float* b,
+                    const int* bShape, int bDim);
+
+/* Sources/Sapphire/operations/optimizers/SGD.cpp:22-28: temp = dz * lr
+ * (orc_scale), z = z - temp (orc_sub through the operator; equal shapes, one
+ * leaf).  pinned: composition of pinned parts. */
+void orc_sgd(float* z, const float* dz, float learningRate, unsigned int size);
+
+/* Sources/Sapphire/operations/Backward/LinearBackward.cpp:27-99 with the SGD
+ * optimizer, as the sequence of operator calls written there:
+ *   Wt = transpose(W); dx += dy*Wt;
+ *   xt = transpose(x); dw = 0; dw += xt*dy; sgd(W, dw);
+ *   ones[1,batch]; dB = 0; dB += ones*dy; dB *= 1/batch; sgd(bias, dB).
+ * x [batch,in], W [in,out], bias [out], dy [batch,out], dx [batch,in].
+ * dx, W and bias are updated in place.
+ * pinned: composition of pinned parts; closed form with one-hot x and dy. */
+void orc_linear_backward(float* dx, float* W, float* bias, const float* dy,
+                         const float* x, unsigned int batch, unsigned int in,
+                         unsigned int outF, float learningRate, int threads);
+
 /* Sources/Sapphire/operations/Forward/Linear.cpp:113-136: y (zero on entry,
  * [batch,out]) receives ones[batch,1]*bias[1,out] through the K=1 GEMM and
  * then x[batch,in]*W[in,out] through a second GEMM, both via the operator.

@@ -18,6 +18,8 @@ HEADER_PATH = os.path.join(os.path.dirname(_PKG), "include", "sapphire_hip.h")
 
 SPH_GEMM_ACCUMULATE = 0
 SPH_GEMM_OVERWRITE = 1
+SPH_GEMM_TRANS_A = 2
+SPH_GEMM_TRANS_B = 4
 
 
 class SphError(RuntimeError):
@@ -75,7 +77,12 @@ SIGNATURES = {
     "sph_relu_f32": [_vp, _vp, _sz],
     "sph_transpose_f32": [_vp, _vp, _u32, _u32, _u32, ctypes.c_int],
     "sph_convert_f32_to_f16": [_vp, _vp, _sz],
+    "sph_scale_f32": [_vp, _vp, ctypes.c_float, _sz],
+    "sph_sub_f32": [_vp, _vp, _vp, _sz, _sz, ctypes.c_int, ctypes.c_int],
+    "sph_relu_backward_f32": [_vp, _vp, _vp, _sz],
+    "sph_sgd_step_f32": [_vp, _vp, ctypes.c_float, _sz],
     "sph_gemm_f32": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64],
+    "sph_gemm_f32_ex": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
     "sph_gemm_f32_grouped": [ctypes.POINTER(SphGemmEntry), _u32, _vp, _vp, _vp, _u32, _u32, _u32],
     "sph_gemm_f16f32": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
     "sph_spmm_csr_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, ctypes.c_int],

@@ -1,8 +1,12 @@
 // One-pass, HBM-bound neighbours of the matrix-multiplication path: constant
-// fill, ReLU, fp32 -> fp16 conversion and the batched 2-D transpose.  All of
-// them move 16 bytes per lane per access where alignment allows and use
-// grid-stride loops sized to a few workgroups per compute unit.
+// fill, ReLU and its backward, scale, subtract, the SGD update, fp32 -> fp16
+// conversion and the batched 2-D transpose.  All of them move 16 bytes per lane
+// per access where alignment allows and use grid-stride loops sized to a few
+// workgroups per compute unit.
 #include "sph_internal.h"
+
+// Products and sums are rounded separately, as in the reference's CPU loops.
+#pragma clang fp contract(off)
 
 #include <hip/hip_fp16.h>
 
@@ -107,6 +111,114 @@ __global__ __launch_bounds__(kThreads) void ConvertKernel(__half* __restrict__ d
         dst[i] = __float2half_rn(src[i]);
 }
 
+// Generic one-pass map over `count` floats: F(i) for the tail and scalar path,
+// F4(i) for 4 consecutive elements starting at 4*i.
+template <typename F4, typename F1>
+__device__ __forceinline__ void MapRange(size_t count, int vec, F4 quad, F1 single)
+{
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t step = static_cast<size_t>(gridDim.x) * kThreads;
+    size_t done = 0;
+    if (vec)
+    {
+        const size_t quads = count / 4;
+        for (size_t i = tid; i < quads; i += step)
+            quad(i);
+        done = quads * 4;
+    }
+    for (size_t i = done + tid; i < count; i += step)
+        single(i);
+}
+
+// out may alias in: every element is read before it is written, by the same lane
+__global__ __launch_bounds__(kThreads) void ScaleKernel(float* out, const float* in, float factor,
+                                                        size_t count, int vec)
+{
+    MapRange(
+        count, vec,
+        [&](size_t i) {
+            float4 v = reinterpret_cast<const float4*>(in)[i];
+            v.x *= factor;
+            v.y *= factor;
+            v.z *= factor;
+            v.w *= factor;
+            reinterpret_cast<float4*>(out)[i] = v;
+        },
+        [&](size_t i) { out[i] = in[i] * factor; });
+}
+
+__global__ __launch_bounds__(kThreads) void SubKernel(float* out, const float* a, const float* b,
+                                                      size_t count, int vec)
+{
+    MapRange(
+        count, vec,
+        [&](size_t i) {
+            const float4 x = reinterpret_cast<const float4*>(a)[i];
+            const float4 y = reinterpret_cast<const float4*>(b)[i];
+            reinterpret_cast<float4*>(out)[i] =
+                make_float4(x.x - y.x, x.y - y.y, x.z - y.z, x.w - y.w);
+        },
+        [&](size_t i) { out[i] = a[i] - b[i]; });
+}
+
+// a and/or b repeat every `la` / `lb` elements
+__global__ __launch_bounds__(kThreads) void SubWrapKernel(float* __restrict__ out,
+                                                          const float* __restrict__ a,
+                                                          const float* __restrict__ b,
+                                                          size_t count, size_t la, size_t lb)
+{
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t step = static_cast<size_t>(gridDim.x) * kThreads;
+    for (size_t i = tid; i < count; i += step)
+        out[i] = a[i % la] - b[i % lb];
+}
+
+__global__ __launch_bounds__(kThreads) void ReluBackwardKernel(float* __restrict__ dx,
+                                                               const float* __restrict__ dy,
+                                                               const float* __restrict__ x,
+                                                               size_t count, int vec)
+{
+    MapRange(
+        count, vec,
+        [&](size_t i) {
+            float4 d = reinterpret_cast<const float4*>(dx)[i];
+            const float4 g = reinterpret_cast<const float4*>(dy)[i];
+            const float4 v = reinterpret_cast<const float4*>(x)[i];
+            d.x += v.x > 0.0f ? g.x : 0.0f;
+            d.y += v.y > 0.0f ? g.y : 0.0f;
+            d.z += v.z > 0.0f ? g.z : 0.0f;
+            d.w += v.w > 0.0f ? g.w : 0.0f;
+            reinterpret_cast<float4*>(dx)[i] = d;
+        },
+        [&](size_t i) { dx[i] += x[i] > 0.0f ? dy[i] : 0.0f; });
+}
+
+// The product is an fp32 value of its own before it is subtracted.  Written with plain
+// operators under this file's contract(off): the rounded-arithmetic intrinsics of the HIP
+// headers are compiled with contraction allowed and would fuse after inlining.
+__device__ __forceinline__ float Rounded(float v)
+{
+    return v;
+}
+
+__global__ __launch_bounds__(kThreads) void SgdStepKernel(float* __restrict__ z,
+                                                          const float* __restrict__ dz, float lr,
+                                                          size_t count, int vec)
+{
+    MapRange(
+        count, vec,
+        [&](size_t i) {
+            float4 w = reinterpret_cast<const float4*>(z)[i];
+            const float4 g = reinterpret_cast<const float4*>(dz)[i];
+            w.x = w.x - Rounded(g.x * lr);
+            w.y = w.y - Rounded(g.y * lr);
+            w.z = w.z - Rounded(g.z * lr);
+            w.w = w.w - Rounded(g.w * lr);
+            reinterpret_cast<float4*>(z)[i] = w;
+        },
+        [&](size_t i) { z[i] = z[i] - Rounded(dz[i] * lr); });
+}
+
 // 64 x 64 tile through LDS; the extra column keeps the column-wise read-out
 // off a single bank.
 constexpr int kTile = 64;
@@ -192,6 +304,81 @@ int sph_convert_f32_to_f16(sph_f16* dst, const float* src, size_t count)
     const int vec = (Aligned16(dst) && Aligned16(src)) ? 1 : 0;
     hipLaunchKernelGGL(ConvertKernel, dim3(GridFor(vec ? count / 8 + 7 : count)), dim3(kThreads),
                        0, stream, reinterpret_cast<__half*>(dst), src, count, vec);
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int sph_scale_f32(float* out, const float* in, float factor, size_t count)
+{
+    if (count == 0)
+        return SPH_OK;
+    SPH_REQUIRE(out != nullptr && in != nullptr, "null pointer");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    const int vec = (Aligned16(out) && Aligned16(in)) ? 1 : 0;
+    hipLaunchKernelGGL(ScaleKernel, dim3(GridFor(vec ? count / 4 + 3 : count)), dim3(kThreads), 0,
+                       stream, out, in, factor, count, vec);
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int sph_sub_f32(float* out, const float* a, const float* b, size_t count, size_t inputStride,
+                int broadcastA, int broadcastB)
+{
+    if (count == 0)
+        return SPH_OK;
+    SPH_REQUIRE(out != nullptr && a != nullptr && b != nullptr, "null pointer");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    if (broadcastA || broadcastB)
+    {
+        SPH_REQUIRE(inputStride != 0, "inputStride must be non-zero with a broadcast operand");
+        SPH_REQUIRE(out != a && out != b, "in-place subtraction with a broadcast operand");
+        const size_t la = broadcastA ? inputStride : count;
+        const size_t lb = broadcastB ? inputStride : count;
+        hipLaunchKernelGGL(SubWrapKernel, dim3(GridFor(count)), dim3(kThreads), 0, stream, out, a,
+                           b, count, la, lb);
+    }
+    else
+    {
+        const int vec = (Aligned16(out) && Aligned16(a) && Aligned16(b)) ? 1 : 0;
+        hipLaunchKernelGGL(SubKernel, dim3(GridFor(vec ? count / 4 + 3 : count)), dim3(kThreads),
+                           0, stream, out, a, b, count, vec);
+    }
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int sph_relu_backward_f32(float* dx, const float* dy, const float* x, size_t count)
+{
+    if (count == 0)
+        return SPH_OK;
+    SPH_REQUIRE(dx != nullptr && dy != nullptr && x != nullptr, "null pointer");
+    SPH_REQUIRE(dx != dy && dx != x, "dx must not alias dy or x");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    const int vec = (Aligned16(dx) && Aligned16(dy) && Aligned16(x)) ? 1 : 0;
+    hipLaunchKernelGGL(ReluBackwardKernel, dim3(GridFor(vec ? count / 4 + 3 : count)),
+                       dim3(kThreads), 0, stream, dx, dy, x, count, vec);
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int sph_sgd_step_f32(float* z, const float* dz, float learningRate, size_t count)
+{
+    if (count == 0)
+        return SPH_OK;
+    SPH_REQUIRE(z != nullptr && dz != nullptr, "null pointer");
+    SPH_REQUIRE(z != dz, "z must not alias dz");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    const int vec = (Aligned16(z) && Aligned16(dz)) ? 1 : 0;
+    hipLaunchKernelGGL(SgdStepKernel, dim3(GridFor(vec ? count / 4 + 3 : count)), dim3(kThreads),
+                       0, stream, z, dz, learningRate, count, vec);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }

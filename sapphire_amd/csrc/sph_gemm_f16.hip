@@ -705,6 +705,9 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
                     int64_t strideB, uint32_t flags)
 {
     SPH_REQUIRE(M != 0 && N != 0 && batch != 0, "M, N and batch must be non-zero");
+    if (flags & (SPH_GEMM_TRANS_A | SPH_GEMM_TRANS_B))
+        return sph::Fail(SPH_ERR_UNSUPPORTED,
+                         "sph_gemm_f16f32 - transposed operands are not supported");
     SPH_REQUIRE((flags & ~SPH_GEMM_OVERWRITE) == 0, "unknown flag");
     SPH_REQUIRE(out != nullptr, "null pointer");
     SPH_REQUIRE(strideOut >= 0 && strideA >= 0 && strideB >= 0, "negative stride");

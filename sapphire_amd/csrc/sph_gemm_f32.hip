@@ -41,11 +41,115 @@ struct GemmF32Args
     const SphGemmEntry* entries;  // device table, or null for stride arithmetic
     uint32_t M, N, K;
     uint32_t tilesM, tilesN;
-    uint32_t outVec;  // 16-byte accesses to out are possible
+    uint32_t outVec;     // 16-byte accesses to out are possible
+    uint32_t overwrite;  // out = A*B instead of out += A*B
     int64_t strideOut, strideA, strideB;
 };
 
-template <int BM, int BN, bool VEC>
+// Slab loaders.  An operand is stored either with K contiguous (A as given, B when it is
+// passed transposed: `rows` indexes M or N) or with the M/N index contiguous (B as given, A
+// when it is passed transposed: `rows` indexes K).  Both end up k-major in LDS, S[k][x].
+template <int BX, int QUADS, bool VEC>
+__device__ __forceinline__ void FetchKContig(float4 (&stage)[QUADS], const float* __restrict__ src,
+                                             uint32_t tid, uint32_t xBase, uint32_t xLimit,
+                                             uint32_t k0, uint32_t K)
+{
+#pragma unroll
+    for (int i = 0; i < QUADS; ++i)
+    {
+        const uint32_t q = tid + i * kThreads;
+        const uint32_t r = q >> 2;
+        const uint32_t kq = (q & 3) * 4;
+        const uint32_t gx = xBase + r;
+        const uint32_t gk = k0 + kq;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (gx < xLimit)
+        {
+            const float* p = src + static_cast<size_t>(gx) * K + gk;
+            if (VEC)
+            {
+                if (gk < K)
+                    v = *reinterpret_cast<const float4*>(p);
+            }
+            else
+            {
+                if (gk + 0 < K) v.x = p[0];
+                if (gk + 1 < K) v.y = p[1];
+                if (gk + 2 < K) v.z = p[2];
+                if (gk + 3 < K) v.w = p[3];
+            }
+        }
+        stage[i] = v;
+    }
+}
+
+template <int BX, int QUADS, bool VEC>
+__device__ __forceinline__ void FetchXContig(float4 (&stage)[QUADS], const float* __restrict__ src,
+                                             uint32_t tid, uint32_t xBase, uint32_t xLimit,
+                                             uint32_t k0, uint32_t K)
+{
+#pragma unroll
+    for (int i = 0; i < QUADS; ++i)
+    {
+        const uint32_t q = tid + i * kThreads;
+        const uint32_t kr = q / (BX / 4);
+        const uint32_t xq = (q % (BX / 4)) * 4;
+        const uint32_t gk = k0 + kr;
+        const uint32_t gx = xBase + xq;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (gk < K)
+        {
+            const float* p = src + static_cast<size_t>(gk) * xLimit + gx;
+            if (VEC)
+            {
+                if (gx < xLimit)
+                    v = *reinterpret_cast<const float4*>(p);
+            }
+            else
+            {
+                if (gx + 0 < xLimit) v.x = p[0];
+                if (gx + 1 < xLimit) v.y = p[1];
+                if (gx + 2 < xLimit) v.z = p[2];
+                if (gx + 3 < xLimit) v.w = p[3];
+            }
+        }
+        stage[i] = v;
+    }
+}
+
+template <int BX, int LD, int QUADS>
+__device__ __forceinline__ void StashKContig(float* __restrict__ slab, const float4 (&stage)[QUADS],
+                                             uint32_t tid)
+{
+#pragma unroll
+    for (int i = 0; i < QUADS; ++i)
+    {
+        const uint32_t q = tid + i * kThreads;
+        const uint32_t r = q >> 2;
+        const uint32_t kq = (q & 3) * 4;
+        float* dst = slab + kq * LD + r;
+        dst[0 * LD] = stage[i].x;
+        dst[1 * LD] = stage[i].y;
+        dst[2 * LD] = stage[i].z;
+        dst[3 * LD] = stage[i].w;
+    }
+}
+
+template <int BX, int LD, int QUADS>
+__device__ __forceinline__ void StashXContig(float* __restrict__ slab, const float4 (&stage)[QUADS],
+                                             uint32_t tid)
+{
+#pragma unroll
+    for (int i = 0; i < QUADS; ++i)
+    {
+        const uint32_t q = tid + i * kThreads;
+        const uint32_t kr = q / (BX / 4);
+        const uint32_t xq = (q % (BX / 4)) * 4;
+        *reinterpret_cast<float4*>(slab + kr * LD + xq) = stage[i];
+    }
+}
+
+template <int BM, int BN, bool VEC, bool TA, bool TB>
 __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args)
 {
     constexpr int WM = BM / 2;   // rows per wavefront
@@ -93,90 +197,32 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
     const uint32_t rowBase = tm * BM;
     const uint32_t colBase = tn * BN;
 
-    // ---- which 4-element groups this lane moves from HBM to LDS ------------
-    // A slab: BM rows x 4 groups; group g covers k = 4g..4g+3 of one row.
-    // B slab: 16 rows x BN/4 groups.
+    // ---- 4-element groups this lane moves from HBM to LDS -----------------------
+    // A as given is M x K (K contiguous); with TA it is K x M.  B as given is K x N (N
+    // contiguous); with TB it is N x K.
     float4 stageA[A_QUADS];
     float4 stageB[B_QUADS];
 
     auto fetch = [&](uint32_t k0) {
-#pragma unroll
-        for (int i = 0; i < A_QUADS; ++i)
-        {
-            const uint32_t q = tid + i * kThreads;
-            const uint32_t r = q >> 2;
-            const uint32_t kq = (q & 3) * 4;
-            const uint32_t gr = rowBase + r;
-            const uint32_t gk = k0 + kq;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (gr < M)
-            {
-                const float* p = A + static_cast<size_t>(gr) * K + gk;
-                if (VEC)
-                {
-                    if (gk < K)
-                        v = *reinterpret_cast<const float4*>(p);
-                }
-                else
-                {
-                    if (gk + 0 < K) v.x = p[0];
-                    if (gk + 1 < K) v.y = p[1];
-                    if (gk + 2 < K) v.z = p[2];
-                    if (gk + 3 < K) v.w = p[3];
-                }
-            }
-            stageA[i] = v;
-        }
-#pragma unroll
-        for (int i = 0; i < B_QUADS; ++i)
-        {
-            const uint32_t q = tid + i * kThreads;
-            const uint32_t kr = q / (BN / 4);
-            const uint32_t nq = (q % (BN / 4)) * 4;
-            const uint32_t gk = k0 + kr;
-            const uint32_t gc = colBase + nq;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (gk < K)
-            {
-                const float* p = B + static_cast<size_t>(gk) * N + gc;
-                if (VEC)
-                {
-                    if (gc < N)
-                        v = *reinterpret_cast<const float4*>(p);
-                }
-                else
-                {
-                    if (gc + 0 < N) v.x = p[0];
-                    if (gc + 1 < N) v.y = p[1];
-                    if (gc + 2 < N) v.z = p[2];
-                    if (gc + 3 < N) v.w = p[3];
-                }
-            }
-            stageB[i] = v;
-        }
+        if constexpr (TA)
+            FetchXContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K);
+        else
+            FetchKContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K);
+        if constexpr (TB)
+            FetchKContig<BN, B_QUADS, VEC>(stageB, B, tid, colBase, N, k0, K);
+        else
+            FetchXContig<BN, B_QUADS, VEC>(stageB, B, tid, colBase, N, k0, K);
     };
 
     auto stash = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < A_QUADS; ++i)
-        {
-            const uint32_t q = tid + i * kThreads;
-            const uint32_t r = q >> 2;
-            const uint32_t kq = (q & 3) * 4;
-            float* dst = &As[buf][kq * LDA + r];
-            dst[0 * LDA] = stageA[i].x;
-            dst[1 * LDA] = stageA[i].y;
-            dst[2 * LDA] = stageA[i].z;
-            dst[3 * LDA] = stageA[i].w;
-        }
-#pragma unroll
-        for (int i = 0; i < B_QUADS; ++i)
-        {
-            const uint32_t q = tid + i * kThreads;
-            const uint32_t kr = q / (BN / 4);
-            const uint32_t nq = (q % (BN / 4)) * 4;
-            *reinterpret_cast<float4*>(&Bs[buf][kr * LDB + nq]) = stageB[i];
-        }
+        if constexpr (TA)
+            StashXContig<BM, LDA, A_QUADS>(As[buf], stageA, tid);
+        else
+            StashKContig<BM, LDA, A_QUADS>(As[buf], stageA, tid);
+        if constexpr (TB)
+            StashKContig<BN, LDB, B_QUADS>(Bs[buf], stageB, tid);
+        else
+            StashXContig<BN, LDB, B_QUADS>(Bs[buf], stageB, tid);
     };
 
     floatx16 acc[TM][TN];
@@ -252,6 +298,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
     constexpr int kQuads = TM * TN * 4;
     float4 old[kQuads];
     const bool wide = args.outVec != 0;  // N % 4 == 0 and 16-byte aligned output rows
+    const bool accumulate = args.overwrite == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -262,7 +309,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
                 const uint32_t r = rowBase + waveM * WM + i * 32 + l32;
                 const uint32_t c = colBase + waveN * WN + j * 32 + 8 * q + 4 * khalf;
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (r < M && c < N)
+                if (accumulate && r < M && c < N)
                 {
                     const float* p = out + static_cast<size_t>(r) * N + c;
                     if (wide)
@@ -322,7 +369,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
 // ---------------------------------------------------------------------------
 constexpr int kSkinnyThreads = 256;
 
-template <bool VEC>
+template <bool VEC, bool TA, bool TB>
 __global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const GemmF32Args args)
 {
     __shared__ float partial[3][32 * 32];
@@ -364,7 +411,6 @@ __global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const Gemm
     const uint32_t gBegin = min(wave * perWave, groups);
     const uint32_t gEnd = min(gBegin + perWave, groups);
 
-    const float* aRow = A + static_cast<size_t>(min(row, M - 1)) * K;
     const bool rowOk = row < M;
     const bool colOk = col < N;
 
@@ -373,39 +419,55 @@ __global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const Gemm
     for (int v = 0; v < 16; ++v)
         acc[v] = 0.f;
 
-    // lane half h holds k = 8*g + 4*h + e for e = 0..3
-    auto loadA = [&](uint32_t g) {
+    // Lane half h holds k = 8*g + 4*h + e for e = 0..3.  An operand stored with K contiguous
+    // (A as given, B passed transposed) is read as one 16-byte segment of its row; one stored
+    // k-major (B as given, A passed transposed) as 4 elements `ld` apart.
+    auto loadAlongK = [&](const float* rowPtr, bool ok, uint32_t g) {
         const uint32_t k = g * 8 + khalf * 4;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (rowOk)
+        if (ok)
         {
             if (VEC)
             {
                 if (k < K)
-                    v = *reinterpret_cast<const float4*>(aRow + k);
+                    v = *reinterpret_cast<const float4*>(rowPtr + k);
             }
             else
             {
-                if (k + 0 < K) v.x = aRow[k + 0];
-                if (k + 1 < K) v.y = aRow[k + 1];
-                if (k + 2 < K) v.z = aRow[k + 2];
-                if (k + 3 < K) v.w = aRow[k + 3];
+                if (k + 0 < K) v.x = rowPtr[k + 0];
+                if (k + 1 < K) v.y = rowPtr[k + 1];
+                if (k + 2 < K) v.z = rowPtr[k + 2];
+                if (k + 3 < K) v.w = rowPtr[k + 3];
             }
         }
         return v;
     };
-    auto loadB = [&](uint32_t g) {
+    auto loadAcrossK = [&](const float* colPtr, size_t ld, bool ok, uint32_t g) {
         const uint32_t k = g * 8 + khalf * 4;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (colOk)
+        if (ok)
         {
-            const float* p = B + static_cast<size_t>(k) * N + col;
+            const float* p = colPtr + static_cast<size_t>(k) * ld;
             if (k + 0 < K) v.x = p[0];
-            if (k + 1 < K) v.y = p[static_cast<size_t>(N)];
-            if (k + 2 < K) v.z = p[2 * static_cast<size_t>(N)];
-            if (k + 3 < K) v.w = p[3 * static_cast<size_t>(N)];
+            if (k + 1 < K) v.y = p[ld];
+            if (k + 2 < K) v.z = p[2 * ld];
+            if (k + 3 < K) v.w = p[3 * ld];
         }
         return v;
+    };
+    const float* aPtr = TA ? A + min(row, M - 1) : A + static_cast<size_t>(min(row, M - 1)) * K;
+    const float* bPtr = TB ? B + static_cast<size_t>(min(col, N - 1)) * K : B + min(col, N - 1);
+    auto loadA = [&](uint32_t g) {
+        if constexpr (TA)
+            return loadAcrossK(aPtr, M, rowOk, g);
+        else
+            return loadAlongK(aPtr, rowOk, g);
+    };
+    auto loadB = [&](uint32_t g) {
+        if constexpr (TB)
+            return loadAlongK(bPtr, colOk, g);
+        else
+            return loadAcrossK(bPtr, N, colOk, g);
     };
 
     constexpr int kDepth = 4;  // groups in flight
@@ -468,7 +530,14 @@ __global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const Gemm
         if (c >= N)
             continue;
         float* p = out + static_cast<size_t>(row) * N + c;
-        if (wide)
+        if (args.overwrite)
+        {
+            p[0] = acc[4 * q + 0];
+            if (c + 1 < N) p[1] = acc[4 * q + 1];
+            if (c + 2 < N) p[2] = acc[4 * q + 2];
+            if (c + 3 < N) p[3] = acc[4 * q + 3];
+        }
+        else if (wide)
         {
             float4 v = *reinterpret_cast<const float4*>(p);
             v.x += acc[4 * q + 0];
@@ -503,17 +572,56 @@ struct EntryTable
 std::mutex gTableMutex;
 EntryTable gTables[16];
 
+template <bool TA, bool TB>
+void LaunchSkinny(const GemmF32Args& args, dim3 grid, bool vec, hipStream_t stream)
+{
+    if (vec)
+        hipLaunchKernelGGL((GemmF32SkinnyKernel<true, TA, TB>), grid, dim3(kSkinnyThreads), 0,
+                           stream, args);
+    else
+        hipLaunchKernelGGL((GemmF32SkinnyKernel<false, TA, TB>), grid, dim3(kSkinnyThreads), 0,
+                           stream, args);
+}
+
+template <bool TA, bool TB>
+void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, hipStream_t stream)
+{
+    const dim3 block(kThreads);
+    if (big)
+    {
+        if (vec)
+            hipLaunchKernelGGL((GemmF32Kernel<128, 128, true, TA, TB>), grid, block, 0, stream,
+                               args);
+        else
+            hipLaunchKernelGGL((GemmF32Kernel<128, 128, false, TA, TB>), grid, block, 0, stream,
+                               args);
+    }
+    else
+    {
+        if (vec)
+            hipLaunchKernelGGL((GemmF32Kernel<64, 64, true, TA, TB>), grid, block, 0, stream,
+                               args);
+        else
+            hipLaunchKernelGGL((GemmF32Kernel<64, 64, false, TA, TB>), grid, block, 0, stream,
+                               args);
+    }
+}
+
+// `transA`: A is stored K x M; `transB`: B is stored N x K.
 int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOffsetsAligned,
-           hipStream_t stream)
+           bool transA, bool transB, hipStream_t stream)
 {
     GemmF32Args args = base;
     args.outVec = (outOffsetsAligned && (args.N % 4 == 0) &&
                    (reinterpret_cast<uintptr_t>(args.out) & 15u) == 0)
                       ? 1u
                       : 0u;
-    const bool aligned =
-        allowVector && (args.K % 4 == 0) && (args.N % 4 == 0) &&
+    const bool basesAligned =
         ((reinterpret_cast<uintptr_t>(args.A) | reinterpret_cast<uintptr_t>(args.B)) & 15u) == 0;
+    // row lengths of the two operands as stored
+    const uint32_t lda = transA ? args.M : args.K;
+    const uint32_t ldb = transB ? args.K : args.N;
+    const bool aligned = allowVector && basesAligned && (lda % 4 == 0) && (ldb % 4 == 0);
 
     // few 64 x 64 tiles and a long K: split K inside the workgroup instead
     const uint64_t tiles64 =
@@ -524,14 +632,20 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         args.tilesN = (args.N + 31) / 32;
         const uint64_t blocks32 = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
         const dim3 grid32(static_cast<uint32_t>(blocks32));
-        const bool aVec = allowVector && (args.K % 4 == 0) &&
-                          (reinterpret_cast<uintptr_t>(args.A) & 15u) == 0;
-        if (aVec)
-            hipLaunchKernelGGL(GemmF32SkinnyKernel<true>, grid32, dim3(kSkinnyThreads), 0, stream,
-                               args);
+        // 16-byte loads are used only for operands stored with K contiguous
+        bool kVec = allowVector && (args.K % 4 == 0);
+        if (!transA)
+            kVec = kVec && (reinterpret_cast<uintptr_t>(args.A) & 15u) == 0;
+        if (transB)
+            kVec = kVec && (reinterpret_cast<uintptr_t>(args.B) & 15u) == 0;
+        if (transA && transB)
+            LaunchSkinny<true, true>(args, grid32, kVec, stream);
+        else if (transA)
+            LaunchSkinny<true, false>(args, grid32, false, stream);
+        else if (transB)
+            LaunchSkinny<false, true>(args, grid32, kVec, stream);
         else
-            hipLaunchKernelGGL(GemmF32SkinnyKernel<false>, grid32, dim3(kSkinnyThreads), 0, stream,
-                               args);
+            LaunchSkinny<false, false>(args, grid32, kVec, stream);
         SPH_CHECK_LAUNCH();
         return SPH_OK;
     }
@@ -547,21 +661,14 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         return sph::Fail(SPH_ERR_INVALID, "sph_gemm_f32 - too many tiles for one launch");
 
     const dim3 grid(static_cast<uint32_t>(blocks));
-    const dim3 block(kThreads);
-    if (big)
-    {
-        if (aligned)
-            hipLaunchKernelGGL((GemmF32Kernel<128, 128, true>), grid, block, 0, stream, args);
-        else
-            hipLaunchKernelGGL((GemmF32Kernel<128, 128, false>), grid, block, 0, stream, args);
-    }
+    if (transA && transB)
+        LaunchTiled<true, true>(args, grid, big, aligned, stream);
+    else if (transA)
+        LaunchTiled<true, false>(args, grid, big, aligned, stream);
+    else if (transB)
+        LaunchTiled<false, true>(args, grid, big, aligned, stream);
     else
-    {
-        if (aligned)
-            hipLaunchKernelGGL((GemmF32Kernel<64, 64, true>), grid, block, 0, stream, args);
-        else
-            hipLaunchKernelGGL((GemmF32Kernel<64, 64, false>), grid, block, 0, stream, args);
-    }
+        LaunchTiled<false, false>(args, grid, big, aligned, stream);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
@@ -596,13 +703,18 @@ int GrowTable(EntryTable& t, size_t count)
 
 extern "C" {
 
-int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M, uint32_t N, uint32_t K,
-                 uint32_t batch, int64_t strideOut, int64_t strideA, int64_t strideB)
+int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M, uint32_t N,
+                    uint32_t K, uint32_t batch, int64_t strideOut, int64_t strideA,
+                    int64_t strideB, uint32_t flags)
 {
     SPH_REQUIRE(M != 0 && N != 0 && batch != 0, "M, N and batch must be non-zero");
-    if (K == 0)
+    SPH_REQUIRE((flags & ~(SPH_GEMM_OVERWRITE | SPH_GEMM_TRANS_A | SPH_GEMM_TRANS_B)) == 0,
+                "unknown flag");
+    const bool overwrite = (flags & SPH_GEMM_OVERWRITE) != 0;
+    if (K == 0 && !overwrite)
         return SPH_OK;
-    SPH_REQUIRE(out != nullptr && A != nullptr && B != nullptr, "null pointer");
+    SPH_REQUIRE(out != nullptr, "null pointer");
+    SPH_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "null pointer");
     SPH_REQUIRE(strideOut >= 0 && strideA >= 0 && strideB >= 0, "negative stride");
     SPH_REQUIRE(batch == 1 || strideOut >= static_cast<int64_t>(M) * N,
                 "output matrices of a batch must not overlap");
@@ -618,11 +730,20 @@ int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M, uint32_
     args.M = M;
     args.N = N;
     args.K = K;
+    args.overwrite = overwrite ? 1u : 0u;
     args.strideOut = strideOut;
     args.strideA = strideA;
     args.strideB = strideB;
     const bool stridesAligned = (strideA % 4 == 0) && (strideB % 4 == 0);
-    return Launch(args, batch, stridesAligned, strideOut % 4 == 0 || batch == 1, stream);
+    return Launch(args, batch, stridesAligned, strideOut % 4 == 0 || batch == 1,
+                  (flags & SPH_GEMM_TRANS_A) != 0, (flags & SPH_GEMM_TRANS_B) != 0, stream);
+}
+
+int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M, uint32_t N, uint32_t K,
+                 uint32_t batch, int64_t strideOut, int64_t strideA, int64_t strideB)
+{
+    return sph_gemm_f32_ex(out, A, B, M, N, K, batch, strideOut, strideA, strideB,
+                           SPH_GEMM_ACCUMULATE);
 }
 
 int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out, const float* A,
@@ -681,7 +802,7 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
         args.M = M;
         args.N = N;
         args.K = K;
-        const int rc = Launch(args, end - begin, offsetsAligned, outAligned, stream);
+        const int rc = Launch(args, end - begin, offsetsAligned, outAligned, false, false, stream);
         if (rc != SPH_OK)
             return rc;
         begin = end;

@@ -3,6 +3,7 @@
 #include <Sapphire/compute/BroadcastPlan.hpp>
 #include <Sapphire/compute/dense/cuda/Gemm.hpp>
 
+#include <algorithm>
 #include <stdexcept>
 #include <string>
 
@@ -91,5 +92,44 @@ void ReLU(TensorData& y, const TensorData& x)
     RequireSameMode(y, x, "ReLU");
     RequireDeviceMode(y, "ReLU");
     Dense::Cuda::ReLU(y.CudaMutableRawPtr(), x.CudaRawPtr(), static_cast<unsigned int>(y.Size()));
+}
+
+void ReLUBackward(TensorData& dx, const TensorData& dy, const TensorData& x)
+{
+    RequireSameMode(dx, dy, "ReLUBackward");
+    RequireSameMode(dx, x, "ReLUBackward");
+    RequireDeviceMode(dx, "ReLUBackward");
+    Dense::Cuda::ReLUBackward(dx.CudaMutableRawPtr(), dy.CudaRawPtr(), x.CudaRawPtr(),
+                              static_cast<unsigned int>(dx.Size()));
+}
+
+void Scale(TensorData& y, const TensorData& x, const float factor)
+{
+    RequireSameMode(y, x, "Scale");
+    RequireDeviceMode(y, "Scale");
+    Dense::Cuda::Scale(y.CudaMutableRawPtr(), x.CudaRawPtr(), factor,
+                       static_cast<unsigned int>(y.GetShape().Size()));
+}
+
+void Sub(TensorData& y, const TensorData& a, const TensorData& b)
+{
+    RequireSameMode(y, a, "Sub");
+    RequireSameMode(y, b, "Sub");
+    RequireDeviceMode(y, "Sub");
+
+    Shape shapeOut = y.GetShape(), shapeA = a.GetShape(), shapeB = b.GetShape();
+    const int maxDim = std::max({ shapeOut.Dim(), shapeA.Dim(), shapeB.Dim() });
+    shapeOut.Expand(maxDim);
+    shapeA.Expand(maxDim);
+    shapeB.Expand(maxDim);
+    const int leafDim = GetMatchingDim({ shapeOut, shapeA, shapeB });
+
+    const auto leaves = PlanBroadcastWith2Inputs(
+        shapeOut, shapeA, shapeB, static_cast<unsigned int>(shapeOut.Size()),
+        static_cast<unsigned int>(shapeA.Size()), static_cast<unsigned int>(shapeB.Size()), 0,
+        static_cast<unsigned int>(leafDim));
+    for (const BroadcastLeaf& leaf : leaves)
+        Dense::Cuda::Sub(leaf.totalSizeOut, y.CudaMutableRawPtr() + leaf.outOff,
+                         a.CudaRawPtr() + leaf.aOff, b.CudaRawPtr() + leaf.bOff, 0, false, false);
 }
 }  // namespace Sapphire::Compute

@@ -1,6 +1,7 @@
 #include <Sapphire/compute/BroadcastPlan.hpp>
 
 #include <algorithm>
+#include <stdexcept>
 
 namespace Sapphire::Compute
 {
@@ -65,6 +66,28 @@ std::vector<BroadcastLeaf> PlanBroadcastWith2Inputs(const Shape& yShape, const S
     const Walker walker{ yShape, aShape, bShape, limit, leaves };
     walker.Visit(totalSizeOut, totalSizeA, totalSizeB, 0, 0, 0, shapeIdx);
     return leaves;
+}
+
+int GetMatchingDim(const std::vector<Shape>& shapes)
+{
+    if (shapes.empty())
+        throw std::runtime_error("Util::GetMatchingDim - shapes is empty");
+    // count trailing positions that exist in every shape and hold the same extent
+    int matched = 0;
+    for (;;)
+    {
+        const int fromLast = matched + 1;
+        bool agree = true;
+        for (const Shape& shape : shapes)
+            if (shape.Dim() < fromLast || shape.At(-fromLast) != shapes.front().At(-fromLast))
+            {
+                agree = false;
+                break;
+            }
+        if (!agree)
+            return matched;
+        ++matched;
+    }
 }
 
 GemmPlan PlanGemm(const Shape& y, const Shape& a, const Shape& b)

@@ -72,6 +72,20 @@ void GemmHalf(float* out, const std::uint16_t* A, const std::uint16_t* B, unsign
           "GemmHalf");
 }
 
+void GemmTransposed(float* out, const float* A, const float* B, unsigned int M, unsigned int N,
+                    unsigned int K, unsigned int batchSize, bool transposeA, bool transposeB,
+                    bool overwrite, int deviceId)
+{
+    Compute::Cuda::CudaSetDevice(deviceId);
+    const std::uint32_t flags = (transposeA ? SPH_GEMM_TRANS_A : 0u) |
+                                (transposeB ? SPH_GEMM_TRANS_B : 0u) |
+                                (overwrite ? SPH_GEMM_OVERWRITE : SPH_GEMM_ACCUMULATE);
+    Check(sph_gemm_f32_ex(out, A, B, M, N, K, batchSize, static_cast<std::int64_t>(M) * N,
+                          static_cast<std::int64_t>(M) * K, static_cast<std::int64_t>(K) * N,
+                          flags),
+          "GemmTransposed");
+}
+
 void ConvertToHalf(std::uint16_t* dst, const float* src, std::size_t size)
 {
     Check(sph_convert_f32_to_f16(dst, src, size), "ConvertToHalf");
@@ -80,6 +94,29 @@ void ConvertToHalf(std::uint16_t* dst, const float* src, std::size_t size)
 void ReLU(float* y, const float* x, unsigned int totalSize)
 {
     Check(sph_relu_f32(y, x, totalSize), "ReLU");
+}
+
+void ReLUBackward(float* dx, const float* dy, const float* x, unsigned int totalSize)
+{
+    Check(sph_relu_backward_f32(dx, dy, x, totalSize), "ReLUBackward");
+}
+
+void Scale(float* y, const float* x, float factor, unsigned int totalSize)
+{
+    Check(sph_scale_f32(y, x, factor, totalSize), "Scale");
+}
+
+void Sub(unsigned int totalSize, float* out, const float* A, const float* B,
+         unsigned int inputStride, bool broadcastInputA, bool broadcastInputB)
+{
+    Check(sph_sub_f32(out, A, B, totalSize, inputStride, broadcastInputA ? 1 : 0,
+                      broadcastInputB ? 1 : 0),
+          "Sub");
+}
+
+void SgdStep(float* z, const float* dz, float learningRate, unsigned int totalSize)
+{
+    Check(sph_sgd_step_f32(z, dz, learningRate, totalSize), "SgdStep");
 }
 
 void Transpose(float* y, const float* x, unsigned int inputNumRows, unsigned int inputNumCols,

@@ -24,6 +24,17 @@ void Transpose(TensorData& y, const TensorData& x);
 
 //! y = x > 0 ? x : 0 (Sources/Sapphire/compute/ActivationOps.cpp:52-67).
 void ReLU(TensorData& y, const TensorData& x);
+
+//! dx += x > 0 ? dy : 0 (Sources/Sapphire/compute/ActivationOps.cpp:69-85).
+void ReLUBackward(TensorData& dx, const TensorData& dy, const TensorData& x);
+
+//! y = x * factor over y's element count (Sources/Sapphire/compute/BasicOps.cpp:250-267).
+void Scale(TensorData& y, const TensorData& x, float factor);
+
+//! y = a - b.  The trailing dimensions on which the three shapes agree form one leaf; the
+//! leading ones are walked by BroadcastWith2Inputs, operands offset by
+//! (index % extent) * stride (Sources/Sapphire/compute/BasicOps.cpp:63-103).
+void Sub(TensorData& y, const TensorData& a, const TensorData& b);
 }  // namespace Sapphire::Compute
 
 #endif

@@ -36,6 +36,10 @@ std::vector<BroadcastLeaf> PlanBroadcastWith2Inputs(const Shape& yShape, const S
                                                     unsigned int shapeIdx,
                                                     unsigned int minimumRequiredDim);
 
+//! Number of trailing dimensions on which every shape agrees
+//! (Includes/Sapphire/util/UnitUtils.hpp:38-73).  Throws std::runtime_error for an empty list.
+int GetMatchingDim(const std::vector<Shape>& shapes);
+
 //! Shape bookkeeping of Compute::Gemm (Sources/Sapphire/compute/BasicOps.cpp:189-230).
 struct GemmPlan
 {

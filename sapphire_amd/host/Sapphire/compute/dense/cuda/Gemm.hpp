@@ -38,11 +38,32 @@ void GemmHalf(float* out, const std::uint16_t* A, const std::uint16_t* B, unsign
               unsigned int N, unsigned int K, unsigned int batchSize, std::size_t strideOut,
               std::size_t strideA, std::size_t strideB, bool overwrite, int deviceId);
 
+//! out[b] (+)= op(A[b]) * op(B[b]) with operands that may be stored transposed (A as K x M, B
+//! as N x K), so that the backward products need no materialised transpose; matrices packed
+//! back to back.  `overwrite` stores the product without reading out.
+void GemmTransposed(float* out, const float* A, const float* B, unsigned int M, unsigned int N,
+                    unsigned int K, unsigned int batchSize, bool transposeA, bool transposeB,
+                    bool overwrite, int deviceId);
+
 //! dst[i] = binary16(src[i]), round to nearest even.
 void ConvertToHalf(std::uint16_t* dst, const float* src, std::size_t size);
 
 //! y = x > 0 ? x : 0 (Sources/Sapphire/compute/dense/cuda/Activation.cu, ReLU).
 void ReLU(float* y, const float* x, unsigned int totalSize);
+
+//! dx += x > 0 ? dy : 0 (Sources/Sapphire/compute/ActivationOps.cpp:69-85).
+void ReLUBackward(float* dx, const float* dy, const float* x, unsigned int totalSize);
+
+//! y = x * factor (device leaf of Compute::Scale, Sources/Sapphire/compute/BasicOps.cpp:250-267).
+void Scale(float* y, const float* x, float factor, unsigned int totalSize);
+
+//! Leaf of Compute::Sub with the reference's argument order
+//! (Sources/Sapphire/compute/dense/naive/NaiveBasic.cpp:28-39).
+void Sub(unsigned int totalSize, float* out, const float* A, const float* B,
+         unsigned int inputStride, bool broadcastInputA, bool broadcastInputB);
+
+//! z -= dz * learningRate in one pass, with the rounding of Scale followed by Sub.
+void SgdStep(float* z, const float* dz, float learningRate, unsigned int totalSize);
 
 //! Batched 2-D transpose (Sources/Sapphire/compute/dense/cuda/Basic.cu:85-102).
 void Transpose(float* y, const float* x, unsigned int inputNumRows, unsigned int inputNumCols,

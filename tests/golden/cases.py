@@ -44,3 +44,21 @@ KAT_GEMM_CASES = [
 ]
 
 SHAPE_CASES = [[5], [3, 4], [2, 3, 4], [2, 3, 4, 5], [1, 1, 6], [7, 1], [2, 2, 2, 2, 2]]
+
+# Compute::Sub host branch: (name, y shape, a shape, b shape, seed)
+SUB_CASES = [
+    ("equal", [6, 5], [6, 5], [6, 5], 200),
+    ("vector", [37], [37], [37], 210),
+    ("b_repeats", [4, 3, 5], [4, 3, 5], [1, 3, 5], 220),
+    ("a_repeats", [2, 3, 4, 5], [1, 1, 4, 5], [2, 3, 4, 5], 230),
+    ("missing_dim", [3, 4, 5], [3, 4, 5], [4, 5], 240),
+    ("last_differs", [3, 4], [3, 4], [3, 1], 250),
+]
+
+# Dense::Naive::Sub leaf: (name, totalSize, inputStride, broadcastA, broadcastB, seed)
+SUB_LEAF_CASES = [
+    ("plain", 101, 0, False, False, 300),
+    ("wrap_a", 60, 12, True, False, 310),
+    ("wrap_b", 60, 5, False, True, 320),
+    ("wrap_both", 64, 16, True, True, 330),
+]

@@ -8,6 +8,8 @@ and Broadcast.hpp.  The fixtures are data only (shapes, seeds, offsets, output b
     naive_gemm_kat.npz   outputs of Dense::Naive::Gemm / the Compute::Gemm host branch /
                          Naive::ReLU / Naive::Transpose on seeded inputs (the inputs are
                          regenerated from the seeds by sapphire_amd.synth)
+    backward_kat.npz     outputs of Naive::Scale / Sub / ReLUBackward and of the Compute::Sub
+                         host branch on seeded inputs
     shape_ops.json       Shape::Expand / Shrink / Rows / Cols / Size / GetNumUnits results
 
     python tests/golden/make_golden.py
@@ -24,7 +26,8 @@ sys.path.insert(0, ROOT)
 
 from oracle import pyoracle as po  # noqa: E402
 from sapphire_amd import synth  # noqa: E402
-from tests.golden.cases import PLAN_CASES, KAT_GEMM_CASES, KAT_OP_CASES, SHAPE_CASES  # noqa: E402
+from tests.golden.cases import (PLAN_CASES, KAT_GEMM_CASES, KAT_OP_CASES, SHAPE_CASES,  # noqa: E402
+                                SUB_CASES, SUB_LEAF_CASES)
 
 
 def main():
@@ -62,6 +65,28 @@ def main():
     r.ref_transpose(po._f(t_out), po._f(t_in), 5, 7, 3, 0)
     kat["transpose"] = t_out
     np.savez_compressed(os.path.join(HERE, "naive_gemm_kat.npz"), **kat)
+
+    back = {}
+    x = synth.normal(950, (1003,))
+    y = np.empty_like(x)
+    r.ref_scale(po._f(y), po._f(x), 0.37, x.size)
+    back["scale"] = y
+    dx = synth.uniform(951, (1003,))
+    dy = synth.uniform(952, (1003,))
+    out = dx.copy()
+    r.ref_relu_backward(po._f(out), po._f(dy), po._f(x), x.size)
+    back["relu_backward"] = out
+    for name, count, stride, bca, bcb, seed in SUB_LEAF_CASES:
+        a = synth.uniform(seed + 1, (count,))
+        b = synth.uniform(seed + 2, (count,))
+        out = np.empty(count, np.float32)
+        r.ref_sub(count, po._f(out), po._f(a), po._f(b), stride, int(bca), int(bcb))
+        back["subleaf_" + name] = out
+    for name, ys, as_, bs, seed in SUB_CASES:
+        a = synth.uniform(seed + 1, as_)
+        b = synth.uniform(seed + 2, bs)
+        back["sub_" + name] = po.compute_sub(ys, a, b, lib="ref")
+    np.savez_compressed(os.path.join(HERE, "backward_kat.npz"), **back)
 
     shapes = []
     for dims in SHAPE_CASES:

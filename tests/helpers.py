@@ -77,3 +77,28 @@ def gpu_spmm(C, V, COL, ROW, M, Kdim, N, B, accumulate, canary=0):
         assert np.array_equal(back[:canary], guard), "write before the start of out"
         assert np.array_equal(back[-canary:], guard), "write past the end of out"
     return back[canary:canary + C.size].reshape(C.shape)
+
+
+def gpu_gemm_f32_ex(C, A, B, M, N, K, flags, batch=1, stride_out=None, stride_a=None,
+                    stride_b=None):
+    """sph_gemm_f32_ex on numpy operands exactly as stored (A is K x M with SPH_GEMM_TRANS_A,
+    B is N x K with SPH_GEMM_TRANS_B)."""
+    so = M * N if stride_out is None else stride_out
+    sa = M * K if stride_a is None else stride_a
+    sb = K * N if stride_b is None else stride_b
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    capi.call("sph_gemm_f32_ex", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, so, sa, sb, flags)
+    out = dC.download(np.float32, C.shape)
+    for d in (dA, dB, dC):
+        d.release()
+    return out
+
+
+def gpu_transpose(x, rows, cols, batch=1):
+    dX = capi.DeviceBuffer.from_array(x)
+    dY = capi.DeviceBuffer(x.nbytes)
+    capi.call("sph_transpose_f32", dY.ptr, dX.ptr, rows, cols, batch, 0)
+    out = dY.download(np.float32, (batch, cols, rows))
+    dX.release()
+    dY.release()
+    return out

@@ -9,6 +9,7 @@
 #include <Sapphire/compute/Initialize.hpp>
 #include <Sapphire/compute/cudaUtil/Memory.hpp>
 #include <Sapphire/compute/sparse/SparseGemm.hpp>
+#include <Sapphire/operations/Backward/LinearBackward.hpp>
 #include <Sapphire/operations/Forward/LinearForward.hpp>
 #include <Sapphire/util/ResourceManager.hpp>
 
@@ -209,6 +210,96 @@ int sphh_transpose(float* yData, const int* y, int yn, const float* xData, const
         TensorData Y(MakeShape(y, yn), Type::Dense, cuda);
         Compute::Transpose(Y, X);
         Download(Y, yData);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// Util::GetMatchingDim over `count` shapes stored back to back, dims[i] extents each
+int sphh_matching_dim(const int* flat, const int* dims, int count)
+{
+    int result = -1;
+    const int rc = Guard([&] {
+        std::vector<Shape> shapes;
+        for (int i = 0; i < count; ++i)
+        {
+            shapes.push_back(MakeShape(flat, dims[i]));
+            flat += dims[i];
+        }
+        result = Compute::GetMatchingDim(shapes);
+    });
+    return rc == 0 ? result : -1;
+}
+
+// y = a - b through Compute::Sub in Cuda mode
+int sphh_sub(float* yData, const int* y, int yn, const float* aData, const int* a, int an,
+             const float* bData, const int* b, int bn)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData A = Upload(MakeShape(a, an), aData, cuda);
+        TensorData B = Upload(MakeShape(b, bn), bData, cuda);
+        TensorData Out = Upload(MakeShape(y, yn), yData, cuda);
+        Compute::Sub(Out, A, B);
+        Download(Out, yData);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// y = x * factor through Compute::Scale; inPlace scales x itself
+int sphh_scale(float* yData, const float* xData, int n, float factor, int inPlace)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData X = Upload(Shape({ n }), xData, cuda);
+        if (inPlace)
+        {
+            Compute::Scale(X, X, factor);
+            Download(X, yData);
+        }
+        else
+        {
+            TensorData Y(Shape({ n }), Type::Dense, cuda);
+            Compute::Scale(Y, X, factor);
+            Download(Y, yData);
+        }
+        Util::ResourceManager::Clean();
+    });
+}
+
+// dx (holding dxData on entry) += x > 0 ? dy : 0 through Compute::ReLUBackward
+int sphh_relu_backward(float* dxData, const float* dyData, const float* xData, int n)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData Dx = Upload(Shape({ n }), dxData, cuda);
+        TensorData Dy = Upload(Shape({ n }), dyData, cuda);
+        TensorData X = Upload(Shape({ n }), xData, cuda);
+        Compute::ReLUBackward(Dx, Dy, X);
+        Download(Dx, dxData);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// BackProp::LinearBackward with an SGD optimizer.  dx, weight and bias are updated in place.
+// sequence: 0 the reference's operator calls, 1 direct; fusedSgd selects the one-pass update.
+int sphh_linear_backward(float* dx, float* weight, float* bias, const float* dy, const float* x,
+                         int batch, int inputs, int outputs, float learningRate, int sequence,
+                         int fusedSgd)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData Dx = Upload(Shape({ batch, inputs }), dx, cuda);
+        TensorData W = Upload(Shape({ inputs, outputs }), weight, cuda);
+        TensorData B = Upload(Shape({ outputs }), bias, cuda);
+        TensorData Dy = Upload(Shape({ batch, outputs }), dy, cuda);
+        TensorData X = Upload(Shape({ batch, inputs }), x, cuda);
+        const Optimizer::SGD sgd(learningRate, fusedSgd != 0);
+        BackProp::LinearBackward(Dx, W, B, Dy, X, static_cast<unsigned int>(batch), sgd,
+                                 sequence == 0 ? BackProp::Sequence::Reference
+                                               : BackProp::Sequence::Direct);
+        Download(Dx, dx);
+        Download(W, weight);
+        Download(B, bias);
         Util::ResourceManager::Clean();
     });
 }

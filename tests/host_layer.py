@@ -31,6 +31,14 @@ def lib():
         h.sphh_sparse_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _fp,
                                        ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint),
                                        _fp, ctypes.c_int]
+        h.sphh_matching_dim.argtypes = [_ip, _ip, ctypes.c_int]
+        h.sphh_sub.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int, _fp, _ip,
+                               ctypes.c_int]
+        h.sphh_scale.argtypes = [_fp, _fp, ctypes.c_int, ctypes.c_float, ctypes.c_int]
+        h.sphh_relu_backward.argtypes = [_fp, _fp, _fp, ctypes.c_int]
+        h.sphh_linear_backward.argtypes = [_fp, _fp, _fp, _fp, _fp, ctypes.c_int, ctypes.c_int,
+                                           ctypes.c_int, ctypes.c_float, ctypes.c_int,
+                                           ctypes.c_int]
         h.sphh_shape_op.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip]
         h.sphh_shape_query.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib = h
@@ -111,3 +119,40 @@ def sparse_gemm(y, V, COL, ROW, M, K, N, B, accumulate):
     _ok(lib().sphh_sparse_gemm(_f(out), M, K, N, _f(Vp), Cp.ctypes.data_as(up),
                                ROW.ctypes.data_as(up), _f(B), 1 if accumulate else 0))
     return out
+
+
+def matching_dim(shapes):
+    flat = [d for s in shapes for d in s]
+    n = lib().sphh_matching_dim(_ints(flat), _ints([len(s) for s in shapes]), len(shapes))
+    if n < 0:
+        raise RuntimeError(lib().sphh_last_error().decode())
+    return n
+
+
+def sub(y_shape, a, b):
+    out = np.zeros(y_shape, np.float32)
+    _ok(lib().sphh_sub(_f(out), _ints(y_shape), len(y_shape), _f(np.ascontiguousarray(a)),
+                       _ints(a.shape), a.ndim, _f(np.ascontiguousarray(b)), _ints(b.shape),
+                       b.ndim))
+    return out
+
+
+def scale(x, factor, in_place=False):
+    out = np.zeros_like(x)
+    _ok(lib().sphh_scale(_f(out), _f(x), x.size, factor, 1 if in_place else 0))
+    return out
+
+
+def relu_backward(dx, dy, x):
+    out = np.ascontiguousarray(dx.copy())
+    _ok(lib().sphh_relu_backward(_f(out), _f(dy), _f(x), x.size))
+    return out
+
+
+def linear_backward(dx, W, bias, dy, x, lr, sequence, fused_sgd):
+    """Returns the updated (dx, W, bias)."""
+    dx, W, bias = (np.ascontiguousarray(v.copy()) for v in (dx, W, bias))
+    batch, inputs = x.shape
+    _ok(lib().sphh_linear_backward(_f(dx), _f(W), _f(bias), _f(dy), _f(x), batch, inputs,
+                                   W.shape[1], lr, sequence, 1 if fused_sgd else 0))
+    return dx, W, bias

@@ -157,3 +157,64 @@ def test_tensor_data_life_cycle_on_device(dev):
     lib = hl.lib()
     rc = lib.sphh_tensor_lifecycle()
     assert rc == 0, (rc, lib.sphh_last_error())
+
+
+# ---- backward neighbours and the Linear backward pass -------------------------------------------
+
+def _bits(x):
+    return np.ascontiguousarray(x).view(np.uint32)
+
+
+def test_compute_sub_matches_recorded_reference_outputs(dev):
+    import os
+    from tests.golden.cases import SUB_CASES
+    kat = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                               "backward_kat.npz"))
+    for name, ys, as_, bs, seed in SUB_CASES:
+        h.announce("Compute::Sub", name, ys, as_, bs)
+        a = synth.uniform(seed + 1, as_)
+        b = synth.uniform(seed + 2, bs)
+        assert np.array_equal(_bits(hl.sub(ys, a, b)), _bits(kat["sub_" + name])), name
+
+
+def test_compute_scale_and_relu_backward(dev):
+    h.announce("Compute::Scale / Compute::ReLUBackward")
+    x = synth.normal(5, (3001,))
+    assert np.array_equal(_bits(hl.scale(x, 0.125)), _bits(po.scale(x, 0.125)))
+    assert np.array_equal(_bits(hl.scale(x, -3.3, in_place=True)), _bits(po.scale(x, -3.3)))
+    dx, dy = synth.uniform(6, (3001,)), synth.uniform(7, (3001,))
+    assert np.array_equal(_bits(hl.relu_backward(dx, dy, x)), _bits(po.relu_backward(dx, dy, x)))
+
+
+@pytest.mark.parametrize("dims", [(1, 1, 1), (4, 3, 2), (33, 20, 7), (128, 784, 64),
+                                  (1024, 1024, 10), (256, 100, 300)])
+def test_linear_backward(dev, dims):
+    """Sources/Sapphire/operations/Backward/LinearBackward.cpp:27-99 + SGD on the device against
+    the same call sequence on the CPU.  dx within the fp32 GEMM tolerance; the updated
+    parameters within learningRate x that tolerance (plus one rounding of the parameter)."""
+    batch, fin, fout = dims
+    lr = 0.01
+    h.announce("BackProp::LinearBackward", dims)
+    x = synth.uniform(81, (batch, fin))
+    W = synth.uniform(82, (fin, fout))
+    bias = synth.uniform(83, (fout,))
+    dy = synth.uniform(84, (batch, fout))
+    dx0 = synth.uniform(85, (batch, fin))
+    ref_dx, ref_W, ref_b = po.linear_backward(dx0, W, bias, dy, x, lr, threads=8)
+
+    seq_ref = hl.linear_backward(dx0, W, bias, dy, x, lr, sequence=0, fused_sgd=False)
+    direct = hl.linear_backward(dx0, W, bias, dy, x, lr, sequence=1, fused_sgd=True)
+    # the direct sequence (transposed reads, overwrite, one-pass SGD) changes no bit
+    for got, want in zip(direct, seq_ref):
+        assert np.array_equal(_bits(got), _bits(want))
+
+    dx, W2, b2 = seq_ref
+    den = np.abs(dy).astype(np.float64) @ np.abs(W.T).astype(np.float64)
+    assert h.normalised_error(dx, ref_dx, None, den, is_denominator=True) <= TOL_F32
+    den = np.abs(x.T).astype(np.float64) @ np.abs(dy).astype(np.float64)
+    slack = np.finfo(np.float32).eps * (np.abs(ref_W) + lr * den)
+    assert np.all(np.abs(W2.astype(np.float64) - ref_W) <= lr * TOL_F32 * den + slack)
+    den = np.abs(dy).astype(np.float64).sum(axis=0) / batch
+    slack = np.finfo(np.float32).eps * (np.abs(ref_b) + lr * den)
+    assert np.all(np.abs(b2.astype(np.float64) - ref_b) <= lr * TOL_F32 * den + slack)
+    assert np.any(W2 != W) and np.any(b2 != bias) and np.any(dx != dx0)

@@ -87,3 +87,12 @@ def test_host_life_cycle_and_error_paths():
     assert b"Host mode is not provided" in h.sphh_last_error()
     with pytest.raises(RuntimeError, match="must be greater than zero"):
         hl.shape_op([2, 3], 0, -1)
+
+
+def test_matching_dim_agrees_with_checker():
+    cases = [[[3, 4], [3, 4], [3, 4]], [[2, 3, 4], [1, 3, 4], [2, 3, 4]], [[3, 4], [3, 5]],
+             [[2, 3, 4], [3, 4]], [[5]], [[2, 3, 4], [2, 5, 4]], [[1, 1, 4, 5], [2, 3, 4, 5]]]
+    for shapes in cases:
+        assert hl.matching_dim(shapes) == po.matching_dim(shapes), shapes
+    with pytest.raises(RuntimeError):
+        hl.matching_dim([])

@@ -16,7 +16,8 @@ import pytest
 
 from oracle import pyoracle as po
 from sapphire_amd import synth
-from tests.golden.cases import KAT_GEMM_CASES, KAT_OP_CASES, PLAN_CASES, SHAPE_CASES
+from tests.golden.cases import (KAT_GEMM_CASES, KAT_OP_CASES, PLAN_CASES, SHAPE_CASES, SUB_CASES,
+                                SUB_LEAF_CASES)
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 needs_ref = pytest.mark.skipif(not po.have_ref(), reason="oracle/_ref not built on this machine")
@@ -258,3 +259,124 @@ def test_csr_brute_force_tiny():
     B = np.array([[1, 2], [3, 4], [5, 6]], np.float32)
     out = po.spmm_csr(np.zeros((4, 2), np.float32), V, COL, ROW, 4, 2, B)
     assert out.tolist() == [[2 * 1 - 5, 2 * 2 - 6], [0, 0], [1.5, 2.0], [20, 24]]
+
+
+# ---- backward neighbours --------------------------------------------------------------------
+
+def test_backward_leaves_match_recorded_reference_outputs():
+    kat = np.load(os.path.join(GOLDEN, "backward_kat.npz"))
+    x = synth.normal(950, (1003,))
+    assert np.array_equal(bits(po.scale(x, 0.37)), bits(kat["scale"]))
+    dx = synth.uniform(951, (1003,))
+    dy = synth.uniform(952, (1003,))
+    assert np.array_equal(bits(po.relu_backward(dx, dy, x)), bits(kat["relu_backward"]))
+    for name, count, stride, bca, bcb, seed in SUB_LEAF_CASES:
+        a = synth.uniform(seed + 1, (count,))
+        b = synth.uniform(seed + 2, (count,))
+        assert np.array_equal(bits(po.sub_leaf(a, b, count, stride, bca, bcb)),
+                              bits(kat["subleaf_" + name])), name
+    for name, ys, as_, bs, seed in SUB_CASES:
+        a = synth.uniform(seed + 1, as_)
+        b = synth.uniform(seed + 2, bs)
+        assert np.array_equal(bits(po.compute_sub(ys, a, b)), bits(kat["sub_" + name])), name
+
+
+@needs_ref
+def test_backward_leaves_bit_exact_against_reference_objects():
+    r = po.ref()
+    for n in (1, 7, 4096):
+        x = synth.normal(n, (n,))
+        dy = synth.uniform(n + 1, (n,))
+        dx = synth.uniform(n + 2, (n,))
+        want = np.empty_like(x)
+        r.ref_scale(po._f(want), po._f(x), -1.25, n)
+        assert np.array_equal(bits(po.scale(x, -1.25)), bits(want))
+        want = dx.copy()
+        r.ref_relu_backward(po._f(want), po._f(dy), po._f(x), n)
+        assert np.array_equal(bits(po.relu_backward(dx, dy, x)), bits(want))
+    for name, ys, as_, bs, seed in SUB_CASES:
+        a = synth.uniform(seed + 5, as_)
+        b = synth.uniform(seed + 6, bs)
+        assert np.array_equal(bits(po.compute_sub(ys, a, b)),
+                              bits(po.compute_sub(ys, a, b, lib="ref"))), name
+
+
+def test_backward_closed_forms():
+    x = np.array([-2.0, -0.0, 0.0, 1e-30, 3.0], np.float32)
+    dy = np.array([10, 20, 30, 40, 50], np.float32)
+    dx = np.ones(5, np.float32)
+    assert po.relu_backward(dx, dy, x).tolist() == [1, 1, 1, 41, 51]      # strict x > 0, adds
+    assert po.scale(np.array([1.5, -4.0], np.float32), 2.0).tolist() == [3.0, -8.0]
+    a = np.arange(6, dtype=np.float32)
+    b = np.array([10, 20], np.float32)
+    # b wraps every inputStride = 2 elements; a does not
+    assert po.sub_leaf(a, b, 6, 2, False, True).tolist() == [-10, -19, -8, -17, -6, -15]
+    # Compute::Sub with equal shapes is elementwise; with b one matrix short it repeats b
+    a3 = synth.uniform(1, (4, 3, 5))
+    b3 = synth.uniform(2, (3, 5))
+    assert np.array_equal(po.compute_sub([4, 3, 5], a3, a3), np.zeros((4, 3, 5), np.float32))
+    assert np.array_equal(po.compute_sub([4, 3, 5], a3, b3), a3 - b3[None])
+
+
+def test_matching_dim_hand_table():
+    table = [
+        ([[3, 4], [3, 4], [3, 4]], 2),
+        ([[2, 3, 4], [1, 3, 4], [2, 3, 4]], 2),       # leading extent differs
+        ([[3, 4], [3, 5]], 0),                        # last extent differs
+        ([[2, 3, 4], [3, 4]], 2),                     # shorter shape stops the count
+        ([[5]], 1),
+        ([[2, 7, 4], [9, 7, 4], [2, 7, 4]], 2),
+        ([[2, 3, 4], [2, 5, 4]], 1),
+    ]
+    for shapes, want in table:
+        assert po.matching_dim(shapes) == want, shapes
+    assert po.matching_dim([]) == -1
+
+
+def test_sgd_rounds_the_product_before_subtracting():
+    # z - fl(dz*lr) differs from the fused z - dz*lr in the last bit for these values
+    z = np.array([1.9026086330413818], np.float32)
+    dz = np.array([1.7237802743911743], np.float32)
+    lr = np.float32(0.5041077733039856)
+    prod = np.float32(dz[0] * lr)                       # rounded to fp32
+    want = np.float32(z[0] - prod)
+    fused = np.float32(np.float64(z[0]) - np.float64(dz[0]) * np.float64(lr))
+    assert want != fused
+    assert po.sgd(z, dz, float(lr))[0] == want
+
+
+def test_linear_backward_closed_form_and_composition():
+    batch, fin, fout, lr = 4, 3, 2, 0.5
+    # one-hot x and dy: x = e0 rows, dy = e1 rows -> dw = batch at [0][1], dB = [0, 1]
+    x = np.zeros((batch, fin), np.float32)
+    x[:, 0] = 1
+    dy = np.zeros((batch, fout), np.float32)
+    dy[:, 1] = 1
+    W = np.arange(fin * fout, dtype=np.float32).reshape(fin, fout)
+    bias = np.array([1.0, 2.0], np.float32)
+    dx0 = np.full((batch, fin), 0.25, np.float32)
+    dx, W2, b2 = po.linear_backward(dx0, W, bias, dy, x, lr)
+    assert np.array_equal(dx, dx0 + W[:, 1][None, :])                     # dy * W^T, W before update
+    wantW = W.copy()
+    wantW[0, 1] -= lr * batch
+    assert np.array_equal(W2, wantW)
+    assert np.array_equal(b2, np.array([1.0, 2.0 - lr], np.float32))
+    # composition out of the pinned parts on seeded data
+    batch, fin, fout = 9, 7, 5
+    x = synth.uniform(31, (batch, fin))
+    dy = synth.uniform(32, (batch, fout))
+    W = synth.uniform(33, (fin, fout))
+    bias = synth.uniform(34, (fout,))
+    dx0 = synth.uniform(35, (batch, fin))
+    dx, W2, b2 = po.linear_backward(dx0, W, bias, dy, x, 0.01)
+    wt = po.transpose(W, fin, fout, 1).reshape(fout, fin)
+    assert np.array_equal(bits(dx), bits(po.naive_gemm(dx0.copy(), dy, wt, batch, fin, fout)))
+    xt = po.transpose(x, batch, fin, 1).reshape(fin, batch)
+    dw = po.naive_gemm(np.zeros((fin, fout), np.float32), xt, dy, fin, fout, batch)
+    assert np.array_equal(bits(W2), bits(po.sgd(W, dw, 0.01)))
+    dB = po.naive_gemm(np.zeros((1, fout), np.float32), np.ones((1, batch), np.float32), dy, 1,
+                       fout, batch)
+    dB = po.scale(dB, np.float32(1.0) / np.float32(batch))
+    assert np.array_equal(bits(b2), bits(po.sgd(bias, dB.reshape(fout), 0.01)))
+    dxT, WT, bT = po.linear_backward(dx0, W, bias, dy, x, 0.01, threads=3)
+    assert np.array_equal(bits(dxT), bits(dx)) and np.array_equal(bits(WT), bits(W2))
