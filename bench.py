@@ -57,7 +57,7 @@ def parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     p.add_argument("--all", action="store_true",
                    help="also time configurations 1, 2 and 4 (reported under 'others')")
-    p.add_argument("--only", choices=["gemm", "spmm", "copy"], default=None,
+    p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
     return p.parse_args()
 
@@ -164,6 +164,102 @@ def bench_mlp(capi, synth, steps, warmup):
     return event_ms, flops
 
 
+def bench_mlp_backward(capi, synth, steps, warmup, direct):
+    """Backward pass + SGD update of configuration 4's three Linear layers through the C ABI
+    (the call sequence of LinearBackProp::m_runBackProp per layer, ReLUBackward between
+    layers).  direct=False materialises the transposes, zero-fills and uses Scale + Sub like
+    the reference; direct=True uses the transposed-read / overwrite flags and the one-pass SGD
+    step.  Parameters drift over the steps; only time is taken here."""
+    d = synth.config4()
+    batch = d["x"].shape[0]
+    sizes = [d["x"].shape[1]] + [w.shape[1] for w in d["W"]]
+    lr = 1e-6
+    W = [capi.DeviceBuffer.from_array(w) for w in d["W"]]
+    b = [capi.DeviceBuffer.from_array(v) for v in d["b"]]
+    acts = [capi.DeviceBuffer.from_array(synth.uniform(400 + l, (batch, sizes[l])))
+            for l in range(3)]                                   # layer inputs x_l
+    pre = [capi.DeviceBuffer.from_array(synth.uniform(410 + l, (batch, sizes[l + 1])))
+           for l in range(2)]                                    # pre-activations of layers 0, 1
+    dy_top = capi.DeviceBuffer.from_array(synth.uniform(420, (batch, sizes[3])))
+    grads = [capi.DeviceBuffer(4 * batch * n) for n in sizes]   # d(x_l), and scratch d(pre)
+    dpre = [capi.DeviceBuffer(4 * batch * n) for n in sizes[1:3]]
+    big = max(sizes[l] * sizes[l + 1] for l in range(3))
+    wt = capi.DeviceBuffer(4 * big)
+    xt = capi.DeviceBuffer(4 * batch * max(sizes))
+    dw = capi.DeviceBuffer(4 * big)
+    temp = capi.DeviceBuffer(4 * big)
+    ones = capi.DeviceBuffer.from_array(np.ones(batch, np.float32))
+    dB = capi.DeviceBuffer(4 * max(sizes))
+    TA, TB, OV = capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B, capi.SPH_GEMM_OVERWRITE
+
+    def sgd(z, dz, count):
+        if direct:
+            capi.call("sph_sgd_step_f32", z.ptr, dz.ptr, lr, count)
+        else:
+            capi.call("sph_scale_f32", temp.ptr, dz.ptr, lr, count)
+            capi.call("sph_sub_f32", z.ptr, z.ptr, temp.ptr, count, 0, 0, 0)
+
+    def layer(l, dy):
+        n_in, n_out = sizes[l], sizes[l + 1]
+        dx, x = grads[l], acts[l]
+        capi.call("sph_fill_f32", dx.ptr, 0.0, batch * n_in)       # a fresh dx tensor
+        if direct:
+            capi.call("sph_gemm_f32_ex", dx.ptr, dy.ptr, W[l].ptr, batch, n_in, n_out, 1,
+                      batch * n_in, batch * n_out, n_in * n_out, TB)
+            capi.call("sph_gemm_f32_ex", dw.ptr, x.ptr, dy.ptr, n_in, n_out, batch, 1,
+                      n_in * n_out, n_in * batch, batch * n_out, TA | OV)
+        else:
+            capi.call("sph_transpose_f32", wt.ptr, W[l].ptr, n_in, n_out, 1, 0)
+            capi.call("sph_gemm_f32", dx.ptr, dy.ptr, wt.ptr, batch, n_in, n_out, 1,
+                      batch * n_in, batch * n_out, n_in * n_out)
+            capi.call("sph_transpose_f32", xt.ptr, x.ptr, batch, n_in, 1, 0)
+            capi.call("sph_fill_f32", dw.ptr, 0.0, n_in * n_out)
+            capi.call("sph_gemm_f32", dw.ptr, xt.ptr, dy.ptr, n_in, n_out, batch, 1,
+                      n_in * n_out, n_in * batch, batch * n_out)
+        sgd(W[l], dw, n_in * n_out)
+        if direct:
+            capi.call("sph_gemm_f32_ex", dB.ptr, ones.ptr, dy.ptr, 1, n_out, batch, 1, n_out,
+                      batch, batch * n_out, OV)
+        else:
+            capi.call("sph_fill_f32", ones.ptr, 1.0, batch)
+            capi.call("sph_fill_f32", dB.ptr, 0.0, n_out)
+            capi.call("sph_gemm_f32", dB.ptr, ones.ptr, dy.ptr, 1, n_out, batch, 1, n_out,
+                      batch, batch * n_out)
+        capi.call("sph_scale_f32", dB.ptr, dB.ptr, 1.0 / batch, n_out)
+        sgd(b[l], dB, n_out)
+
+    def launch():
+        dy = dy_top
+        for l in (2, 1, 0):
+            layer(l, dy)
+            if l > 0:
+                capi.call("sph_fill_f32", dpre[l - 1].ptr, 0.0, batch * sizes[l])
+                capi.call("sph_relu_backward_f32", dpre[l - 1].ptr, grads[l].ptr, pre[l - 1].ptr,
+                          batch * sizes[l])
+                dy = dpre[l - 1]
+
+    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    for buf in W + b + acts + pre + grads + dpre + [dy_top, wt, xt, dw, temp, ones, dB]:
+        buf.release()
+    flops = 2.0 * 2.0 * batch * sum(sizes[l] * sizes[l + 1] for l in range(3))
+    return event_ms, flops
+
+
+def bench_sgd_step(capi, steps, warmup, mib=64):
+    """One-pass SGD update over `mib` MiB of parameters: reads z and dz, writes z."""
+    n = mib * (1 << 20) // 4
+    z = capi.DeviceBuffer.from_array(np.ones(n, np.float32))
+    dz = capi.DeviceBuffer.from_array(np.ones(n, np.float32))
+
+    def launch():
+        capi.call("sph_sgd_step_f32", z.ptr, dz.ptr, 1e-6, n)
+
+    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    z.release()
+    dz.release()
+    return event_ms, 3 * 4 * n
+
+
 def bench_copy(capi, steps, warmup, mib=64):
     """A plain one-pass kernel of known size (ReLU over `mib` MiB: reads it once, writes it
     once), used to calibrate the profiler's FETCH_SIZE / WRITE_SIZE counters."""
@@ -267,6 +363,12 @@ def main():
         result["copy"] = {"kernel": "ReluKernel", "bytes_read": nbytes, "bytes_written": nbytes,
                           "launch_ms": ms, "gbs": 2 * nbytes / (ms * 1e-3) / 1e9}
 
+    if args.only in ("backward", "backward_reference"):
+        ms, fl = bench_mlp_backward(capi, synth, args.steps, args.warmup,
+                                    direct=args.only == "backward")
+        result["backward"] = {"sequence": "direct" if args.only == "backward" else "reference",
+                              "step_ms": ms, "tflops": fl / (ms * 1e-3) / 1e12}
+
     if args.only in (None, "spmm"):
         sp_steps = max(args.steps * 4, 100)
         sp_event, sp_wall, d5, nnz, alg_bytes = bench_spmm(capi, synth, sp_steps, args.warmup)
@@ -304,6 +406,17 @@ def main():
         ms, fl = bench_mlp(capi, synth, 100, 10)
         others["config4_mlp_forward"] = {"forward_ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                                          "kernels_per_forward": 11}
+        ms_ref, fl = bench_mlp_backward(capi, synth, 100, 10, direct=False)
+        ms_dir, _ = bench_mlp_backward(capi, synth, 100, 10, direct=True)
+        others["config4_mlp_backward_sgd"] = {
+            "reference_sequence_ms": ms_ref, "direct_ms": ms_dir,
+            "direct_tflops": fl / (ms_dir * 1e-3) / 1e12,
+            "note": "reference sequence: Transpose + Gemm, Zeros, Scale + Sub; direct: "
+                    "transposed-read / overwrite GEMM flags and the one-pass SGD step "
+                    "(bit-identical results)"}
+        ms, nbytes = bench_sgd_step(capi, 200, 20)
+        others["sgd_step_64MiB"] = {"launch_ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9,
+                                    "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS}
         result["others"] = others
 
     if not args.no_cpu and args.only is None:
