@@ -260,6 +260,33 @@ def bench_sgd_step(capi, steps, warmup, mib=64):
     return event_ms, 3 * 4 * n
 
 
+def bench_csr_conversion(capi, synth, steps, warmup):
+    """Dense -> CSR (row offsets + fill, no host read-back of nnz inside the timed region) and
+    CSR -> dense on configuration 5's matrix (8192 x 8192 fp32 at 1 %)."""
+    d = synth.config5()
+    M, K = d["M"], d["K"]
+    nnz = int(d["V"].size)
+    dense = capi.DeviceBuffer.from_array(synth.densify(d["V"], d["COL"], d["ROW"], M, K))
+    row = capi.DeviceBuffer(4 * (M + 1))
+    val = capi.DeviceBuffer(4 * nnz)
+    col = capi.DeviceBuffer(4 * nnz)
+
+    def to_csr():
+        capi.call("sph_csr_row_offsets_f32", row.ptr, dense.ptr, M, K, K, None)
+        capi.call("sph_csr_fill_f32", val.ptr, col.ptr, row.ptr, dense.ptr, M, K, K)
+
+    def to_dense():
+        capi.call("sph_csr_to_dense_f32", dense.ptr, K, val.ptr, col.ptr, row.ptr, M, K)
+
+    ms_csr, _ = timed_launches(capi, to_csr, steps, warmup)
+    ms_dense, _ = timed_launches(capi, to_dense, steps, warmup)
+    for b in (dense, row, val, col):
+        b.release()
+    dense_bytes = 4 * M * K
+    csr_bytes = 8 * nnz + 4 * (M + 1)
+    return ms_csr, ms_dense, dense_bytes, csr_bytes
+
+
 def bench_copy(capi, steps, warmup, mib=64):
     """A plain one-pass kernel of known size (ReLU over `mib` MiB: reads it once, writes it
     once), used to calibrate the profiler's FETCH_SIZE / WRITE_SIZE counters."""
@@ -417,6 +444,14 @@ def main():
         ms, nbytes = bench_sgd_step(capi, 200, 20)
         others["sgd_step_64MiB"] = {"launch_ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9,
                                     "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS}
+        ms_csr, ms_dense, dense_bytes, csr_bytes = bench_csr_conversion(capi, synth, 50, 5)
+        others["csr_conversion_config5"] = {
+            "dense_to_csr_ms": ms_csr,
+            "dense_to_csr_gbs": (dense_bytes + csr_bytes) / (ms_csr * 1e-3) / 1e9,
+            "dense_to_csr_note": "algorithmic bytes: dense read once + CSR written; the kernels "
+                                 "read the dense matrix twice (count, then fill)",
+            "csr_to_dense_ms": ms_dense,
+            "csr_to_dense_gbs": (dense_bytes + csr_bytes) / (ms_dense * 1e-3) / 1e9}
         result["others"] = others
 
     if not args.no_cpu and args.only is None:

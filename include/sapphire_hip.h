@@ -224,6 +224,32 @@ int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL,
                      const uint32_t* ROW, uint32_t M, uint32_t Kdim, uint32_t N,
                      const float* B, int accumulate);
 
+/* ---- dense <-> CSR ------------------------------------------------------- */
+
+/* The reference declares CreateSparseMatrixWithDenseMatrix(dst, src, m, n,
+ * paddedN, numMatrices) and ConvertSparseMatrixToDenseMatrix(dst, src, m, n,
+ * paddedN, numMatrices) (Includes/Sapphire/compute/sparse/Sparse.hpp:150-160)
+ * and defines neither; these three calls are their device work for one matrix
+ * of M rows, N columns and a row pitch of ld floats (ld = paddedN).  An entry
+ * is kept when its value != 0 (-0.0 is dropped, NaN kept); a row's entries are
+ * stored in ascending column order.
+ *
+ * sph_csr_row_offsets_f32: ROW (device, M + 1 entries) receives the offsets,
+ * ROW[M] = number of kept entries.  With nnzHost != NULL that count is also
+ * copied to *nnzHost and the call returns after the stream has drained, so the
+ * caller can size V and COL; with NULL the call is asynchronous.
+ * sph_csr_fill_f32: writes V and COL (device, ROW[M] entries each) from the
+ * same dense matrix and the ROW just computed.
+ * sph_csr_to_dense_f32: dense[r][c] = the stored value, 0 where none is
+ * stored; columns >= N in COL are ignored; the pitch padding is not written. */
+int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M,
+                            uint32_t N, uint32_t ld, uint32_t* nnzHost);
+int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW,
+                     const float* dense, uint32_t M, uint32_t N, uint32_t ld);
+int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V,
+                         const uint32_t* COL, const uint32_t* ROW, uint32_t M,
+                         uint32_t N);
+
 #ifdef __cplusplus
 }
 #endif

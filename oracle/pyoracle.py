@@ -92,6 +92,12 @@ def oracle():
         o.orc_spmm_csr.argtypes = [_fp, _fp, _up, _up, ctypes.c_uint32, ctypes.c_uint32, _fp,
                                    ctypes.c_int]
         o.orc_spmm_csr.restype = None
+        o.orc_csr_from_dense.argtypes = [_fp, _up, _up, _fp, ctypes.c_uint32, ctypes.c_uint32,
+                                         ctypes.c_uint32]
+        o.orc_csr_from_dense.restype = ctypes.c_uint32
+        o.orc_csr_to_dense.argtypes = [_fp, ctypes.c_uint32, _fp, _up, _up, ctypes.c_uint32,
+                                       ctypes.c_uint32]
+        o.orc_csr_to_dense.restype = None
         for name in ("orc_shape_expand", "orc_shape_shrink"):
             getattr(o, name).argtypes = [ctypes.POINTER(OrcShape), ctypes.c_int]
             getattr(o, name).restype = ctypes.c_int
@@ -291,4 +297,27 @@ def spmm_csr(out, V, COL, ROW, M, N, B, threads=1):
                           COL.ctypes.data_as(_up) if COL.size else
                           np.zeros(1, np.uint32).ctypes.data_as(_up),
                           ROW.ctypes.data_as(_up), M, N, _f(B), threads)
+    return out
+
+
+def csr_from_dense(dense, N=None):
+    """(V, COL, ROW) of a 2-D float32 array; N < dense.shape[1] treats the rest as pitch padding."""
+    M, ld = dense.shape
+    N = ld if N is None else N
+    ROW = np.zeros(M + 1, np.uint32)
+    nnz = oracle().orc_csr_from_dense(None, None, ROW.ctypes.data_as(_up), _f(dense), M, N, ld)
+    V = np.zeros(max(nnz, 1), np.float32)
+    COL = np.zeros(max(nnz, 1), np.uint32)
+    oracle().orc_csr_from_dense(_f(V), COL.ctypes.data_as(_up), ROW.ctypes.data_as(_up),
+                                _f(dense), M, N, ld)
+    return V[:nnz], COL[:nnz], ROW
+
+
+def csr_to_dense(V, COL, ROW, M, N, ld=None, fill=0.0):
+    ld = N if ld is None else ld
+    out = np.full((M, ld), np.float32(fill), np.float32)
+    Vp = V if V.size else np.zeros(1, np.float32)
+    Cp = COL if COL.size else np.zeros(1, np.uint32)
+    oracle().orc_csr_to_dense(_f(out), ld, _f(Vp), Cp.ctypes.data_as(_up),
+                              ROW.ctypes.data_as(_up), M, N)
     return out

@@ -632,3 +632,45 @@ void orc_spmm_csr(float* out, const float* V, const uint32_t* COL,
     run_jobs(spmm_worker, jobs, sizeof(spmm_job), threads);
     free(jobs);
 }
+
+/* -------------------------------------------------------------- dense <-> CSR */
+
+uint32_t orc_csr_from_dense(float* V, uint32_t* COL, uint32_t* ROW,
+                            const float* dense, uint32_t M, uint32_t N,
+                            uint32_t ld)
+{
+    uint32_t nnz = 0;
+    for (uint32_t r = 0; r < M; ++r)
+    {
+        ROW[r] = nnz;
+        for (uint32_t c = 0; c < N; ++c)
+        {
+            const float v = dense[(size_t)r * ld + c];
+            if (v != 0.0f)
+            {
+                if (V)
+                    V[nnz] = v;
+                if (COL)
+                    COL[nnz] = c;
+                ++nnz;
+            }
+        }
+    }
+    ROW[M] = nnz;
+    return nnz;
+}
+
+void orc_csr_to_dense(float* dense, uint32_t ld, const float* V,
+                      const uint32_t* COL, const uint32_t* ROW, uint32_t M,
+                      uint32_t N)
+{
+    for (uint32_t r = 0; r < M; ++r)
+    {
+        float* row = dense + (size_t)r * ld;
+        for (uint32_t c = 0; c < N; ++c)
+            row[c] = 0.0f;
+        for (uint32_t p = ROW[r]; p < ROW[r + 1]; ++p)
+            if (COL[p] < N)
+                row[COL[p]] = V[p];
+    }
+}

@@ -205,6 +205,29 @@ void orc_spmm_csr(float* out, const float* V, const uint32_t* COL,
                   const uint32_t* ROW, uint32_t M, uint32_t N,
                   const float* B, int threads);
 
+/* ---- dense <-> CSR ------------------------------------------------------- */
+
+/* The reference declares the conversions only
+ * (Includes/Sapphire/compute/sparse/Sparse.hpp:150-160:
+ * CreateSparseMatrixWithDenseMatrix / ConvertSparseMatrixToDenseMatrix with m,
+ * n, paddedN) and its tests fill pitched dense matrices the same way
+ * (Tests/UnitTests/Sources/TestUtil.cpp:17-60: element (row, col) of matrix i
+ * at i*m*paddedN + row*paddedN + col).  Restated contract: an entry is kept
+ * when value != 0; row-major, ascending columns; ROW has M + 1 offsets.
+ * Returns nnz.  V and COL may be NULL to count only.
+ * pinned: scipy.sparse.csr_matrix on the same matrices (values, indices,
+ * indptr), count_nonzero, dense -> CSR -> dense round trip, hand example with
+ * -0.0 and NaN. */
+uint32_t orc_csr_from_dense(float* V, uint32_t* COL, uint32_t* ROW,
+                            const float* dense, uint32_t M, uint32_t N,
+                            uint32_t ld);
+
+/* dense[r*ld + COL[p]] = V[p], other columns < N zero; padding untouched.
+ * pinned: scipy toarray(), round trip. */
+void orc_csr_to_dense(float* dense, uint32_t ld, const float* V,
+                      const uint32_t* COL, const uint32_t* ROW, uint32_t M,
+                      uint32_t N);
+
 #ifdef __cplusplus
 }
 #endif

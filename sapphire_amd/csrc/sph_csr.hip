@@ -1,0 +1,422 @@
+// Dense <-> CSR conversion on the device.
+//
+// The container is the reference's SparseMatrix
+// (Includes/Sapphire/compute/sparse/SparseMatrix.hpp:28-38); the reference declares the two
+// conversions (Includes/Sapphire/compute/sparse/Sparse.hpp:150-160,
+// CreateSparseMatrixWithDenseMatrix / ConvertSparseMatrixToDenseMatrix over matrices of m
+// rows, n columns and a row pitch of paddedN floats) and defines neither.  An entry is kept
+// when its value compares unequal to zero (so -0.0 is dropped and NaN is kept); entries of a
+// row are stored in ascending column order.
+//
+// All of this is one- or two-pass integer/byte work bound by HBM:
+//   row offsets   read the dense matrix once, popcount per row, exclusive scan of M+1 counts
+//   fill          read it again, ballot + popcount give every kept entry its slot
+//   to dense      zero the rows, then scatter the entries
+// A row is handled by a group of LPR lanes (a power of two, 4..64, chosen from the row
+// length) so that narrow matrices do not idle most of a wavefront; each lane takes 4
+// consecutive columns (16 bytes) per step.
+#include "sph_internal.h"
+
+#include <algorithm>
+
+namespace
+{
+constexpr int kThreads = 256;
+
+struct DenseView
+{
+    const float* data;
+    uint32_t M, N, ld;
+    int vec;  // rows start 16-byte aligned and N % 4 == 0
+};
+
+// 4 consecutive columns of one row; columns past N read as 0
+__device__ __forceinline__ float4 LoadQuad(const DenseView& d, uint32_t row, uint32_t col,
+                                           bool rowOk)
+{
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (rowOk && col < d.N)
+    {
+        const float* p = d.data + static_cast<size_t>(row) * d.ld + col;
+        if (d.vec)
+            v = *reinterpret_cast<const float4*>(p);
+        else
+        {
+            v.x = p[0];
+            if (col + 1 < d.N) v.y = p[1];
+            if (col + 2 < d.N) v.z = p[2];
+            if (col + 3 < d.N) v.w = p[3];
+        }
+    }
+    return v;
+}
+
+// counts[r] = number of entries != 0 in row r; counts[M] = 0 (the slot the scan turns into nnz)
+template <int LPR>
+__global__ __launch_bounds__(kThreads) void CsrCountKernel(uint32_t* __restrict__ counts,
+                                                           const DenseView d)
+{
+    constexpr uint32_t kGroups = kThreads / LPR;
+    const uint32_t lane = threadIdx.x % LPR;
+    const uint32_t group = threadIdx.x / LPR;
+    const uint32_t rowsPerPass = gridDim.x * kGroups;
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        counts[d.M] = 0;
+    // every group of a wavefront runs the same number of passes and steps
+    const uint32_t passes = (d.M + rowsPerPass - 1) / rowsPerPass;
+    for (uint32_t pass = 0; pass < passes; ++pass)
+    {
+        const uint32_t row = pass * rowsPerPass + blockIdx.x * kGroups + group;
+        const bool rowOk = row < d.M;
+        uint32_t c = 0;
+        for (uint32_t col = lane * 4; col < d.N; col += LPR * 4)
+        {
+            const float4 v = LoadQuad(d, row, col, rowOk);
+            c += (v.x != 0.f) + (v.y != 0.f) + (v.z != 0.f) + (v.w != 0.f);
+        }
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1)
+            c += __shfl_xor(c, off, LPR);
+        if (rowOk && lane == 0)
+            counts[row] = c;
+    }
+}
+
+// ---- exclusive scan of n uint32 in place, 4096 per workgroup -----------------------------
+constexpr int kScanThreads = 1024;
+constexpr int kScanPerBlock = kScanThreads * 4;
+
+// exclusive scan of one value per thread across the workgroup; returns the prefix and leaves
+// the workgroup total in `total`
+__device__ __forceinline__ uint32_t BlockExclusiveScan(uint32_t value, uint32_t& total,
+                                                       uint32_t* waveSums)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    uint32_t inclusive = value;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+    {
+        const uint32_t up = __shfl_up(inclusive, off, 64);
+        if (lane >= static_cast<uint32_t>(off))
+            inclusive += up;
+    }
+    if (lane == 63)
+        waveSums[wave] = inclusive;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kScanThreads / 64; ++w)
+    {
+        const uint32_t s = waveSums[w];
+        if (static_cast<uint32_t>(w) < wave)
+            before += s;
+        all += s;
+    }
+    __syncthreads();  // waveSums may be reused by the caller's next round
+    total = all;
+    return before + inclusive - value;
+}
+
+__global__ __launch_bounds__(kScanThreads) void ScanBlocksKernel(uint32_t* __restrict__ data,
+                                                                 uint32_t* __restrict__ blockSums,
+                                                                 uint32_t n)
+{
+    __shared__ uint32_t waveSums[kScanThreads / 64];
+    const size_t base = static_cast<size_t>(blockIdx.x) * kScanPerBlock + threadIdx.x * 4;
+    uint32_t v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        v[e] = base + e < n ? data[base + e] : 0u;
+    uint32_t total;
+    uint32_t run = BlockExclusiveScan(v[0] + v[1] + v[2] + v[3], total, waveSums);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+    {
+        if (base + e < n)
+            data[base + e] = run;
+        run += v[e];
+    }
+    if (threadIdx.x == 0 && blockSums != nullptr)
+        blockSums[blockIdx.x] = total;
+}
+
+// one workgroup: exclusive scan of the per-block totals in place
+__global__ __launch_bounds__(kScanThreads) void ScanSumsKernel(uint32_t* __restrict__ sums,
+                                                               uint32_t count)
+{
+    __shared__ uint32_t waveSums[kScanThreads / 64];
+    uint32_t carry = 0;
+    for (uint32_t start = 0; start < count; start += kScanThreads)
+    {
+        const uint32_t i = start + threadIdx.x;
+        const uint32_t v = i < count ? sums[i] : 0u;
+        uint32_t total;
+        const uint32_t prefix = BlockExclusiveScan(v, total, waveSums);
+        if (i < count)
+            sums[i] = carry + prefix;
+        carry += total;
+    }
+}
+
+__global__ __launch_bounds__(kScanThreads) void AddBlockOffsetsKernel(
+    uint32_t* __restrict__ data, const uint32_t* __restrict__ blockOffsets, uint32_t n)
+{
+    // block 0 needs no offset: the grid starts at block 1
+    const uint32_t block = blockIdx.x + 1;
+    const uint32_t add = blockOffsets[block];
+    const size_t base = static_cast<size_t>(block) * kScanPerBlock + threadIdx.x * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if (base + e < n)
+            data[base + e] += add;
+}
+
+// V / COL of every kept entry, rows laid out by ROW
+template <int LPR>
+__global__ __launch_bounds__(kThreads) void CsrFillKernel(float* __restrict__ V,
+                                                          uint32_t* __restrict__ COL,
+                                                          const uint32_t* __restrict__ ROW,
+                                                          const DenseView d)
+{
+    constexpr uint32_t kGroups = kThreads / LPR;
+    const uint32_t lane = threadIdx.x % LPR;
+    const uint32_t group = threadIdx.x / LPR;
+    // position of this group inside its wavefront, as a shift for 64-bit ballots
+    const uint32_t shift = (threadIdx.x & 63u) - lane;
+    const uint64_t groupMask = LPR == 64 ? ~0ull : ((1ull << LPR) - 1ull);
+    const uint64_t below = (1ull << lane) - 1ull;
+    const uint32_t rowsPerPass = gridDim.x * kGroups;
+    const uint32_t passes = (d.M + rowsPerPass - 1) / rowsPerPass;
+    for (uint32_t pass = 0; pass < passes; ++pass)
+    {
+        const uint32_t row = pass * rowsPerPass + blockIdx.x * kGroups + group;
+        const bool rowOk = row < d.M;
+        uint32_t slot = rowOk ? ROW[row] : 0u;
+        // a ROW that was not computed from this matrix must not make the stores run past the row
+        const uint32_t rowEnd = rowOk ? ROW[row + 1] : 0u;
+        for (uint32_t col0 = 0; col0 < d.N; col0 += LPR * 4)
+        {
+            const uint32_t col = col0 + lane * 4;
+            const float4 q = LoadQuad(d, row, col, rowOk);
+            const float v[4] = { q.x, q.y, q.z, q.w };
+            // entries are ordered by (lane, element): everything lower lanes keep comes first
+            uint32_t before = 0, kept = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+            {
+                const uint64_t m = (__ballot(v[e] != 0.f) >> shift) & groupMask;
+                before += __popcll(m & below);
+                kept += __popcll(m);
+            }
+            uint32_t at = slot + before;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (v[e] != 0.f && at < rowEnd)
+                {
+                    V[at] = v[e];
+                    COL[at] = col + e;
+                    ++at;
+                }
+            slot += kept;
+        }
+    }
+}
+
+// dense[row][COL[p]] = V[p]; 16 lanes walk one row's entries
+__global__ __launch_bounds__(kThreads) void CsrScatterKernel(float* __restrict__ dense,
+                                                             uint32_t ld, uint32_t M, uint32_t N,
+                                                             const float* __restrict__ V,
+                                                             const uint32_t* __restrict__ COL,
+                                                             const uint32_t* __restrict__ ROW)
+{
+    constexpr uint32_t kLanes = 16;
+    constexpr uint32_t kGroups = kThreads / kLanes;
+    const uint32_t lane = threadIdx.x % kLanes;
+    const uint32_t group = threadIdx.x / kLanes;
+    for (uint32_t row = blockIdx.x * kGroups + group; row < M; row += gridDim.x * kGroups)
+    {
+        const uint32_t end = ROW[row + 1];
+        float* out = dense + static_cast<size_t>(row) * ld;
+        for (uint32_t p = ROW[row] + lane; p < end; p += kLanes)
+        {
+            const uint32_t c = COL[p];
+            if (c < N)  // an entry outside the matrix is dropped, never written
+                out[c] = V[p];
+        }
+    }
+}
+
+// rows x cols block of a pitched matrix set to `value`
+__global__ __launch_bounds__(kThreads) void FillPitchedKernel(float* __restrict__ dst,
+                                                              float value, uint32_t rows,
+                                                              uint32_t cols, uint32_t ld)
+{
+    for (uint32_t r = blockIdx.y; r < rows; r += gridDim.y)
+        for (uint32_t c = blockIdx.x * kThreads + threadIdx.x; c < cols; c += gridDim.x * kThreads)
+            dst[static_cast<size_t>(r) * ld + c] = value;
+}
+
+int LanesPerRow(uint32_t N)
+{
+    const uint32_t quads = (N + 3) / 4;
+    int lpr = 4;
+    while (lpr < 64 && static_cast<uint32_t>(lpr) < quads)
+        lpr *= 2;
+    return lpr;
+}
+
+uint32_t RowGrid(uint32_t M, int lanesPerRow)
+{
+    const uint32_t groups = kThreads / static_cast<uint32_t>(lanesPerRow);
+    const uint64_t blocks = (static_cast<uint64_t>(M) + groups - 1) / groups;
+    const uint64_t cap = static_cast<uint64_t>(sph::ComputeUnits()) * 16;
+    return static_cast<uint32_t>(std::max<uint64_t>(1, std::min(blocks, cap)));
+}
+
+DenseView MakeView(const float* dense, uint32_t M, uint32_t N, uint32_t ld)
+{
+    DenseView d{};
+    d.data = dense;
+    d.M = M;
+    d.N = N;
+    d.ld = ld;
+    d.vec = (N % 4 == 0) && (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(dense) & 15u) == 0;
+    return d;
+}
+
+template <template <int> class Launcher, typename... Args>
+void DispatchLanes(int lanesPerRow, Args&&... args)
+{
+    switch (lanesPerRow)
+    {
+        case 4: Launcher<4>::Run(args...); break;
+        case 8: Launcher<8>::Run(args...); break;
+        case 16: Launcher<16>::Run(args...); break;
+        case 32: Launcher<32>::Run(args...); break;
+        default: Launcher<64>::Run(args...); break;
+    }
+}
+
+template <int LPR>
+struct CountLauncher
+{
+    static void Run(uint32_t grid, hipStream_t stream, uint32_t* counts, const DenseView& d)
+    {
+        hipLaunchKernelGGL(CsrCountKernel<LPR>, dim3(grid), dim3(kThreads), 0, stream, counts, d);
+    }
+};
+
+template <int LPR>
+struct FillLauncher
+{
+    static void Run(uint32_t grid, hipStream_t stream, float* V, uint32_t* COL,
+                    const uint32_t* ROW, const DenseView& d)
+    {
+        hipLaunchKernelGGL(CsrFillKernel<LPR>, dim3(grid), dim3(kThreads), 0, stream, V, COL, ROW,
+                           d);
+    }
+};
+}  // namespace
+
+extern "C" {
+
+int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint32_t N,
+                            uint32_t ld, uint32_t* nnzHost)
+{
+    SPH_REQUIRE(ROW != nullptr, "ROW is null");
+    SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
+    SPH_REQUIRE(M < 0xffffffffu, "too many rows");
+    SPH_REQUIRE(M == 0 || N == 0 || dense != nullptr, "dense is null");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+
+    const DenseView d = MakeView(dense, M, N, ld);
+    const int lanes = LanesPerRow(N);
+    DispatchLanes<CountLauncher>(lanes, RowGrid(M, lanes), stream, ROW, d);
+    SPH_CHECK_LAUNCH();
+
+    const uint32_t n = M + 1;
+    const uint32_t blocks = (n + kScanPerBlock - 1) / kScanPerBlock;
+    if (blocks == 1)
+    {
+        hipLaunchKernelGGL(ScanBlocksKernel, dim3(1), dim3(kScanThreads), 0, stream, ROW,
+                           static_cast<uint32_t*>(nullptr), n);
+        SPH_CHECK_LAUNCH();
+    }
+    else
+    {
+        // per-block totals live in a stream-ordered scratch allocation
+        uint32_t* sums = nullptr;
+        SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&sums), blocks * sizeof(uint32_t),
+                                   stream));
+        hipLaunchKernelGGL(ScanBlocksKernel, dim3(blocks), dim3(kScanThreads), 0, stream, ROW,
+                           sums, n);
+        hipLaunchKernelGGL(ScanSumsKernel, dim3(1), dim3(kScanThreads), 0, stream, sums, blocks);
+        hipLaunchKernelGGL(AddBlockOffsetsKernel, dim3(blocks - 1), dim3(kScanThreads), 0, stream,
+                           ROW, sums, n);
+        const hipError_t launched = hipGetLastError();
+        SPH_HIP_TRY(hipFreeAsync(sums, stream));
+        if (launched != hipSuccess)
+            return sph::Fail(SPH_ERR_DEVICE, std::string("sph_csr_row_offsets_f32 launch failed with ") +
+                                                 hipGetErrorString(launched));
+    }
+    if (nnzHost != nullptr)
+    {
+        SPH_HIP_TRY(hipMemcpyAsync(nnzHost, ROW + M, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                   stream));
+        SPH_HIP_TRY(hipStreamSynchronize(stream));
+    }
+    return SPH_OK;
+}
+
+int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW, const float* dense, uint32_t M,
+                     uint32_t N, uint32_t ld)
+{
+    if (M == 0 || N == 0)
+        return SPH_OK;
+    SPH_REQUIRE(ROW != nullptr && dense != nullptr, "null pointer");
+    SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
+    // V and COL may be null only for a matrix without entries; the kernel then writes nothing
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    const DenseView d = MakeView(dense, M, N, ld);
+    const int lanes = LanesPerRow(N);
+    DispatchLanes<FillLauncher>(lanes, RowGrid(M, lanes), stream, V, COL, ROW, d);
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V, const uint32_t* COL,
+                         const uint32_t* ROW, uint32_t M, uint32_t N)
+{
+    if (M == 0 || N == 0)
+        return SPH_OK;
+    SPH_REQUIRE(dense != nullptr && ROW != nullptr, "null pointer");
+    SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    if (ld == N)
+    {
+        const int rc = sph_fill_f32(dense, 0.0f, static_cast<size_t>(M) * N);
+        if (rc != SPH_OK)
+            return rc;
+    }
+    else
+    {
+        const uint32_t gx = std::min<uint32_t>((N + kThreads - 1) / kThreads, 64u);
+        const uint32_t gy = std::min<uint32_t>(M, 65535u);
+        hipLaunchKernelGGL(FillPitchedKernel, dim3(gx, gy), dim3(kThreads), 0, stream, dense, 0.0f,
+                           M, N, ld);
+        SPH_CHECK_LAUNCH();
+    }
+    hipLaunchKernelGGL(CsrScatterKernel, dim3(RowGrid(M, 16)), dim3(kThreads), 0, stream, dense, ld,
+                       M, N, V, COL, ROW);
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+}  // extern "C"

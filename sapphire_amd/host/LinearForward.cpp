@@ -2,6 +2,7 @@
 
 #include <Sapphire/compute/BasicOps.hpp>
 #include <Sapphire/compute/Initialize.hpp>
+#include <Sapphire/compute/sparse/SparseGemm.hpp>
 
 #include <stdexcept>
 
@@ -37,5 +38,43 @@ void LinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
 
     Compute::Gemm(y2, ones, bias2);
     Compute::Gemm(y2, x2, weight);
+}
+
+void SparseLinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
+                         const SparseMatrix& weightTransposed,
+                         const TensorUtil::TensorData& bias)
+{
+    if (x.Mode() != bias.Mode() || x.Mode() != y.Mode())
+        throw std::invalid_argument("NN::Linear - Device mode inequality");
+    if (x.Mode() != ComputeMode::Cuda)
+        throw std::runtime_error("NN::Linear - Host mode is not provided by the device backend");
+
+    const int batchSize = x.GetShape().GetNumUnits(1);
+    const int inputs = static_cast<int>(weightTransposed.N);
+    const int outputs = static_cast<int>(weightTransposed.M);
+    if (x.Size() != batchSize * inputs || y.Size() != batchSize * outputs ||
+        bias.Size() != outputs)
+        throw std::invalid_argument("NN::Linear - sparse weight shape mismatch");
+    const CudaDevice device = x.GetCudaDevice();
+
+    TensorUtil::TensorData x2 = x, y2 = y, biasColumn = bias;
+    Util::ChangeTensorDataDimension(2, x2);
+    Util::ChangeTensorDataDimension(2, y2);
+    biasColumn.Reshape(Shape({ outputs, 1 }));
+
+    TensorUtil::TensorData xT(Shape({ inputs, batchSize }), Type::Dense, device);
+    TensorUtil::TensorData yT(Shape({ outputs, batchSize }), Type::Dense, device);
+    TensorUtil::TensorData ones(Shape({ 1, batchSize }), Type::Dense, device);
+    xT.SetMode(ComputeMode::Cuda);
+    yT.SetMode(ComputeMode::Cuda);
+    ones.SetMode(ComputeMode::Cuda);
+
+    Compute::Transpose(xT, x2);
+    Compute::Initialize::Ones(ones);
+    Compute::Initialize::Zeros(yT);  // a pooled buffer may hold an earlier result
+    Compute::Gemm(yT, biasColumn, ones);
+    Compute::Sparse::Cuda::Gemm(yT.CudaMutableRawPtr(), &weightTransposed, xT.CudaRawPtr(),
+                                static_cast<unsigned int>(batchSize), true, device.GetID());
+    Compute::Transpose(y2, yT);
 }
 }  // namespace Sapphire::NN

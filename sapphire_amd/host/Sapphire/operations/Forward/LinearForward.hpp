@@ -11,6 +11,7 @@
 #ifndef SAPPHIRE_AMD_OPERATIONS_FORWARD_LINEARFORWARD_HPP
 #define SAPPHIRE_AMD_OPERATIONS_FORWARD_LINEARFORWARD_HPP
 
+#include <Sapphire/compute/sparse/SparseMatrix.hpp>
 #include <Sapphire/tensor/TensorData.hpp>
 
 namespace Sapphire::Util
@@ -24,6 +25,17 @@ namespace Sapphire::NN
 {
 void LinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
                    const TensorUtil::TensorData& weight, const TensorUtil::TensorData& bias);
+
+//! The same layer with a sparse weight, the variant NN::Linear rejects with
+//! "Sparse version not implemented" (Sources/Sapphire/operations/Forward/Linear.cpp:28-30).
+//! `weightTransposed` is a device record of the transposed weight, [out, in] in CSR, so that
+//! the CSR x dense kernel applies:  y^T [out, batch] = bias * ones[1, batch] (K = 1 GEMM),
+//! y^T += weightTransposed * x^T, y = transpose(y^T).  y is overwritten; the result equals
+//! LinearForward on the densified weight with a zero y, bit for bit on the CPU contract
+//! (entries in ascending input index, products and sums rounded separately).
+void SparseLinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
+                         const SparseMatrix& weightTransposed,
+                         const TensorUtil::TensorData& bias);
 }  // namespace Sapphire::NN
 
 #endif

@@ -8,11 +8,13 @@
 #include <Sapphire/compute/BroadcastPlan.hpp>
 #include <Sapphire/compute/Initialize.hpp>
 #include <Sapphire/compute/cudaUtil/Memory.hpp>
+#include <Sapphire/compute/sparse/Sparse.hpp>
 #include <Sapphire/compute/sparse/SparseGemm.hpp>
 #include <Sapphire/operations/Backward/LinearBackward.hpp>
 #include <Sapphire/operations/Forward/LinearForward.hpp>
 #include <Sapphire/util/ResourceManager.hpp>
 
+#include <algorithm>
 #include <cstring>
 #include <exception>
 #include <stdexcept>
@@ -300,6 +302,105 @@ int sphh_linear_backward(float* dx, float* weight, float* bias, const float* dy,
         Download(Dx, dx);
         Download(W, weight);
         Download(B, bias);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// Dense (host, numMatrices x m x paddedN) -> device -> CreateSparseMatrixWithDenseMatrix ->
+// DeepCopyDeviceToDevice into fresh records -> DeepCopyDeviceToHost -> out arrays (entries of
+// all matrices back to back in V / COL, m + 1 offsets per matrix in ROW, counts in nnz), and
+// ConvertSparseMatrixToDenseMatrix of the copied records into denseBack, which is pre-filled
+// with `fill` so that untouched padding stays visible.  capacity bounds V / COL.
+int sphh_csr_round_trip(const float* dense, unsigned m, unsigned n, unsigned paddedN,
+                        unsigned numMatrices, unsigned* nnz, float* V, unsigned* COL,
+                        unsigned* ROW, unsigned long capacity, float* denseBack, float fill)
+{
+    return Guard([&] {
+        const std::size_t total = static_cast<std::size_t>(numMatrices) * m * paddedN;
+        const std::size_t bytes = std::max<std::size_t>(total, 1) * sizeof(float);
+        Compute::Cuda::CudaSetDevice(0);
+        void* dDense = nullptr;
+        void* dBack = nullptr;
+        Compute::Cuda::CudaMalloc(&dDense, bytes);
+        Compute::Cuda::CudaMalloc(&dBack, bytes);
+        SparseMatrix* created = nullptr;
+        SparseMatrix* copied = nullptr;
+        SparseMatrix* host = nullptr;
+        try
+        {
+            Compute::Cuda::CopyHostToDevice(dDense, dense, total * sizeof(float));
+            Compute::CreateSparseMatrixWithDenseMatrix(&created, static_cast<const float*>(dDense),
+                                                       m, n, paddedN, numMatrices, 0);
+            Compute::DeepAllocateSparseCuda(&copied, created, numMatrices, 0);
+            Compute::DeepCopyDeviceToDevice(copied, created, numMatrices, 0);
+            std::vector<uint32_t> counts(numMatrices);
+            for (unsigned i = 0; i < numMatrices; ++i)
+                counts[i] = nnz[i] = copied[i].NNZ;
+            Compute::DeepAllocateSparseHost(&host, m, n, counts.data(), numMatrices);
+            Compute::DeepCopyDeviceToHost(host, copied, numMatrices, 0);
+            std::size_t at = 0;
+            for (unsigned i = 0; i < numMatrices; ++i)
+            {
+                if (at + host[i].NNZ > capacity)
+                    throw std::runtime_error("sphh_csr_round_trip - capacity too small");
+                std::memcpy(V + at, host[i].V, host[i].NNZ * sizeof(float));
+                std::memcpy(COL + at, host[i].COL, host[i].NNZ * sizeof(unsigned));
+                std::memcpy(ROW + static_cast<std::size_t>(i) * (m + 1), host[i].ROW,
+                            (static_cast<std::size_t>(m) + 1) * sizeof(unsigned));
+                at += host[i].NNZ;
+            }
+            Compute::Dense::Cuda::Scalar(static_cast<float*>(dBack), fill, total);
+            Compute::ConvertSparseMatrixToDenseMatrix(static_cast<float*>(dBack), copied, m, n,
+                                                      paddedN, numMatrices, 0);
+            Compute::Cuda::CopyDeviceToHost(denseBack, dBack, total * sizeof(float));
+        }
+        catch (...)
+        {
+            Compute::DeepFreeSparseHost(host, numMatrices);
+            Compute::DeepFreeSparseCuda(copied, numMatrices, 0);
+            Compute::DeepFreeSparseCuda(created, numMatrices, 0);
+            Compute::Cuda::CudaFree(dDense);
+            Compute::Cuda::CudaFree(dBack);
+            throw;
+        }
+        Compute::DeepFreeSparseHost(host, numMatrices);
+        Compute::DeepFreeSparseCuda(copied, numMatrices, 0);
+        Compute::DeepFreeSparseCuda(created, numMatrices, 0);
+        Compute::Cuda::CudaFree(dDense);
+        Compute::Cuda::CudaFree(dBack);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// NN::SparseLinearForward: the weight arrives dense [inputs, outputs] on the host, is sent to
+// the device, transposed there and converted to CSR there.
+int sphh_sparse_linear_forward(const float* x, int batch, int inputs, int outputs,
+                               const float* weight, const float* bias, float* y)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData X = Upload(Shape({ batch, inputs }), x, cuda);
+        TensorData W = Upload(Shape({ inputs, outputs }), weight, cuda);
+        TensorData B = Upload(Shape({ outputs }), bias, cuda);
+        TensorData Wt(Shape({ outputs, inputs }), Type::Dense, cuda);
+        Compute::Transpose(Wt, W);
+        SparseMatrix* record = nullptr;
+        Compute::CreateSparseMatrixWithDenseMatrix(&record, Wt.CudaRawPtr(),
+                                                   static_cast<uint32_t>(outputs),
+                                                   static_cast<uint32_t>(inputs),
+                                                   static_cast<uint32_t>(inputs), 1, 0);
+        TensorData Y(Shape({ batch, outputs }), Type::Dense, cuda);
+        try
+        {
+            NN::SparseLinearForward(Y, X, record[0], B);
+            Download(Y, y);
+        }
+        catch (...)
+        {
+            Compute::DeepFreeSparseCuda(record, 1, 0);
+            throw;
+        }
+        Compute::DeepFreeSparseCuda(record, 1, 0);
         Util::ResourceManager::Clean();
     });
 }

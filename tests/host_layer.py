@@ -39,6 +39,12 @@ def lib():
         h.sphh_linear_backward.argtypes = [_fp, _fp, _fp, _fp, _fp, ctypes.c_int, ctypes.c_int,
                                            ctypes.c_int, ctypes.c_float, ctypes.c_int,
                                            ctypes.c_int]
+        up = ctypes.POINTER(ctypes.c_uint)
+        h.sphh_csr_round_trip.argtypes = [_fp, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint,
+                                          ctypes.c_uint, up, _fp, up, up, ctypes.c_ulong, _fp,
+                                          ctypes.c_float]
+        h.sphh_sparse_linear_forward.argtypes = [_fp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                 _fp, _fp, _fp]
         h.sphh_shape_op.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip]
         h.sphh_shape_query.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib = h
@@ -156,3 +162,30 @@ def linear_backward(dx, W, bias, dy, x, lr, sequence, fused_sgd):
     _ok(lib().sphh_linear_backward(_f(dx), _f(W), _f(bias), _f(dy), _f(x), batch, inputs,
                                    W.shape[1], lr, sequence, 1 if fused_sgd else 0))
     return dx, W, bias
+
+
+def csr_round_trip(dense, n, fill=7.0):
+    """dense: [numMatrices, m, paddedN].  Returns (nnz per matrix, V, COL, ROW [numMatrices, m+1],
+    dense again) through the device-side conversion, copies and back-conversion."""
+    num, m, padded = dense.shape
+    up = ctypes.POINTER(ctypes.c_uint)
+    cap = max(int(np.count_nonzero(dense)) + 8, 8)
+    nnz = np.zeros(max(num, 1), np.uint32)
+    V = np.zeros(cap, np.float32)
+    COL = np.zeros(cap, np.uint32)
+    ROW = np.zeros((max(num, 1), m + 1), np.uint32)
+    back = np.zeros(dense.shape if dense.size else (1,), np.float32)
+    src = np.ascontiguousarray(dense) if dense.size else np.zeros(1, np.float32)
+    _ok(lib().sphh_csr_round_trip(_f(src), m, n, padded, num, nnz.ctypes.data_as(up), _f(V),
+                                  COL.ctypes.data_as(up), ROW.ctypes.data_as(up), cap, _f(back),
+                                  fill))
+    total = int(nnz[:num].sum())
+    return nnz[:num], V[:total], COL[:total], ROW[:num], back.reshape(dense.shape) if dense.size else back
+
+
+def sparse_linear_forward(x, W, bias):
+    batch, inputs = x.shape
+    out = np.zeros((batch, W.shape[1]), np.float32)
+    _ok(lib().sphh_sparse_linear_forward(_f(x), batch, inputs, W.shape[1],
+                                         _f(np.ascontiguousarray(W)), _f(bias), _f(out)))
+    return out

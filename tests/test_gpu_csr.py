@@ -1,0 +1,148 @@
+"""Dense <-> CSR conversion on the device (C ABI and the C++ layer) and the sparse Linear
+forward, bit-exact against the CPU checker."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from sapphire_amd import capi, synth
+from tests import helpers as h
+from tests import host_layer as hl
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(x):
+    return np.ascontiguousarray(x).view(np.uint32)
+
+
+def sparse_dense(seed, shape, density):
+    vals = synth.uniform(seed, shape)
+    keep = synth.uniform(seed + 1, shape, 0.0, 1.0) < density
+    return np.where(keep, vals, np.float32(0)).astype(np.float32)
+
+
+def gpu_csr_from_dense(dense, N):
+    """(V, COL, ROW) through sph_csr_row_offsets_f32 + sph_csr_fill_f32."""
+    M, ld = dense.shape
+    dD = capi.DeviceBuffer.from_array(dense if dense.size else np.zeros(1, np.float32))
+    dRow = capi.DeviceBuffer(4 * (M + 1))
+    nnz = ctypes.c_uint32(0xDEADBEEF)
+    capi.call("sph_csr_row_offsets_f32", dRow.ptr, dD.ptr, M, N, ld, ctypes.byref(nnz))
+    ROW = dRow.download(np.uint32, (M + 1,))
+    assert ROW[M] == nnz.value
+    guard = 4
+    dV = capi.DeviceBuffer.from_array(np.full(nnz.value + guard, -77.0, np.float32))
+    dCol = capi.DeviceBuffer.from_array(np.full(nnz.value + guard, 0xABCDEF, np.uint32))
+    capi.call("sph_csr_fill_f32", dV.ptr, dCol.ptr, dRow.ptr, dD.ptr, M, N, ld)
+    V = dV.download(np.float32, (nnz.value + guard,))
+    COL = dCol.download(np.uint32, (nnz.value + guard,))
+    assert np.all(V[nnz.value:] == -77.0) and np.all(COL[nnz.value:] == 0xABCDEF)
+    for d in (dD, dRow, dV, dCol):
+        d.release()
+    return V[:nnz.value], COL[:nnz.value], ROW
+
+
+def gpu_csr_to_dense(V, COL, ROW, M, N, ld, fill):
+    dOut = capi.DeviceBuffer.from_array(np.full((M, ld), np.float32(fill)))
+    dV = capi.DeviceBuffer.from_array(V if V.size else np.zeros(1, np.float32))
+    dCol = capi.DeviceBuffer.from_array(COL if COL.size else np.zeros(1, np.uint32))
+    dRow = capi.DeviceBuffer.from_array(ROW)
+    capi.call("sph_csr_to_dense_f32", dOut.ptr, ld, dV.ptr, dCol.ptr, dRow.ptr, M, N)
+    out = dOut.download(np.float32, (M, ld))
+    for d in (dOut, dV, dCol, dRow):
+        d.release()
+    return out
+
+
+# rows x columns x pitch x density: every lanes-per-row variant (4..64), ragged widths, the
+# 16-byte and the scalar load path, empty and full rows, more rows than one scan block
+CASES = [(1, 1, 1, 1.0), (3, 2, 2, 0.5), (7, 13, 13, 0.3), (33, 16, 16, 0.2), (50, 31, 32, 0.5),
+         (64, 64, 64, 0.05), (100, 100, 104, 0.1), (9, 257, 260, 0.4), (40, 1000, 1000, 0.01),
+         (5000, 24, 24, 0.1), (9000, 8, 8, 0.0), (300, 300, 300, 1.0), (2, 5000, 5000, 0.02)]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conversion_matches_checker(dev, case):
+    M, N, ld, density = case
+    h.announce("sph_csr_* M N ld density =", case)
+    dense = sparse_dense(1000 + M + N, (M, ld), density)
+    dense[:, N:] = 5.0                                     # junk in the pitch padding
+    wantV, wantCol, wantRow = po.csr_from_dense(dense, N=N)
+    V, COL, ROW = gpu_csr_from_dense(dense, N)
+    assert np.array_equal(ROW, wantRow)
+    assert np.array_equal(COL, wantCol)
+    assert np.array_equal(bits(V), bits(wantV))
+    back = gpu_csr_to_dense(V, COL, ROW, M, N, ld, fill=9.0)
+    assert np.array_equal(bits(back), bits(po.csr_to_dense(wantV, wantCol, wantRow, M, N, ld, 9.0)))
+    assert np.array_equal(bits(back[:, :N]), bits(dense[:, :N]))
+    assert np.all(back[:, N:] == 9.0)
+
+
+def test_special_values_and_unaligned_base(dev):
+    h.announce("sph_csr_* -0.0 / NaN / unaligned base")
+    dense = np.array([[0.0, -0.0, 2.0, 0.0],
+                      [np.nan, 0.0, 0.0, -1.0],
+                      [0.0, 0.0, 0.0, 0.0]], np.float32)
+    V, COL, ROW = gpu_csr_from_dense(dense, 4)
+    assert ROW.tolist() == [0, 1, 3, 3] and COL.tolist() == [2, 0, 3]
+    assert V[0] == 2.0 and np.isnan(V[1]) and V[2] == -1.0
+    # base 4 bytes off a 16-byte boundary: scalar loads
+    flat = np.concatenate([[np.float32(3.0)], sparse_dense(77, (10, 12), 0.4).ravel()])
+    dD = capi.DeviceBuffer.from_array(flat.astype(np.float32))
+    dRow = capi.DeviceBuffer(4 * 11)
+    nnz = ctypes.c_uint32(0)
+    capi.call("sph_csr_row_offsets_f32", dRow.ptr, dD.at(4), 10, 12, 12, ctypes.byref(nnz))
+    want = po.csr_from_dense(np.ascontiguousarray(flat[1:].reshape(10, 12)))
+    assert np.array_equal(dRow.download(np.uint32, (11,)), want[2]) and nnz.value == want[2][-1]
+    dD.release()
+    dRow.release()
+
+
+def test_round_trip_at_configuration_5_size(dev):
+    """8192 x 8192 at 1 %: too slow to restate on the CPU entry by entry in a test, so checked
+    through what the conversion must preserve: counts, ordering, and the round trip."""
+    d = synth.config5()
+    M, K = d["M"], d["K"]
+    h.announce("sph_csr_* configuration 5", M, K)
+    dense = synth.densify(d["V"], d["COL"], d["ROW"], M, K)
+    V, COL, ROW = gpu_csr_from_dense(dense, K)
+    assert np.array_equal(ROW, d["ROW"]) and np.array_equal(COL, d["COL"])
+    assert np.array_equal(bits(V), bits(d["V"]))
+    back = gpu_csr_to_dense(V, COL, ROW, M, K, K, fill=1.0)
+    assert np.array_equal(bits(back), bits(dense))
+
+
+@pytest.mark.parametrize("case", [(1, 5, 7, 7, 0.5), (3, 20, 30, 32, 0.2), (4, 9, 16, 16, 0.0),
+                                  (2, 600, 40, 44, 0.3)])
+def test_host_layer_create_copy_convert(dev, case):
+    num, m, n, padded, density = case
+    h.announce("CreateSparseMatrixWithDenseMatrix / DeepCopy* / ConvertSparseMatrixToDenseMatrix",
+               case)
+    dense = sparse_dense(2000 + m, (num, m, padded), density)
+    dense[:, :, n:] = 5.0
+    nnz, V, COL, ROW, back = hl.csr_round_trip(dense, n, fill=7.0)
+    at = 0
+    for i in range(num):
+        wV, wC, wR = po.csr_from_dense(np.ascontiguousarray(dense[i]), N=n)
+        assert nnz[i] == wR[-1]
+        assert np.array_equal(ROW[i], wR)
+        assert np.array_equal(COL[at:at + nnz[i]], wC)
+        assert np.array_equal(bits(V[at:at + nnz[i]]), bits(wV))
+        at += int(nnz[i])
+    assert np.array_equal(bits(back[:, :, :n]), bits(dense[:, :, :n]))
+    assert np.all(back[:, :, n:] == 7.0)
+
+
+@pytest.mark.parametrize("dims", [(1, 1, 1), (5, 7, 3), (64, 100, 33), (256, 784, 128),
+                                  (1024, 1024, 10)])
+def test_sparse_linear_forward_equals_dense_layer_on_cpu(dev, dims):
+    batch, fin, fout = dims
+    h.announce("NN::SparseLinearForward", dims)
+    x = synth.uniform(91, (batch, fin))
+    W = sparse_dense(92, (fin, fout), 0.1 if fin > 8 else 1.0)
+    bias = synth.uniform(94, (fout,))
+    want = po.linear_forward(x, W, bias, threads=8)
+    got = hl.sparse_linear_forward(x, W, bias)
+    assert np.array_equal(bits(got), bits(want))

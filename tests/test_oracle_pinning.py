@@ -380,3 +380,44 @@ def test_linear_backward_closed_form_and_composition():
     assert np.array_equal(bits(b2), bits(po.sgd(bias, dB.reshape(fout), 0.01)))
     dxT, WT, bT = po.linear_backward(dx0, W, bias, dy, x, 0.01, threads=3)
     assert np.array_equal(bits(dxT), bits(dx)) and np.array_equal(bits(WT), bits(W2))
+
+
+# ---- dense <-> CSR --------------------------------------------------------------------------
+
+def _sparse_dense(seed, M, N, density, ld=None):
+    ld = N if ld is None else ld
+    vals = synth.uniform(seed, (M, ld))
+    keep = synth.uniform(seed + 1, (M, ld), 0.0, 1.0) < density
+    return np.where(keep, vals, np.float32(0)).astype(np.float32)
+
+
+def test_csr_conversion_against_scipy():
+    import scipy.sparse as sp
+    for seed, (M, N, density) in enumerate([(1, 1, 1.0), (5, 7, 0.5), (64, 300, 0.05),
+                                            (200, 33, 0.0), (17, 1024, 0.3), (3, 4, 1.0)]):
+        dense = _sparse_dense(500 + 2 * seed, M, N, density)
+        V, COL, ROW = po.csr_from_dense(dense)
+        want = sp.csr_matrix(dense)
+        want.sort_indices()
+        assert ROW.tolist() == want.indptr.tolist()
+        assert COL.tolist() == want.indices.tolist()
+        assert np.array_equal(bits(V), bits(want.data.astype(np.float32)))
+        assert ROW[-1] == np.count_nonzero(dense)
+        assert np.array_equal(bits(po.csr_to_dense(V, COL, ROW, M, N)), bits(want.toarray()))
+        assert np.array_equal(bits(po.csr_to_dense(V, COL, ROW, M, N)), bits(dense))
+
+
+def test_csr_conversion_pitch_and_special_values():
+    # N = 3 of a pitch of 5: the padding columns hold junk that must not be read or written
+    dense = np.array([[0.0, -0.0, 2.0, 9.0, 9.0],
+                      [np.nan, 0.0, 0.0, 9.0, 9.0],
+                      [0.0, 0.0, 0.0, 9.0, 9.0],
+                      [1.0, -3.0, 4.0, 9.0, 9.0]], np.float32)
+    V, COL, ROW = po.csr_from_dense(dense, N=3)
+    assert ROW.tolist() == [0, 1, 2, 2, 5]                   # -0.0 dropped, NaN kept
+    assert COL.tolist() == [2, 0, 0, 1, 2]
+    assert np.isnan(V[1]) and V[[0, 2, 3, 4]].tolist() == [2.0, 1.0, -3.0, 4.0]
+    back = po.csr_to_dense(V, COL, ROW, 4, 3, ld=5, fill=7.0)
+    assert np.all(back[:, 3:] == 7.0)                        # padding untouched
+    assert back[0, :3].tolist() == [0.0, 0.0, 2.0] and not np.signbit(back[0, 1])
+    assert np.isnan(back[1, 0]) and back[3, :3].tolist() == [1.0, -3.0, 4.0]
