@@ -22,6 +22,7 @@
 // reference's random test sizes (Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:26-33).
 #include "sph_internal.h"
 
+#include <algorithm>
 #include <cstring>
 #include <mutex>
 #include <unordered_set>
@@ -41,6 +42,9 @@ struct GemmF32Args
     const SphGemmEntry* entries;  // device table, or null for stride arithmetic
     uint32_t M, N, K;
     uint32_t tilesM, tilesN;
+    uint32_t tilesTotal;  // tilesM * tilesN * units
+    uint32_t perXcd;      // ceil(tilesTotal / 8): the grid has 8 * perXcd workgroups
+    uint32_t band;        // tile rows per band of the in-unit ordering
     uint32_t outVec;     // 16-byte accesses to out are possible
     uint32_t overwrite;  // out = A*B instead of out += A*B
     int64_t strideOut, strideA, strideB;
@@ -149,6 +153,107 @@ __device__ __forceinline__ void StashXContig(float* __restrict__ slab, const flo
     }
 }
 
+// Workgroup -> tile.  Workgroups are handed to the 8 XCDs round robin (id % 8), and each XCD
+// has its own L2.  Workgroup `id` therefore takes logical tile (id % 8) * perXcd + id / 8, so
+// that an XCD owns one contiguous run of logical tiles; inside a unit the logical order walks
+// bands of `band` tile rows column by column, which makes a run a compact block of the
+// output whose A rows and B columns the XCD's workgroups share.  Returns false for the
+// surplus workgroups of a grid rounded up to 8 * perXcd.
+__device__ __forceinline__ bool MapTile(const GemmF32Args& args, uint32_t& tm, uint32_t& tn,
+                                        uint32_t& unit)
+{
+    const uint32_t id = blockIdx.x;
+    const uint32_t logical = (id & 7u) * args.perXcd + (id >> 3);
+    if (logical >= args.tilesTotal)
+        return false;
+    const uint32_t perUnit = args.tilesM * args.tilesN;
+    unit = logical / perUnit;
+    const uint32_t t = logical - unit * perUnit;
+    const uint32_t perBand = args.band * args.tilesN;
+    const uint32_t bandIdx = t / perBand;
+    const uint32_t within = t - bandIdx * perBand;
+    const uint32_t rows = min(args.band, args.tilesM - bandIdx * args.band);
+    tm = bandIdx * args.band + within % rows;
+    tn = within / rows;
+    return true;
+}
+
+// k index (inside a 16-wide step) that lane half `khalf` feeds to MFMA instruction t
+__device__ __forceinline__ constexpr uint32_t KOfPair(uint32_t t, uint32_t khalf)
+{
+    return 8u * (t / 4u) + 4u * khalf + (t % 4u);
+}
+
+// out (+)= acc for the TM x TN blocks of 32 x 32 one wavefront owns; rowBase / colBase are
+// the wavefront's first row and column.  `wide`: N % 4 == 0 and 16-byte aligned output rows.
+template <int TM, int TN>
+__device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* __restrict__ out,
+                                          uint32_t rowBase, uint32_t colBase, uint32_t M,
+                                          uint32_t N, uint32_t l32, uint32_t khalf, bool wide,
+                                          bool accumulate)
+{
+    // ---- out += acc ---------------------------------------------------------
+    // With the operands swapped, register v of lane l holds row l%32 and column
+    // 8*(v/4) + 4*(l/32) + v%4 of its 32x32 block: registers 4q..4q+3 are 4
+    // consecutive columns.  The old values of the whole wavefront block are requested
+    // in one batch, then added and stored.
+    constexpr int kQuads = TM * TN * 4;
+    float4 old[kQuads];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const uint32_t r = rowBase + i * 32 + l32;
+                const uint32_t c = colBase + j * 32 + 8 * q + 4 * khalf;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (accumulate && r < M && c < N)
+                {
+                    const float* p = out + static_cast<size_t>(r) * N + c;
+                    if (wide)
+                        v = *reinterpret_cast<const float4*>(p);
+                    else
+                    {
+                        v.x = p[0];
+                        if (c + 1 < N) v.y = p[1];
+                        if (c + 2 < N) v.z = p[2];
+                        if (c + 3 < N) v.w = p[3];
+                    }
+                }
+                old[(i * TN + j) * 4 + q] = v;
+            }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const uint32_t r = rowBase + i * 32 + l32;
+                const uint32_t c = colBase + j * 32 + 8 * q + 4 * khalf;
+                if (r < M && c < N)
+                {
+                    float4 v = old[(i * TN + j) * 4 + q];
+                    v.x += acc[i][j][4 * q + 0];
+                    v.y += acc[i][j][4 * q + 1];
+                    v.z += acc[i][j][4 * q + 2];
+                    v.w += acc[i][j][4 * q + 3];
+                    float* p = out + static_cast<size_t>(r) * N + c;
+                    if (wide)
+                        *reinterpret_cast<float4*>(p) = v;
+                    else
+                    {
+                        p[0] = v.x;
+                        if (c + 1 < N) p[1] = v.y;
+                        if (c + 2 < N) p[2] = v.z;
+                        if (c + 3 < N) p[3] = v.w;
+                    }
+                }
+            }
+}
+
 template <int BM, int BN, bool VEC, bool TA, bool TB>
 __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args)
 {
@@ -170,11 +275,9 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
     const uint32_t waveM = wave >> 1;
     const uint32_t waveN = wave & 1;
 
-    uint32_t id = blockIdx.x;
-    const uint32_t tn = id % args.tilesN;
-    id /= args.tilesN;
-    const uint32_t tm = id % args.tilesM;
-    const uint32_t unit = id / args.tilesM;
+    uint32_t tm, tn, unit;
+    if (!MapTile(args, tm, tn, unit))
+        return;
 
     const float* __restrict__ A;
     const float* __restrict__ B;
@@ -242,8 +345,11 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
     }
     __syncthreads();
 
-    // MFMA 32x32x2 operand layout: lane l supplies A[l % 32][l / 32] and
-    // B[l / 32][l % 32]; two k values per instruction.
+    // MFMA 32x32x2 operand layout: lane l supplies A[l % 32][k] and B[k][l % 32] where k is
+    // one value for lanes 0-31 and another for lanes 32-63.  Which two k an instruction takes
+    // is free as long as A and B agree: instruction t of a step takes k = 8*(t/4) + t%4 from
+    // the lower half and that + 4 from the upper half, the assignment every fp32 kernel of
+    // this file uses, so that they all add the K products in the same order.
     const uint32_t l32 = lane & 31;
     const uint32_t khalf = lane >> 5;
 
@@ -261,10 +367,10 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
         auto readPair = [&](int slot, int kk) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                a[slot][i] = as[(kk + khalf) * LDA + i * 32];
+                a[slot][i] = as[KOfPair(kk / 2, khalf) * LDA + i * 32];
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                b[slot][j] = bs[(kk + khalf) * LDB + j * 32];
+                b[slot][j] = bs[KOfPair(kk / 2, khalf) * LDB + j * 32];
         };
         readPair(0, 0);
 #pragma unroll
@@ -290,68 +396,324 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
         __syncthreads();
     }
 
-    // ---- out += acc ---------------------------------------------------------
-    // With the operands swapped, register v of lane l holds row l%32 and column
-    // 8*(v/4) + 4*(l/32) + v%4 of its 32x32 block: registers 4q..4q+3 are 4
-    // consecutive columns.  The old values of the whole wavefront block are requested
-    // in one batch, then added and stored.
-    constexpr int kQuads = TM * TN * 4;
-    float4 old[kQuads];
-    const bool wide = args.outVec != 0;  // N % 4 == 0 and 16-byte aligned output rows
-    const bool accumulate = args.overwrite == 0;
+    StoreTile<TM, TN>(acc, out, rowBase + waveM * WM, colBase + waveN * WN, M, N, l32, khalf,
+                      args.outVec != 0, args.overwrite == 0);
+}
+
+// ---------------------------------------------------------------------------
+// Pipelined variant for aligned operands with K % 16 == 0.
+//
+// The tiled kernel above holds a K step in registers between its global load and its LDS
+// store, so only one step can be in flight; with one workgroup per compute unit (mid-size
+// products) every step then waits out a full memory latency.  Here the slabs travel from
+// global memory straight into a ring of STAGES LDS stages (global_load_lds_dwordx4, no
+// registers in between), STAGES - 2 steps ahead of the one being multiplied, with one barrier
+// per step.
+//
+// LDS layout of one stage (K step BK = 16 or 32).  An operand stored with K contiguous keeps
+// its rows: X rows of BK floats in 16-byte chunks, chunk c of row x at position
+// c ^ ((x >> 2) & 3) for BK = 16 and c ^ ((x >> 1) & 7) for BK = 32, so that the 16-byte
+// fragment reads of 16 consecutive rows touch every bank once.  BK = 32 makes a row segment a
+// whole 128-byte cache line.  A lane then
+// gets k = 4h..4h+3 of its row in one read (h = lane / 32), which is why the k assignment of
+// this file gives lane half h the values 8q + 4h + e.  An operand stored k-major keeps its 16
+// rows of X floats, with 128 bytes of padding after every 4 rows so that the two lane halves
+// of a 4-byte fragment read (rows k and k + 4) fall into different banks.
+// Rows / columns past the matrix edge are clamped to the last valid ones: they only feed
+// output elements that are never stored.
+// ---------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* LdsVoidPtr;
+
+__device__ __forceinline__ void DmaToLds16(uint32_t laneByteOffset, const void* uniformBase,
+                                           uint32_t ldsByteAddr)
+{
+    // lane i reads 16 bytes at uniformBase + laneByteOffset; they land at ldsByteAddr + 16*i
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(ldsByteAddr), "v"(laneByteOffset), "s"(uniformBase)
+                 : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void WaitVmem()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+template <int X, int BK>
+struct DmaTile
+{
+    // K-contiguous slab: X rows of BK floats.  k-major slab: BK rows of X floats.
+    static constexpr uint32_t kCopies = X * BK / 256;     // 1 KiB copies per operand and step
+    static constexpr uint32_t kChunks = BK / 4;           // 16-byte chunks of a K-contiguous row
+    static constexpr uint32_t kRowsPerCopyK = 256 / BK;   // K-contiguous rows per copy
+    static constexpr uint32_t kRowsPer256 = 64 / BK;      // K-contiguous rows per 256 bytes
+    static constexpr uint32_t kRowBytes = X * 4;          // k-major row
+    static constexpr uint32_t kRowsPerCopyX = 1024 / kRowBytes;
+    static constexpr uint32_t kBytesKContig = X * BK * 4;
+    static constexpr uint32_t kBytesXContig = X * BK * 4 + (BK / 4) * 128;
+
+    // position of chunk c of K-contiguous row x
+    static __device__ __forceinline__ uint32_t Swizzle(uint32_t x)
+    {
+        return (x / kRowsPer256) & (kChunks - 1);
+    }
+    // LDS offset of copy j of a k-major slab (128 bytes of padding after every 4 rows)
+    static __device__ __forceinline__ constexpr uint32_t CopyOffsetXContig(uint32_t j)
+    {
+        return j * 1024u + ((j * kRowsPerCopyX) / 4u) * 128u;
+    }
+    static __device__ __forceinline__ constexpr uint32_t RowOffsetXContig(uint32_t k)
+    {
+        return k * kRowBytes + (k / 4u) * 128u;
+    }
+};
+
+template <int BM, int BN, int BK, int STAGES, bool TA, bool TB>
+__global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args args)
+{
+    static_assert(BM == BN, "square tiles only");
+    static_assert(BK == 16 || BK == 32, "K step of 16 or 32");
+    constexpr int WM = BM / 2;
+    constexpr int WN = BN / 2;
+    constexpr int TM = WM / 32;
+    constexpr int TN = WN / 32;
+    using TileA = DmaTile<BM, BK>;
+    using TileB = DmaTile<BN, BK>;
+    constexpr uint32_t kBytesA = TA ? TileA::kBytesXContig : TileA::kBytesKContig;
+    constexpr uint32_t kBytesB = TB ? TileB::kBytesKContig : TileB::kBytesXContig;
+    constexpr uint32_t kStageBytes = kBytesA + kBytesB;
+    constexpr uint32_t kCopiesPerWave = (TileA::kCopies + TileB::kCopies) / 4;  // per step
+    constexpr uint32_t kCopiesA = TileA::kCopies / 4;  // per wavefront
+    constexpr uint32_t kCopiesB = TileB::kCopies / 4;
+    constexpr uint32_t kBlocks = BK / 8;  // 8-wide k blocks (4 MFMAs each) per step
+
+    __shared__ __attribute__((aligned(1024))) char lds[STAGES * kStageBytes];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t waveM = wave >> 1;
+    const uint32_t waveN = wave & 1;
+    const uint32_t l32 = lane & 31;
+    const uint32_t khalf = lane >> 5;
+
+    uint32_t tm, tn, unit;
+    if (!MapTile(args, tm, tn, unit))
+        return;
+
+    const float* A;
+    const float* B;
+    float* out;
+    if (args.entries != nullptr)
+    {
+        const SphGemmEntry e = args.entries[unit];
+        A = args.A + e.aOff;
+        B = args.B + e.bOff;
+        out = args.out + e.outOff;
+    }
+    else
+    {
+        A = args.A + args.strideA * static_cast<int64_t>(unit);
+        B = args.B + args.strideB * static_cast<int64_t>(unit);
+        out = args.out + args.strideOut * static_cast<int64_t>(unit);
+    }
+    const uint32_t M = args.M, N = args.N, K = args.K;
+    const uint32_t rowBase = tm * BM;
+    const uint32_t colBase = tn * BN;
+
+    // ---- what this lane copies every step -------------------------------------------------
+    // Copy j of an operand is taken by wavefront j % 4.  Lane offsets are bytes from the
+    // operand's base at step 0; the base advances by one K step per step.
+    uint32_t aLane[kCopiesA], bLane[kCopiesB];
+    uint32_t aDst[kCopiesA], bDst[kCopiesB];
+    auto laneOffsetKContig = [&](uint32_t j, uint32_t xBase, uint32_t limit) {
+        using T = TileA;  // chunk geometry depends on BK only
+        const uint32_t x = j * T::kRowsPerCopyK + lane / T::kChunks;  // row inside the tile
+        const uint32_t c = (lane % T::kChunks) ^ T::Swizzle(x);
+        const uint32_t gx = min(xBase + x, limit - 1);
+        return (gx * K + c * 4) * 4u;
+    };
+    auto laneOffsetXContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t rowBytes) {
+        const uint32_t b = j * 1024 + lane * 16;  // byte inside the unpadded slab
+        const uint32_t k = b / rowBytes;
+        const uint32_t col = (b % rowBytes) / 4;
+        const uint32_t gx = min(xBase + col, limit - 4);
+        return (k * limit + gx) * 4u;
+    };
+#pragma unroll
+    for (uint32_t i = 0; i < kCopiesA; ++i)
+    {
+        const uint32_t j = wave + 4 * i;
+        if constexpr (TA)
+        {
+            aLane[i] = laneOffsetXContig(j, rowBase, M, TileA::kRowBytes);
+            aDst[i] = TileA::CopyOffsetXContig(j);
+        }
+        else
+        {
+            aLane[i] = laneOffsetKContig(j, rowBase, M);
+            aDst[i] = j * 1024;
+        }
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kCopiesB; ++i)
+    {
+        const uint32_t j = wave + 4 * i;
+        if constexpr (TB)
+        {
+            bLane[i] = laneOffsetKContig(j, colBase, N);
+            bDst[i] = kBytesA + j * 1024;
+        }
+        else
+        {
+            bLane[i] = laneOffsetXContig(j, colBase, N, TileB::kRowBytes);
+            bDst[i] = kBytesA + TileB::CopyOffsetXContig(j);
+        }
+    }
+    const size_t aStepBytes = TA ? static_cast<size_t>(BK) * M * 4 : BK * 4;
+    const size_t bStepBytes = TB ? BK * 4 : static_cast<size_t>(BK) * N * 4;
+    const uint32_t ldsBase =
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsVoidPtr)(lds)));
+    const uint32_t steps = K / BK;
+
+    auto issue = [&](uint32_t step) {
+        // steps past the end fetch the last one again into a stage nobody reads any more,
+        // which keeps the number of outstanding copies the same in every iteration
+        const uint32_t src = min(step, steps - 1);
+        const uint32_t stage = ldsBase + (step % STAGES) * kStageBytes;
+        const char* aBase = reinterpret_cast<const char*>(A) + src * aStepBytes;
+        const char* bBase = reinterpret_cast<const char*>(B) + src * bStepBytes;
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesA; ++i)
+            DmaToLds16(aLane[i], aBase, stage + aDst[i]);
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesB; ++i)
+            DmaToLds16(bLane[i], bBase, stage + bDst[i]);
+    };
+
+    floatx16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                const uint32_t r = rowBase + waveM * WM + i * 32 + l32;
-                const uint32_t c = colBase + waveN * WN + j * 32 + 8 * q + 4 * khalf;
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (accumulate && r < M && c < N)
-                {
-                    const float* p = out + static_cast<size_t>(r) * N + c;
-                    if (wide)
-                        v = *reinterpret_cast<const float4*>(p);
-                    else
-                    {
-                        v.x = p[0];
-                        if (c + 1 < N) v.y = p[1];
-                        if (c + 2 < N) v.z = p[2];
-                        if (c + 3 < N) v.w = p[3];
-                    }
-                }
-                old[(i * TN + j) * 4 + q] = v;
-            }
+            for (int v = 0; v < 16; ++v)
+                acc[i][j][v] = 0.f;
+
+    // ---- fragment addresses inside a stage -------------------------------------------------
+    // K-contiguous operand: byte offset of this lane's row, chunk chosen per 8-wide k block.
+    // k-major operand: byte offset of this lane's column; the row offset is added per k.
+    uint32_t aFrag[TM], bFrag[TN];
+    uint32_t aSwz[TM], bSwz[TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
+    {
+        const uint32_t x = waveM * WM + i * 32 + l32;
+        aFrag[i] = TA ? x * 4 : x * BK * 4;
+        aSwz[i] = TileA::Swizzle(x);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+    {
+        const uint32_t x = waveN * WN + j * 32 + l32;
+        bFrag[j] = kBytesA + (TB ? x * BK * 4 : x * 4);
+        bSwz[j] = TileB::Swizzle(x);
+    }
+
+    // fragments of k block q (k = 8q + 4*khalf + e, e = 0..3)
+    auto loadFragments = [&](float (&a)[TM][4], float (&b)[TN][4], const char* stage,
+                             uint32_t q) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+        {
+            if constexpr (TA)
+            {
+#pragma unroll
+                for (uint32_t e = 0; e < 4; ++e)
+                    a[i][e] = *reinterpret_cast<const float*>(
+                        stage + aFrag[i] + TileA::RowOffsetXContig(8 * q + e) +
+                        khalf * (TileA::RowOffsetXContig(4) - TileA::RowOffsetXContig(0)));
+            }
+            else
+            {
+                const float4 v = *reinterpret_cast<const float4*>(
+                    stage + aFrag[i] + (((2 * q + khalf) ^ aSwz[i]) << 4));
+                a[i][0] = v.x;
+                a[i][1] = v.y;
+                a[i][2] = v.z;
+                a[i][3] = v.w;
+            }
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
+        {
+            if constexpr (TB)
             {
-                const uint32_t r = rowBase + waveM * WM + i * 32 + l32;
-                const uint32_t c = colBase + waveN * WN + j * 32 + 8 * q + 4 * khalf;
-                if (r < M && c < N)
-                {
-                    float4 v = old[(i * TN + j) * 4 + q];
-                    v.x += acc[i][j][4 * q + 0];
-                    v.y += acc[i][j][4 * q + 1];
-                    v.z += acc[i][j][4 * q + 2];
-                    v.w += acc[i][j][4 * q + 3];
-                    float* p = out + static_cast<size_t>(r) * N + c;
-                    if (wide)
-                        *reinterpret_cast<float4*>(p) = v;
-                    else
-                    {
-                        p[0] = v.x;
-                        if (c + 1 < N) p[1] = v.y;
-                        if (c + 2 < N) p[2] = v.z;
-                        if (c + 3 < N) p[3] = v.w;
-                    }
-                }
+                const float4 v = *reinterpret_cast<const float4*>(
+                    stage + bFrag[j] + (((2 * q + khalf) ^ bSwz[j]) << 4));
+                b[j][0] = v.x;
+                b[j][1] = v.y;
+                b[j][2] = v.z;
+                b[j][3] = v.w;
             }
+            else
+            {
+#pragma unroll
+                for (uint32_t e = 0; e < 4; ++e)
+                    b[j][e] = *reinterpret_cast<const float*>(
+                        stage + bFrag[j] + TileB::RowOffsetXContig(8 * q + e) +
+                        khalf * (TileB::RowOffsetXContig(4) - TileB::RowOffsetXContig(0)));
+            }
+        }
+    };
+    auto multiply = [&](const float (&a)[TM][4], const float (&b)[TN][4]) {
+#pragma unroll
+        for (uint32_t e = 0; e < 4; ++e)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] =
+                        __builtin_amdgcn_mfma_f32_32x32x2f32(b[j][e], a[i][e], acc[i][j], 0, 0, 0);
+    };
+
+#pragma unroll
+    for (uint32_t p = 0; p < STAGES - 1; ++p)
+        issue(p);
+
+    // Fragments are read one k block (8 values) ahead of the MFMAs that use them; the first
+    // block of step s+1 is read while the last block of step s is multiplied.
+    float fa[2][TM][4], fb[2][TN][4];
+    WaitVmem<(STAGES - 2) * kCopiesPerWave>();
+    __syncthreads();
+    loadFragments(fa[0], fb[0], lds, 0);
+
+    for (uint32_t s = 0; s < steps; ++s)
+    {
+        // steps s and s+1 have landed once at most the STAGES-3 later ones are pending
+        WaitVmem<(STAGES - 3) * kCopiesPerWave>();
+        __syncthreads();  // everybody's copies are visible; everybody has left step s-1
+        issue(s + STAGES - 1);
+
+        const char* cur = lds + (s % STAGES) * kStageBytes;
+        const char* next = lds + ((s + 1) % STAGES) * kStageBytes;
+#pragma unroll
+        for (uint32_t q = 0; q < kBlocks; ++q)
+        {
+            if (q + 1 < kBlocks)
+                loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], cur, q + 1);
+            else
+                loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], next, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(fa[q & 1], fb[q & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    WaitVmem<0>();  // the surplus copies of the last steps still target LDS
+
+    StoreTile<TM, TN>(acc, out, rowBase + waveM * WM, colBase + waveN * WN, M, N, l32, khalf,
+                      args.outVec != 0, args.overwrite == 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -584,9 +946,25 @@ void LaunchSkinny(const GemmF32Args& args, dim3 grid, bool vec, hipStream_t stre
 }
 
 template <bool TA, bool TB>
-void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, hipStream_t stream)
+void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dma,
+                 hipStream_t stream)
 {
     const dim3 block(kThreads);
+    if (dma)
+    {
+        if (big)
+            hipLaunchKernelGGL((GemmF32DmaKernel<128, 128, 16, 4, TA, TB>), grid, block, 0, stream, args);
+        else
+        {
+            if (args.K % 32 == 0)
+                hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB>), grid, block, 0,
+                                   stream, args);
+            else
+                hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 16, 6, TA, TB>), grid, block, 0,
+                                   stream, args);
+        }
+        return;
+    }
     if (big)
     {
         if (vec)
@@ -657,18 +1035,34 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     args.tilesM = (args.M + bm - 1) / bm;
     args.tilesN = (args.N + bm - 1) / bm;
     const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
-    if (blocks >= (1ull << 31))
+    if (blocks >= (1ull << 31) - 8)
         return sph::Fail(SPH_ERR_INVALID, "sph_gemm_f32 - too many tiles for one launch");
+    args.tilesTotal = static_cast<uint32_t>(blocks);
+    args.perXcd = (args.tilesTotal + 7) / 8;
+    // band height ~ square root of the tiles an XCD works on at once (32 compute units, up
+    // to two resident workgroups each), as a power of two
+    {
+        const uint32_t together = std::min<uint32_t>(args.perXcd, 64);
+        uint32_t band = 1;
+        while (band * band * 4 <= together)
+            band *= 2;
+        args.band = std::min(band, args.tilesM);
+    }
 
-    const dim3 grid(static_cast<uint32_t>(blocks));
+    const dim3 grid(args.perXcd * 8);
+    // straight-to-LDS pipeline: whole K steps, 16-byte chunks everywhere, at least one chunk
+    // per clamped edge, and lane offsets that fit 32 bits
+    const bool dma = aligned && args.K >= kBK && args.K % kBK == 0 && args.M >= 4 && args.N >= 4 &&
+                     static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
+                     static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
     if (transA && transB)
-        LaunchTiled<true, true>(args, grid, big, aligned, stream);
+        LaunchTiled<true, true>(args, grid, big, aligned, dma, stream);
     else if (transA)
-        LaunchTiled<true, false>(args, grid, big, aligned, stream);
+        LaunchTiled<true, false>(args, grid, big, aligned, dma, stream);
     else if (transB)
-        LaunchTiled<false, true>(args, grid, big, aligned, stream);
+        LaunchTiled<false, true>(args, grid, big, aligned, dma, stream);
     else
-        LaunchTiled<false, false>(args, grid, big, aligned, stream);
+        LaunchTiled<false, false>(args, grid, big, aligned, dma, stream);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
