@@ -131,9 +131,10 @@ def bench_f32(capi, A, B, C, M, N, K, batch, sb, steps, warmup):
     return event_ms
 
 
-def bench_mlp(capi, synth, steps, warmup):
+def bench_mlp(capi, synth, steps, warmup, fused=False):
     """Configuration 4 through the C ABI: per layer ones[batch,1] x bias (K = 1 GEMM), x x W,
-    ReLU between layers -- the call sequence of Linear's forward pass."""
+    ReLU between layers -- the call sequence of Linear's forward pass; with `fused` one
+    sph_linear_forward_f32 per layer instead (same result bits)."""
     d = synth.config4()
     batch = d["x"].shape[0]
     sizes = [d["x"].shape[1]] + [w.shape[1] for w in d["W"]]
@@ -148,6 +149,11 @@ def bench_mlp(capi, synth, steps, warmup):
         cur = x
         for l in range(3):
             n_in, n_out = sizes[l], sizes[l + 1]
+            if fused:
+                capi.call("sph_linear_forward_f32", y[l].ptr, cur.ptr, W[l].ptr, b[l].ptr, batch,
+                          n_in, n_out, capi.SPH_LINEAR_RELU if l < 2 else 0)
+                cur = y[l]
+                continue
             capi.call("sph_fill_f32", y[l].ptr, 0.0, batch * n_out)
             capi.call("sph_gemm_f32", y[l].ptr, ones.ptr, b[l].ptr, batch, n_out, 1, 1,
                       batch * n_out, batch, n_out)
@@ -433,6 +439,10 @@ def main():
         ms, fl = bench_mlp(capi, synth, 100, 10)
         others["config4_mlp_forward"] = {"forward_ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                                          "kernels_per_forward": 11}
+        ms, fl = bench_mlp(capi, synth, 100, 10, fused=True)
+        others["config4_mlp_forward_fused"] = {"forward_ms": ms,
+                                               "tflops": fl / (ms * 1e-3) / 1e12,
+                                               "kernels_per_forward": 3}
         ms_ref, fl = bench_mlp_backward(capi, synth, 100, 10, direct=False)
         ms_dir, _ = bench_mlp_backward(capi, synth, 100, 10, direct=True)
         others["config4_mlp_backward_sgd"] = {

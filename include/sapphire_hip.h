@@ -105,7 +105,7 @@ int sph_fill_f32(float* dst, float value, size_t count);
 
 /* out[i] = in[i] > 0 ? in[i] : 0.  Replaces Dense::Cuda::ReLU
  * (Sources/Sapphire/compute/dense/cuda/kernels/ActivationKernel.cu:11-22);
- * CPU counterpart NaiveBasic.cpp:159-165. */
+ * CPU counterpart NaiveBasic.cpp:159-165.  out may alias in. */
 int sph_relu_f32(float* out, const float* in, size_t count);
 
 /* Batched 2-D transpose, out[b][j][i] = in[b][i][j]; with broadcast != 0 the
@@ -177,6 +177,20 @@ int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M,
 int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M,
                     uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,
                     int64_t strideA, int64_t strideB, uint32_t flags);
+
+/* The forward pass of a fully connected layer in one launch:
+ *   y[b][j] = act((0 + bias[j]) + sum_k x[b][k] * W[k][j])
+ * x is batch x inputs, W inputs x outputs, bias has outputs entries, y is
+ * batch x outputs and is not read.  This is what
+ * Sources/Sapphire/operations/Forward/Linear.cpp:113-136 computes with
+ * Gemm(y, ones, bias) and Gemm(y, x, W) on a zero y; with SPH_LINEAR_RELU the
+ * ReLU that follows the layer (Sources/Sapphire/compute/ActivationOps.cpp:52-67)
+ * is applied to the value before it is stored.  The product term and the bits
+ * of the result are those of sph_fill_f32 + two sph_gemm_f32 (+ sph_relu_f32). */
+#define SPH_LINEAR_RELU 1u
+int sph_linear_forward_f32(float* y, const float* x, const float* W,
+                           const float* bias, uint32_t batch, uint32_t inputs,
+                           uint32_t outputs, uint32_t flags);
 
 /* One M x N unit product per entry, out[outOff] += A[aOff] * B[bOff], offsets
  * in elements from the three bases.  Entries are read from host memory.  This

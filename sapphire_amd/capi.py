@@ -20,6 +20,7 @@ SPH_GEMM_ACCUMULATE = 0
 SPH_GEMM_OVERWRITE = 1
 SPH_GEMM_TRANS_A = 2
 SPH_GEMM_TRANS_B = 4
+SPH_LINEAR_RELU = 1
 
 
 class SphError(RuntimeError):
@@ -83,6 +84,7 @@ SIGNATURES = {
     "sph_sgd_step_f32": [_vp, _vp, ctypes.c_float, _sz],
     "sph_gemm_f32": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64],
     "sph_gemm_f32_ex": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
+    "sph_linear_forward_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32],
     "sph_gemm_f32_grouped": [ctypes.POINTER(SphGemmEntry), _u32, _vp, _vp, _vp, _u32, _u32, _u32],
     "sph_gemm_f16f32": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
     "sph_csr_row_offsets_f32": [_vp, _vp, _u32, _u32, _u32, ctypes.POINTER(ctypes.c_uint32)],

@@ -47,8 +47,8 @@ __global__ __launch_bounds__(kThreads) void FillKernel(float* __restrict__ dst, 
         dst[i] = value;
 }
 
-__global__ __launch_bounds__(kThreads) void ReluKernel(float* __restrict__ out,
-                                                       const float* __restrict__ in,
+// out may alias in: every element is read before it is written, by the same lane
+__global__ __launch_bounds__(kThreads) void ReluKernel(float* out, const float* in,
                                                        size_t count, int vec)
 {
     const size_t tid = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;

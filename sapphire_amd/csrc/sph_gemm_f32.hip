@@ -47,6 +47,8 @@ struct GemmF32Args
     uint32_t band;        // tile rows per band of the in-unit ordering
     uint32_t outVec;     // 16-byte accesses to out are possible
     uint32_t overwrite;  // out = A*B instead of out += A*B
+    uint32_t relu;       // out = max(., 0) applied to the value that is stored
+    const float* bias;   // when set: out = (0 + bias[column]) + A*B, out is not read
     int64_t strideOut, strideA, strideB;
 };
 
@@ -190,7 +192,8 @@ template <int TM, int TN>
 __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* __restrict__ out,
                                           uint32_t rowBase, uint32_t colBase, uint32_t M,
                                           uint32_t N, uint32_t l32, uint32_t khalf, bool wide,
-                                          bool accumulate)
+                                          bool accumulate, const float* __restrict__ bias = nullptr,
+                                          bool relu = false)
 {
     // ---- out += acc ---------------------------------------------------------
     // With the operands swapped, register v of lane l holds row l%32 and column
@@ -209,7 +212,15 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
                 const uint32_t r = rowBase + i * 32 + l32;
                 const uint32_t c = colBase + j * 32 + 8 * q + 4 * khalf;
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (accumulate && r < M && c < N)
+                if (bias != nullptr)
+                {
+                    // what the K = 1 product ones x bias leaves in a zero-filled out
+                    if (c + 0 < N) v.x = 0.f + bias[c + 0];
+                    if (c + 1 < N) v.y = 0.f + bias[c + 1];
+                    if (c + 2 < N) v.z = 0.f + bias[c + 2];
+                    if (c + 3 < N) v.w = 0.f + bias[c + 3];
+                }
+                else if (accumulate && r < M && c < N)
                 {
                     const float* p = out + static_cast<size_t>(r) * N + c;
                     if (wide)
@@ -240,6 +251,13 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
                     v.y += acc[i][j][4 * q + 1];
                     v.z += acc[i][j][4 * q + 2];
                     v.w += acc[i][j][4 * q + 3];
+                    if (relu)
+                    {
+                        v.x = v.x > 0 ? v.x : 0;
+                        v.y = v.y > 0 ? v.y : 0;
+                        v.z = v.z > 0 ? v.z : 0;
+                        v.w = v.w > 0 ? v.w : 0;
+                    }
                     float* p = out + static_cast<size_t>(r) * N + c;
                     if (wide)
                         *reinterpret_cast<float4*>(p) = v;
@@ -397,7 +415,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
     }
 
     StoreTile<TM, TN>(acc, out, rowBase + waveM * WM, colBase + waveN * WN, M, N, l32, khalf,
-                      args.outVec != 0, args.overwrite == 0);
+                      args.outVec != 0, args.overwrite == 0, args.bias, args.relu != 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -713,28 +731,28 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     WaitVmem<0>();  // the surplus copies of the last steps still target LDS
 
     StoreTile<TM, TN>(acc, out, rowBase + waveM * WM, colBase + waveN * WN, M, N, l32, khalf,
-                      args.outVec != 0, args.overwrite == 0);
+                      args.outVec != 0, args.overwrite == 0, args.bias, args.relu != 0);
 }
 
 // ---------------------------------------------------------------------------
-// Few-tile shapes (small M x N, long K): 32 x 32 output tile per workgroup, K split four
-// ways across its wavefronts.
+// Few-tile shapes (small M x N, long K): 32 x 32 output tile per workgroup, K split across
+// its WAVES wavefronts (4, or 16 when even these tiles occupy less than a quarter of the chip
+// and K >= 512).
 //
 // With few output tiles the tiled kernel above leaves most compute units idle and is bound by
 // the latency of one load -> LDS -> MFMA chain per K step.  Here every wavefront reads its
 // operands straight from global memory in MFMA layout (A: 16 bytes per lane along K, lines
 // reused from L1 over the next steps; B: one row segment per lane half), keeps several loads
-// in flight, and accumulates a private 32 x 32 partial over its quarter of K.  The four
+// in flight, and accumulates a private 32 x 32 partial over its share of K.  The
 // partials are then added in wavefront order through LDS, so the result does not depend on
 // timing.  The two k values of one MFMA come from lanes 0-31 and 32-63; which k each half
 // holds is free as long as A and B agree, and is chosen so that A is read with float4.
 // ---------------------------------------------------------------------------
-constexpr int kSkinnyThreads = 256;
 
-template <bool VEC, bool TA, bool TB>
-__global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const GemmF32Args args)
+template <bool VEC, bool TA, bool TB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32Args args)
 {
-    __shared__ float partial[3][32 * 32];
+    __shared__ float partial[WAVES - 1][32 * 32];
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
@@ -769,7 +787,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const Gemm
 
     // this wavefront's K range, in groups of 8 (one float4 of A per lane half)
     const uint32_t groups = (K + 7) / 8;
-    const uint32_t perWave = (groups + 3) / 4;
+    const uint32_t perWave = (groups + WAVES - 1) / WAVES;
     const uint32_t gBegin = min(wave * perWave, groups);
     const uint32_t gEnd = min(gBegin + perWave, groups);
 
@@ -870,7 +888,7 @@ __global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const Gemm
     if (wave != 0)
         return;
 #pragma unroll
-    for (int w = 0; w < 3; ++w)
+    for (int w = 0; w < WAVES - 1; ++w)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
         {
@@ -892,7 +910,25 @@ __global__ __launch_bounds__(kSkinnyThreads) void GemmF32SkinnyKernel(const Gemm
         if (c >= N)
             continue;
         float* p = out + static_cast<size_t>(row) * N + c;
-        if (args.overwrite)
+        if (args.bias != nullptr || args.relu)
+        {
+            // fused Linear epilogue: (0 + bias) + product, optional ReLU, out not read
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (c + e < N)
+                {
+                    float old = 0.f;
+                    if (args.bias != nullptr)
+                        old = 0.f + args.bias[c + e];
+                    else if (!args.overwrite)
+                        old = p[e];
+                    float v = old + acc[4 * q + e];
+                    if (args.relu)
+                        v = v > 0 ? v : 0;
+                    p[e] = v;
+                }
+        }
+        else if (args.overwrite)
         {
             p[0] = acc[4 * q + 0];
             if (c + 1 < N) p[1] = acc[4 * q + 1];
@@ -935,14 +971,26 @@ std::mutex gTableMutex;
 EntryTable gTables[16];
 
 template <bool TA, bool TB>
-void LaunchSkinny(const GemmF32Args& args, dim3 grid, bool vec, hipStream_t stream)
+void LaunchSkinny(const GemmF32Args& args, dim3 grid, bool vec, bool wide, hipStream_t stream)
 {
+    // `wide`: 16 wavefronts per tile instead of 4 when even the 32 x 32 tiles leave most of
+    // the chip idle and K is long enough to give each wavefront a few steps
+    if (wide)
+    {
+        if (vec)
+            hipLaunchKernelGGL((GemmF32SkinnyKernel<true, TA, TB, 16>), grid, dim3(1024), 0,
+                               stream, args);
+        else
+            hipLaunchKernelGGL((GemmF32SkinnyKernel<false, TA, TB, 16>), grid, dim3(1024), 0,
+                               stream, args);
+        return;
+    }
     if (vec)
-        hipLaunchKernelGGL((GemmF32SkinnyKernel<true, TA, TB>), grid, dim3(kSkinnyThreads), 0,
-                           stream, args);
+        hipLaunchKernelGGL((GemmF32SkinnyKernel<true, TA, TB, 4>), grid, dim3(256), 0, stream,
+                           args);
     else
-        hipLaunchKernelGGL((GemmF32SkinnyKernel<false, TA, TB>), grid, dim3(kSkinnyThreads), 0,
-                           stream, args);
+        hipLaunchKernelGGL((GemmF32SkinnyKernel<false, TA, TB, 4>), grid, dim3(256), 0, stream,
+                           args);
 }
 
 template <bool TA, bool TB>
@@ -1016,14 +1064,16 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
             kVec = kVec && (reinterpret_cast<uintptr_t>(args.A) & 15u) == 0;
         if (transB)
             kVec = kVec && (reinterpret_cast<uintptr_t>(args.B) & 15u) == 0;
+        const bool wide = blocks32 * 4 <= static_cast<uint64_t>(sph::ComputeUnits()) &&
+                          args.K >= 512;
         if (transA && transB)
-            LaunchSkinny<true, true>(args, grid32, kVec, stream);
+            LaunchSkinny<true, true>(args, grid32, kVec, wide, stream);
         else if (transA)
-            LaunchSkinny<true, false>(args, grid32, false, stream);
+            LaunchSkinny<true, false>(args, grid32, false, wide, stream);
         else if (transB)
-            LaunchSkinny<false, true>(args, grid32, kVec, stream);
+            LaunchSkinny<false, true>(args, grid32, kVec, wide, stream);
         else
-            LaunchSkinny<false, false>(args, grid32, kVec, stream);
+            LaunchSkinny<false, false>(args, grid32, kVec, wide, stream);
         SPH_CHECK_LAUNCH();
         return SPH_OK;
     }
@@ -1131,6 +1181,31 @@ int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M, uint
     const bool stridesAligned = (strideA % 4 == 0) && (strideB % 4 == 0);
     return Launch(args, batch, stridesAligned, strideOut % 4 == 0 || batch == 1,
                   (flags & SPH_GEMM_TRANS_A) != 0, (flags & SPH_GEMM_TRANS_B) != 0, stream);
+}
+
+int sph_linear_forward_f32(float* y, const float* x, const float* W, const float* bias,
+                           uint32_t batch, uint32_t inputs, uint32_t outputs, uint32_t flags)
+{
+    SPH_REQUIRE(batch != 0 && outputs != 0, "batch and outputs must be non-zero");
+    SPH_REQUIRE((flags & ~SPH_LINEAR_RELU) == 0, "unknown flag");
+    SPH_REQUIRE(y != nullptr && bias != nullptr, "null pointer");
+    SPH_REQUIRE(inputs == 0 || (x != nullptr && W != nullptr), "null pointer");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+
+    GemmF32Args args{};
+    args.out = y;
+    args.A = x;
+    args.B = W;
+    args.entries = nullptr;
+    args.M = batch;
+    args.N = outputs;
+    args.K = inputs;
+    args.overwrite = 1u;
+    args.bias = bias;
+    args.relu = (flags & SPH_LINEAR_RELU) ? 1u : 0u;
+    return Launch(args, 1, true, true, false, false, stream);
 }
 
 int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M, uint32_t N, uint32_t K,

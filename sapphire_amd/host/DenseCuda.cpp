@@ -86,6 +86,16 @@ void GemmTransposed(float* out, const float* A, const float* B, unsigned int M, 
           "GemmTransposed");
 }
 
+void LinearForward(float* y, const float* x, const float* W, const float* bias,
+                   unsigned int batch, unsigned int inputs, unsigned int outputs, bool relu,
+                   int deviceId)
+{
+    Compute::Cuda::CudaSetDevice(deviceId);
+    Check(sph_linear_forward_f32(y, x, W, bias, batch, inputs, outputs,
+                                 relu ? SPH_LINEAR_RELU : 0u),
+          "LinearForward");
+}
+
 void ConvertToHalf(std::uint16_t* dst, const float* src, std::size_t size)
 {
     Check(sph_convert_f32_to_f16(dst, src, size), "ConvertToHalf");

@@ -2,6 +2,7 @@
 
 #include <Sapphire/compute/BasicOps.hpp>
 #include <Sapphire/compute/Initialize.hpp>
+#include <Sapphire/compute/dense/cuda/Gemm.hpp>
 #include <Sapphire/compute/sparse/SparseGemm.hpp>
 
 #include <stdexcept>
@@ -38,6 +39,26 @@ void LinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
 
     Compute::Gemm(y2, ones, bias2);
     Compute::Gemm(y2, x2, weight);
+}
+
+void LinearForwardFused(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
+                        const TensorUtil::TensorData& weight,
+                        const TensorUtil::TensorData& bias, bool relu)
+{
+    if (x.Mode() != weight.Mode() || x.Mode() != bias.Mode() || x.Mode() != y.Mode())
+        throw std::invalid_argument("NN::Linear - Device mode inequality");
+    if (x.Mode() != ComputeMode::Cuda)
+        throw std::runtime_error("NN::Linear - Host mode is not provided by the device backend");
+    const int batchSize = x.GetShape().GetNumUnits(1);
+    const int inputs = weight.Rows();
+    const int outputs = weight.Cols();
+    if (x.Size() != batchSize * inputs || y.Size() != batchSize * outputs ||
+        bias.Size() != outputs)
+        throw std::invalid_argument("NN::Linear - shape mismatch");
+    Compute::Dense::Cuda::LinearForward(
+        y.CudaMutableRawPtr(), x.CudaRawPtr(), weight.CudaRawPtr(), bias.CudaRawPtr(),
+        static_cast<unsigned int>(batchSize), static_cast<unsigned int>(inputs),
+        static_cast<unsigned int>(outputs), relu, y.GetCudaDevice().GetID());
 }
 
 void SparseLinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,

@@ -45,6 +45,12 @@ void GemmTransposed(float* out, const float* A, const float* B, unsigned int M, 
                     unsigned int K, unsigned int batchSize, bool transposeA, bool transposeB,
                     bool overwrite, int deviceId);
 
+//! y = act((0 + bias) + x * W) in one launch: the two GEMMs of Linear's forward pass on a zero
+//! y, optionally followed by ReLU, with the same result bits.
+void LinearForward(float* y, const float* x, const float* W, const float* bias,
+                   unsigned int batch, unsigned int inputs, unsigned int outputs, bool relu,
+                   int deviceId);
+
 //! dst[i] = binary16(src[i]), round to nearest even.
 void ConvertToHalf(std::uint16_t* dst, const float* src, std::size_t size);
 

@@ -26,6 +26,13 @@ namespace Sapphire::NN
 void LinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
                    const TensorUtil::TensorData& weight, const TensorUtil::TensorData& bias);
 
+//! The same layer as one launch: the bias row and, with `relu`, the activation that follows
+//! the layer (Compute::ReLU) are applied where the product is stored.  y is overwritten; the
+//! result has the bits of LinearForward on a zero y followed by Compute::ReLU.
+void LinearForwardFused(TensorUtil::TensorData& y, const TensorUtil::TensorData& x,
+                        const TensorUtil::TensorData& weight,
+                        const TensorUtil::TensorData& bias, bool relu);
+
 //! The same layer with a sparse weight, the variant NN::Linear rejects with
 //! "Sparse version not implemented" (Sources/Sapphire/operations/Forward/Linear.cpp:28-30).
 //! `weightTransposed` is a device record of the transposed weight, [out, in] in CSR, so that

@@ -179,7 +179,8 @@ int sphh_gemm_in_host_mode_throws()
 
 // layers Linear -> ReLU -> ... -> Linear (no ReLU after the last), sizes has layers + 1 entries
 int sphh_mlp_forward(const float* x, int batch, const int* sizes, int layers,
-                     const float* const* weights, const float* const* biases, float* out)
+                     const float* const* weights, const float* const* biases, float* out,
+                     int fused)
 {
     return Guard([&] {
         const CudaDevice cuda(0, "device0");
@@ -189,6 +190,13 @@ int sphh_mlp_forward(const float* x, int batch, const int* sizes, int layers,
             TensorData W = Upload(Shape({ sizes[l], sizes[l + 1] }), weights[l], cuda);
             TensorData bias = Upload(Shape({ sizes[l + 1] }), biases[l], cuda);
             TensorData y(Shape({ batch, sizes[l + 1] }), Type::Dense, cuda);  // zero-filled
+            if (fused)
+            {
+                // one launch per layer, activation included
+                NN::LinearForwardFused(y, cur, W, bias, l + 1 < layers);
+                cur = y;
+                continue;
+            }
             NN::LinearForward(y, cur, W, bias);
             if (l + 1 < layers)
             {

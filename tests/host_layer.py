@@ -27,7 +27,7 @@ def lib():
                                         ctypes.c_int]
         h.sphh_transpose.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int]
         h.sphh_mlp_forward.argtypes = [_fp, ctypes.c_int, _ip, ctypes.c_int,
-                                       ctypes.POINTER(_fp), ctypes.POINTER(_fp), _fp]
+                                       ctypes.POINTER(_fp), ctypes.POINTER(_fp), _fp, ctypes.c_int]
         h.sphh_sparse_gemm.argtypes = [_fp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _fp,
                                        ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint),
                                        _fp, ctypes.c_int]
@@ -108,12 +108,13 @@ def transpose(x, y_shape):
     return out
 
 
-def mlp_forward(x, weights, biases):
+def mlp_forward(x, weights, biases, fused=False):
     sizes = [x.shape[1]] + [w.shape[1] for w in weights]
     out = np.zeros((x.shape[0], sizes[-1]), np.float32)
     wp = (_fp * len(weights))(*[_f(w) for w in weights])
     bp = (_fp * len(biases))(*[_f(b) for b in biases])
-    _ok(lib().sphh_mlp_forward(_f(x), x.shape[0], _ints(sizes), len(weights), wp, bp, _f(out)))
+    _ok(lib().sphh_mlp_forward(_f(x), x.shape[0], _ints(sizes), len(weights), wp, bp, _f(out),
+                               1 if fused else 0))
     return out
 
 

@@ -176,3 +176,50 @@ def test_errors_are_statuses_not_crashes(dev):
     with pytest.raises(capi.SphError) as e:
         capi.call("sph_set_device", 99)
     assert "exceeds number of available devices" in str(e.value)
+
+
+@pytest.mark.parametrize("dims", [(1, 1, 1), (5, 0, 3), (7, 9, 5), (64, 64, 64), (100, 784, 130),
+                                  (256, 1024, 10), (1024, 1024, 1024), (130, 100, 257)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_linear_forward_one_launch(dev, dims, relu):
+    """sph_linear_forward_f32 against the CPU layer (bias GEMM + GEMM on a zero y, then ReLU) and,
+    bit for bit, against the unfused device sequence it replaces."""
+    batch, fin, fout = dims
+    h.announce("sph_linear_forward_f32", dims, "relu", relu)
+    x = synth.uniform(31, (batch, max(fin, 1)))[:, :fin].copy()
+    W = synth.uniform(32, (max(fin, 1), fout))[:fin].copy()
+    bias = synth.uniform(33, (fout,))
+    bias[0] = -0.0                                   # 0 + (-0) = +0 on the reference path
+    dX = capi.DeviceBuffer.from_array(x if x.size else np.zeros(1, np.float32))
+    dW = capi.DeviceBuffer.from_array(W if W.size else np.zeros(1, np.float32))
+    dB = capi.DeviceBuffer.from_array(bias)
+    dY = capi.DeviceBuffer.from_array(np.full((batch, fout), np.float32(np.nan)))
+    flags = capi.SPH_LINEAR_RELU if relu else 0
+    capi.call("sph_linear_forward_f32", dY.ptr, dX.ptr, dW.ptr, dB.ptr, batch, fin, fout, flags)
+    got = dY.download(np.float32, (batch, fout))
+
+    # the sequence it replaces, on the device
+    ones = capi.DeviceBuffer.from_array(np.ones(batch, np.float32))
+    dZ = capi.DeviceBuffer(4 * batch * fout)
+    capi.call("sph_fill_f32", dZ.ptr, 0.0, batch * fout)
+    capi.call("sph_gemm_f32", dZ.ptr, ones.ptr, dB.ptr, batch, fout, 1, 1, batch * fout, batch, fout)
+    if fin:
+        capi.call("sph_gemm_f32", dZ.ptr, dX.ptr, dW.ptr, batch, fout, fin, 1, batch * fout,
+                  batch * fin, fin * fout)
+    if relu:
+        capi.call("sph_relu_f32", dZ.ptr, dZ.ptr, batch * fout)
+    want_bits = dZ.download(np.float32, (batch, fout))
+    assert np.array_equal(got.view(np.uint32), want_bits.view(np.uint32))
+
+    ref = np.zeros((batch, fout), np.float32)
+    if fin:
+        ref = po.linear_forward(x, W, bias, threads=8)
+    else:
+        ref += (np.float32(0) + bias)[None, :]
+    if relu:
+        ref = po.relu(ref)
+    den = np.abs(x).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(bias)
+    err = h.normalised_error(got, ref, None, np.maximum(den, 1e-30), is_denominator=True)
+    assert err <= TOL_F32, err
+    for d in (dX, dW, dB, dY, dZ, ones):
+        d.release()

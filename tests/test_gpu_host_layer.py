@@ -125,6 +125,10 @@ def test_config4_mlp_forward(dev):
     assert err <= TOL_F32, err
     # also against the plain magnitude of the output
     assert np.max(np.abs(got - act)) <= 1e-4 * max(1.0, float(np.max(np.abs(act))))
+    # one launch per layer (bias row and ReLU applied where the product is stored): same bits
+    h.announce("config4 MLP forward through NN::LinearForwardFused")
+    fused = hl.mlp_forward(d["x"], d["W"], d["b"], fused=True)
+    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
 
 
 def test_transpose(dev):
