@@ -82,6 +82,17 @@ def timed_launches(capi, launch, steps, warmup):
     return event_ms, wall_ms
 
 
+def timed_maybe_graph(capi, launch, steps, warmup, graph):
+    """Event time per step of `launch`, issued call by call or recorded once and replayed."""
+    if not graph:
+        return timed_launches(capi, launch, steps, warmup)[0]
+    with capi.Graph() as recorded:
+        launch()
+    event_ms, _ = timed_launches(capi, recorded.launch, steps, warmup)
+    recorded.destroy()
+    return event_ms
+
+
 def bench_gemm_f16(capi, synth, steps, warmup, flags=0):
     n = 4096
     d = synth.config3(n)
@@ -131,7 +142,7 @@ def bench_f32(capi, A, B, C, M, N, K, batch, sb, steps, warmup):
     return event_ms
 
 
-def bench_mlp(capi, synth, steps, warmup, fused=False):
+def bench_mlp(capi, synth, steps, warmup, fused=False, graph=False):
     """Configuration 4 through the C ABI: per layer ones[batch,1] x bias (K = 1 GEMM), x x W,
     ReLU between layers -- the call sequence of Linear's forward pass; with `fused` one
     sph_linear_forward_f32 per layer instead (same result bits)."""
@@ -163,14 +174,14 @@ def bench_mlp(capi, synth, steps, warmup, fused=False):
                 capi.call("sph_relu_f32", act[l].ptr, y[l].ptr, batch * n_out)
                 cur = act[l]
 
-    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    event_ms = timed_maybe_graph(capi, launch, steps, warmup, graph)
     for buf in [x, ones] + W + b + y + act:
         buf.release()
     flops = 2.0 * batch * sum(sizes[l] * sizes[l + 1] for l in range(3))
     return event_ms, flops
 
 
-def bench_mlp_backward(capi, synth, steps, warmup, direct):
+def bench_mlp_backward(capi, synth, steps, warmup, direct, graph=False):
     """Backward pass + SGD update of configuration 4's three Linear layers through the C ABI
     (the call sequence of LinearBackProp::m_runBackProp per layer, ReLUBackward between
     layers).  direct=False materialises the transposes, zero-fills and uses Scale + Sub like
@@ -244,7 +255,7 @@ def bench_mlp_backward(capi, synth, steps, warmup, direct):
                           batch * sizes[l])
                 dy = dpre[l - 1]
 
-    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    event_ms = timed_maybe_graph(capi, launch, steps, warmup, graph)
     for buf in W + b + acts + pre + grads + dpre + [dy_top, wt, xt, dw, temp, ones, dB]:
         buf.release()
     flops = 2.0 * 2.0 * batch * sum(sizes[l] * sizes[l + 1] for l in range(3))
@@ -451,6 +462,12 @@ def main():
             "note": "reference sequence: Transpose + Gemm, Zeros, Scale + Sub; direct: "
                     "transposed-read / overwrite GEMM flags and the one-pass SGD step "
                     "(bit-identical results)"}
+        ms_f, _ = bench_mlp(capi, synth, 100, 10, fused=True, graph=True)
+        ms_b, _ = bench_mlp_backward(capi, synth, 100, 10, direct=True, graph=True)
+        others["config4_replayed_as_graphs"] = {
+            "forward_fused_ms": ms_f, "backward_sgd_direct_ms": ms_b,
+            "note": "the same call sequences recorded once with sph_graph_begin_capture / "
+                    "sph_graph_end_capture and replayed with sph_graph_launch"}
         ms, nbytes = bench_sgd_step(capi, 200, 20)
         others["sgd_step_64MiB"] = {"launch_ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9,
                                     "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS}

@@ -95,6 +95,25 @@ int sph_event_record(void* event);
 int sph_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for stop */
 int sph_event_destroy(void* event);
 
+/* ---- graphs -------------------------------------------------------------- */
+
+/* Launch-bound sequences (a layer's forward or backward pass is a handful of
+ * kernels of a few microseconds each) can be recorded once and replayed as one
+ * HIP graph.  Between begin and end the calling thread's entry points enqueue
+ * into the graph instead of running; entry points that wait for the device,
+ * allocate, free, read back or change the stream or device (copies to or from
+ * the host, sph_stream_sync, sph_malloc/sph_free, sph_event_elapsed_ms,
+ * sph_gemm_f32_grouped, sph_csr_row_offsets_f32 with a host count or more
+ * than 4095 rows) return SPH_ERR_UNSUPPORTED and leave the capture intact.
+ * sph_graph_launch enqueues one replay on the thread's stream.  The recorded
+ * pointers and sizes are fixed; change inputs by writing into the same
+ * buffers.  No counterpart in the reference (its cuBLAS calls are issued one
+ * by one). */
+int sph_graph_begin_capture(void);
+int sph_graph_end_capture(void** graph);
+int sph_graph_launch(void* graph);
+int sph_graph_destroy(void* graph);
+
 /* ---- fills and element-wise neighbours ----------------------------------- */
 
 /* dst[i] = value.  Replaces Dense::Cuda::Scalar

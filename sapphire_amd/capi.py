@@ -74,6 +74,10 @@ SIGNATURES = {
     "sph_event_record": [_vp],
     "sph_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(ctypes.c_float)],
     "sph_event_destroy": [_vp],
+    "sph_graph_begin_capture": [],
+    "sph_graph_end_capture": [ctypes.POINTER(_vp)],
+    "sph_graph_launch": [_vp],
+    "sph_graph_destroy": [_vp],
     "sph_fill_f32": [_vp, ctypes.c_float, _sz],
     "sph_relu_f32": [_vp, _vp, _sz],
     "sph_transpose_f32": [_vp, _vp, _u32, _u32, _u32, ctypes.c_int],
@@ -208,6 +212,33 @@ class Event:
         if self.ptr:
             call("sph_event_destroy", self.ptr)
             self.ptr = 0
+
+
+class Graph:
+    """Records the calls made inside the `with` block; launch() replays them."""
+
+    def __init__(self):
+        self.ptr = None
+
+    def __enter__(self):
+        call("sph_graph_begin_capture")
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        handle = _vp()
+        status = lib().sph_graph_end_capture(ctypes.byref(handle))
+        if exc_type is None:
+            check(status)
+            self.ptr = handle.value
+        return False
+
+    def launch(self):
+        call("sph_graph_launch", self.ptr)
+
+    def destroy(self):
+        if self.ptr:
+            call("sph_graph_destroy", self.ptr)
+            self.ptr = None
 
 
 def make_entries(triples):

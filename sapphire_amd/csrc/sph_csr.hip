@@ -328,6 +328,8 @@ int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint3
     SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
     SPH_REQUIRE(M < 0xffffffffu, "too many rows");
     SPH_REQUIRE(M == 0 || N == 0 || dense != nullptr, "dense is null");
+    if (nnzHost != nullptr || M + 1 > kScanPerBlock)
+        SPH_REFUSE_WHILE_CAPTURING();  // reads back, or takes a scratch allocation
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;

@@ -1219,6 +1219,7 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
                          const float* B, uint32_t M, uint32_t N, uint32_t K)
 {
     SPH_REQUIRE(M != 0 && N != 0, "M and N must be non-zero");
+    SPH_REFUSE_WHILE_CAPTURING();  // the offset table is uploaded from a shared staging buffer
     if (count == 0 || K == 0)
         return SPH_OK;
     SPH_REQUIRE(entries != nullptr && out != nullptr && A != nullptr && B != nullptr,

@@ -23,6 +23,10 @@ int CurrentDevice();
 
 // Number of compute units of the current device (cached).
 int ComputeUnits();
+
+// True between sph_graph_begin_capture and sph_graph_end_capture on this thread.  Entry
+// points that must wait for the device or allocate refuse to run while it is set.
+bool Capturing();
 }  // namespace sph
 
 #define SPH_HIP_TRY(expr)                                                      \
@@ -41,6 +45,16 @@ int ComputeUnits();
         if (!(cond))                                                           \
             return ::sph::Fail(SPH_ERR_INVALID, std::string(__func__) +        \
                                                     " - " + (what));           \
+    } while (0)
+
+// For entry points that synchronise, allocate or read back: not recordable into a graph.
+#define SPH_REFUSE_WHILE_CAPTURING()                                           \
+    do                                                                         \
+    {                                                                          \
+        if (::sph::Capturing())                                                \
+            return ::sph::Fail(SPH_ERR_UNSUPPORTED,                            \
+                               std::string(__func__) +                         \
+                                   " - not available while a graph is being captured"); \
     } while (0)
 
 // Checks the launch that was just issued.

@@ -27,6 +27,7 @@ struct ThreadSlots
     int device = 0;
     hipStream_t own[kMaxDevices] = {};
     hipStream_t borrowed[kMaxDevices] = {};
+    hipStream_t capturing = nullptr;  // stream under capture, if any
 
     ~ThreadSlots()
     {
@@ -86,6 +87,11 @@ hipStream_t CurrentStream()
     return tlsSlots.own[d];
 }
 
+bool Capturing()
+{
+    return tlsSlots.capturing != nullptr;
+}
+
 int ComputeUnits()
 {
     const int d = tlsSlots.device;
@@ -131,6 +137,7 @@ int sph_device_count(int* count)
 
 int sph_set_device(int deviceId)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     int n = 0;
     const int rc = sph_device_count(&n);
     if (rc != SPH_OK)
@@ -172,6 +179,7 @@ int sph_device_info(int deviceId, SphDeviceInfo* info)
 
 int sph_malloc(void** ptr, size_t bytes)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     SPH_REQUIRE(ptr != nullptr, "ptr is null");
     SPH_HIP_TRY(hipSetDevice(tlsSlots.device));
     SPH_HIP_TRY(hipMalloc(ptr, bytes));
@@ -180,12 +188,14 @@ int sph_malloc(void** ptr, size_t bytes)
 
 int sph_free(void* ptr)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     SPH_HIP_TRY(hipFree(ptr));
     return SPH_OK;
 }
 
 int sph_host_malloc(void** ptr, size_t bytes)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     SPH_REQUIRE(ptr != nullptr, "ptr is null");
     SPH_HIP_TRY(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
     return SPH_OK;
@@ -193,12 +203,14 @@ int sph_host_malloc(void** ptr, size_t bytes)
 
 int sph_host_free(void* ptr)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     SPH_HIP_TRY(hipHostFree(ptr));
     return SPH_OK;
 }
 
 int sph_memcpy_h2d(void* dev, const void* host, size_t bytes)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     if (bytes == 0)
         return SPH_OK;
     SPH_REQUIRE(dev != nullptr && host != nullptr, "null pointer");
@@ -210,6 +222,7 @@ int sph_memcpy_h2d(void* dev, const void* host, size_t bytes)
 
 int sph_memcpy_d2h(void* host, const void* dev, size_t bytes)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     if (bytes == 0)
         return SPH_OK;
     SPH_REQUIRE(dev != nullptr && host != nullptr, "null pointer");
@@ -221,6 +234,7 @@ int sph_memcpy_d2h(void* host, const void* dev, size_t bytes)
 
 int sph_memcpy_d2d(void* dst, const void* src, size_t bytes)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     if (bytes == 0)
         return SPH_OK;
     SPH_REQUIRE(dst != nullptr && src != nullptr, "null pointer");
@@ -242,6 +256,7 @@ int sph_memcpy_d2d_async(void* dst, const void* src, size_t bytes)
 
 int sph_stream_sync(void)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     SPH_STREAM_OR_FAIL(stream);
     SPH_HIP_TRY(hipStreamSynchronize(stream));
     return SPH_OK;
@@ -257,6 +272,7 @@ int sph_get_stream(void** hipStream)
 
 int sph_set_stream(void* hipStream)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     tlsSlots.borrowed[tlsSlots.device] = static_cast<hipStream_t>(hipStream);
     return SPH_OK;
 }
@@ -280,6 +296,7 @@ int sph_event_record(void* event)
 
 int sph_event_elapsed_ms(void* start, void* stop, float* ms)
 {
+    SPH_REFUSE_WHILE_CAPTURING();
     SPH_REQUIRE(start != nullptr && stop != nullptr && ms != nullptr, "null argument");
     SPH_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
     SPH_HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start),
@@ -291,6 +308,54 @@ int sph_event_destroy(void* event)
 {
     SPH_REQUIRE(event != nullptr, "event is null");
     SPH_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return SPH_OK;
+}
+
+int sph_graph_begin_capture(void)
+{
+    SPH_REQUIRE(!sph::Capturing(), "a capture is already in progress on this thread");
+    // resolve everything that queries the device before the stream goes into capture
+    (void)sph::ComputeUnits();
+    SPH_STREAM_OR_FAIL(stream);
+    SPH_HIP_TRY(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    tlsSlots.capturing = stream;
+    return SPH_OK;
+}
+
+int sph_graph_end_capture(void** graph)
+{
+    SPH_REQUIRE(graph != nullptr, "graph is null");
+    SPH_REQUIRE(sph::Capturing(), "no capture in progress on this thread");
+    hipStream_t stream = tlsSlots.capturing;
+    tlsSlots.capturing = nullptr;
+    *graph = nullptr;
+    hipGraph_t recorded = nullptr;
+    SPH_HIP_TRY(hipStreamEndCapture(stream, &recorded));
+    if (recorded == nullptr)
+        return sph::Fail(SPH_ERR_DEVICE, "sph_graph_end_capture - the capture was invalidated");
+    hipGraphExec_t exec = nullptr;
+    const hipError_t err = hipGraphInstantiate(&exec, recorded, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(recorded);
+    if (err != hipSuccess)
+        return sph::Fail(SPH_ERR_DEVICE, std::string("hipGraphInstantiate failed with ") +
+                                             hipGetErrorString(err));
+    *graph = exec;
+    return SPH_OK;
+}
+
+int sph_graph_launch(void* graph)
+{
+    SPH_REQUIRE(graph != nullptr, "graph is null");
+    SPH_REFUSE_WHILE_CAPTURING();
+    SPH_STREAM_OR_FAIL(stream);
+    SPH_HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), stream));
+    return SPH_OK;
+}
+
+int sph_graph_destroy(void* graph)
+{
+    SPH_REQUIRE(graph != nullptr, "graph is null");
+    SPH_HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
     return SPH_OK;
 }
 
