@@ -57,7 +57,8 @@ def parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     p.add_argument("--all", action="store_true",
                    help="also time configurations 1, 2 and 4 (reported under 'others')")
-    p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference"], default=None,
+    p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
+                                      "csr"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
     return p.parse_args()
 
@@ -412,6 +413,21 @@ def main():
                                     direct=args.only == "backward")
         result["backward"] = {"sequence": "direct" if args.only == "backward" else "reference",
                               "step_ms": ms, "tflops": fl / (ms * 1e-3) / 1e12}
+
+    if args.only == "gemm_f32":
+        c2 = synth.config2()
+        ms = bench_f32(capi, c2["A"], c2["B"], c2["C"], 512, 512, 512, 16, 0, args.steps,
+                       args.warmup)
+        tf = 16 * 2 * 512 ** 3 / (ms * 1e-3) / 1e12
+        result["gemm_f32"] = {"workload": "configuration 2: A[16,512,512] x B[1,512,512] fp32",
+                              "launch_ms": ms, "tflops": tf,
+                              "frac_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
+
+    if args.only == "csr":
+        ms_csr, ms_dense, dense_bytes, csr_bytes = bench_csr_conversion(capi, synth, args.steps,
+                                                                        args.warmup)
+        result["csr"] = {"dense_to_csr_ms": ms_csr, "csr_to_dense_ms": ms_dense,
+                         "dense_bytes": dense_bytes, "csr_bytes": csr_bytes}
 
     if args.only in (None, "spmm"):
         sp_steps = max(args.steps * 4, 100)

@@ -104,7 +104,7 @@ int sph_event_destroy(void* event);
  * allocate, free, read back or change the stream or device (copies to or from
  * the host, sph_stream_sync, sph_malloc/sph_free, sph_event_elapsed_ms,
  * sph_gemm_f32_grouped, sph_csr_row_offsets_f32 with a host count or more
- * than 4095 rows) return SPH_ERR_UNSUPPORTED and leave the capture intact.
+ * than 65535 rows) return SPH_ERR_UNSUPPORTED and leave the capture intact.
  * sph_graph_launch enqueues one replay on the thread's stream.  The recorded
  * pointers and sizes are fixed; change inputs by writing into the same
  * buffers.  No counterpart in the reference (its cuBLAS calls are issued one

@@ -85,6 +85,7 @@ __global__ __launch_bounds__(kThreads) void CsrCountKernel(uint32_t* __restrict_
 // ---- exclusive scan of n uint32 in place, 4096 per workgroup -----------------------------
 constexpr int kScanThreads = 1024;
 constexpr int kScanPerBlock = kScanThreads * 4;
+constexpr uint32_t kScanSingleLimit = 16 * kScanPerBlock;  // scanned by one workgroup
 
 // exclusive scan of one value per thread across the workgroup; returns the prefix and leaves
 // the workgroup total in `total`
@@ -155,6 +156,32 @@ __global__ __launch_bounds__(kScanThreads) void ScanSumsKernel(uint32_t* __restr
         const uint32_t prefix = BlockExclusiveScan(v, total, waveSums);
         if (i < count)
             sums[i] = carry + prefix;
+        carry += total;
+    }
+}
+
+// one workgroup: exclusive scan of n values in place, 4096 per round with a running carry
+__global__ __launch_bounds__(kScanThreads) void ScanSingleKernel(uint32_t* __restrict__ data,
+                                                                 uint32_t n)
+{
+    __shared__ uint32_t waveSums[kScanThreads / 64];
+    uint32_t carry = 0;
+    for (size_t start = 0; start < n; start += kScanPerBlock)
+    {
+        const size_t base = start + threadIdx.x * 4;
+        uint32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            v[e] = base + e < n ? data[base + e] : 0u;
+        uint32_t total;
+        uint32_t run = carry + BlockExclusiveScan(v[0] + v[1] + v[2] + v[3], total, waveSums);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            if (base + e < n)
+                data[base + e] = run;
+            run += v[e];
+        }
         carry += total;
     }
 }
@@ -328,7 +355,7 @@ int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint3
     SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
     SPH_REQUIRE(M < 0xffffffffu, "too many rows");
     SPH_REQUIRE(M == 0 || N == 0 || dense != nullptr, "dense is null");
-    if (nnzHost != nullptr || M + 1 > kScanPerBlock)
+    if (nnzHost != nullptr || M + 1 > kScanSingleLimit)
         SPH_REFUSE_WHILE_CAPTURING();  // reads back, or takes a scratch allocation
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
@@ -341,10 +368,10 @@ int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint3
 
     const uint32_t n = M + 1;
     const uint32_t blocks = (n + kScanPerBlock - 1) / kScanPerBlock;
-    if (blocks == 1)
+    if (n <= kScanSingleLimit)
     {
-        hipLaunchKernelGGL(ScanBlocksKernel, dim3(1), dim3(kScanThreads), 0, stream, ROW,
-                           static_cast<uint32_t*>(nullptr), n);
+        // up to 16 rounds of one workgroup cost less than three launches
+        hipLaunchKernelGGL(ScanSingleKernel, dim3(1), dim3(kScanThreads), 0, stream, ROW, n);
         SPH_CHECK_LAUNCH();
     }
     else

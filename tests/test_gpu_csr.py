@@ -60,7 +60,7 @@ def gpu_csr_to_dense(V, COL, ROW, M, N, ld, fill):
 # 16-byte and the scalar load path, empty and full rows, more rows than one scan block
 CASES = [(1, 1, 1, 1.0), (3, 2, 2, 0.5), (7, 13, 13, 0.3), (33, 16, 16, 0.2), (50, 31, 32, 0.5),
          (64, 64, 64, 0.05), (100, 100, 104, 0.1), (9, 257, 260, 0.4), (40, 1000, 1000, 0.01),
-         (5000, 24, 24, 0.1), (9000, 8, 8, 0.0), (300, 300, 300, 1.0), (2, 5000, 5000, 0.02)]
+         (5000, 24, 24, 0.1), (9000, 8, 8, 0.0), (70000, 6, 8, 0.3), (300, 300, 300, 1.0), (2, 5000, 5000, 0.02)]
 
 
 @pytest.mark.parametrize("case", CASES)
