@@ -305,6 +305,34 @@ def bench_csr_conversion(capi, synth, steps, warmup):
     return ms_csr, ms_dense, dense_bytes, csr_bytes
 
 
+def bench_spgemm(capi, synth, steps, warmup, n=8192, per_row=8.0):
+    """CSR x CSR -> CSR of two n x n matrices with `per_row` entries per row on average: the
+    counting pass (row offsets, no host read-back inside the timed region) and the fill pass."""
+    a = synth.csr_matrix(7001, n, n, per_row)
+    b = synth.csr_matrix(7002, n, n, per_row)
+    bufs = [capi.DeviceBuffer.from_array(x) for x in a + b]
+    row = capi.DeviceBuffer(4 * (n + 1))
+    import ctypes
+    nnz = ctypes.c_uint32(0)
+    ptrs = [x.ptr for x in bufs]
+    capi.call("sph_spgemm_row_offsets_f32", row.ptr, *ptrs, n, n, n, ctypes.byref(nnz))
+    val = capi.DeviceBuffer(4 * max(nnz.value, 1))
+    col = capi.DeviceBuffer(4 * max(nnz.value, 1))
+
+    def launch():
+        capi.call("sph_spgemm_row_offsets_f32", row.ptr, *ptrs, n, n, n, None)
+        capi.call("sph_spgemm_fill_f32", val.ptr, col.ptr, row.ptr, *ptrs, n, n, n)
+
+    event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    for x in bufs + [row, val, col]:
+        x.release()
+    # products: for every entry of A, the length of the matching row of B
+    lengths = np.diff(b[2].astype(np.int64))
+    products = int(lengths[a[1]].sum())
+    nbytes = 8 * (a[0].size + b[0].size + nnz.value) + 3 * 4 * (n + 1)
+    return event_ms, products, nnz.value, nbytes, a[0].size, b[0].size
+
+
 def bench_copy(capi, steps, warmup, mib=64):
     """A plain one-pass kernel of known size (ReLU over `mib` MiB: reads it once, writes it
     once), used to calibrate the profiler's FETCH_SIZE / WRITE_SIZE counters."""
@@ -495,6 +523,15 @@ def main():
                                  "read the dense matrix twice (count, then fill)",
             "csr_to_dense_ms": ms_dense,
             "csr_to_dense_gbs": (dense_bytes + csr_bytes) / (ms_dense * 1e-3) / 1e9}
+        ms, products, nnz_c, nbytes, nnz_a, nnz_b = bench_spgemm(capi, synth, 50, 5)
+        others["spgemm_8192_8_per_row"] = {
+            "workload": "CSR 8192x8192 (nnz %d) x CSR 8192x8192 (nnz %d) -> CSR (nnz %d)"
+                        % (nnz_a, nnz_b, nnz_c),
+            "count_plus_fill_ms": ms, "products": products,
+            "gproducts_per_s": 2 * products / (ms * 1e-3) / 1e9,
+            "algorithmic_gbs": nbytes / (ms * 1e-3) / 1e9,
+            "note": "both passes compute every product (the count pass must see which sums "
+                    "cancel); products counted once per pass in gproducts_per_s"}
         result["others"] = others
 
     if not args.no_cpu and args.only is None:

@@ -283,6 +283,34 @@ int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V,
                          const uint32_t* COL, const uint32_t* ROW, uint32_t M,
                          uint32_t N);
 
+/* ---- CSR x CSR ------------------------------------------------------------ */
+
+/* C = A * B with all three in CSR (A is M x K, B is K x N).  The reference
+ * declares this product (Sparse::Cuda::Gemm over arrays of SparseMatrix,
+ * Includes/Sapphire/compute/sparse/cuda/SparseGemm.cuh:16-42, with device
+ * helpers in Sources/Sapphire/compute/cudaUtil/SparseUtil.cu) and defines no
+ * host entry.  Element (i, j) is the sum over the entries of A's row i, in
+ * storage order, of a * B[k][j], product and sum rounded separately in fp32
+ * from +0 -- what the dense leaf gives on the densified operands; sums that
+ * are exactly 0 are not stored (SparseUtil.cu:55-60 deletes them too); a
+ * row's entries come out in ascending column order.  Column indices of B
+ * must be distinct within a row.
+ *
+ * Two steps, like the dense -> CSR conversion: sph_spgemm_row_offsets_f32
+ * computes ROWC (device, M + 1 entries; ROWC[M] = entries of C, copied to
+ * *nnzHost when that is not NULL, after which the stream has drained), the
+ * caller sizes VC / COLC, and sph_spgemm_fill_f32 writes them. */
+int sph_spgemm_row_offsets_f32(uint32_t* ROWC, const float* VA,
+                               const uint32_t* COLA, const uint32_t* ROWA,
+                               const float* VB, const uint32_t* COLB,
+                               const uint32_t* ROWB, uint32_t M, uint32_t K,
+                               uint32_t N, uint32_t* nnzHost);
+int sph_spgemm_fill_f32(float* VC, uint32_t* COLC, const uint32_t* ROWC,
+                        const float* VA, const uint32_t* COLA,
+                        const uint32_t* ROWA, const float* VB,
+                        const uint32_t* COLB, const uint32_t* ROWB, uint32_t M,
+                        uint32_t K, uint32_t N);
+
 #ifdef __cplusplus
 }
 #endif

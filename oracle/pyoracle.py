@@ -98,6 +98,9 @@ def oracle():
         o.orc_csr_to_dense.argtypes = [_fp, ctypes.c_uint32, _fp, _up, _up, ctypes.c_uint32,
                                        ctypes.c_uint32]
         o.orc_csr_to_dense.restype = None
+        o.orc_spgemm_csr.argtypes = [_fp, _up, _up, _fp, _up, _up, _fp, _up, _up,
+                                     ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
+        o.orc_spgemm_csr.restype = ctypes.c_uint32
         for name in ("orc_shape_expand", "orc_shape_shrink"):
             getattr(o, name).argtypes = [ctypes.POINTER(OrcShape), ctypes.c_int]
             getattr(o, name).restype = ctypes.c_int
@@ -321,3 +324,25 @@ def csr_to_dense(V, COL, ROW, M, N, ld=None, fill=0.0):
     oracle().orc_csr_to_dense(_f(out), ld, _f(Vp), Cp.ctypes.data_as(_up),
                               ROW.ctypes.data_as(_up), M, N)
     return out
+
+
+def _u32p(a):
+    a = a if a.size else np.zeros(1, np.uint32)
+    assert a.dtype == np.uint32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_up)
+
+
+def spgemm_csr(A, B, M, K, N):
+    """(V, COL, ROW) of A * B for CSR triples A = (V, COL, ROW), B likewise."""
+    VA, CA, RA = A
+    VB, CB, RB = B
+    fa = VA if VA.size else np.zeros(1, np.float32)
+    fb = VB if VB.size else np.zeros(1, np.float32)
+    ROW = np.zeros(M + 1, np.uint32)
+    nnz = oracle().orc_spgemm_csr(None, None, _u32p(ROW), _f(fa), _u32p(CA), _u32p(RA), _f(fb),
+                                  _u32p(CB), _u32p(RB), M, K, N)
+    V = np.zeros(max(nnz, 1), np.float32)
+    COL = np.zeros(max(nnz, 1), np.uint32)
+    oracle().orc_spgemm_csr(_f(V), _u32p(COL), _u32p(ROW), _f(fa), _u32p(CA), _u32p(RA), _f(fb),
+                            _u32p(CB), _u32p(RB), M, K, N)
+    return V[:nnz], COL[:nnz], ROW

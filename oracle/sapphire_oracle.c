@@ -674,3 +674,45 @@ void orc_csr_to_dense(float* dense, uint32_t ld, const float* V,
                 row[COL[p]] = V[p];
     }
 }
+
+/* ------------------------------------------------------------------ CSR x CSR */
+
+uint32_t orc_spgemm_csr(float* VC, uint32_t* COLC, uint32_t* ROWC, const float* VA,
+                        const uint32_t* COLA, const uint32_t* ROWA,
+                        const float* VB, const uint32_t* COLB,
+                        const uint32_t* ROWB, uint32_t M, uint32_t K,
+                        uint32_t N)
+{
+    float* acc = (float*)malloc(((size_t)N + 1) * sizeof(float));
+    uint32_t nnz = 0;
+    for (uint32_t i = 0; i < M; ++i)
+    {
+        ROWC[i] = nnz;
+        for (uint32_t j = 0; j < N; ++j)
+            acc[j] = 0.0f;
+        for (uint32_t pa = ROWA[i]; pa < ROWA[i + 1]; ++pa)
+        {
+            const uint32_t k = COLA[pa];
+            const float a = VA[pa];
+            if (k >= K)
+                continue;
+            for (uint32_t pb = ROWB[k]; pb < ROWB[k + 1]; ++pb)
+            {
+                const float prod = a * VB[pb];
+                acc[COLB[pb]] = acc[COLB[pb]] + prod;
+            }
+        }
+        for (uint32_t j = 0; j < N; ++j)
+            if (acc[j] != 0.0f)
+            {
+                if (VC)
+                    VC[nnz] = acc[j];
+                if (COLC)
+                    COLC[nnz] = j;
+                ++nnz;
+            }
+    }
+    ROWC[M] = nnz;
+    free(acc);
+    return nnz;
+}

@@ -228,6 +228,24 @@ void orc_csr_to_dense(float* dense, uint32_t ld, const float* V,
                       const uint32_t* COL, const uint32_t* ROW, uint32_t M,
                       uint32_t N);
 
+/* ---- CSR x CSR ----------------------------------------------------------- */
+
+/* The reference declares the product only
+ * (Includes/Sapphire/compute/sparse/cuda/SparseGemm.cuh:16-42; its device
+ * helper deletes sums that reach 0, Sources/Sapphire/compute/cudaUtil/SparseUtil.cu:55-60).
+ * Restated contract: for each row of A, a dense running row started at +0,
+ * A's entries in storage order, acc[col] = acc[col] + a*b for the entries of
+ * B's row k (unfused); then the non-zero elements in ascending column order.
+ * Returns nnz; VC / COLC may be NULL to count only.  ROWC has M + 1 entries.
+ * pinned: bit-exact against densify + orc_naive_gemm + orc_csr_from_dense;
+ * scipy.sparse product (values to rounding, structure where nothing
+ * cancels); hand example with a cancelling pair. */
+uint32_t orc_spgemm_csr(float* VC, uint32_t* COLC, uint32_t* ROWC, const float* VA,
+                        const uint32_t* COLA, const uint32_t* ROWA,
+                        const float* VB, const uint32_t* COLB,
+                        const uint32_t* ROWB, uint32_t M, uint32_t K,
+                        uint32_t N);
+
 #ifdef __cplusplus
 }
 #endif

@@ -346,6 +346,46 @@ struct FillLauncher
 };
 }  // namespace
 
+namespace sph
+{
+int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStream_t stream)
+{
+    if (lastHost != nullptr || n > kScanSingleLimit)
+        SPH_REFUSE_WHILE_CAPTURING();  // reads back, or takes a scratch allocation
+    const uint32_t blocks = (n + kScanPerBlock - 1) / kScanPerBlock;
+    if (n <= kScanSingleLimit)
+    {
+        // up to 16 rounds of one workgroup cost less than three launches
+        hipLaunchKernelGGL(ScanSingleKernel, dim3(1), dim3(kScanThreads), 0, stream, data, n);
+        SPH_CHECK_LAUNCH();
+    }
+    else
+    {
+        // per-block totals live in a stream-ordered scratch allocation
+        uint32_t* sums = nullptr;
+        SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&sums), blocks * sizeof(uint32_t),
+                                   stream));
+        hipLaunchKernelGGL(ScanBlocksKernel, dim3(blocks), dim3(kScanThreads), 0, stream, data,
+                           sums, n);
+        hipLaunchKernelGGL(ScanSumsKernel, dim3(1), dim3(kScanThreads), 0, stream, sums, blocks);
+        hipLaunchKernelGGL(AddBlockOffsetsKernel, dim3(blocks - 1), dim3(kScanThreads), 0, stream,
+                           data, sums, n);
+        const hipError_t launched = hipGetLastError();
+        SPH_HIP_TRY(hipFreeAsync(sums, stream));
+        if (launched != hipSuccess)
+            return sph::Fail(SPH_ERR_DEVICE, std::string("exclusive scan launch failed with ") +
+                                                 hipGetErrorString(launched));
+    }
+    if (lastHost != nullptr && n != 0)
+    {
+        SPH_HIP_TRY(hipMemcpyAsync(lastHost, data + (n - 1), sizeof(uint32_t),
+                                   hipMemcpyDeviceToHost, stream));
+        SPH_HIP_TRY(hipStreamSynchronize(stream));
+    }
+    return SPH_OK;
+}
+}  // namespace sph
+
 extern "C" {
 
 int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint32_t N,
@@ -355,8 +395,6 @@ int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint3
     SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
     SPH_REQUIRE(M < 0xffffffffu, "too many rows");
     SPH_REQUIRE(M == 0 || N == 0 || dense != nullptr, "dense is null");
-    if (nnzHost != nullptr || M + 1 > kScanSingleLimit)
-        SPH_REFUSE_WHILE_CAPTURING();  // reads back, or takes a scratch allocation
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
@@ -366,38 +404,7 @@ int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint3
     DispatchLanes<CountLauncher>(lanes, RowGrid(M, lanes), stream, ROW, d);
     SPH_CHECK_LAUNCH();
 
-    const uint32_t n = M + 1;
-    const uint32_t blocks = (n + kScanPerBlock - 1) / kScanPerBlock;
-    if (n <= kScanSingleLimit)
-    {
-        // up to 16 rounds of one workgroup cost less than three launches
-        hipLaunchKernelGGL(ScanSingleKernel, dim3(1), dim3(kScanThreads), 0, stream, ROW, n);
-        SPH_CHECK_LAUNCH();
-    }
-    else
-    {
-        // per-block totals live in a stream-ordered scratch allocation
-        uint32_t* sums = nullptr;
-        SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&sums), blocks * sizeof(uint32_t),
-                                   stream));
-        hipLaunchKernelGGL(ScanBlocksKernel, dim3(blocks), dim3(kScanThreads), 0, stream, ROW,
-                           sums, n);
-        hipLaunchKernelGGL(ScanSumsKernel, dim3(1), dim3(kScanThreads), 0, stream, sums, blocks);
-        hipLaunchKernelGGL(AddBlockOffsetsKernel, dim3(blocks - 1), dim3(kScanThreads), 0, stream,
-                           ROW, sums, n);
-        const hipError_t launched = hipGetLastError();
-        SPH_HIP_TRY(hipFreeAsync(sums, stream));
-        if (launched != hipSuccess)
-            return sph::Fail(SPH_ERR_DEVICE, std::string("sph_csr_row_offsets_f32 launch failed with ") +
-                                                 hipGetErrorString(launched));
-    }
-    if (nnzHost != nullptr)
-    {
-        SPH_HIP_TRY(hipMemcpyAsync(nnzHost, ROW + M, sizeof(uint32_t), hipMemcpyDeviceToHost,
-                                   stream));
-        SPH_HIP_TRY(hipStreamSynchronize(stream));
-    }
-    return SPH_OK;
+    return sph::ExclusiveScanInPlace(ROW, M + 1, nnzHost, stream);
 }
 
 int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW, const float* dense, uint32_t M,

@@ -24,6 +24,11 @@ int CurrentDevice();
 // Number of compute units of the current device (cached).
 int ComputeUnits();
 
+// Exclusive prefix sum of n 32-bit counts in place on `stream` (data[i] = sum of data[0..i)).
+// With lastHost the last element (the total, when the last count is 0) is copied to the host
+// and the stream is drained.
+int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStream_t stream);
+
 // True between sph_graph_begin_capture and sph_graph_end_capture on this thread.  Entry
 // points that must wait for the device or allocate refuse to run while it is set.
 bool Capturing();

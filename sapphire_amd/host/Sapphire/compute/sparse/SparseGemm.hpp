@@ -12,6 +12,7 @@
 #include <Sapphire/compute/sparse/SparseMatrix.hpp>
 #include <Sapphire/tensor/TensorData.hpp>
 
+#include <cstddef>
 #include <vector>
 
 namespace Sapphire::Compute::Sparse::Cuda
@@ -30,6 +31,16 @@ SparseMatrix CreateSparseMatrix(const std::vector<float>& values,
                                 const std::vector<uint32_t>& rowOffsets, uint32_t rows,
                                 uint32_t cols, int deviceId);
 void FreeSparseMatrix(SparseMatrix& matrix);
+
+//! Sparse x sparse: output i = cudaA[i] * cudaB[i] for numMatrices device records of shapes
+//! m x k and k x n, with the signature the reference declares
+//! (Includes/Sapphire/compute/sparse/cuda/SparseGemm.cuh:38-42).  *cudaOutput receives a new
+//! array of device records (release with Compute::DeepFreeSparseCuda); with copyResultToHost
+//! *hostOutput receives host copies (release with Compute::DeepFreeSparseHost), otherwise
+//! nullptr.  Sums that are exactly zero are not stored; columns ascend within a row.
+void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cudaA,
+          SparseMatrix* cudaB, uint32_t m, uint32_t n, std::size_t numMatrices, int deviceId,
+          bool copyResultToHost);
 }  // namespace Sapphire::Compute::Sparse::Cuda
 
 namespace Sapphire::Compute

@@ -1,12 +1,15 @@
 #include <Sapphire/compute/sparse/SparseGemm.hpp>
 
 #include <Sapphire/compute/cudaUtil/Memory.hpp>
+#include <Sapphire/compute/sparse/Sparse.hpp>
 #include <Sapphire/util/ResourceManager.hpp>
 
 #include <sapphire_hip.h>
 
+#include <algorithm>
 #include <stdexcept>
 #include <string>
+#include <vector>
 
 namespace Sapphire::Compute::Sparse::Cuda
 {
@@ -57,6 +60,62 @@ void FreeSparseMatrix(SparseMatrix& matrix)
     if (matrix.ROW != nullptr)
         Util::ResourceManager::FreePreservedCuda(matrix.ROW);
     matrix = SparseMatrix{};
+}
+
+void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cudaA,
+          SparseMatrix* cudaB, uint32_t m, uint32_t n, std::size_t numMatrices, int deviceId,
+          bool copyResultToHost)
+{
+    if (cudaOutput == nullptr || (copyResultToHost && hostOutput == nullptr))
+        throw std::invalid_argument("Sparse::Cuda::Gemm - output pointer is null");
+    Compute::Cuda::CudaSetDevice(deviceId);
+    const auto count = static_cast<uint32_t>(numMatrices);
+    auto* result = new SparseMatrix[count]();
+    auto check = [&](int status) {
+        if (status != SPH_OK)
+            throw std::runtime_error(std::string("Sparse::Cuda::Gemm failed with ") +
+                                     sph_last_error());
+    };
+    try
+    {
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            const SparseMatrix& a = cudaA[i];
+            const SparseMatrix& b = cudaB[i];
+            if (a.M != m || b.N != n || a.N != b.M)
+                throw std::invalid_argument("Sparse::Cuda::Gemm - shape mismatch");
+            SparseMatrix& c = result[i];
+            c.M = m;
+            c.N = n;
+            c.ROW = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(
+                (static_cast<std::size_t>(m) + 1) * 4, true));
+            uint32_t nnz = 0;
+            check(sph_spgemm_row_offsets_f32(c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m, a.N,
+                                             n, &nnz));
+            c.NNZ = nnz;
+            const std::size_t bytes = std::max<std::size_t>(nnz, 1) * 4;
+            c.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
+            c.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
+            check(sph_spgemm_fill_f32(c.V, c.COL, c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m,
+                                      a.N, n));
+        }
+        if (copyResultToHost)
+        {
+            std::vector<uint32_t> counts(count);
+            for (uint32_t i = 0; i < count; ++i)
+                counts[i] = result[i].NNZ;
+            DeepAllocateSparseHost(hostOutput, m, n, counts.data(), count);
+            DeepCopyDeviceToHost(*hostOutput, result, count, deviceId);
+        }
+        else if (hostOutput != nullptr)
+            *hostOutput = nullptr;
+    }
+    catch (...)
+    {
+        DeepFreeSparseCuda(result, count, deviceId);
+        throw;
+    }
+    *cudaOutput = result;
 }
 }  // namespace Sapphire::Compute::Sparse::Cuda
 

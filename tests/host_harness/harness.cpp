@@ -413,6 +413,49 @@ int sphh_sparse_linear_forward(const float* x, int batch, int inputs, int output
     });
 }
 
+// Sparse::Cuda::Gemm on one pair of matrices given dense on the host: both are sent to the
+// device and converted to CSR there; the product comes back as host CSR arrays (nnz, ROW with
+// m + 1 entries, V / COL up to `capacity`).
+int sphh_sparse_sparse_gemm(const float* denseA, const float* denseB, unsigned m, unsigned k,
+                            unsigned n, unsigned* nnz, unsigned* ROW, float* V, unsigned* COL,
+                            unsigned long capacity)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData A = Upload(Shape({ static_cast<int>(m), static_cast<int>(k) }), denseA, cuda);
+        TensorData B = Upload(Shape({ static_cast<int>(k), static_cast<int>(n) }), denseB, cuda);
+        SparseMatrix* a = nullptr;
+        SparseMatrix* b = nullptr;
+        SparseMatrix* cDevice = nullptr;
+        SparseMatrix* cHost = nullptr;
+        try
+        {
+            Compute::CreateSparseMatrixWithDenseMatrix(&a, A.CudaRawPtr(), m, k, k, 1, 0);
+            Compute::CreateSparseMatrixWithDenseMatrix(&b, B.CudaRawPtr(), k, n, n, 1, 0);
+            Compute::Sparse::Cuda::Gemm(&cHost, &cDevice, a, b, m, n, 1, 0, true);
+            *nnz = cHost[0].NNZ;
+            if (cHost[0].NNZ > capacity)
+                throw std::runtime_error("sphh_sparse_sparse_gemm - capacity too small");
+            std::memcpy(ROW, cHost[0].ROW, (static_cast<std::size_t>(m) + 1) * sizeof(unsigned));
+            std::memcpy(V, cHost[0].V, cHost[0].NNZ * sizeof(float));
+            std::memcpy(COL, cHost[0].COL, cHost[0].NNZ * sizeof(unsigned));
+        }
+        catch (...)
+        {
+            Compute::DeepFreeSparseHost(cHost, 1);
+            Compute::DeepFreeSparseCuda(cDevice, 1, 0);
+            Compute::DeepFreeSparseCuda(b, 1, 0);
+            Compute::DeepFreeSparseCuda(a, 1, 0);
+            throw;
+        }
+        Compute::DeepFreeSparseHost(cHost, 1);
+        Compute::DeepFreeSparseCuda(cDevice, 1, 0);
+        Compute::DeepFreeSparseCuda(b, 1, 0);
+        Compute::DeepFreeSparseCuda(a, 1, 0);
+        Util::ResourceManager::Clean();
+    });
+}
+
 int sphh_sparse_gemm(float* yData, int M, int K, int N, const float* V, const unsigned* COL,
                      const unsigned* ROW, const float* bData, int accumulate)
 {

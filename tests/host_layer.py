@@ -43,6 +43,8 @@ def lib():
         h.sphh_csr_round_trip.argtypes = [_fp, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint,
                                           ctypes.c_uint, up, _fp, up, up, ctypes.c_ulong, _fp,
                                           ctypes.c_float]
+        h.sphh_sparse_sparse_gemm.argtypes = [_fp, _fp, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint,
+                                              up, up, _fp, up, ctypes.c_ulong]
         h.sphh_sparse_linear_forward.argtypes = [_fp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                  _fp, _fp, _fp]
         h.sphh_shape_op.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip]
@@ -190,3 +192,18 @@ def sparse_linear_forward(x, W, bias):
     _ok(lib().sphh_sparse_linear_forward(_f(x), batch, inputs, W.shape[1],
                                          _f(np.ascontiguousarray(W)), _f(bias), _f(out)))
     return out
+
+
+def sparse_sparse_gemm(dA, dB, capacity):
+    """(V, COL, ROW) of the CSR x CSR product of two dense-given matrices."""
+    m, k = dA.shape
+    n = dB.shape[1]
+    up = ctypes.POINTER(ctypes.c_uint)
+    nnz = ctypes.c_uint(0)
+    ROW = np.zeros(m + 1, np.uint32)
+    V = np.zeros(max(capacity, 1), np.float32)
+    COL = np.zeros(max(capacity, 1), np.uint32)
+    _ok(lib().sphh_sparse_sparse_gemm(_f(np.ascontiguousarray(dA)), _f(np.ascontiguousarray(dB)),
+                                      m, k, n, ctypes.byref(nnz), ROW.ctypes.data_as(up), _f(V),
+                                      COL.ctypes.data_as(up), capacity))
+    return V[:nnz.value], COL[:nnz.value], ROW

@@ -1,0 +1,104 @@
+"""CSR x CSR -> CSR on the device (C ABI and the C++ layer), bit-exact against the CPU checker."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import pyoracle as po
+from sapphire_amd import capi, synth
+from tests import helpers as h
+from tests import host_layer as hl
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(x):
+    return np.ascontiguousarray(x).view(np.uint32)
+
+
+def sparse_dense(seed, shape, density):
+    vals = synth.uniform(seed, shape)
+    keep = synth.uniform(seed + 1, shape, 0.0, 1.0) < density
+    return np.where(keep, vals, np.float32(0)).astype(np.float32)
+
+
+def _dev(a, dtype):
+    return capi.DeviceBuffer.from_array(a if a.size else np.zeros(1, dtype))
+
+
+def gpu_spgemm(A, B, M, K, N):
+    VA, CA, RA = A
+    VB, CB, RB = B
+    bufs = [_dev(VA, np.float32), _dev(CA, np.uint32), _dev(RA, np.uint32),
+            _dev(VB, np.float32), _dev(CB, np.uint32), _dev(RB, np.uint32)]
+    dRow = capi.DeviceBuffer(4 * (M + 1))
+    nnz = ctypes.c_uint32(0xDEADBEEF)
+    capi.call("sph_spgemm_row_offsets_f32", dRow.ptr, *[b.ptr for b in bufs], M, K, N,
+              ctypes.byref(nnz))
+    ROW = dRow.download(np.uint32, (M + 1,))
+    assert ROW[M] == nnz.value
+    guard = 4
+    dV = capi.DeviceBuffer.from_array(np.full(nnz.value + guard, -77.0, np.float32))
+    dCol = capi.DeviceBuffer.from_array(np.full(nnz.value + guard, 0xABCDEF, np.uint32))
+    capi.call("sph_spgemm_fill_f32", dV.ptr, dCol.ptr, dRow.ptr, *[b.ptr for b in bufs], M, K, N)
+    V = dV.download(np.float32, (nnz.value + guard,))
+    COL = dCol.download(np.uint32, (nnz.value + guard,))
+    assert np.all(V[nnz.value:] == -77.0) and np.all(COL[nnz.value:] == 0xABCDEF)
+    for d in bufs + [dRow, dV, dCol]:
+        d.release()
+    return V[:nnz.value], COL[:nnz.value], ROW
+
+
+# M, K, N, density of A, density of B: single entries, rows of A and of B longer than 64
+# entries, empty operands, a width that needs two strips, widths that are not multiples of 64
+CASES = [(1, 1, 1, 1.0, 1.0), (5, 7, 3, 0.5, 0.5), (40, 60, 33, 0.1, 0.2), (64, 300, 200, 0.05, 0.05),
+         (30, 200, 70, 1.0, 0.3), (20, 50, 700, 0.3, 0.5), (25, 25, 25, 0.0, 0.5),
+         (25, 25, 25, 0.5, 0.0), (300, 400, 9000, 0.02, 0.01), (2000, 2000, 2000, 0.004, 0.004)]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_product_matches_checker(dev, case):
+    M, K, N, da, db = case
+    h.announce("sph_spgemm_* M K N dA dB =", case)
+    dA = sparse_dense(3000 + M, (M, K), da)
+    dB = sparse_dense(4000 + N, (K, N), db)
+    A, B = po.csr_from_dense(dA), po.csr_from_dense(dB)
+    wV, wC, wR = po.spgemm_csr(A, B, M, K, N)
+    V, COL, ROW = gpu_spgemm(A, B, M, K, N)
+    assert np.array_equal(ROW, wR)
+    assert np.array_equal(COL, wC)
+    assert np.array_equal(bits(V), bits(wV))
+
+
+def test_cancelling_sums_are_dropped_and_unsorted_b_rows_are_accepted(dev):
+    h.announce("sph_spgemm_* cancellation / unsorted rows of B")
+    A = (np.array([1, -1, 3], np.float32), np.array([0, 1, 2], np.uint32),
+         np.array([0, 2, 3], np.uint32))
+    B = (np.array([2, 5, 2, 7, 4], np.float32), np.array([1, 3, 1, 0, 2], np.uint32),
+         np.array([0, 2, 4, 5], np.uint32))
+    V, COL, ROW = gpu_spgemm(A, B, 2, 3, 4)
+    assert ROW.tolist() == [0, 2, 3] and COL.tolist() == [0, 3, 2]
+    assert V.tolist() == [-7.0, 5.0, 12.0]
+
+
+def test_equals_dense_product_of_the_densified_operands(dev):
+    """Against the dense path of this library's own checker: densify, dense leaf, back to CSR."""
+    M, K, N = 96, 128, 80
+    h.announce("sph_spgemm_* against densify + dense leaf", (M, K, N))
+    dA = sparse_dense(5000, (M, K), 0.08)
+    dB = sparse_dense(5002, (K, N), 0.08)
+    dense = po.naive_gemm(np.zeros((M, N), np.float32), dA, dB, M, N, K)
+    wV, wC, wR = po.csr_from_dense(dense)
+    V, COL, ROW = gpu_spgemm(po.csr_from_dense(dA), po.csr_from_dense(dB), M, K, N)
+    assert np.array_equal(ROW, wR) and np.array_equal(COL, wC) and np.array_equal(bits(V), bits(wV))
+
+
+@pytest.mark.parametrize("case", [(7, 9, 5, 0.5), (130, 90, 300, 0.05)])
+def test_host_layer_sparse_sparse_gemm(dev, case):
+    M, K, N, density = case
+    h.announce("Sparse::Cuda::Gemm (sparse x sparse)", case)
+    dA = sparse_dense(6000 + M, (M, K), density)
+    dB = sparse_dense(6100 + N, (K, N), density)
+    wV, wC, wR = po.spgemm_csr(po.csr_from_dense(dA), po.csr_from_dense(dB), M, K, N)
+    V, COL, ROW = hl.sparse_sparse_gemm(dA, dB, capacity=wV.size + 16)
+    assert np.array_equal(ROW, wR) and np.array_equal(COL, wC) and np.array_equal(bits(V), bits(wV))

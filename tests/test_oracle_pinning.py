@@ -421,3 +421,38 @@ def test_csr_conversion_pitch_and_special_values():
     assert np.all(back[:, 3:] == 7.0)                        # padding untouched
     assert back[0, :3].tolist() == [0.0, 0.0, 2.0] and not np.signbit(back[0, 1])
     assert np.isnan(back[1, 0]) and back[3, :3].tolist() == [1.0, -3.0, 4.0]
+
+
+# ---- CSR x CSR ------------------------------------------------------------------------------
+
+def test_spgemm_equals_dense_leaf_on_densified_operands():
+    for seed, (M, K, N, da, db) in enumerate([(1, 1, 1, 1.0, 1.0), (6, 7, 5, 0.5, 0.5),
+                                              (40, 60, 33, 0.1, 0.2), (64, 300, 200, 0.05, 0.05),
+                                              (30, 20, 70, 1.0, 0.3), (25, 25, 25, 0.0, 0.5)]):
+        dA = _sparse_dense(700 + 2 * seed, M, K, da)
+        dB = _sparse_dense(800 + 2 * seed, K, N, db)
+        A, B = po.csr_from_dense(dA), po.csr_from_dense(dB)
+        dense = po.naive_gemm(np.zeros((M, N), np.float32), dA, dB, M, N, K)
+        wV, wC, wR = po.csr_from_dense(dense)
+        V, COL, ROW = po.spgemm_csr(A, B, M, K, N)
+        assert ROW.tolist() == wR.tolist() and COL.tolist() == wC.tolist()
+        assert np.array_equal(bits(V), bits(wV))
+
+
+def test_spgemm_against_scipy_and_a_cancelling_pair():
+    import scipy.sparse as sp
+    dA = _sparse_dense(900, 50, 80, 0.1)
+    dB = _sparse_dense(902, 80, 40, 0.1)
+    V, COL, ROW = po.spgemm_csr(po.csr_from_dense(dA), po.csr_from_dense(dB), 50, 80, 40)
+    want = (sp.csr_matrix(dA.astype(np.float64)) @ sp.csr_matrix(dB.astype(np.float64))).toarray()
+    got = po.csr_to_dense(V, COL, ROW, 50, 40)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    assert np.array_equal(got != 0, want != 0)               # random values: nothing cancels
+    # (1*2) + (-1*2) = 0 is dropped; entries appear in ascending column order
+    A = (np.array([1, -1, 3], np.float32), np.array([0, 1, 2], np.uint32),
+         np.array([0, 2, 3], np.uint32))                     # [[1,-1,0],[0,0,3]]
+    B = (np.array([2, 5, 2, 7, 4], np.float32), np.array([1, 3, 1, 0, 2], np.uint32),
+         np.array([0, 2, 4, 5], np.uint32))                  # [[0,2,0,5],[7,2,0,0],[0,0,4,0]]
+    V, COL, ROW = po.spgemm_csr(A, B, 2, 3, 4)
+    assert ROW.tolist() == [0, 2, 3] and COL.tolist() == [0, 3, 2]
+    assert V.tolist() == [-7.0, 5.0, 12.0]
