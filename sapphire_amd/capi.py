@@ -233,6 +233,8 @@ class Graph:
         if exc_type is None:
             check(status)
             self.ptr = handle.value
+        elif status == 0 and handle.value:
+            lib().sph_graph_destroy(handle.value)   # the block failed: drop what was recorded
         return False
 
     def launch(self):

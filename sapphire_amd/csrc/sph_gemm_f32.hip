@@ -1190,6 +1190,7 @@ int sph_linear_forward_f32(float* y, const float* x, const float* W, const float
     SPH_REQUIRE((flags & ~SPH_LINEAR_RELU) == 0, "unknown flag");
     SPH_REQUIRE(y != nullptr && bias != nullptr, "null pointer");
     SPH_REQUIRE(inputs == 0 || (x != nullptr && W != nullptr), "null pointer");
+    SPH_REQUIRE(y != x && y != W, "y must not alias an input");
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
