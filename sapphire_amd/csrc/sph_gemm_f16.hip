@@ -495,6 +495,187 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
 }
 
 // ---------------------------------------------------------------------------
+// 128 x 128 x 32 kernel with straight-to-LDS copies, ragged M and N
+// ---------------------------------------------------------------------------
+// For shapes the 256-tile kernel does not take (M or N not a multiple of 256) as long as K is a
+// multiple of 32, N of 8 and everything is 16-byte aligned.  Four wavefronts (2 x 2), each
+// 64 x 64 = 2 x 2 MFMA blocks, four LDS stages of 16 KiB (two workgroups per compute unit),
+// copies issued two steps ahead, one barrier per step, fragments read half a step ahead.
+// A stage: 128 rows of 64 bytes, 16-byte chunk c of row x at position c ^ ((x >> 2) & 3).
+// B stage: 32 k-rows of 256 bytes, 32-byte chunks XOR-swizzled with 2*(k%4), read with the
+// transposing LDS load like the 256-tile kernel.  Rows past M and columns past N are clamped to
+// the last valid ones: they only feed outputs that are not stored.
+constexpr int kD = 128;
+constexpr int kDStages = 4;
+constexpr int kDStageBytes = 2 * kD * kTK * 2;  // A + B
+constexpr int kDCopies = 4;                     // per wavefront and step: 2 of A, 2 of B
+
+__global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
+{
+    __shared__ __attribute__((aligned(1024))) char lds[kDStages * kDStageBytes];
+    constexpr uint32_t kBytesA = kD * kTK * 2;  // 8 KiB
+
+    uint32_t unit, tm, tn;
+    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
+        return;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t waveM = wave >> 1;
+    const uint32_t waveN = wave & 1;
+    const uint32_t M = args.M, N = args.N, K = args.K;
+
+    const _Float16* A = args.A + args.strideA * static_cast<int64_t>(unit);
+    const _Float16* B = args.B + args.strideB * static_cast<int64_t>(unit);
+    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit);
+    const uint32_t rowBase = tm * kD;
+    const uint32_t colBase = tn * kD;
+
+    // ---- copy plan: copy j of an operand (j = wave, wave + 4) ---------------------------
+    uint32_t aLane[2], bLane[2], aDst[2], bDst[2];
+#pragma unroll
+    for (uint32_t i = 0; i < 2; ++i)
+    {
+        const uint32_t j = wave + 4 * i;
+        // A: 16 rows per copy; lane -> row j*16 + lane/4, physical chunk lane%4
+        const uint32_t x = j * 16 + (lane >> 2);
+        const uint32_t c = (lane & 3) ^ ((lane >> 4) & 3);  // (x >> 2) & 3 == (lane >> 4) & 3
+        const uint32_t gx = min(rowBase + x, M - 1);
+        aLane[i] = (gx * K + c * 8) * 2u;
+        aDst[i] = j * 1024;
+        // B: 4 k-rows per copy; lane -> k = j*4 + lane/16, physical 16-byte chunk lane%16
+        const uint32_t k = j * 4 + (lane >> 4);
+        const uint32_t phys16 = lane & 15;
+        const uint32_t logical16 = (((phys16 >> 1) ^ (2 * (k & 3))) << 1) | (phys16 & 1);
+        const uint32_t gc = min(colBase + logical16 * 8, N - 8);
+        bLane[i] = (k * N + gc) * 2u;
+        bDst[i] = kBytesA + j * 1024;
+    }
+    const size_t bStepBytes = static_cast<size_t>(kTK) * N * 2;
+    const uint32_t ldsBase = LdsAddress(lds);
+    const uint32_t steps = K / kTK;
+    auto issue = [&](uint32_t step) {
+        const uint32_t src = min(step, steps - 1);  // surplus steps re-fetch the last one
+        const uint32_t stage = ldsBase + (step % kDStages) * kDStageBytes;
+        const char* aBase = reinterpret_cast<const char*>(A) + static_cast<size_t>(src) * (kTK * 2);
+        const char* bBase = reinterpret_cast<const char*>(B) + static_cast<size_t>(src) * bStepBytes;
+        DmaToLds16<0>(aLane[0], aBase, stage + aDst[0]);
+        DmaToLds16<0>(aLane[1], aBase, stage + aDst[1]);
+        DmaToLds16<0>(bLane[0], bBase, stage + bDst[0]);
+        DmaToLds16<0>(bLane[1], bBase, stage + bDst[1]);
+    };
+
+    // ---- fragment plan ----------------------------------------------------------------
+    const uint32_t l32 = lane & 31;
+    const uint32_t khalf = lane >> 5;
+    const uint32_t g = lane >> 4;
+    const uint32_t s = lane & 15;
+    uint32_t aOff[2][2], bOff[2][2];  // [ks][block], bytes inside a stage
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+        {
+            const uint32_t x = waveM * 64 + b * 32 + l32;
+            aOff[ks][b] = x * 64 + (((ks * 2 + khalf) ^ ((x >> 2) & 3)) << 4);
+            const uint32_t k = ks * 16 + 8 * (g >> 1) + (s >> 2);  // + 4 for the second read
+            const uint32_t chunk32 = (waveN * 4 + b * 2 + (g & 1)) ^ (2 * ((s >> 2) & 3));
+            bOff[ks][b] = kBytesA + k * 256 + chunk32 * 32 + (s & 3) * 8;
+        }
+    auto loadFragments = [&](halfx8 (&af)[2], halfx8 (&bf)[2], const char* stage, int ks) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+        {
+            af[b] = *reinterpret_cast<const halfx8*>(stage + aOff[ks][b]);
+            const _Float16* p = reinterpret_cast<const _Float16*>(stage + bOff[ks][b]);
+            bf[b] = Join(LdsReadTr(p), LdsReadTr(p + 4 * 128));
+        }
+    };
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                acc[i][j][v] = 0.f;
+    auto multiply = [&](const halfx8 (&af)[2], const halfx8 (&bf)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[i][j] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+    };
+
+#pragma unroll
+    for (uint32_t p = 0; p < kDStages - 1; ++p)
+        issue(p);
+    halfx8 af[2][2], bf[2][2];
+    WaitVmem<(kDStages - 2) * kDCopies>();
+    __syncthreads();
+    loadFragments(af[0], bf[0], lds, 0);
+
+    for (uint32_t st = 0; st < steps; ++st)
+    {
+        // steps st and st+1 have landed once at most one later step is pending
+        WaitVmem<(kDStages - 3) * kDCopies>();
+        __syncthreads();
+        issue(st + kDStages - 1);
+        const char* cur = lds + (st % kDStages) * kDStageBytes;
+        const char* next = lds + ((st + 1) % kDStages) * kDStageBytes;
+        loadFragments(af[1], bf[1], cur, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(af[0], bf[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        loadFragments(af[0], bf[0], next, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(af[1], bf[1]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    WaitVmem<0>();  // the surplus copies of the last steps still target LDS
+
+    // ---- epilogue: lane holds row l%32 of a block, columns 8q + 4*(l/32) + 0..3 -----------
+    const bool accumulate = args.overwrite == 0;
+    float4 old[16];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const uint32_t r = rowBase + waveM * 64 + i * 32 + l32;
+                const uint32_t c = colBase + waveN * 64 + j * 32 + 8 * q + 4 * khalf;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (accumulate && r < M && c < N)  // N % 8 == 0: whole quads only
+                    v = *reinterpret_cast<const float4*>(out + static_cast<size_t>(r) * N + c);
+                old[(i * 2 + j) * 4 + q] = v;
+            }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const uint32_t r = rowBase + waveM * 64 + i * 32 + l32;
+                const uint32_t c = colBase + waveN * 64 + j * 32 + 8 * q + 4 * khalf;
+                if (r < M && c < N)
+                {
+                    float4 v = old[(i * 2 + j) * 4 + q];
+                    v.x += acc[i][j][4 * q + 0];
+                    v.y += acc[i][j][4 * q + 1];
+                    v.z += acc[i][j][4 * q + 2];
+                    v.w += acc[i][j][4 * q + 3];
+                    *reinterpret_cast<float4*>(out + static_cast<size_t>(r) * N + c) = v;
+                }
+            }
+}
+
+// ---------------------------------------------------------------------------
 // general kernel: 128 x 128 x 32, any shape
 // ---------------------------------------------------------------------------
 constexpr int kG = 128;
@@ -756,7 +937,11 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
           reinterpret_cast<uintptr_t>(out)) & 15u) == 0 &&
         (strideA % 8 == 0) && (strideB % 8 == 0) && (strideOut % 4 == 0);
 
-    const bool tile256 = aligned16 && (M % kT == 0) && (N % kT == 0) && (K % kTK == 0);
+    // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
+    // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
+    const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
+    const bool tile256 = aligned16 && (M % kT == 0) && (N % kT == 0) && (K % kTK == 0) &&
+                         static_cast<uint64_t>(M / kT) * (N / kT) * batch >= minTiles;
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -768,6 +953,13 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     if (tile256)
     {
         hipLaunchKernelGGL(GemmF16Tile256<8>, dim3(grid), dim3(512), 0, stream, args);
+    }
+    else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
+             static_cast<uint64_t>(M) * K < (1ull << 31) &&
+             static_cast<uint64_t>(kTK) * N < (1ull << 31))
+    {
+        // whole K steps and 16-byte chunks everywhere: straight-to-LDS 128-tile kernel
+        hipLaunchKernelGGL(GemmF16Dma128, dim3(grid), dim3(256), 0, stream, args);
     }
     else
     {

@@ -22,18 +22,20 @@ def _oracle(C, A16, B16, M, N, K, batch=1, sa=None, sb=None):
     return po.gemm_rows(C.copy(), A, B, M, N, K, batch=batch, stride_a=sa, stride_b=sb, threads=8)
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 64), (256, 512, 128), (512, 256, 192),
-                                   (768, 1024, 256)])
+# the 256-tile kernel is chosen from 192 tiles up (three quarters of the compute units): the
+# batch count brings these small shapes there
+@pytest.mark.parametrize("shape", [(256, 256, 64, 192), (256, 512, 128, 96), (512, 256, 192, 96),
+                                   (768, 1024, 256, 16), (4096, 3072, 32, 1)])
 def test_tile256_exact_on_integers(dev, shape):
-    M, N, K = shape
+    M, N, K, batch = shape
     h.announce("sph_gemm_f16f32 tile256 integer exactness", shape)
-    A = synth.small_integers(1, (M, K)).astype(np.float16)
-    B = synth.small_integers(2, (K, N)).astype(np.float16)
-    C = synth.small_integers(3, (M, N), span=100)
-    ref = _oracle(C, A, B, M, N, K)
-    got = h.gpu_gemm_f16(C, A, B, M, N, K)
+    A = synth.small_integers(1, (batch, M, K)).astype(np.float16)
+    B = synth.small_integers(2, (batch, K, N)).astype(np.float16)
+    C = synth.small_integers(3, (batch, M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K, batch=batch)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch)
     assert np.array_equal(got, ref)
-    got = h.gpu_gemm_f16(C, A, B, M, N, K, flags=capi.SPH_GEMM_OVERWRITE)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, flags=capi.SPH_GEMM_OVERWRITE)
     assert np.array_equal(got, ref - C)
 
 
@@ -50,9 +52,41 @@ def test_general_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref)
 
 
+# K % 32 == 0 and N % 8 == 0 without being whole 256-tiles: the straight-to-LDS 128-tile kernel,
+# with clamped rows (M ragged) and clamped column chunks (N ragged), one and many tiles
+@pytest.mark.parametrize("shape", [(1, 8, 32), (64, 64, 32), (100, 136, 64), (130, 72, 96),
+                                   (257, 264, 32), (128, 128, 512), (300, 520, 160),
+                                   (1000, 1000, 992), (512, 384, 2048)])
+def test_dma128_exact_on_integers(dev, shape):
+    M, N, K = shape
+    h.announce("sph_gemm_f16f32 128-tile integer exactness", shape)
+    A = synth.small_integers(14, (M, K), span=3).astype(np.float16)
+    B = synth.small_integers(15, (K, N), span=3).astype(np.float16)
+    C = synth.small_integers(16, (M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K)
+    assert np.array_equal(got, ref)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, flags=capi.SPH_GEMM_OVERWRITE)
+    assert np.array_equal(got, ref - C)
+
+
+def test_dma128_batched_with_shared_operand(dev):
+    h.announce("sph_gemm_f16f32 128-tile path, batch 3, strideA = 0")
+    M, N, K, batch = 200, 136, 96, 3
+    A = synth.normal(17, (1, M, K), 0.1).astype(np.float16)
+    B = synth.normal(18, (batch, K, N), 0.1).astype(np.float16)
+    C = synth.uniform(19, (batch, M, N))
+    ref = _oracle(C, A, B, M, N, K, batch=batch, sa=0)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, stride_a=0)
+    for b in range(batch):
+        err = h.normalised_error(got[b], ref[b], np.abs(A[0]).astype(np.float32),
+                                 np.abs(B[b]).astype(np.float32))
+        assert err <= TOL_F16
+
+
 def test_batched_and_broadcast(dev):
-    h.announce("sph_gemm_f16f32 batch 3, strideB = 0, tile256 path")
-    M, N, K, batch = 256, 256, 128, 3
+    h.announce("sph_gemm_f16f32 batch 192, strideB = 0, tile256 path")
+    M, N, K, batch = 256, 256, 128, 192
     A = synth.normal(7, (batch, M, K), 0.1).astype(np.float16)
     B = synth.normal(8, (1, K, N), 0.1).astype(np.float16)
     C = synth.uniform(9, (batch, M, N))
