@@ -11,6 +11,7 @@
 #include <Sapphire/compute/sparse/Sparse.hpp>
 #include <Sapphire/compute/sparse/SparseGemm.hpp>
 #include <Sapphire/operations/Backward/LinearBackward.hpp>
+#include <Sapphire/operations/Backward/MathBackward.hpp>
 #include <Sapphire/operations/Forward/LinearForward.hpp>
 #include <Sapphire/util/ResourceManager.hpp>
 
@@ -452,6 +453,27 @@ int sphh_sparse_sparse_gemm(const float* denseA, const float* denseB, unsigned m
         Compute::DeepFreeSparseCuda(cDevice, 1, 0);
         Compute::DeepFreeSparseCuda(b, 1, 0);
         Compute::DeepFreeSparseCuda(a, 1, 0);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// BackProp::MatMulBackward: da and db hold values on entry and are accumulated into.
+int sphh_matmul_backward(float* da, float* db, const float* dy, const float* a, const float* b,
+                         const int* aShape, int an, const int* bShape, int bn, const int* yShape,
+                         int yn, int sequence)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData A = Upload(MakeShape(aShape, an), a, cuda);
+        TensorData B = Upload(MakeShape(bShape, bn), b, cuda);
+        TensorData Dy = Upload(MakeShape(yShape, yn), dy, cuda);
+        TensorData Da = Upload(MakeShape(aShape, an), da, cuda);
+        TensorData Db = Upload(MakeShape(bShape, bn), db, cuda);
+        BackProp::MatMulBackward(Da, Db, Dy, A, B,
+                                 sequence == 0 ? BackProp::Sequence::Reference
+                                               : BackProp::Sequence::Direct);
+        Download(Da, da);
+        Download(Db, db);
         Util::ResourceManager::Clean();
     });
 }

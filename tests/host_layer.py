@@ -45,6 +45,8 @@ def lib():
                                           ctypes.c_float]
         h.sphh_sparse_sparse_gemm.argtypes = [_fp, _fp, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint,
                                               up, up, _fp, up, ctypes.c_ulong]
+        h.sphh_matmul_backward.argtypes = [_fp, _fp, _fp, _fp, _fp, _ip, ctypes.c_int, _ip,
+                                           ctypes.c_int, _ip, ctypes.c_int, ctypes.c_int]
         h.sphh_sparse_linear_forward.argtypes = [_fp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                  _fp, _fp, _fp]
         h.sphh_shape_op.argtypes = [_ip, ctypes.c_int, ctypes.c_int, ctypes.c_int, _ip]
@@ -207,3 +209,13 @@ def sparse_sparse_gemm(dA, dB, capacity):
                                       m, k, n, ctypes.byref(nnz), ROW.ctypes.data_as(up), _f(V),
                                       COL.ctypes.data_as(up), capacity))
     return V[:nnz.value], COL[:nnz.value], ROW
+
+
+def matmul_backward(da, db, dy, a, b, sequence):
+    """Returns the accumulated (da, db)."""
+    da, db = np.ascontiguousarray(da.copy()), np.ascontiguousarray(db.copy())
+    _ok(lib().sphh_matmul_backward(_f(da), _f(db), _f(np.ascontiguousarray(dy)),
+                                   _f(np.ascontiguousarray(a)), _f(np.ascontiguousarray(b)),
+                                   _ints(a.shape), a.ndim, _ints(b.shape), b.ndim,
+                                   _ints(dy.shape), dy.ndim, sequence))
+    return da, db

@@ -222,3 +222,38 @@ def test_linear_backward(dev, dims):
     slack = np.finfo(np.float32).eps * (np.abs(ref_b) + lr * den)
     assert np.all(np.abs(b2.astype(np.float64) - ref_b) <= lr * TOL_F32 * den + slack)
     assert np.any(W2 != W) and np.any(b2 != bias) and np.any(dx != dx0)
+
+
+@pytest.mark.parametrize("shapes", [((1, 3, 2), (1, 2, 4)), ((5, 33, 20), (5, 20, 17)),
+                                    ((64, 48), (48, 80)), ((2, 3, 40, 64), (2, 3, 64, 24)),
+                                    ((4, 9, 6), (6, 5))])
+def test_matmul_backward(dev, shapes):
+    """Sources/Sapphire/operations/Backward/MathBackward.cpp:35-51 (the reference's TestMatMul
+    uses {1,3,2} x {1,2,4}): da += dy b^T, db += a^T dy against the same operator calls on the
+    CPU; the last case has a 2-D b, which the direct sequence hands to the reference one."""
+    sa, sb = shapes
+    h.announce("BackProp::MatMulBackward", shapes)
+    a = synth.uniform(101, sa)
+    b = synth.uniform(102, sb)
+    sy = tuple(sa[:-1]) + (sb[-1],)
+    dy = synth.uniform(103, sy)
+    da0 = synth.uniform(104, sa)
+    db0 = synth.uniform(105, sb)
+    # CPU: Transpose + Compute::Gemm as written in the reference
+    rows_a, cols_a = sa[-2], sa[-1]
+    rows_b, cols_b = sb[-2], sb[-1]
+    nb_a = int(np.prod(sa[:-2])) if len(sa) > 2 else 1
+    nb_b = int(np.prod(sb[:-2])) if len(sb) > 2 else 1
+    ta = po.transpose(a, rows_a, cols_a, nb_a).reshape(tuple(sa[:-2]) + (cols_a, rows_a))
+    tb = po.transpose(b, rows_b, cols_b, nb_b).reshape(tuple(sb[:-2]) + (cols_b, rows_b))
+    ref_da = po.compute_gemm(da0.copy(), dy, tb)
+    ref_db = po.compute_gemm(db0.copy(), ta, dy)
+    seq_ref = hl.matmul_backward(da0, db0, dy, a, b, 0)
+    direct = hl.matmul_backward(da0, db0, dy, a, b, 1)
+    for got, want in zip(direct, seq_ref):
+        assert np.array_equal(_bits(got), _bits(want))
+    den_a = po.compute_gemm(np.zeros_like(da0), np.abs(dy), np.abs(tb))
+    den_b = po.compute_gemm(np.zeros_like(db0), np.abs(ta), np.abs(dy))
+    for got, ref, den in ((seq_ref[0], ref_da, den_a), (seq_ref[1], ref_db, den_b)):
+        err = float(np.max(np.abs(got.astype(np.float64) - ref) / np.maximum(den, 1e-30)))
+        assert err <= TOL_F32, err
