@@ -954,6 +954,70 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
     }
 }
 
+// ---------------------------------------------------------------------------
+// One output row (M = 1):  out[1 x N] (+)= a[1 x K] * B[K x N], e.g. the column sums
+// ones x dy of the bias gradient.  A matrix-core tile would use one of its 32 rows; this is a
+// plain reduction bound by reading B once.  A workgroup owns 64 consecutive columns (one per
+// lane, 256-byte row segments) and splits K over its 16 wavefronts; the 16 partial sums are
+// added in wavefront order through LDS, so the result does not depend on timing.
+// ---------------------------------------------------------------------------
+constexpr int kGemvWaves = 16;
+
+__global__ __launch_bounds__(kGemvWaves * 64) void GemvRowKernel(const GemmF32Args args)
+{
+    __shared__ float partial[kGemvWaves][64];
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t unit = blockIdx.y;
+    const float* __restrict__ a = args.A + args.strideA * static_cast<int64_t>(unit);
+    const float* __restrict__ B = args.B + args.strideB * static_cast<int64_t>(unit);
+    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit);
+    const uint32_t N = args.N, K = args.K;
+    const uint32_t col = blockIdx.x * 64 + lane;
+    const bool colOk = col < N;
+
+    const uint32_t perWave = (K + kGemvWaves - 1) / kGemvWaves;
+    const uint32_t kBegin = min(wave * perWave, K);
+    const uint32_t kEnd = min(kBegin + perWave, K);
+    // four independent chains keep loads in flight; they are combined in a fixed order
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (colOk)
+    {
+        const float* p = B + static_cast<size_t>(kBegin) * N + col;
+        uint32_t k = kBegin;
+        for (; k + 4 <= kEnd; k += 4)
+        {
+            s0 = fmaf(a[k + 0], p[0], s0);
+            s1 = fmaf(a[k + 1], p[static_cast<size_t>(N)], s1);
+            s2 = fmaf(a[k + 2], p[2 * static_cast<size_t>(N)], s2);
+            s3 = fmaf(a[k + 3], p[3 * static_cast<size_t>(N)], s3);
+            p += 4 * static_cast<size_t>(N);
+        }
+        for (; k < kEnd; ++k)
+        {
+            s0 = fmaf(a[k], p[0], s0);
+            p += N;
+        }
+    }
+    partial[wave][lane] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (wave != 0 || !colOk)
+        return;
+    float sum = partial[0][lane];
+#pragma unroll
+    for (int w = 1; w < kGemvWaves; ++w)
+        sum += partial[w][lane];
+    float old = 0.f;
+    if (args.bias != nullptr)
+        old = 0.f + args.bias[col];
+    else if (!args.overwrite)
+        old = out[col];
+    float v = old + sum;
+    if (args.relu)
+        v = v > 0 ? v : 0;
+    out[col] = v;
+}
+
 // Device table for grouped launches: one growing buffer per device with a
 // pinned staging copy.  The table is shared by every caller, so its use is
 // serialised by a mutex and, across streams, by waiting for the stream that
@@ -1048,6 +1112,15 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const uint32_t lda = transA ? args.M : args.K;
     const uint32_t ldb = transB ? args.K : args.N;
     const bool aligned = allowVector && basesAligned && (lda % 4 == 0) && (ldb % 4 == 0);
+
+    // a single output row is a reduction over the rows of B, not a matrix-core job
+    if (args.M == 1 && !transB && args.entries == nullptr && args.K >= 64 && units <= 65535)
+    {
+        hipLaunchKernelGGL(GemvRowKernel, dim3((args.N + 63) / 64, units), dim3(kGemvWaves * 64),
+                           0, stream, args);
+        SPH_CHECK_LAUNCH();
+        return SPH_OK;
+    }
 
     // few 64 x 64 tiles and a long K: split K inside the workgroup instead
     const uint64_t tiles64 =

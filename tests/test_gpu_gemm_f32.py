@@ -223,3 +223,26 @@ def test_linear_forward_one_launch(dev, dims, relu):
     assert err <= TOL_F32, err
     for d in (dX, dW, dB, dY, dZ, ones):
         d.release()
+
+
+@pytest.mark.parametrize("case", [(1024, 1024, 1), (70, 300, 1), (10, 64, 1), (1000, 4099, 1),
+                                  (96, 200, 5)])
+def test_single_output_row(dev, case):
+    """M = 1 with a long K (the ones x dy column sums of the bias gradient) runs on the row
+    reduction kernel; accumulate, overwrite, the stored-transposed A flag and a batch."""
+    N, K, batch = case
+    h.announce("sph_gemm_f32 M = 1", case)
+    A = synth.uniform(41, (batch, 1, K))
+    B = synth.uniform(42, (batch, K, N))
+    C = synth.uniform(43, (batch, 1, N))
+    ref = po.gemm_rows(C.copy(), A, B, 1, N, K, batch=batch)
+    got = h.gpu_gemm_f32(C, A, B, 1, N, K, batch=batch)
+    for b in range(batch):
+        _check(got[b], ref[b], A[b], B[b], "unit %d" % b)
+    over = h.gpu_gemm_f32_ex(np.full_like(C, np.nan), A, B, 1, N, K, capi.SPH_GEMM_OVERWRITE,
+                             batch=batch)
+    for b in range(batch):
+        _check(over[b], ref[b] - C[b], A[b], B[b], "overwrite unit %d" % b)
+    # a 1 x K operand is its own transpose
+    flagged = h.gpu_gemm_f32_ex(C, A, B, 1, N, K, capi.SPH_GEMM_TRANS_A, batch=batch)
+    assert np.array_equal(flagged.view(np.uint32), got.view(np.uint32))
