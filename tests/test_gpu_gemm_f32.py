@@ -246,3 +246,29 @@ def test_single_output_row(dev, case):
     # a 1 x K operand is its own transpose
     flagged = h.gpu_gemm_f32_ex(C, A, B, 1, N, K, capi.SPH_GEMM_TRANS_A, batch=batch)
     assert np.array_equal(flagged.view(np.uint32), got.view(np.uint32))
+
+
+@pytest.mark.parametrize("dims", [(2, 64, 32, 48), (3, 160, 64, 136), (2, 96, 512, 8)])
+def test_grouped_plan_on_aligned_shapes(dev, dims):
+    """The same modulo walk at sizes that take the straight-to-LDS kernels (K a multiple of 16
+    or 32, 16-byte aligned offsets) and, for the last one, the K-split kernel, with the unit
+    offsets coming from the device table."""
+    b, M, K, N = dims
+    ys, as_, bs = [b, 2, M, N], [b, 1, M, K], [b, 2, K, N]
+    _, leaves = po.gemm_plan(ys, as_, bs)
+    h.announce("sph_gemm_f32_grouped aligned", dims, len(leaves), "leaves")
+    A = synth.uniform(81, as_)
+    B = synth.uniform(82, bs)
+    C = synth.uniform(83, ys)
+    ref = po.compute_gemm(C.copy(), A, B, threads=4)
+    triples = []
+    for o, a, bb, total in leaves:
+        for u in range(total // (M * N)):
+            triples.append((o + u * M * N, a + u * M * K, bb + u * K * N))
+    got = h.gpu_gemm_grouped(C, A, B, M, N, K, triples)
+    flatA, flatB = A.reshape(-1, M, K), B.reshape(-1, K, N)
+    den = np.full((len(triples), M, N), 1e-30)
+    for o, a, bb in triples:
+        den[o // (M * N)] = np.abs(flatA[a // (M * K)]).astype(np.float64) @ np.abs(flatB[bb // (K * N)])
+    err = h.normalised_error(got.reshape(-1, M, N), ref.reshape(-1, M, N), None, den, True)
+    assert err <= TOL_F32
