@@ -333,6 +333,33 @@ def bench_spgemm(capi, synth, steps, warmup, n=8192, per_row=8.0):
     return event_ms, products, nnz.value, nbytes, a[0].size, b[0].size
 
 
+def bench_elementwise(capi, steps, warmup, n=4096):
+    """The one-pass kernels over n x n floats (64 MiB at n = 4096): algorithmic GB/s each."""
+    count = n * n
+    x = capi.DeviceBuffer.from_array(np.ones((n, n), np.float32))
+    z = capi.DeviceBuffer.from_array(np.ones((n, n), np.float32))
+    y = capi.DeviceBuffer(4 * count)
+    half = capi.DeviceBuffer(2 * count)
+    runs = [
+        ("transpose", lambda: capi.call("sph_transpose_f32", y.ptr, x.ptr, n, n, 1, 0), 8),
+        ("relu", lambda: capi.call("sph_relu_f32", y.ptr, x.ptr, count), 8),
+        ("relu_backward", lambda: capi.call("sph_relu_backward_f32", y.ptr, x.ptr, z.ptr, count), 16),
+        ("scale", lambda: capi.call("sph_scale_f32", y.ptr, x.ptr, 2.0, count), 8),
+        ("sub", lambda: capi.call("sph_sub_f32", y.ptr, x.ptr, z.ptr, count, 0, 0, 0), 12),
+        ("sgd_step", lambda: capi.call("sph_sgd_step_f32", y.ptr, x.ptr, 1e-6, count), 12),
+        ("fill", lambda: capi.call("sph_fill_f32", y.ptr, 0.0, count), 4),
+        ("convert_f32_to_f16", lambda: capi.call("sph_convert_f32_to_f16", half.ptr, x.ptr, count), 6),
+    ]
+    out = {}
+    for name, fn, bytes_per_element in runs:
+        ms, _ = timed_launches(capi, fn, steps, warmup)
+        gbs = bytes_per_element * count / (ms * 1e-3) / 1e9
+        out[name] = {"launch_ms": ms, "gbs": gbs, "frac_hbm_peak": gbs / PEAK_HBM_GBS}
+    for b in (x, z, y, half):
+        b.release()
+    return out
+
+
 def bench_copy(capi, steps, warmup, mib=64):
     """A plain one-pass kernel of known size (ReLU over `mib` MiB: reads it once, writes it
     once), used to calibrate the profiler's FETCH_SIZE / WRITE_SIZE counters."""
@@ -532,6 +559,7 @@ def main():
             "algorithmic_gbs": nbytes / (ms * 1e-3) / 1e9,
             "note": "both passes compute every product (the count pass must see which sums "
                     "cancel); products counted once per pass in gproducts_per_s"}
+        others["one_pass_kernels_4096x4096"] = bench_elementwise(capi, 50, 5)
         result["others"] = others
 
     if not args.no_cpu and args.only is None:
