@@ -71,6 +71,15 @@ int sph_device_info(int deviceId, SphDeviceInfo* info);
 
 int sph_malloc(void** ptr, size_t bytes);              /* Memory.cpp:30-36 */
 int sph_free(void* ptr);                               /* Memory.cpp:38-44 */
+/* Stream-ordered allocation on the calling thread's stream (hipMallocAsync):
+ * the block may be used by work enqueued after the call and is returned to
+ * the device's pool, not to the driver, when it is freed, so neither call
+ * waits for the device.  The pool behind the reference's ResourceManager
+ * (Sources/Sapphire/util/ResourceManager.cpp:38-72 calls cudaMalloc / cudaFree,
+ * both of which synchronise).  sph_mem_pool_trim hands idle pool memory back. */
+int sph_malloc_async(void** ptr, size_t bytes);
+int sph_free_async(void* ptr);
+int sph_mem_pool_trim(void);
 int sph_memcpy_h2d(void* dev, const void* host, size_t bytes); /* :46-53 */
 int sph_memcpy_d2h(void* host, const void* dev, size_t bytes); /* :55-63 */
 int sph_memcpy_d2d(void* dst, const void* src, size_t bytes);  /* :65-72 */

@@ -61,6 +61,9 @@ SIGNATURES = {
     "sph_device_info": [ctypes.c_int, ctypes.POINTER(SphDeviceInfo)],
     "sph_malloc": [ctypes.POINTER(_vp), _sz],
     "sph_free": [_vp],
+    "sph_malloc_async": [ctypes.POINTER(_vp), _sz],
+    "sph_free_async": [_vp],
+    "sph_mem_pool_trim": [],
     "sph_memcpy_h2d": [_vp, _vp, _sz],
     "sph_memcpy_d2h": [_vp, _vp, _sz],
     "sph_memcpy_d2d": [_vp, _vp, _sz],

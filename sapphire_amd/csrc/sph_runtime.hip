@@ -21,6 +21,7 @@ thread_local std::string tlsLastError;
 std::mutex gPoolMutex;
 std::vector<hipStream_t> gIdleStreams[kMaxDevices];
 int gComputeUnits[kMaxDevices] = {};
+bool gPoolRetains[kMaxDevices] = {};
 
 struct ThreadSlots
 {
@@ -190,6 +191,47 @@ int sph_free(void* ptr)
 {
     SPH_REFUSE_WHILE_CAPTURING();
     SPH_HIP_TRY(hipFree(ptr));
+    return SPH_OK;
+}
+
+int sph_malloc_async(void** ptr, size_t bytes)
+{
+    SPH_REFUSE_WHILE_CAPTURING();
+    SPH_REQUIRE(ptr != nullptr, "ptr is null");
+    SPH_STREAM_OR_FAIL(stream);
+    const int d = tlsSlots.device;
+    {
+        // freed blocks stay in the device's pool instead of going back to the driver
+        std::lock_guard<std::mutex> lock(gPoolMutex);
+        if (!gPoolRetains[d])
+        {
+            hipMemPool_t pool = nullptr;
+            SPH_HIP_TRY(hipDeviceGetDefaultMemPool(&pool, d));
+            uint64_t keep = ~0ull;
+            SPH_HIP_TRY(hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep));
+            gPoolRetains[d] = true;
+        }
+    }
+    SPH_HIP_TRY(hipMallocAsync(ptr, bytes != 0 ? bytes : 1, stream));
+    return SPH_OK;
+}
+
+int sph_free_async(void* ptr)
+{
+    SPH_REFUSE_WHILE_CAPTURING();
+    if (ptr == nullptr)
+        return SPH_OK;
+    SPH_STREAM_OR_FAIL(stream);
+    SPH_HIP_TRY(hipFreeAsync(ptr, stream));
+    return SPH_OK;
+}
+
+int sph_mem_pool_trim(void)
+{
+    SPH_REFUSE_WHILE_CAPTURING();
+    hipMemPool_t pool = nullptr;
+    SPH_HIP_TRY(hipDeviceGetDefaultMemPool(&pool, tlsSlots.device));
+    SPH_HIP_TRY(hipMemPoolTrimTo(pool, 0));
     return SPH_OK;
 }
 

@@ -34,6 +34,21 @@ void CudaFree(void* ptr)
     Check(sph_free(ptr), "CudaFree");
 }
 
+void CudaMallocAsync(void** ptr, std::size_t byteSize)
+{
+    Check(sph_malloc_async(ptr, byteSize), "CudaMallocAsync");
+}
+
+void CudaFreeAsync(void* ptr)
+{
+    Check(sph_free_async(ptr), "CudaFreeAsync");
+}
+
+void CudaTrimPool()
+{
+    Check(sph_mem_pool_trim(), "CudaTrimPool");
+}
+
 void CopyHostToDevice(void* devicePtr, const void* hostPtr, std::size_t byteSize)
 {
     Check(sph_memcpy_h2d(devicePtr, hostPtr, byteSize), "CopyHostToDevice");

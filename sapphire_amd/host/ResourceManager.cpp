@@ -130,16 +130,19 @@ void ReleaseHost(void* ptr)
     std::free(ptr);
 }
 
+// Device blocks come from the stream-ordered allocator: a request that misses the exact-size
+// free list costs no device synchronisation, and a released block goes back to the device's
+// pool in stream order instead of waiting for the device like cudaFree.
 void* AllocateCuda(std::size_t size)
 {
     void* ptr = nullptr;
-    Compute::Cuda::CudaMalloc(&ptr, size);
+    Compute::Cuda::CudaMallocAsync(&ptr, size);
     return ptr;
 }
 
 void ReleaseCuda(void* ptr)
 {
-    Compute::Cuda::CudaFree(ptr);
+    Compute::Cuda::CudaFreeAsync(ptr);
 }
 
 std::mutex gMutex;
@@ -236,6 +239,11 @@ void ResourceManager::ClearAll()
     ClearPreservedPool();
     ClearVolatilePool();
     ClearFreePool();
+    if (deviceBlocks)
+    {
+        Compute::Cuda::Synchronize();  // the stream-ordered releases have to run first
+        Compute::Cuda::CudaTrimPool();
+    }
 }
 
 PoolStatistics ResourceManager::Statistics()

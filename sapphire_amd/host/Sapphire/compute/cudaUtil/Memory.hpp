@@ -18,6 +18,12 @@ using StreamHandle = void*;
 void CudaSetDevice(int deviceId);
 void CudaMalloc(void** ptr, std::size_t byteSize);
 void CudaFree(void* ptr);
+//! Stream-ordered counterparts on the calling thread's stream: neither waits for the device,
+//! freed blocks stay in the device's pool.
+void CudaMallocAsync(void** ptr, std::size_t byteSize);
+void CudaFreeAsync(void* ptr);
+//! Returns idle pool memory to the driver.
+void CudaTrimPool();
 void CopyHostToDevice(void* devicePtr, const void* hostPtr, std::size_t byteSize);
 void CopyDeviceToHost(void* hostPtr, const void* devicePtr, std::size_t byteSize);
 void CopyDeviceToDevice(void* dst, const void* src, std::size_t byteSize);

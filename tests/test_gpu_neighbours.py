@@ -115,3 +115,28 @@ def test_sub_with_wrapping_operands(dev, case):
         capi.call("sph_sub_f32", dY.ptr, dA.ptr, dB.ptr, count, 0, 1, 0)
     for d in (dA, dB, dY):
         d.release()
+
+
+def test_stream_ordered_allocation(dev):
+    h.announce("sph_malloc_async / sph_free_async / sph_mem_pool_trim")
+    import ctypes
+    n = 1 << 16
+    seen = set()
+    for rep in range(5):
+        ptr = capi._vp()
+        capi.call("sph_malloc_async", ctypes.byref(ptr), 4 * n)
+        assert ptr.value
+        seen.add(ptr.value)
+        capi.call("sph_fill_f32", ptr.value, float(rep), n)      # ordered after the allocation
+        out = np.empty(n, np.float32)
+        capi.call("sph_memcpy_d2h", out.ctypes.data, ptr.value, 4 * n)
+        assert np.all(out == rep)
+        capi.call("sph_free_async", ptr.value)
+    assert len(seen) <= 5
+    capi.call("sph_free_async", None)                             # a null pointer is accepted
+    capi.sync()
+    capi.call("sph_mem_pool_trim")
+    empty = capi._vp()
+    capi.call("sph_malloc_async", ctypes.byref(empty), 0)        # zero bytes still gives a block
+    assert empty.value
+    capi.call("sph_free_async", empty.value)
