@@ -400,6 +400,24 @@ def cpu_gemm_baseline(d, rows=96):
     }
 
 
+def cpu_gemm_all_cores(d):
+    """The same per-element arithmetic (k ascending, unfused, bit-identical output) on the whole
+    of configuration 3, rows split over the host's cores and B walked with unit stride."""
+    from oracle import pyoracle as po
+    n = d["A"].shape[0]
+    A = d["A"].astype(np.float32)
+    B = d["B"].astype(np.float32)
+    out = np.zeros((n, n), np.float32)
+    threads = max(1, min(os.cpu_count() or 1, 16))
+    t0 = time.perf_counter()
+    po.gemm_rows(out, A, B, n, n, n, threads=threads)
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * n ** 3 / dt / 1e12, "unit": "TFLOP/s", "cores": threads,
+            "kind": "port",
+            "sample": "whole configuration 3, row-accumulator form of the reference loop "
+                      "(bit-identical results), %.1f s" % dt}
+
+
 def cpu_spmm_baseline(d):
     from oracle import pyoracle as po
     out = np.zeros((d["M"], d["N"]), np.float32)
@@ -564,6 +582,7 @@ def main():
 
     if not args.no_cpu and args.only is None:
         result["cpu_baseline"] = cpu_gemm_baseline(d3)
+        result["cpu_baseline_all_cores"] = cpu_gemm_all_cores(d3)
 
     print(json.dumps(result))
 
