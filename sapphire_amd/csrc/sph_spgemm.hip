@@ -220,24 +220,46 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
                     touched[t0 + lane] = 0;
                 while (pending != 0)
                 {
-                    const uint32_t t = t0 + static_cast<uint32_t>(__builtin_ctzll(pending));
-                    pending &= pending - 1;
-                    const uint32_t x = t * 64 + lane;
-                    const float v = strip[x];
-                    strip[x] = 0.0f;
-                    const bool keep = v != 0.0f;
-                    const uint64_t m = __ballot(keep);
-                    if (FILL)
+                    // up to four touched blocks per round, read together so that their LDS
+                    // latencies overlap, then emitted in order
+                    uint32_t x[4];
+                    float v[4];
+                    uint32_t rounds = 0;
+#pragma unroll
+                    for (uint32_t u = 0; u < 4; ++u)
                     {
-                        const uint32_t at =
-                            rowBase + emitted + __popcll(m & ((1ull << lane) - 1ull));
-                        if (keep && at < rowLimit)
+                        x[u] = 0;
+                        v[u] = 0.0f;
+                        if (pending != 0)
                         {
-                            args.VC[at] = v;
-                            args.COLC[at] = c0 + x;
+                            const uint32_t t =
+                                t0 + static_cast<uint32_t>(__builtin_ctzll(pending));
+                            pending &= pending - 1;
+                            x[u] = t * 64 + lane;
+                            v[u] = strip[x[u]];
+                            strip[x[u]] = 0.0f;
+                            rounds = u + 1;
                         }
                     }
-                    emitted += __popcll(m);
+#pragma unroll
+                    for (uint32_t u = 0; u < 4; ++u)
+                    {
+                        if (u >= rounds)
+                            break;
+                        const bool keep = v[u] != 0.0f;
+                        const uint64_t m = __ballot(keep);
+                        if (FILL)
+                        {
+                            const uint32_t at =
+                                rowBase + emitted + __popcll(m & ((1ull << lane) - 1ull));
+                            if (keep && at < rowLimit)
+                            {
+                                args.VC[at] = v[u];
+                                args.COLC[at] = c0 + x[u];
+                            }
+                        }
+                        emitted += __popcll(m);
+                    }
                 }
             }
         }
