@@ -4,19 +4,20 @@
 // Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50): half
 // inputs, fp32 accumulation, row-major operands, result added into out.
 //
-// Two kernels:
+// Three kernels:
 //
-//   GemmF16Tile256  M, N multiples of 256, K a multiple of 64, 16-byte aligned
-//     rows.  One workgroup of 8 wavefronts (2 x 4) owns a 256 x 256 output
-//     tile; each wavefront a 128 x 64 part of it (4 x 2 MFMA tiles, 128
-//     accumulator registers).  K advances 64 at a time through two LDS stages
-//     of 64 KiB (A 256x64, B 64x256).  Global memory is copied straight into
-//     LDS (global_load_lds, 16 bytes per lane, no VGPR staging); the copy of
-//     stage i+1 is in flight while the MFMAs of stage i run.  LDS is written
-//     lane-linear by those copies, so bank conflicts are removed by choosing
-//     WHICH global chunk each lane fetches: A rows are XOR-swizzled in 16-byte
-//     chunks (chunk ^ row%8), B rows in 32-byte chunks (chunk ^ 2*(k%4)); both
-//     patterns measured conflict-free for the reads below.
+//   GemmF16Tile256  M, N multiples of 256, K a multiple of 32, 16-byte aligned
+//     rows, and at least three quarters as many tiles as compute units.  One
+//     workgroup of 8 wavefronts (2 x 4) owns a 256 x 256 output tile; each
+//     wavefront a 128 x 64 part of it (4 x 2 MFMA tiles, 128 accumulator
+//     registers).  K advances 32 at a time through four LDS stages of 32 KiB
+//     (A 256x32, B 32x256).  Global memory is copied straight into LDS
+//     (global_load_lds, 16 bytes per lane, no VGPR staging), three to four
+//     steps ahead of the MFMAs.  LDS is written lane-linear by those copies,
+//     so bank conflicts are removed by choosing WHICH global chunk each lane
+//     fetches: A rows are XOR-swizzled in 16-byte chunks (chunk ^ row%8), B
+//     rows in 32-byte chunks (chunk ^ 2*(k%4)); both patterns measured
+//     conflict-free for the reads below.
 //     A fragments are read with ds_read_b128 (8 consecutive k of one row); B is
 //     stored k-major, so its fragments (8 consecutive k of one column) come
 //     from two ds_read_b64_tr_b16 transposing reads.  The MFMA operands are
@@ -26,9 +27,13 @@
 //     XCD (ids congruent mod 8) cover a compact 8 x 4 block of tiles and share
 //     their A and B panels through that XCD's L2.
 //
-//   GemmF16General  any shape.  128 x 128 tile, 4 wavefronts, K step 32, global
-//     loads staged through registers with per-element predication (16-byte
-//     loads when K, N and the bases allow), padded LDS rows.
+//   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned, any M: the
+//     same ingredients on 128 x 128 tiles with 4 wavefronts, for ragged shapes
+//     and for shapes with too few 256-tiles to fill the chip.
+//
+//   GemmF16General  everything else.  128 x 128 tile, 4 wavefronts, K step 32,
+//     global loads staged through registers with per-element predication
+//     (16-byte loads when K, N and the bases allow), padded LDS rows.
 #include "sph_internal.h"
 
 #include <cstdlib>

@@ -5,21 +5,23 @@
 // (Sources/Sapphire/compute/dense/naive/NaiveGemm.cpp:12-38) is the order in
 // which the K products are summed.
 //
-// Work decomposition
-//   * one workgroup (4 wavefronts of 64 lanes, arranged 2 x 2) owns a
-//     BM x BN tile of one M x N unit; BM = BN = 128 when that still gives at
-//     least one tile per compute unit, 64 otherwise;
-//   * the K loop advances 16 columns at a time: the A slab (BM x 16) is stored
-//     k-major in LDS and the B slab (16 x BN) row-major, so that both MFMA
-//     operands are read with lane-consecutive addresses (no bank conflicts);
-//   * the slab for step i+1 is fetched from HBM into registers while the MFMAs
-//     of step i run, and written to the other LDS buffer afterwards;
-//   * units come either from (batch, stride) arithmetic -- stride 0 repeats an
-//     operand -- or from a table of element offsets in device memory.
-//
-// Loads are 16 bytes wide when K, N and every base/stride allow it; otherwise
-// a scalar, fully predicated path handles arbitrary shapes such as the
-// reference's random test sizes (Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:26-33).
+// Four kernels, chosen from the shape and the alignment of the operands:
+//   GemmF32DmaKernel     aligned operands with K a multiple of 16: slabs travel global -> LDS
+//                        without staging registers, several K steps ahead (the fast path);
+//   GemmF32Kernel        any shape and alignment: register-staged double buffering, 16-byte
+//                        loads when possible, scalar predicated loads otherwise (e.g. the
+//                        reference's random test sizes,
+//                        Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:26-33);
+//   GemmF32SkinnyKernel  few output tiles and a long K: K split over the wavefronts of a
+//                        workgroup;
+//   GemvRowKernel        a single output row.
+// The first two share one decomposition: a workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile
+// of one M x N unit, BM = BN = 128 when that still gives a tile per compute unit and 64
+// otherwise, and they add the K products of an element in the same order, so which of them
+// runs never changes a bit.  Either operand may be stored transposed (template flags), the
+// result may overwrite out or take a bias row and a ReLU in the epilogue, and units come from
+// (batch, stride) arithmetic -- stride 0 repeats an operand -- or from a table of element
+// offsets in device memory.
 #include "sph_internal.h"
 
 #include <algorithm>
