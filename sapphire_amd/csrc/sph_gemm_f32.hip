@@ -597,19 +597,27 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsVoidPtr)(lds)));
     const uint32_t steps = K / BK;
 
-    auto issue = [&](uint32_t step) {
-        // steps past the end fetch the last one again into a stage nobody reads any more,
-        // which keeps the number of outstanding copies the same in every iteration
-        const uint32_t src = min(step, steps - 1);
-        const uint32_t stage = ldsBase + (step % STAGES) * kStageBytes;
-        const char* aBase = reinterpret_cast<const char*>(A) + src * aStepBytes;
-        const char* bBase = reinterpret_cast<const char*>(B) + src * bStepBytes;
-#pragma unroll
-        for (uint32_t i = 0; i < kCopiesA; ++i)
-            DmaToLds16(aLane[i], aBase, stage + aDst[i]);
-#pragma unroll
-        for (uint32_t i = 0; i < kCopiesB; ++i)
-            DmaToLds16(bLane[i], bBase, stage + bDst[i]);
+    // Copy n (0 .. kCopiesPerWave-1) of this wavefront's share of the next step to fetch, into
+    // stage `stage`.  aSrc / bSrc point at that step's slab; steps past the end fetch the last
+    // one again into a stage nobody reads any more, which keeps the number of outstanding
+    // copies the same in every iteration.
+    const char* aSrc = reinterpret_cast<const char*>(A);
+    const char* bSrc = reinterpret_cast<const char*>(B);
+    uint32_t stepsToAdvance = steps - 1;
+    auto issueOne = [&](uint32_t stage, uint32_t n) {
+        const uint32_t base = ldsBase + stage * kStageBytes;
+        if (n < kCopiesA)
+            DmaToLds16(aLane[n], aSrc, base + aDst[n]);
+        else
+            DmaToLds16(bLane[n - kCopiesA], bSrc, base + bDst[n - kCopiesA]);
+    };
+    auto advance = [&]() {
+        if (stepsToAdvance != 0)
+        {
+            aSrc += aStepBytes;
+            bSrc += bStepBytes;
+            --stepsToAdvance;
+        }
     };
 
     floatx16 acc[TM][TN];
@@ -697,37 +705,82 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
                     acc[i][j] =
                         __builtin_amdgcn_mfma_f32_32x32x2f32(b[j][e], a[i][e], acc[i][j], 0, 0, 0);
     };
+    // First k block of step s.  The step's housekeeping sits between its MFMAs, where the
+    // matrix pipe is already busy: behind the first one the wait for step s+1's copies and the
+    // barrier, behind each of the next ones one copy of step s+STAGES-1.
+    static_assert(kCopiesPerWave <= 4 * TM * TN, "one copy per MFMA of the first block");
+    auto multiplyAndFeed = [&](const float (&a)[TM][4], const float (&b)[TN][4],
+                               uint32_t fillStage) {
+#pragma unroll
+        for (uint32_t e = 0; e < 4; ++e)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                {
+                    const uint32_t n = (e * TM + i) * TN + j;
+                    acc[i][j] =
+                        __builtin_amdgcn_mfma_f32_32x32x2f32(b[j][e], a[i][e], acc[i][j], 0, 0, 0);
+                    if (n == 0)
+                    {
+                        // steps up to s+1 have landed once at most the STAGES-3 later ones
+                        // are pending; behind the barrier everybody's copies are visible and
+                        // everybody has read the last fragment of step s-1
+                        WaitVmem<(STAGES - 3) * kCopiesPerWave>();
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
+                    }
+                    if (n < kCopiesPerWave)
+                    {
+                        issueOne(fillStage, n);
+                        if (n + 1 == kCopiesPerWave)
+                            advance();
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+    };
 
 #pragma unroll
     for (uint32_t p = 0; p < STAGES - 1; ++p)
-        issue(p);
+    {
+#pragma unroll
+        for (uint32_t n = 0; n < kCopiesPerWave; ++n)
+            issueOne(p, n);
+        advance();
+    }
 
     // Fragments are read one k block (8 values) ahead of the MFMAs that use them; the first
-    // block of step s+1 is read while the last block of step s is multiplied.
+    // block of step s+1 is read while the last block of step s is multiplied.  Stage s+1 is
+    // known to be complete from the barrier inside the first block of step s.
     float fa[2][TM][4], fb[2][TN][4];
     WaitVmem<(STAGES - 2) * kCopiesPerWave>();
     __syncthreads();
     loadFragments(fa[0], fb[0], lds, 0);
 
-    for (uint32_t s = 0; s < steps; ++s)
+    // The loop is unrolled over the ring so that every stage offset is a constant.
+    for (uint32_t s0 = 0; s0 < steps; s0 += STAGES)
     {
-        // steps s and s+1 have landed once at most the STAGES-3 later ones are pending
-        WaitVmem<(STAGES - 3) * kCopiesPerWave>();
-        __syncthreads();  // everybody's copies are visible; everybody has left step s-1
-        issue(s + STAGES - 1);
-
-        const char* cur = lds + (s % STAGES) * kStageBytes;
-        const char* next = lds + ((s + 1) % STAGES) * kStageBytes;
 #pragma unroll
-        for (uint32_t q = 0; q < kBlocks; ++q)
+        for (uint32_t u = 0; u < STAGES; ++u)
         {
-            if (q + 1 < kBlocks)
-                loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], cur, q + 1);
-            else
-                loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], next, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            multiply(fa[q & 1], fb[q & 1]);
-            __builtin_amdgcn_sched_barrier(0);
+            if (s0 + u >= steps)
+                break;
+            const char* cur = lds + u * kStageBytes;
+            const char* next = lds + ((u + 1) % STAGES) * kStageBytes;
+#pragma unroll
+            for (uint32_t q = 0; q < kBlocks; ++q)
+            {
+                if (q + 1 < kBlocks)
+                    loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], cur, q + 1);
+                else
+                    loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], next, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (q == 0)
+                    multiplyAndFeed(fa[0], fb[0], (u + STAGES - 1) % STAGES);
+                else
+                    multiply(fa[q & 1], fb[q & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     }
     WaitVmem<0>();  // the surplus copies of the last steps still target LDS
