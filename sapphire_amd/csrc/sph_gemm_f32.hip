@@ -1206,9 +1206,16 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         return SPH_OK;
     }
 
+    // Tile edge: the matrix pipes bound these kernels, so a launch lasts as long as the
+    // compute unit with the most tiles needs.  A 128-tile costs four 64-tiles and moves half
+    // the operand bytes per flop (measured 7 % faster at equal load); pick the edge with the
+    // smaller cost of the busiest compute unit.
+    const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
     const uint64_t tiles128 =
         static_cast<uint64_t>((args.M + 127) / 128) * ((args.N + 127) / 128) * units;
-    const bool big = tiles128 >= static_cast<uint64_t>(sph::ComputeUnits());
+    const uint64_t cost128 = ((tiles128 + cus - 1) / cus) * 400;
+    const uint64_t cost64 = ((tiles64 + cus - 1) / cus) * 107;
+    const bool big = cost128 <= cost64;
     const uint32_t bm = big ? 128 : 64;
     args.tilesM = (args.M + bm - 1) / bm;
     args.tilesN = (args.N + bm - 1) / bm;
