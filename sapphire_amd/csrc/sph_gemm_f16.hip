@@ -505,7 +505,8 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
 // For shapes the 256-tile kernel does not take (M or N not a multiple of 256) as long as K is a
 // multiple of 32, N of 8 and everything is 16-byte aligned.  Four wavefronts (2 x 2), each
 // 64 x 64 = 2 x 2 MFMA blocks, four LDS stages of 16 KiB (two workgroups per compute unit),
-// copies issued two steps ahead, one barrier per step, fragments read half a step ahead.
+// copies issued two steps ahead, one barrier per step (placed, with the copies, between the
+// MFMAs of the step's first half), fragments read half a step ahead.
 // A stage: 128 rows of 64 bytes, 16-byte chunk c of row x at position c ^ ((x >> 2) & 3).
 // B stage: 32 k-rows of 256 bytes, 32-byte chunks XOR-swizzled with 2*(k%4), read with the
 // transposing LDS load like the 256-tile kernel.  Rows past M and columns past N are clamped to
@@ -560,15 +561,26 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     const size_t bStepBytes = static_cast<size_t>(kTK) * N * 2;
     const uint32_t ldsBase = LdsAddress(lds);
     const uint32_t steps = K / kTK;
-    auto issue = [&](uint32_t step) {
-        const uint32_t src = min(step, steps - 1);  // surplus steps re-fetch the last one
-        const uint32_t stage = ldsBase + (step % kDStages) * kDStageBytes;
-        const char* aBase = reinterpret_cast<const char*>(A) + static_cast<size_t>(src) * (kTK * 2);
-        const char* bBase = reinterpret_cast<const char*>(B) + static_cast<size_t>(src) * bStepBytes;
-        DmaToLds16<0>(aLane[0], aBase, stage + aDst[0]);
-        DmaToLds16<0>(aLane[1], aBase, stage + aDst[1]);
-        DmaToLds16<0>(bLane[0], bBase, stage + bDst[0]);
-        DmaToLds16<0>(bLane[1], bBase, stage + bDst[1]);
+    // Copy n (0..3: two of A, two of B) of the next step to fetch, into stage `stage`.  aSrc /
+    // bSrc point at that step's slabs; surplus steps re-fetch the last one into a stage nobody
+    // reads any more, which keeps the number of outstanding copies the same in every iteration.
+    const char* aSrc = reinterpret_cast<const char*>(A);
+    const char* bSrc = reinterpret_cast<const char*>(B);
+    uint32_t stepsToAdvance = steps - 1;
+    auto issueOne = [&](uint32_t stage, uint32_t n) {
+        const uint32_t base = ldsBase + stage * kDStageBytes;
+        if (n < 2)
+            DmaToLds16<0>(aLane[n], aSrc, base + aDst[n]);
+        else
+            DmaToLds16<0>(bLane[n - 2], bSrc, base + bDst[n - 2]);
+    };
+    auto advance = [&]() {
+        if (stepsToAdvance != 0)
+        {
+            aSrc += kTK * 2;
+            bSrc += bStepBytes;
+            --stepsToAdvance;
+        }
     };
 
     // ---- fragment plan ----------------------------------------------------------------
@@ -615,30 +627,67 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
                     __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
     };
 
+    // First half of a step.  The step's housekeeping sits between its MFMAs, where the matrix
+    // pipe is already busy: behind the first one the wait for the copies of step st+1 and the
+    // barrier, behind every one a copy of step st+3.
+    auto multiplyAndFeed = [&](const halfx8 (&af)[2], const halfx8 (&bf)[2], uint32_t fillStage) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+            {
+                acc[i][j] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+                if (i == 0 && j == 0)
+                {
+                    // steps up to st+1 have landed once at most one later step is pending;
+                    // behind the barrier everybody's copies are visible and everybody has
+                    // read the last fragment of step st-1
+                    WaitVmem<(kDStages - 3) * kDCopies>();
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                }
+                issueOne(fillStage, i * 2 + j);
+                if (i == 1 && j == 1)
+                    advance();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    };
+
 #pragma unroll
     for (uint32_t p = 0; p < kDStages - 1; ++p)
-        issue(p);
+    {
+#pragma unroll
+        for (uint32_t n = 0; n < kDCopies; ++n)
+            issueOne(p, n);
+        advance();
+    }
     halfx8 af[2][2], bf[2][2];
     WaitVmem<(kDStages - 2) * kDCopies>();
     __syncthreads();
     loadFragments(af[0], bf[0], lds, 0);
 
-    for (uint32_t st = 0; st < steps; ++st)
+    // Fragments are read half a step ahead of their MFMAs; stage st+1 is known to be complete
+    // from the barrier inside the first half of step st.  The loop is unrolled over the ring
+    // so that every stage offset is a constant.
+    for (uint32_t s0 = 0; s0 < steps; s0 += kDStages)
     {
-        // steps st and st+1 have landed once at most one later step is pending
-        WaitVmem<(kDStages - 3) * kDCopies>();
-        __syncthreads();
-        issue(st + kDStages - 1);
-        const char* cur = lds + (st % kDStages) * kDStageBytes;
-        const char* next = lds + ((st + 1) % kDStages) * kDStageBytes;
-        loadFragments(af[1], bf[1], cur, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(af[0], bf[0]);
-        __builtin_amdgcn_sched_barrier(0);
-        loadFragments(af[0], bf[0], next, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(af[1], bf[1]);
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t u = 0; u < kDStages; ++u)
+        {
+            if (s0 + u >= steps)
+                break;
+            const char* cur = lds + u * kDStageBytes;
+            const char* next = lds + ((u + 1) % kDStages) * kDStageBytes;
+            loadFragments(af[1], bf[1], cur, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            multiplyAndFeed(af[0], bf[0], (u + kDStages - 1) % kDStages);
+            __builtin_amdgcn_sched_barrier(0);
+            loadFragments(af[0], bf[0], next, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(af[1], bf[1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     WaitVmem<0>();  // the surplus copies of the last steps still target LDS
 
