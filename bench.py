@@ -60,6 +60,9 @@ def parse():
     p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
                                       "csr"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
+    p.add_argument("--zero-operands", action="store_true",
+                   help="with --only gemm: all-zero A and B, to see how far the clock (and the "
+                        "rate) depends on operand values; the line says data = zeros")
     return p.parse_args()
 
 
@@ -94,9 +97,12 @@ def timed_maybe_graph(capi, launch, steps, warmup, graph):
     return event_ms
 
 
-def bench_gemm_f16(capi, synth, steps, warmup, flags=0):
+def bench_gemm_f16(capi, synth, steps, warmup, flags=0, zero_operands=False):
     n = 4096
     d = synth.config3(n)
+    if zero_operands:
+        d["A"][...] = 0
+        d["B"][...] = 0
     dA = capi.DeviceBuffer.from_array(d["A"])
     dB = capi.DeviceBuffer.from_array(d["B"])
     dC = capi.DeviceBuffer.from_array(d["C"])
@@ -443,7 +449,9 @@ def main():
     n = 4096
     flops = 2.0 * n ** 3
     if args.only in (None, "gemm"):
-        event_ms, wall_ms, d3 = bench_gemm_f16(capi, synth, args.steps, args.warmup)
+        zeros = args.zero_operands and args.only == "gemm"
+        event_ms, wall_ms, d3 = bench_gemm_f16(capi, synth, args.steps, args.warmup,
+                                               zero_operands=zeros)
         tflops = flops / (wall_ms * 1e-3) / 1e12
         kernel_tflops = flops / (event_ms * 1e-3) / 1e12
         result.update({
@@ -451,7 +459,7 @@ def main():
             "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": wall_ms, "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "f16 in / f32 accumulate",
-            "data": "synthetic",
+            "data": "zeros" if zeros else "synthetic",
             "config": {"workload": "configuration 3: out[4096,4096] f32 += A[4096,4096] f16 * "
                                    "B[4096,4096] f16, N(0,1/sqrt(K)) inputs, row-major, one launch "
                                    "per step, inputs resident in HBM",
