@@ -11,16 +11,18 @@
 // them as well); a row's entries come out in ascending column order.
 //
 // One wavefront owns one output row.  Instead of a hash table and a sort it keeps a dense
-// strip of the row in LDS (up to 8192 columns, 32 KiB; wider matrices are done strip by
+// strip of the row in LDS (up to 4096 columns, 16 KiB; wider matrices are done strip by
 // strip): A's entries are taken in order, the entries of the matching row of B are spread
 // over the 64 lanes and added into the strip, and because the columns of one row of B are
 // distinct no two lanes touch the same element in one step, which makes the sum order fixed
-// and the result bit-identical to the CPU loop.  The strip is then swept in column order,
-// which yields the sorted row without sorting.  A byte per block of 64 columns records which
-// blocks were touched; only those are swept, and they are set back to zero as they are read,
-// so the strip is cleared once per workgroup and the cost of a row follows the entries it
-// produces, not the width of the matrix.  The same kernel runs twice: once to count the
-// entries of every row (the caller then allocates), once to write them.
+// and the result bit-identical to the CPU loop.  A bit per column records which elements were
+// touched.  The strip is then swept in column order, which yields the sorted row without
+// sorting: every lane owns a run of consecutive columns (its words of the bit map), counts the
+// touched elements of its run that are not zero, a prefix sum over the lanes turns the counts
+// into output positions, and the lane writes its entries.  Touched elements are set back to
+// zero as they are read, so the strip is cleared once per workgroup and the cost of a strip
+// follows the entries it produces, not its width.  The same kernel runs twice: once to count
+// the entries of every row (the caller then allocates), once to write them.
 //
 // Requirements on the operands: column indices of B below N and distinct within a row;
 // column indices of A below the row count of B.
@@ -32,9 +34,11 @@
 
 namespace
 {
-constexpr uint32_t kStripMax = 8192;  // columns per LDS strip
+constexpr uint32_t kStripMax = 4096;  // columns per LDS strip
 constexpr uint32_t kAhead = 8;        // rows of B whose first 64 entries are in flight together
-constexpr uint32_t kRowsPerTurn = 8;  // consecutive output rows a wavefront takes at a time
+constexpr uint32_t kRowsPerTurnMax = 8;  // consecutive output rows a wavefront takes at a time
+constexpr uint32_t kWordsPerLaneMax = kStripMax / 32 / 64;  // bit-map words a lane owns
+static_assert(kWordsPerLaneMax <= 4, "the sweep takes a lane's words as two pairs");
 
 struct SpgemmArgs
 {
@@ -46,6 +50,7 @@ struct SpgemmArgs
     const uint32_t* ROWB;
     uint32_t M, K, N;
     uint32_t strip;  // columns per strip (multiple of 64)
+    uint32_t rowsPerTurn;  // 1 .. kRowsPerTurnMax
     // count pass: counts (M + 1 entries, counts[M] = 0).  fill pass: ROWC, VC, COLC.
     uint32_t* counts;
     const uint32_t* ROWC;
@@ -64,29 +69,37 @@ __device__ __forceinline__ float Uniform(float v, uint32_t lane)
         float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), static_cast<int>(lane)));
 }
 
+__device__ __forceinline__ void Touch(uint32_t* bits, uint32_t column)
+{
+    __hip_atomic_fetch_or(&bits[column >> 5], 1u << (column & 31), __ATOMIC_RELAXED,
+                          __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 template <bool FILL>
 __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
 {
     extern __shared__ float strip[];
-    // one flag per block of 64 columns, after the strip
-    unsigned char* touched = reinterpret_cast<unsigned char*>(strip + args.strip);
-    const uint32_t blocksInStrip = args.strip / 64;
+    // one bit per column, after the strip; lane l owns words l*wordsPerLane .. +wordsPerLane-1
+    uint32_t* bits = reinterpret_cast<uint32_t*>(strip + args.strip);
+    const uint32_t wordsInStrip = args.strip / 32;
+    const uint32_t wordsPerLane = (wordsInStrip + 63) / 64;  // at most kStripMax / 2048
     const uint32_t lane = threadIdx.x;
     if (!FILL && blockIdx.x == 0 && lane == 0)
         args.counts[args.M] = 0;
     // cleared once; every block that is touched is cleared again when it is swept
     for (uint32_t x = lane; x < args.strip; x += 64)
         strip[x] = 0.0f;
-    for (uint32_t t = lane; t < blocksInStrip; t += 64)
-        touched[t] = 0;
+    for (uint32_t t = lane; t < wordsInStrip; t += 64)
+        bits[t] = 0;
 
-    // A wavefront takes kRowsPerTurn consecutive rows per turn.  Their extents are read in one
+    // A wavefront takes rowsPerTurn consecutive rows per turn.  Their extents are read in one
     // go, and the loads that lead to a row's products form a pipeline over the rows of the
     // turn: while row i is multiplied, the first 64 (column, value) pairs of A's row i+2 and
     // the extents of the rows of B that row i+1 needs are already on their way.
-    for (uint32_t turn = blockIdx.x * kRowsPerTurn; turn < args.M; turn += gridDim.x * kRowsPerTurn)
+    for (uint32_t turn = blockIdx.x * args.rowsPerTurn; turn < args.M;
+         turn += gridDim.x * args.rowsPerTurn)
     {
-        const uint32_t rowsHere = min(kRowsPerTurn, args.M - turn);
+        const uint32_t rowsHere = min(args.rowsPerTurn, args.M - turn);
         uint32_t extentA = 0, extentC = 0;
         if (lane <= rowsHere)
         {
@@ -195,7 +208,7 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
                         if (col[u] - c0 < width)  // also false for the 0xffffffff of idle lanes
                         {
                             strip[col[u] - c0] = strip[col[u] - c0] + a[u] * b[u];
-                            touched[(col[u] - c0) >> 6] = 1;
+                            Touch(bits, col[u] - c0);
                         }
                         // rows of B with more than 64 entries: the rest, 64 at a time
                         for (uint32_t pb = s[u] + 64 + lane; pb < e[u]; pb += 64)
@@ -204,64 +217,93 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
                             if (c - c0 < width)
                             {
                                 strip[c - c0] = strip[c - c0] + a[u] * args.VB[pb];
-                                touched[(c - c0) >> 6] = 1;
+                                Touch(bits, c - c0);
                             }
                         }
                     }
                 }
             }
 
-            // sweep the touched blocks in column order and leave them zero again
-            for (uint32_t t0 = 0; t0 < blocksInStrip; t0 += 64)
-            {
-                const bool mine = t0 + lane < blocksInStrip && touched[t0 + lane] != 0;
-                uint64_t pending = __ballot(mine);
-                if (mine)
-                    touched[t0 + lane] = 0;
-                while (pending != 0)
+            // sweep: this lane's touched columns in ascending order, as two 64-column runs
+            // (a pair of bit-map words each)
+            auto fetchPair = [&](uint32_t first) {
+                uint32_t lo = 0, hi = 0;
+                const uint32_t w = lane * wordsPerLane + first;
+                if (first < wordsPerLane && w < wordsInStrip)
                 {
-                    // up to four touched blocks per round, read together so that their LDS
-                    // latencies overlap, then emitted in order
-                    uint32_t x[4];
-                    float v[4];
-                    uint32_t rounds = 0;
+                    lo = bits[w];
+                    if (lo != 0)
+                        bits[w] = 0;
+                }
+                if (first + 1 < wordsPerLane && w + 1 < wordsInStrip)
+                {
+                    hi = bits[w + 1];
+                    if (hi != 0)
+                        bits[w + 1] = 0;
+                }
+                return (static_cast<uint64_t>(hi) << 32) | lo;
+            };
+            const uint64_t mine0 = fetchPair(0);
+            const uint64_t mine1 = fetchPair(2);
+            const uint32_t base0 = lane * wordsPerLane * 32;  // first column of run 0
+            const uint32_t base1 = base0 + 64;
+
+            // next touched column of this lane's runs, removed from the set
+            auto take = [&](uint64_t& set0, uint64_t& set1) {
+                if (set0 != 0)
+                {
+                    const uint32_t b = static_cast<uint32_t>(__builtin_ctzll(set0));
+                    set0 &= set0 - 1;
+                    return base0 + b;
+                }
+                const uint32_t b = static_cast<uint32_t>(__builtin_ctzll(set1));
+                set1 &= set1 - 1;
+                return base1 + b;
+            };
+            // pass 1: how many of them hold a value that is not zero (the count pass
+            // clears them here; the fill pass needs them once more)
+            uint32_t kept = 0;
+            {
+                uint64_t set0 = mine0, set1 = mine1;
+                while ((set0 | set1) != 0)
+                {
+                    const uint32_t x = take(set0, set1);
+                    if (strip[x] != 0.0f)
+                        ++kept;
+                    if (!FILL)
+                        strip[x] = 0.0f;
+                }
+            }
+            // positions: exclusive prefix sum of `kept` over the lanes
+            uint32_t inclusive = kept;
 #pragma unroll
-                    for (uint32_t u = 0; u < 4; ++u)
+            for (uint32_t d = 1; d < 64; d *= 2)
+            {
+                const uint32_t other = __shfl_up(inclusive, d, 64);
+                if (lane >= d)
+                    inclusive += other;
+            }
+            if (FILL)
+            {
+                uint32_t at = rowBase + emitted + inclusive - kept;
+                uint64_t set0 = mine0, set1 = mine1;
+                while ((set0 | set1) != 0)
+                {
+                    const uint32_t x = take(set0, set1);
+                    const float v = strip[x];
+                    strip[x] = 0.0f;
+                    if (v != 0.0f)
                     {
-                        x[u] = 0;
-                        v[u] = 0.0f;
-                        if (pending != 0)
+                        if (at < rowLimit)
                         {
-                            const uint32_t t =
-                                t0 + static_cast<uint32_t>(__builtin_ctzll(pending));
-                            pending &= pending - 1;
-                            x[u] = t * 64 + lane;
-                            v[u] = strip[x[u]];
-                            strip[x[u]] = 0.0f;
-                            rounds = u + 1;
+                            args.VC[at] = v;
+                            args.COLC[at] = c0 + x;
                         }
-                    }
-#pragma unroll
-                    for (uint32_t u = 0; u < 4; ++u)
-                    {
-                        if (u >= rounds)
-                            break;
-                        const bool keep = v[u] != 0.0f;
-                        const uint64_t m = __ballot(keep);
-                        if (FILL)
-                        {
-                            const uint32_t at =
-                                rowBase + emitted + __popcll(m & ((1ull << lane) - 1ull));
-                            if (keep && at < rowLimit)
-                            {
-                                args.VC[at] = v[u];
-                                args.COLC[at] = c0 + x[u];
-                            }
-                        }
-                        emitted += __popcll(m);
+                        ++at;
                     }
                 }
             }
+            emitted += Uniform(inclusive, 63);
         }
         if (!FILL && lane == 0)
             args.counts[turn + i] = emitted;
@@ -275,10 +317,18 @@ uint32_t StripFor(uint32_t N)
     return std::max<uint32_t>(64u, std::min(padded, kStripMax));
 }
 
-uint32_t GridFor(uint32_t M)
+// Rows per turn: long turns let the loads of consecutive rows overlap, short ones give a small
+// matrix enough workgroups to fill the chip (about eight resident per compute unit).
+uint32_t RowsPerTurnFor(uint32_t M)
+{
+    const uint32_t wanted = static_cast<uint32_t>(sph::ComputeUnits()) * 8;
+    return std::max<uint32_t>(1, std::min<uint32_t>(kRowsPerTurnMax, M / std::max<uint32_t>(wanted, 1)));
+}
+
+uint32_t GridFor(uint32_t M, uint32_t rowsPerTurn)
 {
     const uint64_t cap = static_cast<uint64_t>(sph::ComputeUnits()) * 64;
-    const uint64_t turns = (static_cast<uint64_t>(M) + kRowsPerTurn - 1) / kRowsPerTurn;
+    const uint64_t turns = (static_cast<uint64_t>(M) + rowsPerTurn - 1) / rowsPerTurn;
     return static_cast<uint32_t>(std::max<uint64_t>(1, std::min<uint64_t>(turns, cap)));
 }
 }  // namespace
@@ -307,9 +357,10 @@ int sph_spgemm_row_offsets_f32(uint32_t* ROWC, const float* VA, const uint32_t* 
     args.K = K;
     args.N = N;
     args.strip = StripFor(N);
+    args.rowsPerTurn = RowsPerTurnFor(M);
     args.counts = ROWC;
-    hipLaunchKernelGGL(SpgemmRowKernel<false>, dim3(GridFor(M)), dim3(64),
-                       args.strip * sizeof(float) + args.strip / 64, stream, args);
+    hipLaunchKernelGGL(SpgemmRowKernel<false>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
+                       args.strip * sizeof(float) + args.strip / 8, stream, args);
     SPH_CHECK_LAUNCH();
     return sph::ExclusiveScanInPlace(ROWC, M + 1, nnzHost, stream);
 }
@@ -337,11 +388,12 @@ int sph_spgemm_fill_f32(float* VC, uint32_t* COLC, const uint32_t* ROWC, const f
     args.K = K;
     args.N = N;
     args.strip = StripFor(N);
+    args.rowsPerTurn = RowsPerTurnFor(M);
     args.ROWC = ROWC;
     args.VC = VC;
     args.COLC = COLC;
-    hipLaunchKernelGGL(SpgemmRowKernel<true>, dim3(GridFor(M)), dim3(64),
-                       args.strip * sizeof(float) + args.strip / 64, stream, args);
+    hipLaunchKernelGGL(SpgemmRowKernel<true>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
+                       args.strip * sizeof(float) + args.strip / 8, stream, args);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
