@@ -6,8 +6,10 @@
 //
 // Three kernels:
 //
-//   GemmF16Tile256  M, N multiples of 256, K a multiple of 32, 16-byte aligned
-//     rows, and at least three quarters as many tiles as compute units.  One
+//   GemmF16Tile256  K a multiple of 32, N of 8, 16-byte aligned rows, at least three
+//     quarters as many 256 x 256 tiles as compute units and at least three quarters of
+//     the tiled area inside the matrix (a variant with clamped copies and a guarded
+//     epilogue serves M, N that are not multiples of 256).  One
 //     workgroup of 8 wavefronts (2 x 4) owns a 256 x 256 output tile; each
 //     wavefront a 128 x 64 part of it (4 x 2 MFMA tiles, 128 accumulator
 //     registers).  K advances 32 at a time through four LDS stages of 32 KiB
@@ -28,8 +30,8 @@
 //     their A and B panels through that XCD's L2.
 //
 //   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned, any M: the
-//     same ingredients on 128 x 128 tiles with 4 wavefronts, for ragged shapes
-//     and for shapes with too few 256-tiles to fill the chip.
+//     same ingredients on 128 x 128 tiles with 4 wavefronts, for shapes with too
+//     few 256-tiles to fill the chip.
 //
 //   GemmF16General  everything else.  128 x 128 tile, 4 wavefronts, K step 32,
 //     global loads staged through registers with per-element predication
@@ -144,7 +146,10 @@ constexpr int kStageHalfs = kT * kTK;
 
 // WAVES wavefronts arranged 2 x (WAVES/2): each owns 128 rows and 512/WAVES columns of
 // the tile, i.e. 4 x TJ MFMA tiles with TJ = 16/WAVES.
-template <int WAVES>
+// RAGGED: M and N need not be multiples of 256 (N still a multiple of 8).  Rows past M and
+// 16-byte column chunks past N are clamped to the last valid ones when they are copied (they
+// feed only outputs that are never stored) and the epilogue skips what lies outside.
+template <int WAVES, bool RAGGED>
 __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args args)
 {
     constexpr int WN = WAVES / 2;          // wavefront columns
@@ -172,6 +177,9 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     const uint32_t waveN = wave % WN;
 
     const uint32_t K = args.K, N = args.N;
+    // rows and columns of this tile that exist
+    const uint32_t rowsLeft = RAGGED ? min(static_cast<uint32_t>(kT), args.M - tm * kT) : kT;
+    const uint32_t colsLeft = RAGGED ? min(static_cast<uint32_t>(kT), N - tn * kT) : kT;
     const _Float16* __restrict__ A =
         args.A + args.strideA * static_cast<int64_t>(unit) + static_cast<size_t>(tm) * kT * K;
     const _Float16* __restrict__ B =
@@ -197,14 +205,14 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         const uint32_t aRow0 = wave * (8 * ROUNDS) + (lane >> 3) + ((aL & 4) ? 128u : 0u);
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r)
-            aLane[r] = ((aRow0 + 8 * r) * K + (aL & 3) * 8) * 2 + kBias - r * 1024;
+            aLane[r] = (min(aRow0 + 8 * r, rowsLeft - 1) * K + (aL & 3) * 8) * 2 + kBias - r * 1024;
         const uint32_t phys16 = lane & 31;
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r)
         {
             const uint32_t k = wave * (2 * ROUNDS) + r * 2 + (lane >> 5);
             const uint32_t logical16 = (((phys16 >> 1) ^ (2 * (k & 3))) << 1) | (phys16 & 1);
-            bLane[r] = (k * N + logical16 * 8) * 2 + kBias - r * 1024;
+            bLane[r] = (k * N + min(logical16 * 8, colsLeft - 8)) * 2 + kBias - r * 1024;
         }
     }
     const uint32_t waveU = __builtin_amdgcn_readfirstlane(wave);
@@ -433,6 +441,12 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         float* outBlock = out + static_cast<size_t>(waveM * 128 + rdRow) * N +
                           waveN * (32 * TJ) + rdChunk * 4;
         const size_t rowStep = static_cast<size_t>(4) * N;  // between consecutive t
+        // what of this lane's part exists: rows rowFirst + 4*t of the tile, 4 columns at colFirst
+        const uint32_t rowFirst = waveM * 128 + rdRow;
+        const bool colExists = !RAGGED || waveN * (32 * TJ) + rdChunk * 4 < colsLeft;
+        auto exists = [&](int half, int t) {
+            return !RAGGED || (colExists && rowFirst + 4 * (half * 16 + t) < rowsLeft);
+        };
 
         auto stageHalf = [&](int half) {
 #pragma unroll
@@ -456,7 +470,11 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         auto loadOld = [&](int half, float4 (&old)[16]) {
 #pragma unroll
             for (int t = 0; t < 16; ++t)
-                old[t] = *reinterpret_cast<const float4*>(outBlock + (half * 16 + t) * rowStep);
+            {
+                old[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (exists(half, t))
+                    old[t] = *reinterpret_cast<const float4*>(outBlock + (half * 16 + t) * rowStep);
+            }
         };
         auto storeHalf = [&](int half, const float4 (&old)[16], auto accumulate) {
 #pragma unroll
@@ -472,7 +490,8 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
                     v.z += old[t].z;
                     v.w += old[t].w;
                 }
-                *reinterpret_cast<float4*>(outBlock + (half * 16 + t) * rowStep) = v;
+                if (exists(half, t))
+                    *reinterpret_cast<float4*>(outBlock + (half * 16 + t) * rowStep) = v;
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         };
@@ -994,8 +1013,15 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
     // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
     const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
-    const bool tile256 = aligned16 && (M % kT == 0) && (N % kT == 0) && (K % kTK == 0) &&
-                         static_cast<uint64_t>(M / kT) * (N / kT) * batch >= minTiles;
+    const uint64_t tiles256 =
+        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * batch;
+    const bool whole256 = (M % kT == 0) && (N % kT == 0);
+    // ragged shapes only while at least three quarters of the tiled area is real output
+    const bool fills256 =
+        static_cast<uint64_t>(M) * N * 4 >=
+        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * kT * kT * 3;
+    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) && N >= 8 &&
+                         tiles256 >= minTiles && fills256;
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -1006,7 +1032,10 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
 
     if (tile256)
     {
-        hipLaunchKernelGGL(GemmF16Tile256<8>, dim3(grid), dim3(512), 0, stream, args);
+        if (whole256)
+            hipLaunchKernelGGL((GemmF16Tile256<8, false>), dim3(grid), dim3(512), 0, stream, args);
+        else
+            hipLaunchKernelGGL((GemmF16Tile256<8, true>), dim3(grid), dim3(512), 0, stream, args);
     }
     else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
              static_cast<uint64_t>(M) * K < (1ull << 31) &&

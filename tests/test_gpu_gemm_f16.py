@@ -39,6 +39,23 @@ def test_tile256_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref - C)
 
 
+# the same kernel with M and N that are not multiples of 256 (rows and column chunks clamped
+# when copied, guarded epilogue): at least 192 tiles and three quarters of the tiled area real
+@pytest.mark.parametrize("shape", [(250, 248, 64, 192), (500, 504, 96, 48), (4000, 3592, 32, 1),
+                                   (3841, 4096, 64, 1)])
+def test_tile256_ragged_exact_on_integers(dev, shape):
+    M, N, K, batch = shape
+    h.announce("sph_gemm_f16f32 ragged tile256 integer exactness", shape)
+    A = synth.small_integers(21, (batch, M, K)).astype(np.float16)
+    B = synth.small_integers(22, (batch, K, N)).astype(np.float16)
+    C = synth.small_integers(23, (batch, M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K, batch=batch)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch)
+    assert np.array_equal(got, ref)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, flags=capi.SPH_GEMM_OVERWRITE)
+    assert np.array_equal(got, ref - C)
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 2), (31, 33, 17), (64, 64, 32), (100, 72, 40),
                                    (128, 128, 64), (130, 254, 96), (200, 8, 1000), (257, 255, 63)])
 def test_general_exact_on_integers(dev, shape):
