@@ -60,15 +60,36 @@ def parse():
     p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
                                       "csr"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
+    p.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                   help="untimed run-up before each timed leg that lets the clock reach its "
+                        "working frequency (0 = none)")
     p.add_argument("--zero-operands", action="store_true",
                    help="with --only gemm: all-zero A and B, to see how far the clock (and the "
                         "rate) depends on operand values; the line says data = zeros")
     return p.parse_args()
 
 
+# The shader clock idles at ~160 MHz and takes about half a second of load to reach its working
+# frequency (rocm-smi polled beside a run: 150 -> 2140 -> 2370 -> 2394 MHz at 0.2 s intervals).
+# Every timed leg is therefore preceded by SETTLE_MS of the same launches, untimed and not
+# counted as warm-up steps, so that the figure is the sustained one.
+SETTLE_MS = 600.0
+
+
+def settle(capi, launch):
+    if SETTLE_MS <= 0:
+        return
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(20):
+            launch()
+        capi.sync()
+
+
 def timed_launches(capi, launch, steps, warmup):
     """Average milliseconds per launch from HIP events on the launch stream, and the wall-clock
     milliseconds per step between two stream synchronisations."""
+    settle(capi, launch)
     for _ in range(warmup):
         launch()
     capi.sync()
@@ -440,6 +461,8 @@ def main():
               "collectives and every box here has one GPU)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    global SETTLE_MS
+    SETTLE_MS = args.settle_ms
     from sapphire_amd import capi, synth
     capi.call("sph_set_device", 0)
     info = capi.device_info(0)
@@ -457,7 +480,8 @@ def main():
         result.update({
             "metric": "GEMM TFLOP/s + % MFMA peak (4096^3 fp16->fp32); SpMM GB/s + % HBM peak",
             "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-            "warmup": args.warmup, "ms_per_step": wall_ms, "higher_is_better": True,
+            "warmup": args.warmup, "settle_ms": args.settle_ms, "ms_per_step": wall_ms,
+            "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "f16 in / f32 accumulate",
             "data": "zeros" if zeros else "synthetic",
             "config": {"workload": "configuration 3: out[4096,4096] f32 += A[4096,4096] f16 * "
