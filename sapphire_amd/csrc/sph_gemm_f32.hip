@@ -1,6 +1,7 @@
 // fp32 GEMM  out[u] += A[u] * B[u]  on the CDNA4 matrix cores.
 //
-// Storage, products and accumulation are all fp32 (v_mfma_f32_32x32x2_f32), so
+// Storage, products and accumulation are all fp32 (v_mfma_f32_32x32x2_f32, and
+// v_mfma_f32_16x16x4_f32 in the few-tile kernel), so
 // the only difference from the reference's scalar CPU loop
 // (Sources/Sapphire/compute/dense/naive/NaiveGemm.cpp:12-38) is the order in
 // which the K products are summed.
@@ -12,12 +13,12 @@
 //                        loads when possible, scalar predicated loads otherwise (e.g. the
 //                        reference's random test sizes,
 //                        Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:26-33);
-//   GemmF32SkinnyKernel  few output tiles and a long K: K split over the wavefronts of a
-//                        workgroup;
+//   GemmF32SkinnyKernel  few output tiles: 16 x 16 or 32 x 32 tiles with K split over the
+//                        wavefronts of a workgroup;
 //   GemvRowKernel        a single output row.
 // The first two share one decomposition: a workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile
-// of one M x N unit, BM = BN = 128 when that still gives a tile per compute unit and 64
-// otherwise, and they add the K products of an element in the same order, so which of them
+// of one M x N unit, BM = BN = 128 or 64 (whichever loads the busiest compute unit less),
+// and they add the K products of an element in the same order, so which of them
 // runs never changes a bit.  Either operand may be stored transposed (template flags), the
 // result may overwrite out or take a bias row and a ReLU in the epilogue, and units come from
 // (batch, stride) arithmetic -- stride 0 repeats an operand -- or from a table of element
@@ -27,6 +28,7 @@
 #include <algorithm>
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 #include <unordered_set>
 
 namespace
@@ -790,29 +792,41 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 }
 
 // ---------------------------------------------------------------------------
-// Few-tile shapes (small M x N, long K): 32 x 32 output tile per workgroup, K split across
-// its WAVES wavefronts (4, or 16 when even these tiles occupy less than a quarter of the chip
-// and K >= 512).
+// Few-tile shapes (small M x N, long K): a TILE x TILE output tile per workgroup (32, or 16
+// when even 32 x 32 tiles leave most of the chip idle or most of a tile outside the matrix),
+// K split across its WAVES wavefronts (4, or 16 when K >= 512).
 //
 // With few output tiles the tiled kernel above leaves most compute units idle and is bound by
 // the latency of one load -> LDS -> MFMA chain per K step.  Here every wavefront reads its
 // operands straight from global memory in MFMA layout (A: 16 bytes per lane along K, lines
-// reused from L1 over the next steps; B: one row segment per lane half), keeps several loads
-// in flight, and accumulates a private 32 x 32 partial over its share of K.  The
-// partials are then added in wavefront order through LDS, so the result does not depend on
-// timing.  The two k values of one MFMA come from lanes 0-31 and 32-63; which k each half
-// holds is free as long as A and B agree, and is chosen so that A is read with float4.
+// reused from L1 over the next steps; B: one row segment per group of TILE lanes), keeps
+// several loads in flight, and accumulates a private TILE x TILE partial over its share of K.
+// The partials are then added in wavefront order through LDS, so the result does not depend on
+// timing.  One MFMA (32x32x2 or 16x16x4) takes its 64 / TILE values of k from the 64 / TILE
+// groups of TILE lanes; which k each group holds is free as long as A and B agree, and is
+// chosen so that A is read with float4: group h holds k = (256 / TILE) * g + 4 * h + e.
+// A workgroup's matrix pipes are the bound once K is long (one tile's K runs on one compute
+// unit), which is why the 16-wide tile, a quarter of the work per workgroup on four times as
+// many compute units, is preferred whenever its tiles still fit the chip.
 // ---------------------------------------------------------------------------
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-template <bool VEC, bool TA, bool TB, int WAVES>
+template <int TILE, bool VEC, bool TA, bool TB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32Args args)
 {
-    __shared__ float partial[WAVES - 1][32 * 32];
+    static_assert(TILE == 32 || TILE == 16, "MFMA shapes 32x32x2 and 16x16x4");
+    constexpr uint32_t kLaneGroups = 64 / TILE;       // values of k per MFMA
+    constexpr uint32_t kGroupK = 4 * kLaneGroups;     // k per float4 round: 8 or 16
+    constexpr int kAcc = TILE * TILE / 64;            // accumulator registers: 16 or 4
+    constexpr int kQuads = kAcc / 4;
+    using Acc = typename std::conditional<TILE == 32, floatx16, floatx4>::type;
+
+    __shared__ float partial[WAVES - 1][TILE * TILE];
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t l32 = lane & 31;
-    const uint32_t khalf = lane >> 5;
+    const uint32_t lt = lane % TILE;   // row of A / column of B this lane feeds
+    const uint32_t kh = lane / TILE;   // which k of an MFMA
 
     uint32_t id = blockIdx.x;
     const uint32_t tn = id % args.tilesN;
@@ -837,11 +851,11 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         out = args.out + args.strideOut * static_cast<int64_t>(unit);
     }
     const uint32_t M = args.M, N = args.N, K = args.K;
-    const uint32_t row = tm * 32 + l32;
-    const uint32_t col = tn * 32 + l32;
+    const uint32_t row = tm * TILE + lt;
+    const uint32_t col = tn * TILE + lt;
 
-    // this wavefront's K range, in groups of 8 (one float4 of A per lane half)
-    const uint32_t groups = (K + 7) / 8;
+    // this wavefront's K range, in groups of kGroupK (one float4 of A per lane)
+    const uint32_t groups = (K + kGroupK - 1) / kGroupK;
     const uint32_t perWave = (groups + WAVES - 1) / WAVES;
     const uint32_t gBegin = min(wave * perWave, groups);
     const uint32_t gEnd = min(gBegin + perWave, groups);
@@ -849,16 +863,16 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
     const bool rowOk = row < M;
     const bool colOk = col < N;
 
-    floatx16 acc;
+    Acc acc;
 #pragma unroll
-    for (int v = 0; v < 16; ++v)
+    for (int v = 0; v < kAcc; ++v)
         acc[v] = 0.f;
 
-    // Lane half h holds k = 8*g + 4*h + e for e = 0..3.  An operand stored with K contiguous
-    // (A as given, B passed transposed) is read as one 16-byte segment of its row; one stored
-    // k-major (B as given, A passed transposed) as 4 elements `ld` apart.
+    // Lane group h holds k = kGroupK*g + 4*h + e for e = 0..3.  An operand stored with K
+    // contiguous (A as given, B passed transposed) is read as one 16-byte segment of its row;
+    // one stored k-major (B as given, A passed transposed) as 4 elements `ld` apart.
     auto loadAlongK = [&](const float* rowPtr, bool ok, uint32_t g) {
-        const uint32_t k = g * 8 + khalf * 4;
+        const uint32_t k = g * kGroupK + kh * 4;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok)
         {
@@ -878,7 +892,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         return v;
     };
     auto loadAcrossK = [&](const float* colPtr, size_t ld, bool ok, uint32_t g) {
-        const uint32_t k = g * 8 + khalf * 4;
+        const uint32_t k = g * kGroupK + kh * 4;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (ok)
         {
@@ -904,6 +918,14 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         else
             return loadAcrossK(bPtr, N, colOk, g);
     };
+    // operands swapped: the result block comes out indexed [column][row], which leaves 4
+    // consecutive columns of one row in a lane
+    auto multiply = [&](float b, float a) {
+        if constexpr (TILE == 32)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b, a, acc, 0, 0, 0);
+        else
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b, a, acc, 0, 0, 0);
+    };
 
     constexpr int kDepth = 4;  // groups in flight
     float4 fa[kDepth], fb[kDepth];
@@ -924,19 +946,21 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
             fa[d] = next < gEnd ? loadA(next) : make_float4(0.f, 0.f, 0.f, 0.f);
             fb[d] = next < gEnd ? loadB(next) : make_float4(0.f, 0.f, 0.f, 0.f);
             // groups past gEnd carry zeros and add nothing
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.x, a.x, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.y, a.y, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.z, a.z, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b.w, a.w, acc, 0, 0, 0);
+            multiply(b.x, a.x);
+            multiply(b.y, a.y);
+            multiply(b.z, a.z);
+            multiply(b.w, a.w);
         }
     }
 
-    // partial sums of wavefronts 1..3 go through LDS; wavefront 0 adds them in order
+    // lane l holds row l % TILE, columns 4*kLaneGroups*q + 4*(l / TILE) + 0..3 of the tile;
+    // partial sums of the other wavefronts go through LDS, wavefront 0 adds them in order
     if (wave != 0)
     {
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-            *reinterpret_cast<float4*>(&partial[wave - 1][l32 * 32 + 8 * q + 4 * khalf]) =
+        for (int q = 0; q < kQuads; ++q)
+            *reinterpret_cast<float4*>(
+                &partial[wave - 1][lt * TILE + 4 * kLaneGroups * q + 4 * kh]) =
                 make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
     }
     __syncthreads();
@@ -945,23 +969,22 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
 #pragma unroll
     for (int w = 0; w < WAVES - 1; ++w)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < kQuads; ++q)
         {
-            const float4 p =
-                *reinterpret_cast<const float4*>(&partial[w][l32 * 32 + 8 * q + 4 * khalf]);
+            const float4 p = *reinterpret_cast<const float4*>(
+                &partial[w][lt * TILE + 4 * kLaneGroups * q + 4 * kh]);
             acc[4 * q + 0] += p.x;
             acc[4 * q + 1] += p.y;
             acc[4 * q + 2] += p.z;
             acc[4 * q + 3] += p.w;
         }
-    // operands were swapped: lane l holds row l%32, columns 8q + 4*(l/32) + 0..3
     if (!rowOk)
         return;
     const bool wide = args.outVec != 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int q = 0; q < kQuads; ++q)
     {
-        const uint32_t c = tn * 32 + 8 * q + 4 * khalf;
+        const uint32_t c = tn * TILE + 4 * kLaneGroups * q + 4 * kh;
         if (c >= N)
             continue;
         float* p = out + static_cast<size_t>(row) * N + c;
@@ -1089,27 +1112,37 @@ struct EntryTable
 std::mutex gTableMutex;
 EntryTable gTables[16];
 
-template <bool TA, bool TB>
-void LaunchSkinny(const GemmF32Args& args, dim3 grid, bool vec, bool wide, hipStream_t stream)
+template <int TILE, bool TA, bool TB>
+void LaunchSkinnyTile(const GemmF32Args& args, dim3 grid, bool vec, bool wide, hipStream_t stream)
 {
-    // `wide`: 16 wavefronts per tile instead of 4 when even the 32 x 32 tiles leave most of
-    // the chip idle and K is long enough to give each wavefront a few steps
+    // `wide`: 16 wavefronts per tile instead of 4 when K is long enough to give each
+    // wavefront a few steps
     if (wide)
     {
         if (vec)
-            hipLaunchKernelGGL((GemmF32SkinnyKernel<true, TA, TB, 16>), grid, dim3(1024), 0,
+            hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, true, TA, TB, 16>), grid, dim3(1024), 0,
                                stream, args);
         else
-            hipLaunchKernelGGL((GemmF32SkinnyKernel<false, TA, TB, 16>), grid, dim3(1024), 0,
+            hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, false, TA, TB, 16>), grid, dim3(1024), 0,
                                stream, args);
         return;
     }
     if (vec)
-        hipLaunchKernelGGL((GemmF32SkinnyKernel<true, TA, TB, 4>), grid, dim3(256), 0, stream,
-                           args);
+        hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, true, TA, TB, 4>), grid, dim3(256), 0,
+                           stream, args);
     else
-        hipLaunchKernelGGL((GemmF32SkinnyKernel<false, TA, TB, 4>), grid, dim3(256), 0, stream,
-                           args);
+        hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, false, TA, TB, 4>), grid, dim3(256), 0,
+                           stream, args);
+}
+
+template <bool TA, bool TB>
+void LaunchSkinny(const GemmF32Args& args, dim3 grid, uint32_t tile, bool vec, bool wide,
+                  hipStream_t stream)
+{
+    if (tile == 16)
+        LaunchSkinnyTile<16, TA, TB>(args, grid, vec, wide, stream);
+    else
+        LaunchSkinnyTile<32, TA, TB>(args, grid, vec, wide, stream);
 }
 
 template <bool TA, bool TB>
@@ -1182,26 +1215,34 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
     if (tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) && args.K >= 64)
     {
-        args.tilesM = (args.M + 31) / 32;
-        args.tilesN = (args.N + 31) / 32;
-        const uint64_t blocks32 = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
-        const dim3 grid32(static_cast<uint32_t>(blocks32));
+        // 16 x 16 tiles while there are at most four per compute unit: a quarter of the
+        // matrix-core work per workgroup on four times as many compute units, and less of a
+        // tile outside a narrow matrix (measured: 256^3 6.5 -> 4.1 us, 1024 x 10 x 1024
+        // 13.3 -> 6.1 us, 256 x 256 x 4096 40 -> 16.5 us; 640^3 is better off on 32 x 32)
+        const uint64_t blocks16 =
+            static_cast<uint64_t>((args.M + 15) / 16) * ((args.N + 15) / 16) * units;
+        const uint32_t tile =
+            blocks16 <= static_cast<uint64_t>(sph::ComputeUnits()) * 4 ? 16u : 32u;
+        args.tilesM = (args.M + tile - 1) / tile;
+        args.tilesN = (args.N + tile - 1) / tile;
+        const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
+        const dim3 gridSkinny(static_cast<uint32_t>(blocks));
         // 16-byte loads are used only for operands stored with K contiguous
         bool kVec = allowVector && (args.K % 4 == 0);
         if (!transA)
             kVec = kVec && (reinterpret_cast<uintptr_t>(args.A) & 15u) == 0;
         if (transB)
             kVec = kVec && (reinterpret_cast<uintptr_t>(args.B) & 15u) == 0;
-        const bool wide = blocks32 * 4 <= static_cast<uint64_t>(sph::ComputeUnits()) &&
+        const bool wide = blocks * 4 <= static_cast<uint64_t>(sph::ComputeUnits()) * (tile == 16 ? 4 : 1) &&
                           args.K >= 512;
         if (transA && transB)
-            LaunchSkinny<true, true>(args, grid32, kVec, wide, stream);
+            LaunchSkinny<true, true>(args, gridSkinny, tile, kVec, wide, stream);
         else if (transA)
-            LaunchSkinny<true, false>(args, grid32, false, wide, stream);
+            LaunchSkinny<true, false>(args, gridSkinny, tile, false, wide, stream);
         else if (transB)
-            LaunchSkinny<false, true>(args, grid32, kVec, wide, stream);
+            LaunchSkinny<false, true>(args, gridSkinny, tile, kVec, wide, stream);
         else
-            LaunchSkinny<false, false>(args, grid32, kVec, wide, stream);
+            LaunchSkinny<false, false>(args, gridSkinny, tile, kVec, wide, stream);
         SPH_CHECK_LAUNCH();
         return SPH_OK;
     }
