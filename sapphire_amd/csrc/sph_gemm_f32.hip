@@ -793,8 +793,8 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 
 // ---------------------------------------------------------------------------
 // Few-tile shapes (small M x N, long K): a TILE x TILE output tile per workgroup (32, or 16
-// when even 32 x 32 tiles leave most of the chip idle or most of a tile outside the matrix),
-// K split across its WAVES wavefronts (4, or 16 when K >= 512).
+// when at most four of those per compute unit cover the output), K split across its WAVES
+// wavefronts (4, or 16 for 16-wide tiles that fit the chip once and K >= 512).
 //
 // With few output tiles the tiled kernel above leaves most compute units idle and is bound by
 // the latency of one load -> LDS -> MFMA chain per K step.  Here every wavefront reads its
@@ -1115,17 +1115,20 @@ EntryTable gTables[16];
 template <int TILE, bool TA, bool TB>
 void LaunchSkinnyTile(const GemmF32Args& args, dim3 grid, bool vec, bool wide, hipStream_t stream)
 {
-    // `wide`: 16 wavefronts per tile instead of 4 when K is long enough to give each
-    // wavefront a few steps
-    if (wide)
+    // `wide` (16 x 16 tiles only): 16 wavefronts per tile instead of 4 when K is long enough to
+    // give each wavefront a few steps
+    if constexpr (TILE == 16)
     {
-        if (vec)
-            hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, true, TA, TB, 16>), grid, dim3(1024), 0,
-                               stream, args);
-        else
-            hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, false, TA, TB, 16>), grid, dim3(1024), 0,
-                               stream, args);
-        return;
+        if (wide)
+        {
+            if (vec)
+                hipLaunchKernelGGL((GemmF32SkinnyKernel<16, true, TA, TB, 16>), grid, dim3(1024),
+                                   0, stream, args);
+            else
+                hipLaunchKernelGGL((GemmF32SkinnyKernel<16, false, TA, TB, 16>), grid, dim3(1024),
+                                   0, stream, args);
+            return;
+        }
     }
     if (vec)
         hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, true, TA, TB, 4>), grid, dim3(256), 0,
@@ -1233,7 +1236,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
             kVec = kVec && (reinterpret_cast<uintptr_t>(args.A) & 15u) == 0;
         if (transB)
             kVec = kVec && (reinterpret_cast<uintptr_t>(args.B) & 15u) == 0;
-        const bool wide = blocks * 4 <= static_cast<uint64_t>(sph::ComputeUnits()) * (tile == 16 ? 4 : 1) &&
+        const bool wide = tile == 16 && blocks <= static_cast<uint64_t>(sph::ComputeUnits()) &&
                           args.K >= 512;
         if (transA && transB)
             LaunchSkinny<true, true>(args, gridSkinny, tile, kVec, wide, stream);
@@ -1249,12 +1252,15 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
 
     // Tile edge: the matrix pipes bound these kernels, so a launch lasts as long as the
     // compute unit with the most tiles needs.  A 128-tile costs four 64-tiles and moves half
-    // the operand bytes per flop (measured 7 % faster at equal load); pick the edge with the
-    // smaller cost of the busiest compute unit.
+    // the operand bytes per flop (measured 7 % faster at equal load), but a compute unit with
+    // a single 128-tile has nothing to run beside that tile's first loads and epilogue, which
+    // four 64-tiles overlap (measured 6 % slower then); pick the edge with the smaller cost of
+    // the busiest compute unit.
     const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
     const uint64_t tiles128 =
         static_cast<uint64_t>((args.M + 127) / 128) * ((args.N + 127) / 128) * units;
-    const uint64_t cost128 = ((tiles128 + cus - 1) / cus) * 400;
+    const uint64_t rounds128 = (tiles128 + cus - 1) / cus;
+    const uint64_t cost128 = rounds128 * 400 + (rounds128 == 1 ? 32 : 0);
     const uint64_t cost64 = ((tiles64 + cus - 1) / cus) * 107;
     const bool big = cost128 <= cost64;
     const uint32_t bm = big ? 128 : 64;

@@ -19,11 +19,12 @@ TOL_F32 = 1e-4
 FLAG_SETS = [capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
              capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B]
 
-# shapes chosen to reach every kernel: 64- and 128-tiles, the K-split kernel (few tiles, long
-# K), 16-byte and scalar load paths, ragged edges
+# shapes chosen to reach every kernel: 64-tiles, 128-tiles (two per compute unit: 4096 x 2048),
+# the K-split kernel on 16 x 16 and 32 x 32 tiles (few tiles, long K), 16-byte and scalar load
+# paths, ragged edges
 SHAPES = [(1, 1, 1), (3, 5, 7), (64, 64, 64), (65, 33, 17), (128, 96, 40), (257, 130, 31),
-          (512, 384, 100), (2048, 2048, 64), (32, 32, 1024), (40, 24, 515), (8, 200, 4096),
-          (1000, 10, 1000)]
+          (512, 384, 100), (2048, 2048, 64), (4096, 2048, 32), (32, 32, 1024), (40, 24, 515),
+          (8, 200, 4096), (1000, 10, 1000), (256, 256, 96), (640, 600, 72)]
 
 
 def bits(x):
