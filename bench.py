@@ -360,6 +360,28 @@ def bench_spgemm(capi, synth, steps, warmup, n=8192, per_row=8.0):
     return event_ms, products, nnz.value, nbytes, a[0].size, b[0].size
 
 
+def bench_allocation(capi, nbytes=64 << 20, rounds=200):
+    """Host-side cost of taking and returning one device block of `nbytes`: the blocking pair
+    (hipMalloc / hipFree) against the stream-ordered pair the buffer pool uses on a miss."""
+    import ctypes
+    out = {}
+    for name, take, give in (("malloc_free", "sph_malloc", "sph_free"),
+                             ("malloc_async_free_async", "sph_malloc_async", "sph_free_async")):
+        ptr = ctypes.c_void_p()
+        for _ in range(5):
+            capi.call(take, ctypes.byref(ptr), nbytes)
+            capi.call(give, ptr)
+        capi.sync()
+        t0 = time.perf_counter()
+        for _ in range(rounds):
+            capi.call(take, ctypes.byref(ptr), nbytes)
+            capi.call(give, ptr)
+        capi.sync()
+        out[name + "_us"] = (time.perf_counter() - t0) * 1e6 / rounds
+    out["block_bytes"] = nbytes
+    return out
+
+
 def bench_elementwise(capi, steps, warmup, n=4096):
     """The one-pass kernels over n x n floats (64 MiB at n = 4096): algorithmic GB/s each."""
     count = n * n
@@ -610,6 +632,7 @@ def main():
             "note": "both passes compute every product (the count pass must see which sums "
                     "cancel); products counted once per pass in gproducts_per_s"}
         others["one_pass_kernels_4096x4096"] = bench_elementwise(capi, 50, 5)
+        others["device_block_64MiB"] = bench_allocation(capi)
         result["others"] = others
 
     if not args.no_cpu and args.only is None:
