@@ -38,12 +38,7 @@
 //     (16-byte loads when K, N and the bases allow), padded LDS rows.
 #include "sph_internal.h"
 
-#include <cstdlib>
 #include <type_traits>
-
-#ifndef SPH_ABLATE
-#define SPH_ABLATE 0
-#endif
 
 namespace
 {
@@ -64,9 +59,6 @@ struct GemmF16Args
     uint32_t totalTiles;  // tilesM * tilesN * batch
     int64_t strideOut, strideA, strideB;
     uint32_t overwrite;
-#if SPH_ABLATE & 16
-    long long* trace;
-#endif
 };
 
 // Transposing LDS read: within each group of 16 lanes, lane s supplies the
@@ -306,8 +298,6 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
                         halfx8 (&BFN)[TJ], int stageN, int ksN, uint32_t ktCopy, int stageCopy,
                         bool copyIsA) {
         auto copy = [&](auto round) {
-            if (SPH_ABLATE & 1)
-                return;
             if (copyIsA)
                 copyA(ktCopy, stageCopy, round);
             else
@@ -318,19 +308,15 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
             {
-                if (!(SPH_ABLATE & 2))
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(BF[j], AF[i], acc[i][j],
-                                                                       0, 0, 0);
+                acc[i][j] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_f16(BF[j], AF[i], acc[i][j], 0, 0, 0);
                 SPH_FENCE();
-                if (!(SPH_ABLATE & 4))
+                if (j == 0)
+                    AFN[i] = loadA(stageN, ksN, i);
+                if constexpr (i < TJ)
                 {
-                    if (j == 0)
-                        AFN[i] = loadA(stageN, ksN, i);
-                    if constexpr (i < TJ)
-                    {
-                        if (j == 1)
-                            BFN[i] = loadB(stageN, ksN, i);
-                    }
+                    if (j == 1)
+                        BFN[i] = loadB(stageN, ksN, i);
                 }
                 SPH_FENCE();
             }
@@ -395,7 +381,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         halfStep(af0, bf0, af1, bf1, cur, 1, kt + 3, (cur + 3) % kTStages, false);
         // step kt+1 has landed for every wavefront, and every wavefront is done reading
         // step kt, whose buffer now takes step kt+4
-        WaitVmem<(SPH_ABLATE & 1) ? 0 : 2 * COPIES_PER_STAGE>();
+        WaitVmem<2 * COPIES_PER_STAGE>();
         __syncthreads();
         // second half: multiply sub-step 1, fetch sub-step 0 of step kt+1, request A of kt+4
         halfStep(af1, bf1, af0, bf0, nxt, 0, kt + 4, cur, true);
@@ -426,8 +412,6 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     // instead, each wavefront turns its 128 x (32*TJ) block round through a private 16 KiB
     // piece of LDS, 64 rows at a time: after that a lane holds 4 consecutive columns and 16
     // consecutive lanes cover one row of the block.
-    if ((SPH_ABLATE & 8) && args.M != 1)
-        return;
     static_assert(TJ == 2, "the staged epilogue is written for 64-column wavefront blocks");
     WaitVmem<0>();      // clamped copies of the last steps still target LDS
     __syncthreads();    // ... and every wavefront is done with the stage buffers
@@ -998,12 +982,6 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.strideA = strideA;
     args.strideB = strideB;
     args.overwrite = (flags & SPH_GEMM_OVERWRITE) ? 1u : 0u;
-#if SPH_ABLATE & 16
-    {
-        const char* t = getenv("SPH_TRACE_PTR");
-        args.trace = t ? reinterpret_cast<long long*>(strtoull(t, nullptr, 0)) : nullptr;
-    }
-#endif
 
     const bool aligned16 =
         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
