@@ -1063,6 +1063,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void GemvRowKernel(const GemmF32Ar
     {
         const float* p = B + static_cast<size_t>(kBegin) * N + col;
         uint32_t k = kBegin;
+#pragma unroll 4
         for (; k + 4 <= kEnd; k += 4)
         {
             s0 = fmaf(a[k + 0], p[0], s0);
