@@ -55,6 +55,7 @@ struct GemmF16Args
     const _Float16* A;
     const _Float16* B;
     uint32_t M, N, K;
+    uint32_t lda;  // halves between consecutive rows of A (K unless a launch covers part of K)
     uint32_t tilesM, tilesN;
     uint32_t totalTiles;  // tilesM * tilesN * batch
     int64_t strideOut, strideA, strideB;
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     const uint32_t rowsLeft = RAGGED ? min(static_cast<uint32_t>(kT), args.M - tm * kT) : kT;
     const uint32_t colsLeft = RAGGED ? min(static_cast<uint32_t>(kT), N - tn * kT) : kT;
     const _Float16* __restrict__ A =
-        args.A + args.strideA * static_cast<int64_t>(unit) + static_cast<size_t>(tm) * kT * K;
+        args.A + args.strideA * static_cast<int64_t>(unit) + static_cast<size_t>(tm) * kT * args.lda;
     const _Float16* __restrict__ B =
         args.B + args.strideB * static_cast<int64_t>(unit) + static_cast<size_t>(tn) * kT;
     float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit) +
@@ -197,7 +198,8 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         const uint32_t aRow0 = wave * (8 * ROUNDS) + (lane >> 3) + ((aL & 4) ? 128u : 0u);
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r)
-            aLane[r] = (min(aRow0 + 8 * r, rowsLeft - 1) * K + (aL & 3) * 8) * 2 + kBias - r * 1024;
+            aLane[r] =
+                (min(aRow0 + 8 * r, rowsLeft - 1) * args.lda + (aL & 3) * 8) * 2 + kBias - r * 1024;
         const uint32_t phys16 = lane & 31;
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r)
@@ -551,7 +553,7 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
         const uint32_t x = j * 16 + (lane >> 2);
         const uint32_t c = (lane & 3) ^ ((lane >> 4) & 3);  // (x >> 2) & 3 == (lane >> 4) & 3
         const uint32_t gx = min(rowBase + x, M - 1);
-        aLane[i] = (gx * K + c * 8) * 2u;
+        aLane[i] = (gx * args.lda + c * 8) * 2u;
         aDst[i] = j * 1024;
         // B: 4 k-rows per copy; lane -> k = j*4 + lane/16, physical 16-byte chunk lane%16
         const uint32_t k = j * 4 + (lane >> 4);
@@ -776,7 +778,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
             halfx8 v = { 0, 0, 0, 0, 0, 0, 0, 0 };
             if (gr < M)
             {
-                const _Float16* p = A + static_cast<size_t>(gr) * K + gk;
+                const _Float16* p = A + static_cast<size_t>(gr) * args.lda + gk;
                 if (VEC)
                 {
                     if (gk < K)
@@ -934,6 +936,57 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
             }
     }
 }
+
+// Picks the kernel for one launch over args.K columns of A (rows args.lda apart).
+int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, hipStream_t stream)
+{
+    const uint32_t M = args.M, N = args.N, K = args.K;
+    // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
+    // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
+    const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
+    const uint64_t tiles256 =
+        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * batch;
+    const bool whole256 = (M % kT == 0) && (N % kT == 0);
+    // ragged shapes only while at least three quarters of the tiled area is real output
+    const bool fills256 =
+        static_cast<uint64_t>(M) * N * 4 >=
+        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * kT * kT * 3;
+    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) && N >= 8 &&
+                         tiles256 >= minTiles && fills256;
+    const uint32_t edge = tile256 ? kT : kG;
+    args.tilesM = (M + edge - 1) / edge;
+    args.tilesN = (N + edge - 1) / edge;
+    const uint64_t total = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
+    SPH_REQUIRE(total < (1ull << 31) - 8, "too many tiles for one launch");
+    args.totalTiles = static_cast<uint32_t>(total);
+    const uint32_t grid = ((args.totalTiles + 7) / 8) * 8;
+
+    if (tile256)
+    {
+        if (whole256)
+            hipLaunchKernelGGL((GemmF16Tile256<8, false>), dim3(grid), dim3(512), 0, stream, args);
+        else
+            hipLaunchKernelGGL((GemmF16Tile256<8, true>), dim3(grid), dim3(512), 0, stream, args);
+    }
+    else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
+             static_cast<uint64_t>(M) * args.lda < (1ull << 31) &&
+             static_cast<uint64_t>(kTK) * N < (1ull << 31))
+    {
+        // whole K steps and 16-byte chunks everywhere: straight-to-LDS 128-tile kernel
+        hipLaunchKernelGGL(GemmF16Dma128, dim3(grid), dim3(256), 0, stream, args);
+    }
+    else
+    {
+        const bool vec = aligned16 && (K % 8 == 0) && (args.lda % 8 == 0) && (N % 8 == 0);
+        if (vec)
+            hipLaunchKernelGGL(GemmF16General<true>, dim3(grid), dim3(kGThreads), 0, stream, args);
+        else
+            hipLaunchKernelGGL(GemmF16General<false>, dim3(grid), dim3(kGThreads), 0, stream,
+                               args);
+    }
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
 }  // namespace
 
 extern "C" {
@@ -971,6 +1024,11 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     }
     SPH_REQUIRE(A != nullptr && B != nullptr, "null pointer");
 
+    const bool aligned16 =
+        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
+          reinterpret_cast<uintptr_t>(out)) & 15u) == 0 &&
+        (strideA % 8 == 0) && (strideB % 8 == 0) && (strideOut % 4 == 0);
+
     GemmF16Args args{};
     args.out = out;
     args.A = reinterpret_cast<const _Float16*>(A);
@@ -978,61 +1036,29 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.M = M;
     args.N = N;
     args.K = K;
+    args.lda = K;
     args.strideOut = strideOut;
     args.strideA = strideA;
     args.strideB = strideB;
     args.overwrite = (flags & SPH_GEMM_OVERWRITE) ? 1u : 0u;
 
-    const bool aligned16 =
-        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
-          reinterpret_cast<uintptr_t>(out)) & 15u) == 0 &&
-        (strideA % 8 == 0) && (strideB % 8 == 0) && (strideOut % 4 == 0);
-
-    // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
-    // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
-    const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
-    const uint64_t tiles256 =
-        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * batch;
-    const bool whole256 = (M % kT == 0) && (N % kT == 0);
-    // ragged shapes only while at least three quarters of the tiled area is real output
-    const bool fills256 =
-        static_cast<uint64_t>(M) * N * 4 >=
-        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * kT * kT * 3;
-    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) && N >= 8 &&
-                         tiles256 >= minTiles && fills256;
-    const uint32_t edge = tile256 ? kT : kG;
-    args.tilesM = (M + edge - 1) / edge;
-    args.tilesN = (N + edge - 1) / edge;
-    const uint64_t total = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
-    SPH_REQUIRE(total < (1ull << 31) - 8, "too many tiles for one launch");
-    args.totalTiles = static_cast<uint32_t>(total);
-    const uint32_t grid = ((args.totalTiles + 7) / 8) * 8;
-
-    if (tile256)
+    // K = 32 q + r with r a multiple of 8: the straight-to-LDS kernels take whole K steps only,
+    // so they multiply the first 32 q columns of A and the general kernel adds the last r
+    // (measured 4096 x 4096 x 4080: 229 us on the general kernel alone, 175 us this way)
+    const uint32_t tail = K % kTK;
+    if (tail != 0 && K % 8 == 0 && K >= 2 * kTK && aligned16 && N % 8 == 0)
     {
-        if (whole256)
-            hipLaunchKernelGGL((GemmF16Tile256<8, false>), dim3(grid), dim3(512), 0, stream, args);
-        else
-            hipLaunchKernelGGL((GemmF16Tile256<8, true>), dim3(grid), dim3(512), 0, stream, args);
+        GemmF16Args head = args;
+        head.K = K - tail;
+        const int rc = LaunchF16(head, batch, aligned16, stream);
+        if (rc != SPH_OK)
+            return rc;
+        args.A += head.K;
+        args.B += static_cast<size_t>(head.K) * N;
+        args.K = tail;
+        args.overwrite = 0;
     }
-    else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
-             static_cast<uint64_t>(M) * K < (1ull << 31) &&
-             static_cast<uint64_t>(kTK) * N < (1ull << 31))
-    {
-        // whole K steps and 16-byte chunks everywhere: straight-to-LDS 128-tile kernel
-        hipLaunchKernelGGL(GemmF16Dma128, dim3(grid), dim3(256), 0, stream, args);
-    }
-    else
-    {
-        const bool vec = aligned16 && (K % 8 == 0) && (N % 8 == 0);
-        if (vec)
-            hipLaunchKernelGGL(GemmF16General<true>, dim3(grid), dim3(kGThreads), 0, stream, args);
-        else
-            hipLaunchKernelGGL(GemmF16General<false>, dim3(grid), dim3(kGThreads), 0, stream,
-                               args);
-    }
-    SPH_CHECK_LAUNCH();
-    return SPH_OK;
+    return LaunchF16(args, batch, aligned16, stream);
 }
 
 }  // extern "C"

@@ -56,6 +56,23 @@ def test_tile256_ragged_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref - C)
 
 
+# K = 32 q + r, r in {8, 16, 24}: the straight-to-LDS kernels multiply the first 32 q columns and
+# the general kernel adds the rest (256-tile, ragged 256-tile and 128-tile cases)
+@pytest.mark.parametrize("shape", [(256, 256, 72, 192), (250, 248, 80, 192), (4096, 3072, 88, 1),
+                                   (300, 520, 168, 1), (128, 128, 72, 3), (1000, 1000, 1000, 1)])
+def test_k_tail_split_exact_on_integers(dev, shape):
+    M, N, K, batch = shape
+    h.announce("sph_gemm_f16f32 K tail integer exactness", shape)
+    A = synth.small_integers(31, (batch, M, K), span=3).astype(np.float16)
+    B = synth.small_integers(32, (batch, K, N), span=3).astype(np.float16)
+    C = synth.small_integers(33, (batch, M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K, batch=batch)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch)
+    assert np.array_equal(got, ref)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, flags=capi.SPH_GEMM_OVERWRITE)
+    assert np.array_equal(got, ref - C)
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 2), (31, 33, 17), (64, 64, 32), (100, 72, 40),
                                    (128, 128, 64), (130, 254, 96), (200, 8, 1000), (257, 255, 63)])
 def test_general_exact_on_integers(dev, shape):
