@@ -34,8 +34,11 @@
 //     few 256-tiles to fill the chip.
 //
 //   GemmF16General  everything else.  128 x 128 tile, 4 wavefronts, K step 32,
-//     global loads staged through registers with per-element predication
-//     (16-byte loads when K, N and the bases allow), padded LDS rows.
+//     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
+//     widest that K, N, the strides and the bases allow), padded LDS rows.
+//
+// K = 32 q + r with r in {8, 16, 24} goes to the first two kernels for the first 32 q
+// columns of A and to the general kernel for the rest (two launches).
 #include "sph_internal.h"
 
 #include <type_traits>
@@ -44,6 +47,7 @@ namespace
 {
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* LdsPtr;
 typedef short shortx4 __attribute__((ext_vector_type(4)));
@@ -60,6 +64,7 @@ struct GemmF16Args
     uint32_t totalTiles;  // tilesM * tilesN * batch
     int64_t strideOut, strideA, strideB;
     uint32_t overwrite;
+    uint32_t outVec;  // general kernel: out may be accessed 16 bytes at a time
 };
 
 // Transposing LDS read: within each group of 16 lanes, lane s supplies the
@@ -743,7 +748,9 @@ constexpr int kGThreads = 256;
 constexpr int kGLda = kGK + 8;   // halves per A row in LDS (80 B)
 constexpr int kGLdb = kG + 32;   // halves per B row in LDS (320 B)
 
-template <bool VEC>
+// VEC: halves per global load (8, 4, 2 or 1), the largest power of two that divides K, the row
+// stride of A, N and the alignment of the bases.
+template <int VEC>
 __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args args)
 {
     __shared__ __attribute__((aligned(16))) _Float16 As[2][kG * kGLda];
@@ -768,6 +775,49 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
 
     halfx8 stageA[2], stageB[2];
 
+    // 8 consecutive halves starting at p, of which those with index + first < limit exist; read
+    // in pieces of VEC halves (the row stride and the base are multiples of VEC halves, so a
+    // piece is aligned and lies wholly inside or outside the row)
+    auto load8 = [&](const _Float16* p, uint32_t first, uint32_t limit) {
+        halfx8 v = { 0, 0, 0, 0, 0, 0, 0, 0 };
+        if constexpr (VEC == 8)
+        {
+            if (first < limit)
+                v = *reinterpret_cast<const halfx8*>(p);
+        }
+        else if constexpr (VEC == 4)
+        {
+#pragma unroll
+            for (int e = 0; e < 8; e += 4)
+                if (first + e < limit)
+                {
+                    const halfx4 w = *reinterpret_cast<const halfx4*>(p + e);
+                    v[e] = w[0];
+                    v[e + 1] = w[1];
+                    v[e + 2] = w[2];
+                    v[e + 3] = w[3];
+                }
+        }
+        else if constexpr (VEC == 2)
+        {
+#pragma unroll
+            for (int e = 0; e < 8; e += 2)
+                if (first + e < limit)
+                {
+                    const halfx2 w = *reinterpret_cast<const halfx2*>(p + e);
+                    v[e] = w[0];
+                    v[e + 1] = w[1];
+                }
+        }
+        else
+        {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (first + e < limit)
+                    v[e] = p[e];
+        }
+        return v;
+    };
     auto fetch = [&](uint32_t k0) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -777,21 +827,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
             const uint32_t gk = k0 + (q % 4) * 8;
             halfx8 v = { 0, 0, 0, 0, 0, 0, 0, 0 };
             if (gr < M)
-            {
-                const _Float16* p = A + static_cast<size_t>(gr) * args.lda + gk;
-                if (VEC)
-                {
-                    if (gk < K)
-                        v = *reinterpret_cast<const halfx8*>(p);
-                }
-                else
-                {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (gk + e < K)
-                            v[e] = p[e];
-                }
-            }
+                v = load8(A + static_cast<size_t>(gr) * args.lda + gk, gk, K);
             stageA[i] = v;
         }
 #pragma unroll
@@ -802,21 +838,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
             const uint32_t gc = colBase + (q % 16) * 8;
             halfx8 v = { 0, 0, 0, 0, 0, 0, 0, 0 };
             if (gk < K)
-            {
-                const _Float16* p = B + static_cast<size_t>(gk) * N + gc;
-                if (VEC)
-                {
-                    if (gc < N)
-                        v = *reinterpret_cast<const halfx8*>(p);
-                }
-                else
-                {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (gc + e < N)
-                            v[e] = p[e];
-                }
-            }
+                v = load8(B + static_cast<size_t>(gk) * N + gc, gc, N);
             stageB[i] = v;
         }
     };
@@ -907,7 +929,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
             {
                 const uint32_t c = colBase + waveN * 64 + j * 32 + 8 * q + 4 * khalf;
                 float* p = out + static_cast<size_t>(r) * N + c;
-                if (VEC && (N % 4 == 0))
+                if (args.outVec)
                 {
                     if (c < N)
                     {
@@ -977,12 +999,26 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, hipStream_t stre
     }
     else
     {
-        const bool vec = aligned16 && (K % 8 == 0) && (args.lda % 8 == 0) && (N % 8 == 0);
-        if (vec)
-            hipLaunchKernelGGL(GemmF16General<true>, dim3(grid), dim3(kGThreads), 0, stream, args);
+        // widest load every row start and every base allows (in halves)
+        const uint64_t mix = static_cast<uint64_t>(K) | args.lda | N |
+                             static_cast<uint64_t>(args.strideA) |
+                             static_cast<uint64_t>(args.strideB) |
+                             (reinterpret_cast<uintptr_t>(args.A) / 2) |
+                             (reinterpret_cast<uintptr_t>(args.B) / 2) | 8u;
+        const uint32_t vec = static_cast<uint32_t>(mix & (~mix + 1));  // lowest set bit: 1, 2, 4, 8
+        args.outVec = ((reinterpret_cast<uintptr_t>(args.out) & 15u) == 0 && args.strideOut % 4 == 0 &&
+                       N % 4 == 0)
+                          ? 1u
+                          : 0u;
+        const dim3 g(grid), b(kGThreads);
+        if (vec == 8)
+            hipLaunchKernelGGL(GemmF16General<8>, g, b, 0, stream, args);
+        else if (vec == 4)
+            hipLaunchKernelGGL(GemmF16General<4>, g, b, 0, stream, args);
+        else if (vec == 2)
+            hipLaunchKernelGGL(GemmF16General<2>, g, b, 0, stream, args);
         else
-            hipLaunchKernelGGL(GemmF16General<false>, dim3(grid), dim3(kGThreads), 0, stream,
-                               args);
+            hipLaunchKernelGGL(GemmF16General<1>, g, b, 0, stream, args);
     }
     SPH_CHECK_LAUNCH();
     return SPH_OK;

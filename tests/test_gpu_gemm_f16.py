@@ -74,7 +74,8 @@ def test_k_tail_split_exact_on_integers(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 2), (31, 33, 17), (64, 64, 32), (100, 72, 40),
-                                   (128, 128, 64), (130, 254, 96), (200, 8, 1000), (257, 255, 63)])
+                                   (128, 128, 64), (130, 254, 96), (200, 8, 1000), (257, 255, 63),
+                                   (100, 68, 44), (300, 132, 100), (64, 70, 34)])
 def test_general_exact_on_integers(dev, shape):
     M, N, K = shape
     h.announce("sph_gemm_f16f32 general integer exactness", shape)
