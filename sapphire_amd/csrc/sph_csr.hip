@@ -11,7 +11,7 @@
 // All of this is one- or two-pass integer/byte work bound by HBM:
 //   row offsets   read the dense matrix once, popcount per row, exclusive scan of M+1 counts
 //   fill          read it again, ballot + popcount give every kept entry its slot
-//   to dense      zero the rows, then scatter the entries
+//   to dense      one wavefront per row clears it and writes its entries over the zeros
 // A row is handled by a group of LPR lanes (a power of two, 4..64, chosen from the row
 // length) so that narrow matrices do not idle most of a wavefront; each lane takes 4
 // consecutive columns (16 bytes) per step.
@@ -250,38 +250,44 @@ __global__ __launch_bounds__(kThreads) void CsrFillKernel(float* __restrict__ V,
     }
 }
 
-// dense[row][COL[p]] = V[p]; 16 lanes walk one row's entries
-__global__ __launch_bounds__(kThreads) void CsrScatterKernel(float* __restrict__ dense,
-                                                             uint32_t ld, uint32_t M, uint32_t N,
-                                                             const float* __restrict__ V,
-                                                             const uint32_t* __restrict__ COL,
-                                                             const uint32_t* __restrict__ ROW)
+// One wavefront per row: the row is cleared, then its entries are written over the zeros, in
+// one pass over the dense matrix.  VEC: rows start on 16-byte boundaries and N % 4 == 0.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void CsrToDenseRowKernel(float* __restrict__ dense,
+                                                                uint32_t ld, uint32_t M,
+                                                                uint32_t N,
+                                                                const float* __restrict__ V,
+                                                                const uint32_t* __restrict__ COL,
+                                                                const uint32_t* __restrict__ ROW)
 {
-    constexpr uint32_t kLanes = 16;
-    constexpr uint32_t kGroups = kThreads / kLanes;
-    const uint32_t lane = threadIdx.x % kLanes;
-    const uint32_t group = threadIdx.x / kLanes;
-    for (uint32_t row = blockIdx.x * kGroups + group; row < M; row += gridDim.x * kGroups)
+    constexpr uint32_t kWaves = kThreads / 64;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    for (uint32_t row = blockIdx.x * kWaves + wave; row < M; row += gridDim.x * kWaves)
     {
-        const uint32_t end = ROW[row + 1];
         float* out = dense + static_cast<size_t>(row) * ld;
-        for (uint32_t p = ROW[row] + lane; p < end; p += kLanes)
+        const uint32_t begin = ROW[row];
+        const uint32_t end = ROW[row + 1];
+        if (VEC)
+        {
+            for (uint32_t c = lane * 4; c < N; c += 256)
+                *reinterpret_cast<float4*>(out + c) = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        else
+        {
+            for (uint32_t c = lane; c < N; c += 64)
+                out[c] = 0.f;
+        }
+        // An entry is written by another lane than the one that cleared its place: the zeros
+        // have to be acknowledged by the cache before the entries follow them.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        for (uint32_t p = begin + lane; p < end; p += 64)
         {
             const uint32_t c = COL[p];
             if (c < N)  // an entry outside the matrix is dropped, never written
                 out[c] = V[p];
         }
     }
-}
-
-// rows x cols block of a pitched matrix set to `value`
-__global__ __launch_bounds__(kThreads) void FillPitchedKernel(float* __restrict__ dst,
-                                                              float value, uint32_t rows,
-                                                              uint32_t cols, uint32_t ld)
-{
-    for (uint32_t r = blockIdx.y; r < rows; r += gridDim.y)
-        for (uint32_t c = blockIdx.x * kThreads + threadIdx.x; c < cols; c += gridDim.x * kThreads)
-            dst[static_cast<size_t>(r) * ld + c] = value;
 }
 
 int LanesPerRow(uint32_t N)
@@ -435,22 +441,15 @@ int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V, const uint32
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
-    if (ld == N)
-    {
-        const int rc = sph_fill_f32(dense, 0.0f, static_cast<size_t>(M) * N);
-        if (rc != SPH_OK)
-            return rc;
-    }
+    const bool vec = (N % 4 == 0) && (ld % 4 == 0) &&
+                     (reinterpret_cast<uintptr_t>(dense) & 15u) == 0;
+    const uint32_t grid = RowGrid(M, 64);
+    if (vec)
+        hipLaunchKernelGGL(CsrToDenseRowKernel<true>, dim3(grid), dim3(kThreads), 0, stream, dense,
+                           ld, M, N, V, COL, ROW);
     else
-    {
-        const uint32_t gx = std::min<uint32_t>((N + kThreads - 1) / kThreads, 64u);
-        const uint32_t gy = std::min<uint32_t>(M, 65535u);
-        hipLaunchKernelGGL(FillPitchedKernel, dim3(gx, gy), dim3(kThreads), 0, stream, dense, 0.0f,
-                           M, N, ld);
-        SPH_CHECK_LAUNCH();
-    }
-    hipLaunchKernelGGL(CsrScatterKernel, dim3(RowGrid(M, 16)), dim3(kThreads), 0, stream, dense, ld,
-                       M, N, V, COL, ROW);
+        hipLaunchKernelGGL(CsrToDenseRowKernel<false>, dim3(grid), dim3(kThreads), 0, stream, dense,
+                           ld, M, N, V, COL, ROW);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
