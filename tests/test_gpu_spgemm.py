@@ -102,3 +102,25 @@ def test_host_layer_sparse_sparse_gemm(dev, case):
     wV, wC, wR = po.spgemm_csr(po.csr_from_dense(dA), po.csr_from_dense(dB), M, K, N)
     V, COL, ROW = hl.sparse_sparse_gemm(dA, dB, capacity=wV.size + 16)
     assert np.array_equal(ROW, wR) and np.array_equal(COL, wC) and np.array_equal(bits(V), bits(wV))
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_shapes_and_densities(dev, block):
+    """Widths on both sides of the bit-map word, run and strip boundaries (32, 64, 4096, several
+    strips), short and long rows, empty results."""
+    rng = np.random.default_rng(4200 + block)
+    widths = [1, 7, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 500, 2047, 2048, 2049, 4095, 4096,
+              4097, 5000, 8191, 8193, 12289]
+    for it in range(10):
+        M, K = int(rng.integers(1, 300)), int(rng.integers(1, 300))
+        N = int(rng.choice(widths))
+        da = float(rng.choice([0.01, 0.05, 0.2, 0.6]))
+        db = float(rng.choice([0.002, 0.01, 0.05] if N > 3000 else [0.002, 0.01, 0.05, 0.3]))
+        h.announce("sph_spgemm_* random M K N dA dB =", (M, K, N, da, db))
+        dA = sparse_dense(100000 + 100 * block + it, (M, K), da)
+        dB = sparse_dense(200000 + 100 * block + it, (K, N), db)
+        A, B = po.csr_from_dense(dA), po.csr_from_dense(dB)
+        wV, wC, wR = po.spgemm_csr(A, B, M, K, N)
+        V, COL, ROW = gpu_spgemm(A, B, M, K, N)
+        assert np.array_equal(ROW, wR) and np.array_equal(COL, wC)
+        assert np.array_equal(bits(V), bits(wV))
