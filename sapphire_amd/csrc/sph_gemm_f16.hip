@@ -750,7 +750,10 @@ constexpr int kGLdb = kG + 32;   // halves per B row in LDS (320 B)
 
 // VEC: halves per global load (8, 4, 2 or 1), the largest power of two that divides K, the row
 // stride of A, N and the alignment of the bases.
-template <int VEC>
+// TA: A is stored K x M; TB: B is stored N x K.  A transposed operand is read along its
+// contiguous dimension like the other one and turned round on its way into LDS (8 two-byte
+// stores per chunk instead of one 16-byte store), so the MFMA side does not change.
+template <int VEC, bool TA, bool TB>
 __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args args)
 {
     __shared__ __attribute__((aligned(16))) _Float16 As[2][kG * kGLda];
@@ -823,22 +826,44 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
         for (int i = 0; i < 2; ++i)
         {
             const uint32_t q = tid + i * kGThreads;
-            const uint32_t gr = rowBase + q / 4;
-            const uint32_t gk = k0 + (q % 4) * 8;
             halfx8 v = { 0, 0, 0, 0, 0, 0, 0, 0 };
-            if (gr < M)
-                v = load8(A + static_cast<size_t>(gr) * args.lda + gk, gk, K);
+            if constexpr (TA)
+            {
+                // 8 consecutive rows m of one k
+                const uint32_t gk = k0 + q / 16;
+                const uint32_t gr = rowBase + (q % 16) * 8;
+                if (gk < K)
+                    v = load8(A + static_cast<size_t>(gk) * M + gr, gr, M);
+            }
+            else
+            {
+                const uint32_t gr = rowBase + q / 4;
+                const uint32_t gk = k0 + (q % 4) * 8;
+                if (gr < M)
+                    v = load8(A + static_cast<size_t>(gr) * args.lda + gk, gk, K);
+            }
             stageA[i] = v;
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i)
         {
             const uint32_t q = tid + i * kGThreads;
-            const uint32_t gk = k0 + q / 16;
-            const uint32_t gc = colBase + (q % 16) * 8;
             halfx8 v = { 0, 0, 0, 0, 0, 0, 0, 0 };
-            if (gk < K)
-                v = load8(B + static_cast<size_t>(gk) * N + gc, gc, N);
+            if constexpr (TB)
+            {
+                // 8 consecutive k of one column n
+                const uint32_t gc = colBase + q / 4;
+                const uint32_t gk = k0 + (q % 4) * 8;
+                if (gc < N)
+                    v = load8(B + static_cast<size_t>(gc) * K + gk, gk, K);
+            }
+            else
+            {
+                const uint32_t gk = k0 + q / 16;
+                const uint32_t gc = colBase + (q % 16) * 8;
+                if (gk < K)
+                    v = load8(B + static_cast<size_t>(gk) * N + gc, gc, N);
+            }
             stageB[i] = v;
         }
     };
@@ -848,13 +873,27 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
         for (int i = 0; i < 2; ++i)
         {
             const uint32_t q = tid + i * kGThreads;
-            *reinterpret_cast<halfx8*>(&As[buf][(q / 4) * kGLda + (q % 4) * 8]) = stageA[i];
+            if constexpr (TA)
+            {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    As[buf][((q % 16) * 8 + e) * kGLda + q / 16] = stageA[i][e];
+            }
+            else
+                *reinterpret_cast<halfx8*>(&As[buf][(q / 4) * kGLda + (q % 4) * 8]) = stageA[i];
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i)
         {
             const uint32_t q = tid + i * kGThreads;
-            *reinterpret_cast<halfx8*>(&Bs[buf][(q / 16) * kGLdb + (q % 16) * 8]) = stageB[i];
+            if constexpr (TB)
+            {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    Bs[buf][((q % 4) * 8 + e) * kGLdb + q / 4] = stageB[i][e];
+            }
+            else
+                *reinterpret_cast<halfx8*>(&Bs[buf][(q / 16) * kGLdb + (q % 16) * 8]) = stageB[i];
         }
     };
 
@@ -960,9 +999,11 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
 }
 
 // Picks the kernel for one launch over args.K columns of A (rows args.lda apart).
-int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, hipStream_t stream)
+int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, bool transB,
+              hipStream_t stream)
 {
     const uint32_t M = args.M, N = args.N, K = args.K;
+    const bool plain = !transA && !transB;  // only the general kernel reads transposed operands
     // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
     // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
     const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
@@ -973,8 +1014,8 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, hipStream_t stre
     const bool fills256 =
         static_cast<uint64_t>(M) * N * 4 >=
         static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * kT * kT * 3;
-    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) && N >= 8 &&
-                         tiles256 >= minTiles && fills256;
+    const bool tile256 = plain && aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) &&
+                         N >= 8 && tiles256 >= minTiles && fills256;
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -990,7 +1031,7 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, hipStream_t stre
         else
             hipLaunchKernelGGL((GemmF16Tile256<8, true>), dim3(grid), dim3(512), 0, stream, args);
     }
-    else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
+    else if (plain && aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
              static_cast<uint64_t>(M) * args.lda < (1ull << 31) &&
              static_cast<uint64_t>(kTK) * N < (1ull << 31))
     {
@@ -999,8 +1040,10 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, hipStream_t stre
     }
     else
     {
-        // widest load every row start and every base allows (in halves)
-        const uint64_t mix = static_cast<uint64_t>(K) | args.lda | N |
+        // widest load every row start, every row length and every base allows (in halves);
+        // an operand is read along its contiguous dimension: K (A), N (B), M (A stored K x M)
+        // or K (B stored N x K)
+        const uint64_t mix = static_cast<uint64_t>(K) | (transA ? M : args.lda) | (transB ? K : N) |
                              static_cast<uint64_t>(args.strideA) |
                              static_cast<uint64_t>(args.strideB) |
                              (reinterpret_cast<uintptr_t>(args.A) / 2) |
@@ -1011,14 +1054,36 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, hipStream_t stre
                           ? 1u
                           : 0u;
         const dim3 g(grid), b(kGThreads);
-        if (vec == 8)
-            hipLaunchKernelGGL(GemmF16General<8>, g, b, 0, stream, args);
-        else if (vec == 4)
-            hipLaunchKernelGGL(GemmF16General<4>, g, b, 0, stream, args);
-        else if (vec == 2)
-            hipLaunchKernelGGL(GemmF16General<2>, g, b, 0, stream, args);
+        if (plain)
+        {
+            if (vec == 8)
+                hipLaunchKernelGGL((GemmF16General<8, false, false>), g, b, 0, stream, args);
+            else if (vec == 4)
+                hipLaunchKernelGGL((GemmF16General<4, false, false>), g, b, 0, stream, args);
+            else if (vec == 2)
+                hipLaunchKernelGGL((GemmF16General<2, false, false>), g, b, 0, stream, args);
+            else
+                hipLaunchKernelGGL((GemmF16General<1, false, false>), g, b, 0, stream, args);
+        }
+        else if (vec == 8)
+        {
+            // transposed operands: 16-byte loads or single halves
+            if (transA && transB)
+                hipLaunchKernelGGL((GemmF16General<8, true, true>), g, b, 0, stream, args);
+            else if (transA)
+                hipLaunchKernelGGL((GemmF16General<8, true, false>), g, b, 0, stream, args);
+            else
+                hipLaunchKernelGGL((GemmF16General<8, false, true>), g, b, 0, stream, args);
+        }
         else
-            hipLaunchKernelGGL(GemmF16General<1>, g, b, 0, stream, args);
+        {
+            if (transA && transB)
+                hipLaunchKernelGGL((GemmF16General<1, true, true>), g, b, 0, stream, args);
+            else if (transA)
+                hipLaunchKernelGGL((GemmF16General<1, true, false>), g, b, 0, stream, args);
+            else
+                hipLaunchKernelGGL((GemmF16General<1, false, true>), g, b, 0, stream, args);
+        }
     }
     SPH_CHECK_LAUNCH();
     return SPH_OK;
@@ -1032,10 +1097,10 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
                     int64_t strideB, uint32_t flags)
 {
     SPH_REQUIRE(M != 0 && N != 0 && batch != 0, "M, N and batch must be non-zero");
-    if (flags & (SPH_GEMM_TRANS_A | SPH_GEMM_TRANS_B))
-        return sph::Fail(SPH_ERR_UNSUPPORTED,
-                         "sph_gemm_f16f32 - transposed operands are not supported");
-    SPH_REQUIRE((flags & ~SPH_GEMM_OVERWRITE) == 0, "unknown flag");
+    SPH_REQUIRE((flags & ~(SPH_GEMM_OVERWRITE | SPH_GEMM_TRANS_A | SPH_GEMM_TRANS_B)) == 0,
+                "unknown flag");
+    const bool transA = (flags & SPH_GEMM_TRANS_A) != 0;
+    const bool transB = (flags & SPH_GEMM_TRANS_B) != 0;
     SPH_REQUIRE(out != nullptr, "null pointer");
     SPH_REQUIRE(strideOut >= 0 && strideA >= 0 && strideB >= 0, "negative stride");
     SPH_REQUIRE(batch == 1 || strideOut >= static_cast<int64_t>(M) * N,
@@ -1082,11 +1147,11 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     // so they multiply the first 32 q columns of A and the general kernel adds the last r
     // (measured 4096 x 4096 x 4080: 229 us on the general kernel alone, 175 us this way)
     const uint32_t tail = K % kTK;
-    if (tail != 0 && K % 8 == 0 && K >= 2 * kTK && aligned16 && N % 8 == 0)
+    if (tail != 0 && !transA && !transB && K % 8 == 0 && K >= 2 * kTK && aligned16 && N % 8 == 0)
     {
         GemmF16Args head = args;
         head.K = K - tail;
-        const int rc = LaunchF16(head, batch, aligned16, stream);
+        const int rc = LaunchF16(head, batch, aligned16, false, false, stream);
         if (rc != SPH_OK)
             return rc;
         args.A += head.K;
@@ -1094,7 +1159,7 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
         args.K = tail;
         args.overwrite = 0;
     }
-    return LaunchF16(args, batch, aligned16, stream);
+    return LaunchF16(args, batch, aligned16, transA, transB, stream);
 }
 
 }  // extern "C"

@@ -105,6 +105,29 @@ def test_dma128_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref - C)
 
 
+@pytest.mark.parametrize("flags", [capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
+                                   capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (5, 3, 2, 1), (64, 64, 32, 1), (100, 72, 40, 2),
+                                   (130, 254, 96, 1), (257, 255, 63, 1), (256, 512, 128, 3),
+                                   (300, 136, 1000, 1)])
+def test_transposed_operands_exact_on_integers(dev, shape, flags):
+    """A stored K x M and / or B stored N x K: the same product as with the operands stored
+    plainly, bit for bit on integer-valued inputs (16-byte loads when M, N, K allow, single
+    halves otherwise)."""
+    M, N, K, batch = shape
+    h.announce("sph_gemm_f16f32 transposed operands", shape, "flags", flags)
+    A = synth.small_integers(41, (batch, M, K), span=3).astype(np.float16)
+    B = synth.small_integers(42, (batch, K, N), span=3).astype(np.float16)
+    C = synth.small_integers(43, (batch, M, N), span=100)
+    As = np.ascontiguousarray(A.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_A else A
+    Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
+    ref = _oracle(C, A, B, M, N, K, batch=batch)
+    got = h.gpu_gemm_f16(C, As, Bs, M, N, K, batch=batch, flags=flags)
+    assert np.array_equal(got, ref)
+    got = h.gpu_gemm_f16(C, As, Bs, M, N, K, batch=batch, flags=flags | capi.SPH_GEMM_OVERWRITE)
+    assert np.array_equal(got, ref - C)
+
+
 def test_dma128_batched_with_shared_operand(dev):
     h.announce("sph_gemm_f16f32 128-tile path, batch 3, strideA = 0")
     M, N, K, batch = 200, 136, 96, 3
