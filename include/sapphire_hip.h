@@ -244,8 +244,7 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
  * flags: SPH_GEMM_OVERWRITE stores A*B without reading out (for callers that
  * know out holds zeros); default accumulates like the reference.
  * SPH_GEMM_TRANS_A / SPH_GEMM_TRANS_B read an operand stored transposed
- * (A as K x M, B as N x K), as in sph_gemm_f32_ex; such launches run on the
- * general (register-staged) kernel, not on the straight-to-LDS ones. */
+ * (A as K x M, B as N x K), as in sph_gemm_f32_ex. */
 
 int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M,
                     uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,

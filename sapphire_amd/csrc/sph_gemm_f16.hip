@@ -31,7 +31,7 @@
 //
 //   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned, any M: the
 //     same ingredients on 128 x 128 tiles with 4 wavefronts, for shapes with too
-//     few 256-tiles to fill the chip.
+//     few 256-tiles to fill the chip and for operands stored transposed.
 //
 //   GemmF16General  everything else.  128 x 128 tile, 4 wavefronts, K step 32,
 //     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
@@ -521,11 +521,15 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
 // B stage: 32 k-rows of 256 bytes, 32-byte chunks XOR-swizzled with 2*(k%4), read with the
 // transposing LDS load like the 256-tile kernel.  Rows past M and columns past N are clamped to
 // the last valid ones: they only feed outputs that are not stored.
+// TA (A stored K x M) / TB (B stored N x K): an operand stored the other way round simply takes
+// the other operand's stage layout and fragment read -- an A stored k-major is copied and read
+// like B, a B stored with K contiguous like A -- so the MFMAs and their order do not change.
 constexpr int kD = 128;
 constexpr int kDStages = 4;
 constexpr int kDStageBytes = 2 * kD * kTK * 2;  // A + B
 constexpr int kDCopies = 4;                     // per wavefront and step: 2 of A, 2 of B
 
+template <bool TA, bool TB>
 __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
 {
     __shared__ __attribute__((aligned(1024))) char lds[kDStages * kDStageBytes];
@@ -549,26 +553,35 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     const uint32_t colBase = tn * kD;
 
     // ---- copy plan: copy j of an operand (j = wave, wave + 4) ---------------------------
+    // K-contiguous operand (x = row of A / column of a transposed B, `pitch` halves apart):
+    // 16 x per copy; lane -> x = j*16 + lane/4, physical chunk lane%4.
+    auto laneKContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t pitch) {
+        const uint32_t x = j * 16 + (lane >> 2);
+        const uint32_t c = (lane & 3) ^ ((lane >> 4) & 3);  // (x >> 2) & 3 == (lane >> 4) & 3
+        const uint32_t gx = min(xBase + x, limit - 1);
+        return (gx * pitch + c * 8) * 2u;
+    };
+    // k-major operand (x = column of B / row of a transposed A, rows `pitch` halves apart):
+    // 4 k-rows per copy; lane -> k = j*4 + lane/16, physical 16-byte chunk lane%16.
+    auto laneKMajor = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t pitch) {
+        const uint32_t k = j * 4 + (lane >> 4);
+        const uint32_t phys16 = lane & 15;
+        const uint32_t logical16 = (((phys16 >> 1) ^ (2 * (k & 3))) << 1) | (phys16 & 1);
+        const uint32_t gx = min(xBase + logical16 * 8, limit - 8);
+        return (k * pitch + gx) * 2u;
+    };
     uint32_t aLane[2], bLane[2], aDst[2], bDst[2];
 #pragma unroll
     for (uint32_t i = 0; i < 2; ++i)
     {
         const uint32_t j = wave + 4 * i;
-        // A: 16 rows per copy; lane -> row j*16 + lane/4, physical chunk lane%4
-        const uint32_t x = j * 16 + (lane >> 2);
-        const uint32_t c = (lane & 3) ^ ((lane >> 4) & 3);  // (x >> 2) & 3 == (lane >> 4) & 3
-        const uint32_t gx = min(rowBase + x, M - 1);
-        aLane[i] = (gx * args.lda + c * 8) * 2u;
+        aLane[i] = TA ? laneKMajor(j, rowBase, M, M) : laneKContig(j, rowBase, M, args.lda);
+        bLane[i] = TB ? laneKContig(j, colBase, N, K) : laneKMajor(j, colBase, N, N);
         aDst[i] = j * 1024;
-        // B: 4 k-rows per copy; lane -> k = j*4 + lane/16, physical 16-byte chunk lane%16
-        const uint32_t k = j * 4 + (lane >> 4);
-        const uint32_t phys16 = lane & 15;
-        const uint32_t logical16 = (((phys16 >> 1) ^ (2 * (k & 3))) << 1) | (phys16 & 1);
-        const uint32_t gc = min(colBase + logical16 * 8, N - 8);
-        bLane[i] = (k * N + gc) * 2u;
         bDst[i] = kBytesA + j * 1024;
     }
-    const size_t bStepBytes = static_cast<size_t>(kTK) * N * 2;
+    const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * M * 2 : kTK * 2;
+    const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * N * 2;
     const uint32_t ldsBase = LdsAddress(lds);
     const uint32_t steps = K / kTK;
     // Copy n (0..3: two of A, two of B) of the next step to fetch, into stage `stage`.  aSrc /
@@ -587,7 +600,7 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     auto advance = [&]() {
         if (stepsToAdvance != 0)
         {
-            aSrc += kTK * 2;
+            aSrc += aStepBytes;
             bSrc += bStepBytes;
             --stepsToAdvance;
         }
@@ -598,25 +611,43 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     const uint32_t khalf = lane >> 5;
     const uint32_t g = lane >> 4;
     const uint32_t s = lane & 15;
-    uint32_t aOff[2][2], bOff[2][2];  // [ks][block], bytes inside a stage
+    // bytes inside an operand's part of a stage, [ks][block]
+    auto offKContig = [&](int ks, uint32_t x) {
+        return x * 64 + (((ks * 2 + khalf) ^ ((x >> 2) & 3)) << 4);
+    };
+    auto offKMajor = [&](int ks, uint32_t chunkBase) {
+        const uint32_t k = ks * 16 + 8 * (g >> 1) + (s >> 2);  // + 4 for the second read
+        const uint32_t chunk32 = (chunkBase + (g & 1)) ^ (2 * ((s >> 2) & 3));
+        return k * 256 + chunk32 * 32 + (s & 3) * 8;
+    };
+    uint32_t aOff[2][2], bOff[2][2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
         for (int b = 0; b < 2; ++b)
         {
-            const uint32_t x = waveM * 64 + b * 32 + l32;
-            aOff[ks][b] = x * 64 + (((ks * 2 + khalf) ^ ((x >> 2) & 3)) << 4);
-            const uint32_t k = ks * 16 + 8 * (g >> 1) + (s >> 2);  // + 4 for the second read
-            const uint32_t chunk32 = (waveN * 4 + b * 2 + (g & 1)) ^ (2 * ((s >> 2) & 3));
-            bOff[ks][b] = kBytesA + k * 256 + chunk32 * 32 + (s & 3) * 8;
+            aOff[ks][b] = TA ? offKMajor(ks, waveM * 4 + b * 2)
+                             : offKContig(ks, waveM * 64 + b * 32 + l32);
+            bOff[ks][b] = kBytesA + (TB ? offKContig(ks, waveN * 64 + b * 32 + l32)
+                                        : offKMajor(ks, waveN * 4 + b * 2));
         }
+    auto readKContig = [&](const char* p) { return *reinterpret_cast<const halfx8*>(p); };
+    auto readKMajor = [&](const char* p) {
+        const _Float16* h = reinterpret_cast<const _Float16*>(p);
+        return Join(LdsReadTr(h), LdsReadTr(h + 4 * 128));
+    };
     auto loadFragments = [&](halfx8 (&af)[2], halfx8 (&bf)[2], const char* stage, int ks) {
 #pragma unroll
         for (int b = 0; b < 2; ++b)
         {
-            af[b] = *reinterpret_cast<const halfx8*>(stage + aOff[ks][b]);
-            const _Float16* p = reinterpret_cast<const _Float16*>(stage + bOff[ks][b]);
-            bf[b] = Join(LdsReadTr(p), LdsReadTr(p + 4 * 128));
+            if constexpr (TA)
+                af[b] = readKMajor(stage + aOff[ks][b]);
+            else
+                af[b] = readKContig(stage + aOff[ks][b]);
+            if constexpr (TB)
+                bf[b] = readKContig(stage + bOff[ks][b]);
+            else
+                bf[b] = readKMajor(stage + bOff[ks][b]);
         }
     };
 
@@ -1003,7 +1034,7 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
               hipStream_t stream)
 {
     const uint32_t M = args.M, N = args.N, K = args.K;
-    const bool plain = !transA && !transB;  // only the general kernel reads transposed operands
+    const bool plain = !transA && !transB;  // the 256-tile kernel takes plain storage only
     // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
     // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
     const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
@@ -1031,12 +1062,21 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
         else
             hipLaunchKernelGGL((GemmF16Tile256<8, true>), dim3(grid), dim3(512), 0, stream, args);
     }
-    else if (plain && aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
-             static_cast<uint64_t>(M) * args.lda < (1ull << 31) &&
-             static_cast<uint64_t>(kTK) * N < (1ull << 31))
+    else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
+             (!transA || (M % 8 == 0 && M >= 8)) &&
+             static_cast<uint64_t>(M) * (transA ? kTK : args.lda) < (1ull << 31) &&
+             static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31))
     {
         // whole K steps and 16-byte chunks everywhere: straight-to-LDS 128-tile kernel
-        hipLaunchKernelGGL(GemmF16Dma128, dim3(grid), dim3(256), 0, stream, args);
+        const dim3 g(grid), b(256);
+        if (transA && transB)
+            hipLaunchKernelGGL((GemmF16Dma128<true, true>), g, b, 0, stream, args);
+        else if (transA)
+            hipLaunchKernelGGL((GemmF16Dma128<true, false>), g, b, 0, stream, args);
+        else if (transB)
+            hipLaunchKernelGGL((GemmF16Dma128<false, true>), g, b, 0, stream, args);
+        else
+            hipLaunchKernelGGL((GemmF16Dma128<false, false>), g, b, 0, stream, args);
     }
     else
     {
