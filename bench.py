@@ -58,7 +58,7 @@ def parse():
     p.add_argument("--all", action="store_true",
                    help="also time configurations 1, 2 and 4 (reported under 'others')")
     p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
-                                      "csr"], default=None,
+                                      "csr", "spgemm"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
     p.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                    help="untimed run-up before each timed leg that lets the clock reach its "
@@ -555,6 +555,11 @@ def main():
                                                                         args.warmup)
         result["csr"] = {"dense_to_csr_ms": ms_csr, "csr_to_dense_ms": ms_dense,
                          "dense_bytes": dense_bytes, "csr_bytes": csr_bytes}
+
+    if args.only == "spgemm":
+        ms, products, nnz_c, nbytes, nnz_a, nnz_b = bench_spgemm(capi, synth, args.steps, args.warmup)
+        result["spgemm"] = {"count_plus_fill_ms": ms, "products": products, "nnz_a": nnz_a,
+                            "nnz_b": nnz_b, "nnz_c": nnz_c, "algorithmic_bytes": nbytes}
 
     if args.only in (None, "spmm"):
         sp_steps = max(args.steps * 4, 100)
