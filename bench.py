@@ -360,6 +360,41 @@ def bench_spgemm(capi, synth, steps, warmup, n=8192, per_row=8.0):
     return event_ms, products, nnz.value, nbytes, a[0].size, b[0].size
 
 
+def bench_sparse_linear(capi, synth, steps, warmup, batch=256):
+    """Forward of a Linear layer whose weight is configuration 5's matrix kept as CSR
+    (8192 inputs, 8192 outputs, 1 % of the weights), batch 256, issued as the C++ layer's
+    NN::SparseLinearForward issues it: x transposed, ones, zero fill, bias x ones (K = 1 GEMM),
+    CSR x dense accumulating, result transposed back.  Returns the milliseconds per forward and
+    of the CSR x dense launch alone."""
+    d = synth.config5()
+    outs, ins = d["M"], d["K"]
+    x = capi.DeviceBuffer.from_array(synth.uniform(6100, (batch, ins)))
+    bias = capi.DeviceBuffer.from_array(synth.uniform(6101, (outs,), -0.1, 0.1))
+    dV, dCol, dRow = (capi.DeviceBuffer.from_array(d[k]) for k in ("V", "COL", "ROW"))
+    xT = capi.DeviceBuffer(4 * ins * batch)
+    yT = capi.DeviceBuffer(4 * outs * batch)
+    y = capi.DeviceBuffer(4 * outs * batch)
+    ones = capi.DeviceBuffer(4 * batch)
+
+    def product():
+        capi.call("sph_spmm_csr_f32", yT.ptr, dV.ptr, dCol.ptr, dRow.ptr, outs, ins, batch, xT.ptr, 1)
+
+    def forward():
+        capi.call("sph_transpose_f32", xT.ptr, x.ptr, batch, ins, 1, 0)
+        capi.call("sph_fill_f32", ones.ptr, 1.0, batch)
+        capi.call("sph_fill_f32", yT.ptr, 0.0, outs * batch)
+        capi.call("sph_gemm_f32", yT.ptr, bias.ptr, ones.ptr, outs, batch, 1, 1, outs * batch, outs,
+                  batch)
+        product()
+        capi.call("sph_transpose_f32", y.ptr, yT.ptr, outs, batch, 1, 0)
+
+    ms, _ = timed_launches(capi, forward, steps, warmup)
+    ms_product, _ = timed_launches(capi, product, steps, warmup)
+    for b in (x, bias, dV, dCol, dRow, xT, yT, y, ones):
+        b.release()
+    return ms, ms_product, int(d["V"].size)
+
+
 def bench_allocation(capi, nbytes=64 << 20, rounds=200):
     """Host-side cost of taking and returning one device block of `nbytes`: the blocking pair
     (hipMalloc / hipFree) against the stream-ordered pair the buffer pool uses on a miss."""
@@ -636,6 +671,13 @@ def main():
             "algorithmic_gbs": nbytes / (ms * 1e-3) / 1e9,
             "note": "both passes compute every product (the count pass must see which sums "
                     "cancel); products counted once per pass in gproducts_per_s"}
+        ms, ms_product, nnz_w = bench_sparse_linear(capi, synth, 50, 5)
+        others["sparse_linear_forward_8192x8192_batch256"] = {
+            "forward_ms": ms, "csr_x_dense_ms": ms_product, "launches_per_forward": 6,
+            "weights_kept": nnz_w,
+            "gflops": 2.0 * nnz_w * 256 / (ms * 1e-3) / 1e9,
+            "note": "the NN::SparseLinearForward sequence through the C ABI: transpose x, ones, "
+                    "zero fill, bias x ones (K = 1 GEMM), CSR x dense (accumulating), transpose y"}
         others["one_pass_kernels_4096x4096"] = bench_elementwise(capi, 50, 5)
         others["device_block_64MiB"] = bench_allocation(capi)
         result["others"] = others
