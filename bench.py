@@ -671,6 +671,14 @@ def main():
             "algorithmic_gbs": nbytes / (ms * 1e-3) / 1e9,
             "note": "both passes compute every product (the count pass must see which sums "
                     "cancel); products counted once per pass in gproducts_per_s"}
+        ms, products, nnz_c, nbytes, nnz_a, nnz_b = bench_spgemm(capi, synth, 20, 3, n=65536)
+        others["spgemm_65536_8_per_row"] = {
+            "workload": "CSR 65536x65536 (nnz %d) x CSR 65536x65536 (nnz %d) -> CSR (nnz %d)"
+                        % (nnz_a, nnz_b, nnz_c),
+            "count_plus_fill_ms": ms, "products": products,
+            "gproducts_per_s": 2 * products / (ms * 1e-3) / 1e9,
+            "algorithmic_gbs": nbytes / (ms * 1e-3) / 1e9,
+            "note": "16 strips wide: rows with few products go through the hash-table kernel"}
         ms, ms_product, nnz_w = bench_sparse_linear(capi, synth, 50, 5)
         others["sparse_linear_forward_8192x8192_batch256"] = {
             "forward_ms": ms, "csr_x_dense_ms": ms_product, "launches_per_forward": 6,

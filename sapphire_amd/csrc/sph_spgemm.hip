@@ -24,6 +24,10 @@
 // follows the entries it produces, not its width.  The same kernel runs twice: once to count
 // the entries of every row (the caller then allocates), once to write them.
 //
+// Matrices wider than two strips: rows with few products (A's row at most 64 entries, at most
+// 256 products) go to SpgemmHashKernel, which keeps the row in a hash table instead and whose
+// cost does not depend on the width; the strip kernel then takes only the remaining rows.
+//
 // Requirements on the operands: column indices of B below N and distinct within a row;
 // column indices of A below the row count of B.
 #include "sph_internal.h"
@@ -38,6 +42,14 @@ constexpr uint32_t kStripMax = 4096;  // columns per LDS strip
 constexpr uint32_t kAhead = 8;        // rows of B whose first 64 entries are in flight together
 constexpr uint32_t kRowsPerTurnMax = 8;  // consecutive output rows a wavefront takes at a time
 constexpr uint32_t kWordsPerLaneMax = kStripMax / 32 / 64;  // bit-map words a lane owns
+// Wide matrices (more than one strip): rows with few products go through a hash table instead
+constexpr uint32_t kHashSlots = 512;            // power of two
+constexpr uint32_t kHashProducts = kHashSlots / 2;  // a row with at most this many products is "light"
+constexpr uint32_t kEmpty = 0xffffffffu;
+// two strips still cost less than the table and its sort (8192 columns, 8 entries per row on
+// both sides: 82 us on strips, 96 us through the table); from three strips on the table wins
+constexpr uint32_t kHashFromWidth = 2 * kStripMax;
+static_assert(kHashSlots == 512, "the hash takes the top 9 bits of a product");
 static_assert(kWordsPerLaneMax <= 4, "the sweep takes a lane's words as two pairs");
 
 struct SpgemmArgs
@@ -51,6 +63,7 @@ struct SpgemmArgs
     uint32_t M, K, N;
     uint32_t strip;  // columns per strip (multiple of 64)
     uint32_t rowsPerTurn;  // 1 .. kRowsPerTurnMax
+    uint32_t heavyOnly;    // strip kernel: leave the rows SpgemmHashKernel takes alone
     // count pass: counts (M + 1 entries, counts[M] = 0).  fill pass: ROWC, VC, COLC.
     uint32_t* counts;
     const uint32_t* ROWC;
@@ -73,6 +86,247 @@ __device__ __forceinline__ void Touch(uint32_t* bits, uint32_t column)
 {
     __hip_atomic_fetch_or(&bits[column >> 5], 1u << (column & 31), __ATOMIC_RELAXED,
                           __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+__device__ __forceinline__ uint32_t WaveSum(uint32_t v)
+{
+#pragma unroll
+    for (uint32_t d = 1; d < 64; d *= 2)
+        v += __shfl_xor(v, d, 64);
+    return v;
+}
+
+// A row is light when A's row has at most 64 entries and the rows of B they select hold at
+// most kHashProducts entries together.  Both kernels decide from these two numbers.
+__device__ __forceinline__ bool LightRow(uint32_t entriesOfA, uint32_t products)
+{
+    return entriesOfA <= 64 && products <= kHashProducts;
+}
+
+// Light rows of a wide product.  The strip kernel walks all products of a row once per strip
+// of 4096 columns, which is wasted on a row whose few products fall into a matrix of, say,
+// 65536 columns.  Here a wavefront keeps the row in an LDS hash table keyed by column instead
+// (the design the reference sketches, SparseGemm.cuh:16-36): the products are generated in the
+// same order as in the strip kernel -- A's entries in storage order, the entries of one row of
+// B across the lanes, so no two lanes of a step hold the same column -- a lane finds or claims
+// (compare-and-swap on the key) the slot of its column and adds into it, which keeps the sum
+// order of every element fixed.  Claimed slots are listed as they are claimed; at the end of
+// the row the listed (column, sum) pairs are sorted by column (bitonic, in LDS), sums that are
+// exactly zero are dropped, and the table is reset through the list.  The cost of a row follows
+// its products, not the width of the matrix.
+template <bool FILL>
+__global__ __launch_bounds__(64) void SpgemmHashKernel(const SpgemmArgs args)
+{
+    __shared__ uint32_t keys[kHashSlots];
+    __shared__ float sums[kHashSlots];
+    __shared__ uint32_t sortKey[kHashProducts];  // first the list of claimed slots, then columns
+    __shared__ float sortVal[kHashProducts];
+    const uint32_t lane = threadIdx.x;
+    const uint64_t below = (1ull << lane) - 1ull;
+    for (uint32_t t = lane; t < kHashSlots; t += 64)
+    {
+        keys[t] = kEmpty;
+        sums[t] = 0.0f;
+    }
+
+    // A wavefront takes rows blockIdx.x, blockIdx.x + gridDim.x, ... in turns of up to 64: their
+    // extents are read in one go (one row per lane), and the loads that lead to a row's
+    // products form a pipeline over the rows of the turn: while row i is multiplied, the
+    // entries of A's row i+2 and the extents of the rows of B that row i+1 selects are on
+    // their way.
+    for (uint64_t first = blockIdx.x; first < args.M; first += 64ull * gridDim.x)
+    {
+        const uint64_t mine = first + static_cast<uint64_t>(lane) * gridDim.x;
+        const uint32_t rowsHere = static_cast<uint32_t>(
+            min(static_cast<uint64_t>(64), (args.M - first + gridDim.x - 1) / gridDim.x));
+        uint32_t extentBegin = 0, extentEnd = 0, outBegin = 0, outEnd = 0;
+        if (mine < args.M)
+        {
+            extentBegin = args.ROWA[mine];
+            extentEnd = args.ROWA[mine + 1];
+            if (FILL)
+            {
+                outBegin = args.ROWC[mine];
+                outEnd = args.ROWC[mine + 1];
+            }
+        }
+        // stage 1: this lane's entry of A's row i (rows with more than 64 entries are not ours)
+        auto loadStage1 = [&](uint32_t i, uint32_t& k, float& value) {
+            k = kEmpty;
+            value = 0.0f;
+            if (i < rowsHere)
+            {
+                const uint32_t begin = Uniform(extentBegin, i), end = Uniform(extentEnd, i);
+                if (end - begin <= 64 && begin + lane < end)
+                {
+                    k = args.COLA[begin + lane];
+                    value = args.VA[begin + lane];
+                }
+            }
+        };
+        // stage 2: the extent of the row of B that entry selects
+        auto loadStage2 = [&](uint32_t k, uint32_t& begin, uint32_t& end) {
+            begin = 0;
+            end = 0;
+            if (k < args.K)
+            {
+                begin = args.ROWB[k];
+                end = args.ROWB[k + 1];
+            }
+        };
+        uint32_t k1, k2, nextBegin, nextEnd;
+        float value1, value2;
+        loadStage1(0, k2, value2);
+        loadStage2(k2, nextBegin, nextEnd);
+        loadStage1(1, k1, value1);
+
+      for (uint32_t i = 0; i < rowsHere; ++i)
+      {
+        const uint32_t row = static_cast<uint32_t>(first + static_cast<uint64_t>(i) * gridDim.x);
+        const uint32_t entriesOfA = Uniform(extentEnd, i) - Uniform(extentBegin, i);
+        const uint32_t bBegin = nextBegin, bEnd = nextEnd;
+        const float aValue = value2;
+        k2 = k1;
+        value2 = value1;
+        loadStage2(k2, nextBegin, nextEnd);
+        loadStage1(i + 2, k1, value1);
+        if (!LightRow(entriesOfA, WaveSum(bEnd - bBegin)))
+            continue;  // heavy: the strip kernel's row
+
+        uint32_t listed = 0;  // claimed slots so far (uniform)
+        for (uint32_t j0 = 0; j0 < entriesOfA; j0 += kAhead)
+        {
+            // the first 64 entries of kAhead rows of B are requested before the first is used
+            uint32_t s[kAhead], e[kAhead], col[kAhead];
+            float a[kAhead], b[kAhead];
+#pragma unroll
+            for (uint32_t u = 0; u < kAhead; ++u)
+            {
+                const uint32_t j = min(j0 + u, 63u);
+                s[u] = Uniform(bBegin, j);
+                e[u] = j0 + u < entriesOfA ? Uniform(bEnd, j) : s[u];
+                a[u] = Uniform(aValue, j);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < kAhead; ++u)
+            {
+                col[u] = kEmpty;
+                b[u] = 0.0f;
+                if (s[u] + lane < e[u])
+                {
+                    col[u] = args.COLB[s[u] + lane];
+                    b[u] = args.VB[s[u] + lane];
+                }
+            }
+            // one product per lane: find or claim the column's slot and add into it
+            auto insert = [&](uint32_t c, float product, bool have) {
+                bool claimed = false;
+                uint32_t h = 0;
+                if (have)
+                {
+                    h = (c * 2654435761u) >> 23;  // top 9 bits: kHashSlots = 512
+                    for (uint32_t tries = 0; tries < kHashSlots; ++tries)
+                    {
+                        const uint32_t k = keys[h];
+                        if (k == c)
+                            break;
+                        if (k == kEmpty)
+                        {
+                            const uint32_t old = atomicCAS(&keys[h], kEmpty, c);
+                            if (old == kEmpty)
+                            {
+                                claimed = true;
+                                break;
+                            }
+                            if (old == c)
+                                break;
+                        }
+                        h = (h + 1) & (kHashSlots - 1);
+                    }
+                    sums[h] = sums[h] + product;
+                }
+                const uint64_t m = __ballot(claimed);
+                if (claimed)
+                    sortKey[listed + static_cast<uint32_t>(__popcll(m & below))] = h;
+                listed += static_cast<uint32_t>(__popcll(m));
+            };
+#pragma unroll
+            for (uint32_t u = 0; u < kAhead; ++u)
+            {
+                insert(col[u], a[u] * b[u], col[u] < args.N);
+                // rows of B with more than 64 entries: the rest, 64 at a time
+                for (uint32_t pb0 = s[u] + 64; pb0 < e[u]; pb0 += 64)
+                {
+                    const bool have = pb0 + lane < e[u];
+                    const uint32_t c = have ? args.COLB[pb0 + lane] : kEmpty;
+                    const float bv = have ? args.VB[pb0 + lane] : 0.0f;
+                    insert(c, a[u] * bv, have && c < args.N);
+                }
+            }
+        }
+
+        // the listed slots become (column, sum) pairs, and the table is empty again
+        uint32_t padded = 64;
+        while (padded < listed)
+            padded *= 2;
+        for (uint32_t q = lane; q < padded; q += 64)
+        {
+            uint32_t c = kEmpty;
+            float v = 0.0f;
+            if (q < listed)
+            {
+                const uint32_t h = sortKey[q];
+                c = keys[h];
+                v = sums[h];
+                keys[h] = kEmpty;
+                sums[h] = 0.0f;
+            }
+            sortKey[q] = c;
+            sortVal[q] = v;
+        }
+        // bitonic sort by column; the padding (kEmpty) ends up behind the entries
+        for (uint32_t size = 2; size <= padded; size *= 2)
+            for (uint32_t stride = size / 2; stride > 0; stride /= 2)
+                for (uint32_t t = lane; t < padded / 2; t += 64)
+                {
+                    const uint32_t lo = 2 * t - (t & (stride - 1));  // lower index of pair t
+                    const uint32_t hi = lo + stride;
+                    const bool ascending = (lo & size) == 0;
+                    const uint32_t kLo = sortKey[lo], kHi = sortKey[hi];
+                    if ((kLo > kHi) == ascending)
+                    {
+                        const float vLo = sortVal[lo], vHi = sortVal[hi];
+                        sortKey[lo] = kHi;
+                        sortKey[hi] = kLo;
+                        sortVal[lo] = vHi;
+                        sortVal[hi] = vLo;
+                    }
+                }
+        // entries in column order; sums that are exactly zero are not stored
+        uint32_t emitted = 0;
+        const uint32_t rowBase = FILL ? Uniform(outBegin, i) : 0u;
+        const uint32_t rowLimit = FILL ? Uniform(outEnd, i) : 0u;
+        for (uint32_t i0 = 0; i0 < listed; i0 += 64)
+        {
+            const uint32_t x = i0 + lane;
+            const float v = x < listed ? sortVal[x] : 0.0f;
+            const bool keep = v != 0.0f;
+            const uint64_t m = __ballot(keep);
+            if (FILL)
+            {
+                const uint32_t at = rowBase + emitted + static_cast<uint32_t>(__popcll(m & below));
+                if (keep && at < rowLimit)
+                {
+                    args.VC[at] = v;
+                    args.COLC[at] = sortKey[x];
+                }
+            }
+            emitted += static_cast<uint32_t>(__popcll(m));
+        }
+        if (!FILL && lane == 0)
+            args.counts[row] = emitted;
+      }
+    }
 }
 
 template <bool FILL>
@@ -150,6 +404,9 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
         value2 = value1;
         loadStage2(k2, nextBegin, nextEnd);
         loadStage1(i + 2, k1, value1);
+        // in a wide product the light rows belong to SpgemmHashKernel
+        if (args.heavyOnly != 0 && LightRow(aEnd - aBegin, WaveSum(firstEnd - firstBegin)))
+            continue;
 
         for (uint32_t c0 = 0; c0 < args.N; c0 += args.strip)
         {
@@ -325,6 +582,13 @@ uint32_t RowsPerTurnFor(uint32_t M)
     return std::max<uint32_t>(1, std::min<uint32_t>(kRowsPerTurnMax, M / std::max<uint32_t>(wanted, 1)));
 }
 
+// one wavefront per workgroup, rows dealt round robin; 6 KiB of LDS each
+uint32_t HashGridFor(uint32_t M)
+{
+    const uint64_t cap = static_cast<uint64_t>(sph::ComputeUnits()) * 32;
+    return static_cast<uint32_t>(std::max<uint64_t>(1, std::min<uint64_t>(M, cap)));
+}
+
 uint32_t GridFor(uint32_t M, uint32_t rowsPerTurn)
 {
     const uint64_t cap = static_cast<uint64_t>(sph::ComputeUnits()) * 64;
@@ -359,6 +623,9 @@ int sph_spgemm_row_offsets_f32(uint32_t* ROWC, const float* VA, const uint32_t* 
     args.strip = StripFor(N);
     args.rowsPerTurn = RowsPerTurnFor(M);
     args.counts = ROWC;
+    args.heavyOnly = N > kHashFromWidth ? 1u : 0u;
+    if (args.heavyOnly != 0 && M != 0)
+        hipLaunchKernelGGL(SpgemmHashKernel<false>, dim3(HashGridFor(M)), dim3(64), 0, stream, args);
     hipLaunchKernelGGL(SpgemmRowKernel<false>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
                        args.strip * sizeof(float) + args.strip / 8, stream, args);
     SPH_CHECK_LAUNCH();
@@ -392,6 +659,9 @@ int sph_spgemm_fill_f32(float* VC, uint32_t* COLC, const uint32_t* ROWC, const f
     args.ROWC = ROWC;
     args.VC = VC;
     args.COLC = COLC;
+    args.heavyOnly = N > kHashFromWidth ? 1u : 0u;
+    if (args.heavyOnly != 0)
+        hipLaunchKernelGGL(SpgemmHashKernel<true>, dim3(HashGridFor(M)), dim3(64), 0, stream, args);
     hipLaunchKernelGGL(SpgemmRowKernel<true>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
                        args.strip * sizeof(float) + args.strip / 8, stream, args);
     SPH_CHECK_LAUNCH();

@@ -124,3 +124,41 @@ def test_random_shapes_and_densities(dev, block):
         V, COL, ROW = gpu_spgemm(A, B, M, K, N)
         assert np.array_equal(ROW, wR) and np.array_equal(COL, wC)
         assert np.array_equal(bits(V), bits(wV))
+
+
+def test_wide_product_mixes_table_rows_and_strip_rows(dev):
+    """More than two strips of columns: rows with few products are kept in the hash table,
+    the others stay with the strips.  The operands mix both kinds: rows of A that select rows of
+    B longer than 64 entries, rows of A with more than 64 entries, rows with more than 256
+    products, empty rows, and a pair of entries whose contributions cancel exactly."""
+    M, K, N = 260, 300, 20000
+    h.announce("sph_spgemm_* wide product with light and heavy rows", (M, K, N))
+    rng = np.random.default_rng(77)
+    dB = np.zeros((K, N), np.float32)
+    for k in range(K):
+        count = 100 if k < 10 else 10
+        cols = rng.choice(N, size=count, replace=False)
+        dB[k, cols] = synth.uniform(9000 + k, (count,))
+    dB[21] = dB[20]  # rows 20 and 21 of B are equal: +1 and -1 times them cancel
+    dA = np.zeros((M, K), np.float32)
+    for m in range(M):
+        kind = m % 5
+        if kind == 0:    # one or two long rows of B: light, with the 64-at-a-time tail
+            ks = rng.choice(10, size=1 + m % 2, replace=False)
+        elif kind == 1:  # a handful of short rows of B: light
+            ks = 10 + rng.choice(K - 10, size=6, replace=False)
+        elif kind == 2:  # more than 64 entries: the strips' row
+            ks = rng.choice(K, size=150, replace=False)
+        elif kind == 3:  # few entries, more than 256 products: the strips' row
+            ks = rng.choice(10, size=6, replace=False)
+        else:            # empty
+            ks = np.zeros(0, np.int64)
+        dA[m, ks] = synth.uniform(9500 + m, (len(ks),))
+    dA[1, :] = 0
+    dA[1, 20], dA[1, 21], dA[1, 30] = 1.0, -1.0, 0.5  # cancelling pair plus one survivor
+    A, B = po.csr_from_dense(dA), po.csr_from_dense(dB)
+    wV, wC, wR = po.spgemm_csr(A, B, M, K, N)
+    assert wR[2] - wR[1] == np.count_nonzero(dB[30])  # the cancelled columns are not stored
+    V, COL, ROW = gpu_spgemm(A, B, M, K, N)
+    assert np.array_equal(ROW, wR) and np.array_equal(COL, wC)
+    assert np.array_equal(bits(V), bits(wV))
