@@ -265,63 +265,105 @@ __global__ __launch_bounds__(64) void SpgemmHashKernel(const SpgemmArgs args)
             }
         }
 
-        // the listed slots become (column, sum) pairs, and the table is empty again
-        uint32_t padded = 64;
-        while (padded < listed)
-            padded *= 2;
-        for (uint32_t q = lane; q < padded; q += 64)
+        uint32_t emitted = 0;
+        const uint32_t rowBase = FILL ? Uniform(outBegin, i) : 0u;
+        const uint32_t rowLimit = FILL ? Uniform(outEnd, i) : 0u;
+        if (listed <= 64)
         {
+            // one (column, sum) pair per lane: sorted in registers with cross-lane exchanges
             uint32_t c = kEmpty;
             float v = 0.0f;
-            if (q < listed)
+            if (lane < listed)
             {
-                const uint32_t h = sortKey[q];
+                const uint32_t h = sortKey[lane];
                 c = keys[h];
                 v = sums[h];
                 keys[h] = kEmpty;
                 sums[h] = 0.0f;
             }
-            sortKey[q] = c;
-            sortVal[q] = v;
-        }
-        // bitonic sort by column; the padding (kEmpty) ends up behind the entries
-        for (uint32_t size = 2; size <= padded; size *= 2)
-            for (uint32_t stride = size / 2; stride > 0; stride /= 2)
-                for (uint32_t t = lane; t < padded / 2; t += 64)
+#pragma unroll
+            for (uint32_t size = 2; size <= 64; size *= 2)
+#pragma unroll
+                for (uint32_t stride = size / 2; stride > 0; stride /= 2)
                 {
-                    const uint32_t lo = 2 * t - (t & (stride - 1));  // lower index of pair t
-                    const uint32_t hi = lo + stride;
-                    const bool ascending = (lo & size) == 0;
-                    const uint32_t kLo = sortKey[lo], kHi = sortKey[hi];
-                    if ((kLo > kHi) == ascending)
-                    {
-                        const float vLo = sortVal[lo], vHi = sortVal[hi];
-                        sortKey[lo] = kHi;
-                        sortKey[hi] = kLo;
-                        sortVal[lo] = vHi;
-                        sortVal[hi] = vLo;
-                    }
+                    const uint32_t oc = __shfl_xor(c, stride, 64);
+                    const float ov = __shfl_xor(v, stride, 64);
+                    // in an ascending run the lower lane of a pair keeps the smaller column
+                    const bool wantsSmaller = ((lane & stride) == 0) == ((lane & size) == 0);
+                    const bool takeOther = wantsSmaller ? oc < c : oc > c;
+                    c = takeOther ? oc : c;
+                    v = takeOther ? ov : v;
                 }
-        // entries in column order; sums that are exactly zero are not stored
-        uint32_t emitted = 0;
-        const uint32_t rowBase = FILL ? Uniform(outBegin, i) : 0u;
-        const uint32_t rowLimit = FILL ? Uniform(outEnd, i) : 0u;
-        for (uint32_t i0 = 0; i0 < listed; i0 += 64)
-        {
-            const uint32_t x = i0 + lane;
-            const float v = x < listed ? sortVal[x] : 0.0f;
-            const bool keep = v != 0.0f;
+            const bool keep = c != kEmpty && v != 0.0f;  // exact zeros are not stored
             const uint64_t m = __ballot(keep);
             if (FILL)
             {
-                const uint32_t at = rowBase + emitted + static_cast<uint32_t>(__popcll(m & below));
+                const uint32_t at = rowBase + static_cast<uint32_t>(__popcll(m & below));
                 if (keep && at < rowLimit)
                 {
                     args.VC[at] = v;
-                    args.COLC[at] = sortKey[x];
+                    args.COLC[at] = c;
                 }
             }
-            emitted += static_cast<uint32_t>(__popcll(m));
+            emitted = static_cast<uint32_t>(__popcll(m));
+        }
+        else
+        {
+            // the listed slots become (column, sum) pairs, and the table is empty again
+            uint32_t padded = 64;
+            while (padded < listed)
+                padded *= 2;
+            for (uint32_t q = lane; q < padded; q += 64)
+            {
+                uint32_t c = kEmpty;
+                float v = 0.0f;
+                if (q < listed)
+                {
+                    const uint32_t h = sortKey[q];
+                    c = keys[h];
+                    v = sums[h];
+                    keys[h] = kEmpty;
+                    sums[h] = 0.0f;
+                }
+                sortKey[q] = c;
+                sortVal[q] = v;
+            }
+            // bitonic sort by column; the padding (kEmpty) ends up behind the entries
+            for (uint32_t size = 2; size <= padded; size *= 2)
+                for (uint32_t stride = size / 2; stride > 0; stride /= 2)
+                    for (uint32_t t = lane; t < padded / 2; t += 64)
+                    {
+                        const uint32_t lo = 2 * t - (t & (stride - 1));  // lower index of pair t
+                        const uint32_t hi = lo + stride;
+                        const bool ascending = (lo & size) == 0;
+                        const uint32_t kLo = sortKey[lo], kHi = sortKey[hi];
+                        if ((kLo > kHi) == ascending)
+                        {
+                            const float vLo = sortVal[lo], vHi = sortVal[hi];
+                            sortKey[lo] = kHi;
+                            sortKey[hi] = kLo;
+                            sortVal[lo] = vHi;
+                            sortVal[hi] = vLo;
+                        }
+                    }
+            // entries in column order; sums that are exactly zero are not stored
+            for (uint32_t i0 = 0; i0 < listed; i0 += 64)
+            {
+                const uint32_t x = i0 + lane;
+                const float v = x < listed ? sortVal[x] : 0.0f;
+                const bool keep = v != 0.0f;
+                const uint64_t m = __ballot(keep);
+                if (FILL)
+                {
+                    const uint32_t at = rowBase + emitted + static_cast<uint32_t>(__popcll(m & below));
+                    if (keep && at < rowLimit)
+                    {
+                        args.VC[at] = v;
+                        args.COLC[at] = sortKey[x];
+                    }
+                }
+                emitted += static_cast<uint32_t>(__popcll(m));
+            }
         }
         if (!FILL && lane == 0)
             args.counts[row] = emitted;
