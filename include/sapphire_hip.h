@@ -287,6 +287,20 @@ int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL,
  * stored; columns >= N in COL are ignored; the pitch padding is not written. */
 int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M,
                             uint32_t N, uint32_t ld, uint32_t* nnzHost);
+/* sph_csr_row_offsets_f32 for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops that must not reach the
+ * allocator, harnesses that forbid it).  No counterpart in the reference.
+ * Same ROW, bit for bit, for any M, including the M + 1 > 65536 case in which
+ * sph_csr_row_offsets_f32 takes a stream-ordered scratch block: the per-block
+ * totals of the scan live in a fixed 16 KiB array inside the library (one copy
+ * per device, held until the process ends) instead.  Allocates nothing, waits
+ * for nothing, copies nothing to the host (read ROW[M] yourself) and can be
+ * recorded into a graph.  M above 16777215 is SPH_ERR_INVALID.  All calls on
+ * one device share the array: calls that overlap in time on different streams
+ * of one device race; calls on one stream are ordered and need no clearing
+ * between them. */
+int sph_csr_row_offsets_noalloc_f32(uint32_t* ROW, const float* dense,
+                                    uint32_t M, uint32_t N, uint32_t ld);
 int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW,
                      const float* dense, uint32_t M, uint32_t N, uint32_t ld);
 int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V,

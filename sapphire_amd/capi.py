@@ -95,6 +95,7 @@ SIGNATURES = {
     "sph_gemm_f32_grouped": [ctypes.POINTER(SphGemmEntry), _u32, _vp, _vp, _vp, _u32, _u32, _u32],
     "sph_gemm_f16f32": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
     "sph_csr_row_offsets_f32": [_vp, _vp, _u32, _u32, _u32, ctypes.POINTER(ctypes.c_uint32)],
+    "sph_csr_row_offsets_noalloc_f32": [_vp, _vp, _u32, _u32, _u32],
     "sph_csr_fill_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32],
     "sph_csr_to_dense_f32": [_vp, _u32, _vp, _vp, _vp, _u32, _u32],
     "sph_spgemm_row_offsets_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,

@@ -18,10 +18,21 @@
 #include "sph_internal.h"
 
 #include <algorithm>
+#include <mutex>
 
 namespace
 {
 constexpr int kThreads = 256;
+
+// Block totals of the row-offset scan for sph_csr_row_offsets_noalloc_f32: one 32-bit total
+// per 4096 counts, 4096 totals = 16 KiB per device for the life of the process.  In host code
+// this name is only a handle for hipGetSymbolAddress; kernels get the resolved pointer.
+constexpr uint32_t kNoAllocMaxBlocks = 4096;
+static __device__ __align__(256) uint32_t scratch[kNoAllocMaxBlocks];
+
+constexpr int kMaxScratchDevices = 16;
+std::mutex gScratchMutex;
+uint32_t* gScratchPtr[kMaxScratchDevices] = {};
 
 struct DenseView
 {
@@ -354,9 +365,36 @@ struct FillLauncher
 
 namespace sph
 {
-int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStream_t stream)
+bool ScanWaitsOrAllocates(uint32_t n, const uint32_t* lastHost)
 {
-    if (lastHost != nullptr || n > kScanSingleLimit)
+    return lastHost != nullptr || n > kScanSingleLimit;
+}
+
+int ResolveCsrScratch(uint32_t** out)
+{
+    const int device = sph::CurrentDevice();
+    if (device < 0 || device >= kMaxScratchDevices)
+        return sph::Fail(SPH_ERR_INVALID, "ResolveCsrScratch - device id out of range");
+    std::lock_guard<std::mutex> lock(gScratchMutex);
+    if (gScratchPtr[device] == nullptr)
+    {
+        // every device holds its own copy of the array at its own address
+        SPH_HIP_TRY(hipSetDevice(device));
+        uint32_t* ptr = nullptr;
+        SPH_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+        if (ptr == nullptr)
+            return sph::Fail(SPH_ERR_DEVICE, "ResolveCsrScratch - null symbol address");
+        gScratchPtr[device] = ptr;
+    }
+    if (out != nullptr)
+        *out = gScratchPtr[device];
+    return SPH_OK;
+}
+
+int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStream_t stream,
+                         uint32_t* sums)
+{
+    if (lastHost != nullptr || (n > kScanSingleLimit && sums == nullptr))
         SPH_REFUSE_WHILE_CAPTURING();  // reads back, or takes a scratch allocation
     const uint32_t blocks = (n + kScanPerBlock - 1) / kScanPerBlock;
     if (n <= kScanSingleLimit)
@@ -367,17 +405,19 @@ int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStre
     }
     else
     {
-        // per-block totals live in a stream-ordered scratch allocation
-        uint32_t* sums = nullptr;
-        SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&sums), blocks * sizeof(uint32_t),
-                                   stream));
+        // per-block totals: the caller's workspace, or a stream-ordered scratch allocation
+        const bool own = sums == nullptr;
+        if (own)
+            SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&sums),
+                                       blocks * sizeof(uint32_t), stream));
         hipLaunchKernelGGL(ScanBlocksKernel, dim3(blocks), dim3(kScanThreads), 0, stream, data,
                            sums, n);
         hipLaunchKernelGGL(ScanSumsKernel, dim3(1), dim3(kScanThreads), 0, stream, sums, blocks);
         hipLaunchKernelGGL(AddBlockOffsetsKernel, dim3(blocks - 1), dim3(kScanThreads), 0, stream,
                            data, sums, n);
         const hipError_t launched = hipGetLastError();
-        SPH_HIP_TRY(hipFreeAsync(sums, stream));
+        if (own)
+            SPH_HIP_TRY(hipFreeAsync(sums, stream));
         if (launched != hipSuccess)
             return sph::Fail(SPH_ERR_DEVICE, std::string("exclusive scan launch failed with ") +
                                                  hipGetErrorString(launched));
@@ -401,6 +441,8 @@ int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint3
     SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
     SPH_REQUIRE(M < 0xffffffffu, "too many rows");
     SPH_REQUIRE(M == 0 || N == 0 || dense != nullptr, "dense is null");
+    if (sph::ScanWaitsOrAllocates(M + 1, nnzHost))
+        SPH_REFUSE_WHILE_CAPTURING();  // before anything is enqueued into the graph
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
@@ -411,6 +453,31 @@ int sph_csr_row_offsets_f32(uint32_t* ROW, const float* dense, uint32_t M, uint3
     SPH_CHECK_LAUNCH();
 
     return sph::ExclusiveScanInPlace(ROW, M + 1, nnzHost, stream);
+}
+
+int sph_csr_row_offsets_noalloc_f32(uint32_t* ROW, const float* dense, uint32_t M, uint32_t N,
+                                    uint32_t ld)
+{
+    SPH_REQUIRE(ROW != nullptr, "ROW is null");
+    SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
+    SPH_REQUIRE(M == 0 || N == 0 || dense != nullptr, "dense is null");
+    SPH_REQUIRE(M < static_cast<uint64_t>(kNoAllocMaxBlocks) * kScanPerBlock,
+                "more than 16777215 rows exceed the fixed scratch array");
+    uint32_t* sums = nullptr;
+    const int rc = sph::ResolveCsrScratch(&sums);
+    if (rc != SPH_OK)
+        return rc;
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+
+    const DenseView d = MakeView(dense, M, N, ld);
+    const int lanes = LanesPerRow(N);
+    DispatchLanes<CountLauncher>(lanes, RowGrid(M, lanes), stream, ROW, d);
+    SPH_CHECK_LAUNCH();
+
+    // every total the scan reads is written by the same call first: nothing has to be cleared
+    return sph::ExclusiveScanInPlace(ROW, M + 1, nullptr, stream, sums);
 }
 
 int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW, const float* dense, uint32_t M,

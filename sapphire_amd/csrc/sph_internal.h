@@ -27,7 +27,19 @@ int ComputeUnits();
 // Exclusive prefix sum of n 32-bit counts in place on `stream` (data[i] = sum of data[0..i)).
 // With lastHost the last element (the total, when the last count is 0) is copied to the host
 // and the stream is drained.
-int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStream_t stream);
+// Scans of more than ScanSingleLimit() values need one 32-bit total per 4096 values: taken from
+// `sums` when that is not null (device memory, at least ScanBlocks(n) entries, contents
+// irrelevant), from a stream-ordered allocation otherwise.
+int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStream_t stream,
+                         uint32_t* sums = nullptr);
+
+// True when ExclusiveScanInPlace(data, n, lastHost, stream) would read back or allocate, which
+// a stream under capture cannot record.  Entry points ask before they enqueue anything.
+bool ScanWaitsOrAllocates(uint32_t n, const uint32_t* lastHost);
+
+// Resolves, once per device, the address of the scratch array behind
+// sph_csr_row_offsets_noalloc_f32 on the calling thread's device.
+int ResolveCsrScratch(uint32_t** scratch);
 
 // True between sph_graph_begin_capture and sph_graph_end_capture on this thread.  Entry
 // points that must wait for the device or allocate refuse to run while it is set.

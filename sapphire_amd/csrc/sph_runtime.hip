@@ -358,6 +358,11 @@ int sph_graph_begin_capture(void)
     SPH_REQUIRE(!sph::Capturing(), "a capture is already in progress on this thread");
     // resolve everything that queries the device before the stream goes into capture
     (void)sph::ComputeUnits();
+    {
+        const int rc = sph::ResolveCsrScratch(nullptr);
+        if (rc != SPH_OK)
+            return rc;
+    }
     SPH_STREAM_OR_FAIL(stream);
     SPH_HIP_TRY(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
     tlsSlots.capturing = stream;

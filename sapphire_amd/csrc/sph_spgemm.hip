@@ -649,6 +649,8 @@ int sph_spgemm_row_offsets_f32(uint32_t* ROWC, const float* VA, const uint32_t* 
     SPH_REQUIRE(ROWC != nullptr && ROWA != nullptr, "null pointer");
     SPH_REQUIRE(M < 0xffffffffu, "too many rows");
     SPH_REQUIRE(K == 0 || ROWB != nullptr, "null pointer");
+    if (sph::ScanWaitsOrAllocates(M + 1, nnzHost))
+        SPH_REFUSE_WHILE_CAPTURING();  // before anything is enqueued into the graph
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
