@@ -13,6 +13,8 @@ steps (2*4096^3 flop each).  The same line carries
                 the stream the kernel runs on;
   spmm          the CSR x dense product of configuration 5 (8192 x 8192 at 1 % times
                 8192 x 256), timed the same way, against the HBM peak on algorithmic bytes;
+  configs       configurations 1, 2 and 4 (fp32 GEMM, batched fp32 GEMM with a shared B, the
+                3-layer MLP forward), each with its own roofline object;
   cpu_baseline  the reference's own scalar CPU GEMM (built into oracle/_ref from the
                 reference's NaiveGemm.cpp; the plain-C port when that build is absent) timed
                 on a bounded slice of the same workload on this machine's host cores.
@@ -56,7 +58,8 @@ def parse():
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     p.add_argument("--all", action="store_true",
-                   help="also time configurations 1, 2 and 4 (reported under 'others')")
+                   help="also time the neighbouring kernels (backward pass, conversions, CSR x "
+                        "CSR, one-pass kernels; reported under 'others')")
     p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
                                       "csr", "spgemm"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
@@ -460,7 +463,18 @@ def bench_copy(capi, steps, warmup, mib=64):
     return event_ms, 4 * n
 
 
-def cpu_gemm_baseline(d, rows=96):
+def f32_roofline(workload, entry, kernel, ms, flops, alg_bytes):
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"workload": workload, "entry_point": entry, "launch_ms": ms, "value": tf,
+            "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "kernel": kernel, "achieved": tf,
+                         "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tf / PEAK_FP32_TFLOPS, "flop_per_step": flops,
+                         "algorithmic_bytes_per_step": alg_bytes,
+                         "hbm_gbs_on_algorithmic_bytes": alg_bytes / (ms * 1e-3) / 1e9}}
+
+
+def cpu_gemm_baseline(d, rows=32):
     """The reference's scalar loop on rows [0, rows) of configuration 3 (inputs widened to fp32
     exactly), one thread, as the reference runs it."""
     from oracle import pyoracle as po
@@ -620,23 +634,43 @@ def main():
                                               "(the reference has no sparse x dense code), %.2f s" % dt}
         result["spmm"] = spmm
 
-    if args.all and args.only is None:
-        others = {}
+    if args.only is None:
+        # configurations 1, 2 and 4, each against the fp32 MFMA peak (configuration 1 is a
+        # single 33.6 MFLOP launch and is bound by launch latency, not by any roofline)
+        configs = {}
         c1 = synth.config1()
         ms = bench_f32(capi, c1["A"], c1["B"], c1["C"], 256, 256, 256, 1, 256 * 256, 1000, 50)
-        others["config1_f32_256"] = {"launch_ms": ms, "tflops": 2 * 256 ** 3 / (ms * 1e-3) / 1e12}
+        configs["config1_f32_256"] = f32_roofline(
+            "configuration 1: out[256,256] += A[256,256] * B[256,256] fp32, one launch",
+            "sph_gemm_f32", "GemmF32SkinnyKernel", ms, 2.0 * 256 ** 3, 4 * 4 * 256 * 256)
         c2 = synth.config2()
         ms = bench_f32(capi, c2["A"], c2["B"], c2["C"], 512, 512, 512, 16, 0, 200, 20)
-        tf = 16 * 2 * 512 ** 3 / (ms * 1e-3) / 1e12
-        others["config2_f32_batched"] = {"launch_ms": ms, "tflops": tf,
-                                         "frac_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
-        ms, fl = bench_mlp(capi, synth, 100, 10)
-        others["config4_mlp_forward"] = {"forward_ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
-                                         "kernels_per_forward": 11}
+        configs["config2_f32_batched"] = f32_roofline(
+            "configuration 2: out[16,512,512] += A[16,512,512] * B[1,512,512] fp32, B shared "
+            "(stride 0), one launch", "sph_gemm_f32", "GemmF32DmaKernel<64>", ms,
+            16 * 2.0 * 512 ** 3, 4 * 512 * 512 * (16 + 1 + 16 + 16))
+        c4 = synth.config4()
+        sizes = [c4["x"].shape[1]] + [w.shape[1] for w in c4["W"]]
+        batch = c4["x"].shape[0]
+        # x, W, bias read once, every layer's y written once and read once by the next layer
+        mlp_bytes = 4 * (batch * sizes[0] + sum(sizes[l] * sizes[l + 1] + sizes[l + 1]
+                                                for l in range(3))
+                         + batch * (2 * sizes[1] + 2 * sizes[2] + sizes[3]))
         ms, fl = bench_mlp(capi, synth, 100, 10, fused=True)
-        others["config4_mlp_forward_fused"] = {"forward_ms": ms,
-                                               "tflops": fl / (ms * 1e-3) / 1e12,
-                                               "kernels_per_forward": 3}
+        configs["config4_mlp_forward"] = f32_roofline(
+            "configuration 4: 3-layer MLP forward 784-1024-1024-10 on x[1024,784] fp32, bias and "
+            "ReLU fused into each layer's launch (3 launches per step)",
+            "sph_linear_forward_f32 x 3", "GemmF32DmaKernel / GemmF32SkinnyKernel (fused epilogue)",
+            ms, fl, mlp_bytes)
+        ms, fl = bench_mlp(capi, synth, 100, 10)
+        configs["config4_mlp_forward"]["reference_call_sequence"] = {
+            "note": "the reference's operator calls one for one: fill, K = 1 bias GEMM, GEMM, "
+                    "ReLU (11 launches per step); same result bits as the fused form",
+            "launch_ms": ms, "tflops": fl / (ms * 1e-3) / 1e12}
+        result["configs"] = configs
+
+    if args.all and args.only is None:
+        others = {}
         ms_ref, fl = bench_mlp_backward(capi, synth, 100, 10, direct=False)
         ms_dir, _ = bench_mlp_backward(capi, synth, 100, 10, direct=True)
         others["config4_mlp_backward_sgd"] = {
