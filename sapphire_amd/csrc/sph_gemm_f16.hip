@@ -17,9 +17,9 @@
 //     (global_load_lds, 16 bytes per lane, no VGPR staging), three to four
 //     steps ahead of the MFMAs.  LDS is written lane-linear by those copies,
 //     so bank conflicts are removed by choosing WHICH global chunk each lane
-//     fetches: A rows are XOR-swizzled in 16-byte chunks (chunk ^ row%8), B
+//     fetches: A rows are XOR-swizzled in 16-byte chunks (chunk ^ (row/2)%8), B
 //     rows in 32-byte chunks (chunk ^ 2*(k%4)); both patterns measured
-//     conflict-free for the reads below.
+//     conflict-free for the reads below (4.6 and 2.6 clocks per wavefront read).
 //     A fragments are read with ds_read_b128 (8 consecutive k of one row); B is
 //     stored k-major, so its fragments (8 consecutive k of one column) come
 //     from two ds_read_b64_tr_b16 transposing reads.  The MFMA operands are
@@ -158,7 +158,11 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     constexpr uint32_t kBias = 4096;       // keeps every lane offset non-negative
 
     // A stage: 128 LDS rows of 128 bytes; LDS row R holds A[R][k0..k0+31] in its first 64
-    // bytes and A[R+128][k0..k0+31] in the last 64, 16-byte chunks XOR-swizzled with R%8.
+    // bytes and A[R+128][k0..k0+31] in the last 64, 16-byte chunks XOR-swizzled with
+    // (R/2)%8: the LDS serves a 16-byte read to 16 lanes per clock from 64 banks, and 16
+    // consecutive 128-byte rows are 8 even ones on banks 0-31 and 8 odd ones on banks 32-63,
+    // so the 8 rows of either parity must take 8 different chunk positions (with R%8 they
+    // take 4, and every fragment read costs 8 clocks instead of 4).
     // B stage: 32 k-rows of 512 bytes, 32-byte chunks XOR-swizzled with 2*(k%4).
     __shared__ __attribute__((aligned(1024))) _Float16 Lds[2][kTStages][kStageHalfs];
     auto& As = Lds[0];
@@ -190,8 +194,8 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     // at w*WAVE_LDS of a stage in ROUNDS copies; copy r puts lane i's 16 bytes at
     // w*WAVE_LDS + r*1024 + i*16.
     //   A: that is LDS row R = w*8*ROUNDS + r*8 + i/8, physical chunk i%8, which must hold
-    //      logical chunk L = (i%8) ^ (R%8) = (i%8) ^ (i/8): matrix row R (L < 4) or R+128
-    //      (L >= 4), k offset (L%4)*8.
+    //      logical chunk L = (i%8) ^ ((R/2)%8): matrix row R (L < 4) or R+128 (L >= 4),
+    //      k offset (L%4)*8.
     //   B: k = w*2*ROUNDS + r*2 + i/32, physical 16-byte chunk i%32, 32-byte chunks
     //      swizzled with 2*(k%4).
     // The global address of a copy is a uniform base that advances with the K step plus a
@@ -199,12 +203,14 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     // both the LDS and the global address, so the lane offsets subtract it again.
     uint32_t aLane[ROUNDS], bLane[ROUNDS];
     {
-        const uint32_t aL = (lane & 7) ^ (lane >> 3);
-        const uint32_t aRow0 = wave * (8 * ROUNDS) + (lane >> 3) + ((aL & 4) ? 128u : 0u);
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r)
-            aLane[r] =
-                (min(aRow0 + 8 * r, rowsLeft - 1) * args.lda + (aL & 3) * 8) * 2 + kBias - r * 1024;
+        {
+            const uint32_t R = wave * (8 * ROUNDS) + 8 * r + (lane >> 3);
+            const uint32_t aL = (lane & 7) ^ ((R >> 1) & 7);
+            const uint32_t row = R + ((aL & 4) ? 128u : 0u);
+            aLane[r] = (min(row, rowsLeft - 1) * args.lda + (aL & 3) * 8) * 2 + kBias - r * 1024;
+        }
         const uint32_t phys16 = lane & 31;
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r)
@@ -243,7 +249,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     //   logical chunk waveM*4 + ks*2 + l/32.
     const uint32_t l32 = lane & 31;
     const uint32_t khalf = lane >> 5;
-    const uint32_t aSwz = l32 & 7;
+    const uint32_t aSwz = (l32 >> 1) & 7;
     const uint32_t aChunkBase = waveM * 4 + khalf;  // + ks*2
     // B fragment (column block j, sub-step ks): 16-lane group g = l/16, s = l%16;
     //   columns waveN*(32*TJ) + j*32 + 16*(g%2) + 4*(s%4)..+3,
