@@ -41,6 +41,7 @@
 // columns of A and to the general kernel for the rest (two launches).
 #include "sph_internal.h"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace
@@ -103,6 +104,21 @@ __device__ __forceinline__ uint32_t LdsAddress(const void* p)
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsPtr)(p)));
 }
 
+// 16-byte accesses to out with the streaming hint: the tile is read once and written once, so
+// it should neither displace the A and B panels in the L2 nor stay there dirty until the end of
+// the kernel.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 NtLoad4(const float* p)
+{
+    const floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(p));
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void NtStore4(float* p, float4 v)
+{
+    const floatx4 w = { v.x, v.y, v.z, v.w };
+    __builtin_nontemporal_store(w, reinterpret_cast<floatx4*>(p));
+}
+
 __device__ __forceinline__ halfx8 Join(halfx4 lo, halfx4 hi)
 {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -147,9 +163,16 @@ constexpr int kStageHalfs = kT * kTK;
 // RAGGED: M and N need not be multiples of 256 (N still a multiple of 8).  Rows past M and
 // 16-byte column chunks past N are clamped to the last valid ones when they are copied (they
 // feed only outputs that are never stored) and the epilogue skips what lies outside.
-template <int WAVES, bool RAGGED>
+// CLOOP (whole tiles, accumulating, at least kCLoopSteps K steps): the old contents of out are
+// not read in the epilogue, when every workgroup would ask for them at once, but during the
+// first K steps: every second step a wavefront has one of its eight 32 x 32 blocks copied
+// straight into a 4 KiB LDS mailbox in accumulator layout and, two steps later, adds it to
+// the accumulators of that block.  The epilogue then only stores.
+constexpr int kCLoopSteps = 20;
+template <int WAVES, bool RAGGED, bool CLOOP>
 __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args args)
 {
+    static_assert(!(CLOOP && RAGGED), "old values are added in the loop for whole tiles only");
     constexpr int WN = WAVES / 2;          // wavefront columns
     constexpr int TJ = 8 / WN;             // 32-column MFMA blocks per wavefront
     constexpr int ROUNDS = 16 / WAVES;     // copies per lane per operand per stage
@@ -165,6 +188,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     // take 4, and every fragment read costs 8 clocks instead of 4).
     // B stage: 32 k-rows of 512 bytes, 32-byte chunks XOR-swizzled with 2*(k%4).
     __shared__ __attribute__((aligned(1024))) _Float16 Lds[2][kTStages][kStageHalfs];
+    __shared__ __attribute__((aligned(1024))) float CMail[CLOOP ? WAVES * 1024 : 4];
     auto& As = Lds[0];
     auto& Bs = Lds[1];
 
@@ -386,35 +410,109 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
     for (int j = 0; j < TJ; ++j)
         bf0[j] = loadB(0, 0, j);
 
-    // one K step with its stage index known at compile time
-    auto step = [&](auto stageC, uint32_t kt) {
+    // one K step with its stage index known at compile time; EXTRA = vector memory
+    // operations other than stage copies issued since the first half of the step before
+    auto step = [&](auto stageC, uint32_t kt, auto extraC) {
         constexpr int cur = decltype(stageC)::value;
         constexpr int nxt = (cur + 1) % kTStages;
+        constexpr int EXTRA = decltype(extraC)::value;
         // first half: multiply sub-step 0, fetch sub-step 1, request B of step kt+3
         halfStep(af0, bf0, af1, bf1, cur, 1, kt + 3, (cur + 3) % kTStages, false);
         // step kt+1 has landed for every wavefront, and every wavefront is done reading
         // step kt, whose buffer now takes step kt+4
-        WaitVmem<2 * COPIES_PER_STAGE>();
+        WaitVmem<2 * COPIES_PER_STAGE + EXTRA>();
         __syncthreads();
         // second half: multiply sub-step 1, fetch sub-step 0 of step kt+1, request A of kt+4
         halfStep(af1, bf1, af0, bf0, nxt, 0, kt + 4, cur, true);
     };
 
-    for (uint32_t kt = 0;; kt += 4)
+    constexpr std::integral_constant<int, 0> kNoExtra{};
+    if constexpr (CLOOP)
     {
-        step(std::integral_constant<int, 0>{}, kt);
-        if (kt + 1 >= steps)
-            break;
-        step(std::integral_constant<int, 1>{}, kt + 1);
-        if (kt + 2 >= steps)
-            break;
-        step(std::integral_constant<int, 2>{}, kt + 2);
-        if (kt + 3 >= steps)
-            break;
-        step(std::integral_constant<int, 3>{}, kt + 3);
-        if (kt + 4 >= steps)
-            break;
+        // Block b = 2*i + j of this wavefront: register 4q + r of lane l is row i*32 + l%32,
+        // column j*32 + 8q + 4*(l/32) + r of its 128 x 64 part.  Copy q of a block moves, per
+        // lane, those 4 floats to mailbox + q*1024 + 16*l; the instruction offset 128*j + 32*q
+        // (added to both addresses) selects block column and q, so M0 takes it off again.
+        const uint32_t mail = LdsAddress(&CMail[0]) + waveU * 4096;
+        const uint32_t cLane0 = ((waveM * 128 + l32) * N + waveN * (32 * TJ) + 4 * khalf) * 4;
+        const uint32_t cRowStep = 32 * N * 4;
+        auto issueC = [&](auto bC) {
+            constexpr int b = decltype(bC)::value;
+            constexpr int i = b / TJ, j = b % TJ;
+            const uint32_t laneOff = cLane0 + i * cRowStep;
+            DmaToLds16<j * 128 + 0>(laneOff, out, mail + 0 * 992 - j * 128);
+            DmaToLds16<j * 128 + 32>(laneOff, out, mail + 1 * 992 - j * 128);
+            DmaToLds16<j * 128 + 64>(laneOff, out, mail + 2 * 992 - j * 128);
+            DmaToLds16<j * 128 + 96>(laneOff, out, mail + 3 * 992 - j * 128);
+        };
+        auto addC = [&](auto bC) {
+            constexpr int b = decltype(bC)::value;
+            constexpr int i = b / TJ, j = b % TJ;
+            const float* box = &CMail[wave * 1024 + lane * 4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const float4 c = *reinterpret_cast<const float4*>(box + q * 256);
+                acc[i][j][4 * q + 0] += c.x;
+                acc[i][j][4 * q + 1] += c.y;
+                acc[i][j][4 * q + 2] += c.z;
+                acc[i][j][4 * q + 3] += c.w;
+            }
+        };
+        // Step s = 2b requests block b; step s + 2 adds it.  Ahead of the mid-step wait of
+        // step s lie the stage copies counted there plus the 4 block copies of step s or s-1
+        // (while blocks are still being requested, s <= 15); ahead of the wait for block b at
+        // the start of step 2b + 2 lie the 8 stage copies of steps 2b and 2b + 1.
+        auto cStep = [&](auto stageC, auto sC) {
+            constexpr int st = decltype(sC)::value;
+            if constexpr (st % 2 == 0 && st >= 2 && st <= 2 * 4 * TJ)
+            {
+                WaitVmem<2 * COPIES_PER_STAGE>();
+                addC(std::integral_constant<int, st / 2 - 1>{});
+            }
+            if constexpr (st % 2 == 0 && st < 2 * 4 * TJ)
+                issueC(std::integral_constant<int, st / 2>{});
+            step(stageC, static_cast<uint32_t>(st),
+                 std::integral_constant<int, (st <= 2 * 4 * TJ - 1) ? 4 : 0>{});
+        };
+        static_assert(kCLoopSteps % 4 == 0 && kCLoopSteps > 2 * 4 * TJ, "prefix covers all blocks");
+        auto cRound = [&](auto rC) {
+            constexpr int r = decltype(rC)::value;
+            cStep(std::integral_constant<int, 0>{}, std::integral_constant<int, 4 * r + 0>{});
+            cStep(std::integral_constant<int, 1>{}, std::integral_constant<int, 4 * r + 1>{});
+            cStep(std::integral_constant<int, 2>{}, std::integral_constant<int, 4 * r + 2>{});
+            cStep(std::integral_constant<int, 3>{}, std::integral_constant<int, 4 * r + 3>{});
+        };
+        cRound(std::integral_constant<int, 0>{});
+        cRound(std::integral_constant<int, 1>{});
+        cRound(std::integral_constant<int, 2>{});
+        cRound(std::integral_constant<int, 3>{});
+        cRound(std::integral_constant<int, 4>{});
     }
+    auto regularSteps = [&](uint32_t first) {
+        for (uint32_t kt = first;; kt += 4)
+        {
+            step(std::integral_constant<int, 0>{}, kt, kNoExtra);
+            if (kt + 1 >= steps)
+                break;
+            step(std::integral_constant<int, 1>{}, kt + 1, kNoExtra);
+            if (kt + 2 >= steps)
+                break;
+            step(std::integral_constant<int, 2>{}, kt + 2, kNoExtra);
+            if (kt + 3 >= steps)
+                break;
+            step(std::integral_constant<int, 3>{}, kt + 3, kNoExtra);
+            if (kt + 4 >= steps)
+                break;
+        }
+    };
+    if constexpr (CLOOP)
+    {
+        if (steps > kCLoopSteps)
+            regularSteps(kCLoopSteps);
+    }
+    else
+        regularSteps(0);
 #undef SPH_FENCE
 
     // ---- epilogue -------------------------------------------------------------
@@ -470,7 +568,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
             {
                 old[t] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (exists(half, t))
-                    old[t] = *reinterpret_cast<const float4*>(outBlock + (half * 16 + t) * rowStep);
+                    old[t] = NtLoad4(outBlock + (half * 16 + t) * rowStep);
             }
         };
         auto storeHalf = [&](int half, const float4 (&old)[16], auto accumulate) {
@@ -494,7 +592,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         };
 
         float4 old[16];
-        if (args.overwrite)
+        if (CLOOP || args.overwrite)
         {
             stageHalf(0);
             storeHalf(0, old, std::false_type{});
@@ -1063,10 +1161,13 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
 
     if (tile256)
     {
-        if (whole256)
-            hipLaunchKernelGGL((GemmF16Tile256<8, false>), dim3(grid), dim3(512), 0, stream, args);
+        static const bool cloopOff = std::getenv("SPH_F16_NO_CLOOP") != nullptr;
+        if (whole256 && !args.overwrite && K / kTK >= kCLoopSteps && !cloopOff)
+            hipLaunchKernelGGL((GemmF16Tile256<8, false, true>), dim3(grid), dim3(512), 0, stream, args);
+        else if (whole256)
+            hipLaunchKernelGGL((GemmF16Tile256<8, false, false>), dim3(grid), dim3(512), 0, stream, args);
         else
-            hipLaunchKernelGGL((GemmF16Tile256<8, true>), dim3(grid), dim3(512), 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Tile256<8, true, false>), dim3(grid), dim3(512), 0, stream, args);
     }
     else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
              (!transA || (M % 8 == 0 && M >= 8)) &&

@@ -24,13 +24,19 @@ def _oracle(C, A16, B16, M, N, K, batch=1, sa=None, sb=None):
 
 # the 256-tile kernel is chosen from 192 tiles up (three quarters of the compute units): the
 # batch count brings these small shapes there
+# from 20 K steps up (K >= 640) the accumulating launch adds the old contents of out during the
+# first steps of the loop instead of in the epilogue: K = 640 (no step after the prefix), 672,
+# 704 (one and two steps after it) and longer
 @pytest.mark.parametrize("shape", [(256, 256, 64, 192), (256, 512, 128, 96), (512, 256, 192, 96),
-                                   (768, 1024, 256, 16), (4096, 3072, 32, 1)])
+                                   (768, 1024, 256, 16), (4096, 3072, 32, 1), (256, 256, 640, 192),
+                                   (4096, 3072, 672, 1), (512, 256, 704, 96), (1024, 768, 1280, 16),
+                                   (256, 512, 608, 96)])
 def test_tile256_exact_on_integers(dev, shape):
     M, N, K, batch = shape
     h.announce("sph_gemm_f16f32 tile256 integer exactness", shape)
-    A = synth.small_integers(1, (batch, M, K)).astype(np.float16)
-    B = synth.small_integers(2, (batch, K, N)).astype(np.float16)
+    span = 4 if K <= 256 else 3      # every partial sum stays an exact fp32 integer
+    A = synth.small_integers(1, (batch, M, K), span=span).astype(np.float16)
+    B = synth.small_integers(2, (batch, K, N), span=span).astype(np.float16)
     C = synth.small_integers(3, (batch, M, N), span=100)
     ref = _oracle(C, A, B, M, N, K, batch=batch)
     got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch)
@@ -188,7 +194,16 @@ def test_config3_4096_cubed(dev):
     twice = dC.download(np.float32, got.shape)
     for x in (dA, dB, dC):
         x.release()
-    assert np.array_equal(twice, got + got)
+    # the old contents join the sum during the first K steps, so out + A*B is associated
+    # differently from "sum, then one add": equal within the accumulation error, not bit for bit
+    assert h.normalised_error(twice, got + got, None, den.astype(np.float64), True) <= 1e-5
+    # real-valued out of the size of the product
+    C = synth.uniform(91, (n, n))
+    ref = _oracle(C, d["A"], d["B"], n, n, n)
+    got = h.gpu_gemm_f16(C, d["A"], d["B"], n, n, n)
+    err = h.normalised_error(got, ref, None, den.astype(np.float64) + np.abs(C), True)
+    assert err <= TOL_F16, err
+    assert float(np.max(np.abs(got - ref))) <= 1e-4
 
 
 def test_convert_f32_to_f16_matches_numpy_rounding(dev):
