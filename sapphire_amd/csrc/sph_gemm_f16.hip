@@ -168,10 +168,17 @@ constexpr int kStageHalfs = kT * kTK;
 // first K steps: every second step a wavefront has one of its eight 32 x 32 blocks copied
 // straight into a 4 KiB LDS mailbox in accumulator layout and, two steps later, adds it to
 // the accumulators of that block.  The epilogue then only stores.
-constexpr int kCLoopSteps = 20;
-template <int WAVES, bool RAGGED, bool CLOOP>
+// CSP = K steps between two blocks (0 = the epilogue reads out); the prefix that handles the 8
+// blocks is written out step by step and takes CLoopSteps(CSP) steps.
+constexpr int CLoopSteps(int csp)
+{
+    return (8 * csp + 1 + 3) / 4 * 4;
+}
+template <int WAVES, bool RAGGED, int CSP>
 __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args args)
 {
+    constexpr bool CLOOP = CSP != 0;
+    constexpr int kCLoopSteps = CLoopSteps(CSP);
     static_assert(!(CLOOP && RAGGED), "old values are added in the loop for whole tiles only");
     constexpr int WN = WAVES / 2;          // wavefront columns
     constexpr int TJ = 8 / WN;             // 32-column MFMA blocks per wavefront
@@ -459,35 +466,54 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
                 acc[i][j][4 * q + 3] += c.w;
             }
         };
-        // Step s = 2b requests block b; step s + 2 adds it.  Ahead of the mid-step wait of
-        // step s lie the stage copies counted there plus the 4 block copies of step s or s-1
-        // (while blocks are still being requested, s <= 15); ahead of the wait for block b at
-        // the start of step 2b + 2 lie the 8 stage copies of steps 2b and 2b + 1.
+        // Step s = CSP*b requests block b; step s + CSP adds it.  Ahead of the mid-step wait
+        // of step s lie the stage copies counted there plus the 4 block copies of step s or
+        // s-1, if one of the two requested a block; ahead of the wait for block b at the start
+        // of step CSP*(b+1) lie the stage copies of the CSP steps since its request.
+        constexpr int kBlocks = 4 * TJ;
         auto cStep = [&](auto stageC, auto sC) {
             constexpr int st = decltype(sC)::value;
-            if constexpr (st % 2 == 0 && st >= 2 && st <= 2 * 4 * TJ)
+            constexpr bool requests = st % CSP == 0 && st / CSP < kBlocks;
+            constexpr bool requestedBefore = st >= 1 && (st - 1) % CSP == 0 && (st - 1) / CSP < kBlocks;
+            if constexpr (st % CSP == 0 && st >= CSP && st / CSP <= kBlocks)
             {
-                WaitVmem<2 * COPIES_PER_STAGE>();
-                addC(std::integral_constant<int, st / 2 - 1>{});
+                WaitVmem<CSP * COPIES_PER_STAGE>();
+                addC(std::integral_constant<int, st / CSP - 1>{});
             }
-            if constexpr (st % 2 == 0 && st < 2 * 4 * TJ)
-                issueC(std::integral_constant<int, st / 2>{});
+            if constexpr (requests)
+                issueC(std::integral_constant<int, requests ? st / CSP : 0>{});
             step(stageC, static_cast<uint32_t>(st),
-                 std::integral_constant<int, (st <= 2 * 4 * TJ - 1) ? 4 : 0>{});
+                 std::integral_constant<int, (requests || requestedBefore) ? 4 : 0>{});
         };
-        static_assert(kCLoopSteps % 4 == 0 && kCLoopSteps > 2 * 4 * TJ, "prefix covers all blocks");
+        static_assert(CSP * COPIES_PER_STAGE <= 63, "vmcnt holds 6 bits");
         auto cRound = [&](auto rC) {
             constexpr int r = decltype(rC)::value;
-            cStep(std::integral_constant<int, 0>{}, std::integral_constant<int, 4 * r + 0>{});
-            cStep(std::integral_constant<int, 1>{}, std::integral_constant<int, 4 * r + 1>{});
-            cStep(std::integral_constant<int, 2>{}, std::integral_constant<int, 4 * r + 2>{});
-            cStep(std::integral_constant<int, 3>{}, std::integral_constant<int, 4 * r + 3>{});
+            if constexpr (4 * r < kCLoopSteps)
+            {
+                cStep(std::integral_constant<int, 0>{}, std::integral_constant<int, 4 * r + 0>{});
+                cStep(std::integral_constant<int, 1>{}, std::integral_constant<int, 4 * r + 1>{});
+                cStep(std::integral_constant<int, 2>{}, std::integral_constant<int, 4 * r + 2>{});
+                cStep(std::integral_constant<int, 3>{}, std::integral_constant<int, 4 * r + 3>{});
+            }
         };
+        static_assert(kCLoopSteps <= 4 * 17, "rounds written out below");
         cRound(std::integral_constant<int, 0>{});
         cRound(std::integral_constant<int, 1>{});
         cRound(std::integral_constant<int, 2>{});
         cRound(std::integral_constant<int, 3>{});
         cRound(std::integral_constant<int, 4>{});
+        cRound(std::integral_constant<int, 5>{});
+        cRound(std::integral_constant<int, 6>{});
+        cRound(std::integral_constant<int, 7>{});
+        cRound(std::integral_constant<int, 8>{});
+        cRound(std::integral_constant<int, 9>{});
+        cRound(std::integral_constant<int, 10>{});
+        cRound(std::integral_constant<int, 11>{});
+        cRound(std::integral_constant<int, 12>{});
+        cRound(std::integral_constant<int, 13>{});
+        cRound(std::integral_constant<int, 14>{});
+        cRound(std::integral_constant<int, 15>{});
+        cRound(std::integral_constant<int, 16>{});
     }
     auto regularSteps = [&](uint32_t first) {
         for (uint32_t kt = first;; kt += 4)
@@ -603,6 +629,396 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args a
         {
             // the old contents of a half are requested in one batch, in flight while its
             // accumulators are staged
+            loadOld(0, old);
+            stageHalf(0);
+            storeHalf(0, old, std::true_type{});
+            loadOld(1, old);
+            stageHalf(1);
+            storeHalf(1, old, std::true_type{});
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// 256 x 256 tile on v_mfma_f32_16x16x32_f16
+// ---------------------------------------------------------------------------
+// The same tile, stages, copies and epilogue as GemmF16Tile256, multiplied with the 16x16x32
+// instruction: a wavefront's 128 x 64 part is 8 x 4 blocks of 16 x 16 (4 accumulator registers
+// each) and a K step of 32 is one instruction deep.  Every accumulator is read and written
+// once per 32 products instead of once per 16, and under the power limit that bounds this
+// kernel on real operands the deeper instruction delivers about a tenth more (matrix cores fed
+// from LDS only, N(0, 1/64) operands: 72.8 against 80.6 us for the flops of 4096^3).
+//   A fragment i (rows 16i..16i+15 of the wavefront's 128): lane l holds row l%16, k 8*(l/16)..+7:
+//     one 16-byte LDS read from the A stage layout described above.
+//   B fragment j (columns 16j..16j+15 of its 64): lane l holds column l%16, k 8*(l/16)..+7: two
+//     transposing reads, each 16-lane group g reading the 4 x 16 block at k = 8g + 4h.  The
+//     32-byte chunks of a k-row are XOR-swizzled with 2*(k%4) + (k/8)%2, so that the two groups
+//     served in one clock (k and k + 8) fall on different banks.
+//   With the operands swapped, register v of lane l is row l%16, column 4*(l/16) + v of a block.
+// A step is split by rows: blocks 0-3 before the barrier, 4-7 after it.  The A fragments of a
+// step's second half are read during its first half; behind the barrier the first half's A
+// registers take the next step's rows 0-63 and a second set of B registers its B fragments.
+template <bool RAGGED, int CSP>
+__global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
+{
+    constexpr int WAVES = 8;
+    constexpr int ROUNDS = 2;               // copies per lane per operand per stage
+    constexpr int WAVE_LDS = ROUNDS * 1024;
+    constexpr int COPIES_PER_STAGE = 2 * ROUNDS;
+    constexpr uint32_t kBias = 4096;
+    constexpr bool CLOOP = CSP != 0;
+    constexpr int kCLoopSteps = CLoopSteps(CSP);
+    static_assert(!(CLOOP && RAGGED), "old values are added in the loop for whole tiles only");
+
+    __shared__ __attribute__((aligned(1024))) _Float16 Lds[2][kTStages][kStageHalfs];
+    __shared__ __attribute__((aligned(1024))) float CMail[CLOOP ? WAVES * 1024 : 4];
+    auto& As = Lds[0];
+    auto& Bs = Lds[1];
+
+    uint32_t unit, tm, tn;
+    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
+        return;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t waveM = wave >> 2;  // 0..1 -> 128 rows each
+    const uint32_t waveN = wave & 3;   // 0..3 -> 64 columns each
+
+    const uint32_t K = args.K, N = args.N;
+    const uint32_t rowsLeft = RAGGED ? min(static_cast<uint32_t>(kT), args.M - tm * kT) : kT;
+    const uint32_t colsLeft = RAGGED ? min(static_cast<uint32_t>(kT), N - tn * kT) : kT;
+    const _Float16* __restrict__ A =
+        args.A + args.strideA * static_cast<int64_t>(unit) + static_cast<size_t>(tm) * kT * args.lda;
+    const _Float16* __restrict__ B =
+        args.B + args.strideB * static_cast<int64_t>(unit) + static_cast<size_t>(tn) * kT;
+    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit) +
+                              static_cast<size_t>(tm) * kT * N + static_cast<size_t>(tn) * kT;
+
+    // ---- global -> LDS copy plan (as in GemmF16Tile256; B rows with the swizzle above) ----
+    uint32_t aLane[ROUNDS], bLane[ROUNDS];
+    {
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r)
+        {
+            const uint32_t R = wave * (8 * ROUNDS) + 8 * r + (lane >> 3);
+            const uint32_t aL = (lane & 7) ^ ((R >> 1) & 7);
+            const uint32_t row = R + ((aL & 4) ? 128u : 0u);
+            aLane[r] = (min(row, rowsLeft - 1) * args.lda + (aL & 3) * 8) * 2 + kBias - r * 1024;
+        }
+        const uint32_t phys16 = lane & 31;
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r)
+        {
+            const uint32_t k = wave * (2 * ROUNDS) + r * 2 + (lane >> 5);
+            const uint32_t swz = 2 * (k & 3) + ((k >> 3) & 1);
+            const uint32_t logical16 = (((phys16 >> 1) ^ swz) << 1) | (phys16 & 1);
+            bLane[r] = (k * N + min(logical16 * 8, colsLeft - 8)) * 2 + kBias - r * 1024;
+        }
+    }
+    const uint32_t waveU = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t aLds = LdsAddress(&As[0][0]) + waveU * WAVE_LDS;
+    const uint32_t bLds = LdsAddress(&Bs[0][0]) + waveU * WAVE_LDS;
+    const char* aGlobal = reinterpret_cast<const char*>(A) - kBias;
+    const char* bGlobal = reinterpret_cast<const char*>(B) - kBias;
+    const size_t bStepBytes = static_cast<size_t>(kTK) * N * 2;
+
+    const uint32_t steps = K / kTK;
+    auto copyA = [&](uint32_t kt, int stage, auto round) {
+        constexpr int r = decltype(round)::value;
+        const uint32_t src = min(kt, steps - 1);
+        DmaToLds16<r * 1024>(aLane[r], aGlobal + static_cast<size_t>(src) * (kTK * 2),
+                             aLds + stage * kStageBytes);
+    };
+    auto copyB = [&](uint32_t kt, int stage, auto round) {
+        constexpr int r = decltype(round)::value;
+        const uint32_t src = min(kt, steps - 1);
+        DmaToLds16<r * 1024>(bLane[r], bGlobal + static_cast<size_t>(src) * bStepBytes,
+                             bLds + stage * kStageBytes);
+    };
+
+    // ---- LDS -> fragment read plan ---------------------------------------------------
+    const uint32_t l16 = lane & 15;
+    const uint32_t g = lane >> 4;
+    // A: LDS row 16i + l16, half waveM of it, logical chunk waveM*4 + g, swizzle (row/2)%8
+    const uint32_t aOff = l16 * 64 + (((waveM * 4 + g) ^ ((l16 >> 1) & 7)) * 8);  // + i*16*64
+    // B: k-row 8g + 4h + l16/4, 32-byte chunk waveN*4 + j swizzled, halves 4*(l16%4)..+3 of it
+    uint32_t bOff[4];
+    {
+        const uint32_t kRow = 8 * g + (l16 >> 2);
+        const uint32_t swz = 2 * ((l16 >> 2) & 3) + (g & 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            bOff[j] = kRow * kT + (((waveN * 4 + j) ^ swz) * 16) + (l16 & 3) * 4;
+    }
+    auto loadA = [&](int stage, int i) {
+        return *reinterpret_cast<const halfx8*>(&As[stage][aOff + i * 16 * 64]);
+    };
+    auto loadB = [&](int stage, int j) {
+        const _Float16* p = &Bs[stage][bOff[j]];
+        return Join(LdsReadTr(p), LdsReadTr(p + 4 * kT));
+    };
+
+    floatx4 acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            acc[i][j] = floatx4{ 0.f, 0.f, 0.f, 0.f };
+
+#define SPH_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+#pragma unroll
+    for (int st = 0; st < 3; ++st)
+    {
+        copyA(st, st, std::integral_constant<int, 0>{});
+        copyA(st, st, std::integral_constant<int, 1>{});
+        copyB(st, st, std::integral_constant<int, 0>{});
+        copyB(st, st, std::integral_constant<int, 1>{});
+    }
+    copyA(3, 3, std::integral_constant<int, 0>{});
+    copyA(3, 3, std::integral_constant<int, 1>{});
+    // stage 0 is followed by 2.5 stages' worth of copies
+    WaitVmem<(5 * COPIES_PER_STAGE) / 2>();
+    __syncthreads();
+
+    halfx8 af[8], bf0[4], bf1[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        af[i] = loadA(0, i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        bf0[j] = loadB(0, j);
+
+    // One K step, stage index known at compile time.  BF holds this step's B fragments, BFN
+    // receives the next step's.  EXTRA = vector memory operations other than stage copies
+    // issued since the first half of the step before.
+    auto stepWith = [&](auto stageC, uint32_t kt, auto extraC, const halfx8 (&BF)[4],
+                        halfx8 (&BFN)[4]) {
+        constexpr int cur = decltype(stageC)::value;
+        constexpr int nxt = (cur + 1) % kTStages;
+        constexpr int EXTRA = decltype(extraC)::value;
+        // first half: rows 0-63, fetch this step's rows 64-127, request B of step kt+3
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(BF[j], af[i], acc[i][j], 0, 0, 0);
+                SPH_FENCE();
+                if (i < 2 && (j & 1) == 0)
+                    af[4 + 2 * i + j / 2] = loadA(cur, 4 + 2 * i + j / 2);
+                SPH_FENCE();
+            }
+            if (i == 1)
+                copyB(kt + 3, (cur + 3) % kTStages, std::integral_constant<int, 0>{});
+            if (i == 3)
+                copyB(kt + 3, (cur + 3) % kTStages, std::integral_constant<int, 1>{});
+            SPH_FENCE();
+        }
+        // step kt+1 has landed for every wavefront, and every wavefront is done reading
+        // step kt, whose A buffer now takes step kt+4
+        WaitVmem<2 * COPIES_PER_STAGE + EXTRA>();
+        __syncthreads();
+        // second half: rows 64-127, fetch the next step's rows 0-63 and B, request A of kt+4
+#pragma unroll
+        for (int i = 4; i < 8; ++i)
+        {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(BF[j], af[i], acc[i][j], 0, 0, 0);
+                SPH_FENCE();
+                if (i < 6)
+                {
+                    if ((j & 1) == 0)
+                        af[2 * (i - 4) + j / 2] = loadA(nxt, 2 * (i - 4) + j / 2);
+                    else
+                        BFN[2 * (i - 4) + j / 2] = loadB(nxt, 2 * (i - 4) + j / 2);
+                }
+                SPH_FENCE();
+            }
+            if (i == 5)
+                copyA(kt + 4, cur, std::integral_constant<int, 0>{});
+            if (i == 7)
+                copyA(kt + 4, cur, std::integral_constant<int, 1>{});
+            SPH_FENCE();
+        }
+    };
+    auto step = [&](auto stageC, uint32_t kt, auto extraC) {
+        if constexpr (decltype(stageC)::value % 2 == 0)
+            stepWith(stageC, kt, extraC, bf0, bf1);
+        else
+            stepWith(stageC, kt, extraC, bf1, bf0);
+    };
+
+    constexpr std::integral_constant<int, 0> kNoExtra{};
+    if constexpr (CLOOP)
+    {
+        // Row block i of this wavefront (16 rows x 64 columns = 4 accumulator blocks): copy j
+        // moves, per lane, the 4 floats of block (i, j) to mailbox + j*1024 + 16*l; the
+        // instruction offset 64*j (added to both addresses) selects the block, so M0 takes it
+        // off again.
+        const uint32_t mail = LdsAddress(&CMail[0]) + waveU * 4096;
+        const uint32_t cLane0 = ((waveM * 128 + l16) * N + waveN * 64 + 4 * g) * 4;
+        const uint32_t cRowStep = 16 * N * 4;
+        auto issueC = [&](auto bC) {
+            constexpr int i = decltype(bC)::value;
+            const uint32_t laneOff = cLane0 + i * cRowStep;
+            DmaToLds16<0>(laneOff, out, mail);
+            DmaToLds16<64>(laneOff, out, mail + 960);
+            DmaToLds16<128>(laneOff, out, mail + 2 * 960);
+            DmaToLds16<192>(laneOff, out, mail + 3 * 960);
+        };
+        auto addC = [&](auto bC) {
+            constexpr int i = decltype(bC)::value;
+            const float* box = &CMail[wave * 1024 + lane * 4];
+            // two blocks at a time: the four reads at once would not fit the register budget
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                const float4 c = *reinterpret_cast<const float4*>(box + j * 256);
+                acc[i][j][0] += c.x;
+                acc[i][j][1] += c.y;
+                acc[i][j][2] += c.z;
+                acc[i][j][3] += c.w;
+                if (j == 1)
+                    SPH_FENCE();
+            }
+        };
+        // Step s = CSP*b requests row block b; step s + CSP adds it (vmcnt accounting as in
+        // GemmF16Tile256).
+        constexpr int kBlocks = 8;
+        auto cStep = [&](auto stageC, auto sC) {
+            constexpr int st = decltype(sC)::value;
+            constexpr bool requests = st % CSP == 0 && st / CSP < kBlocks;
+            constexpr bool requestedBefore = st >= 1 && (st - 1) % CSP == 0 && (st - 1) / CSP < kBlocks;
+            if constexpr (st % CSP == 0 && st >= CSP && st / CSP <= kBlocks)
+            {
+                WaitVmem<CSP * COPIES_PER_STAGE>();
+                addC(std::integral_constant<int, st / CSP - 1>{});
+            }
+            if constexpr (requests)
+                issueC(std::integral_constant<int, requests ? st / CSP : 0>{});
+            step(stageC, static_cast<uint32_t>(st),
+                 std::integral_constant<int, (requests || requestedBefore) ? 4 : 0>{});
+        };
+        static_assert(CSP * COPIES_PER_STAGE <= 63, "vmcnt holds 6 bits");
+        auto cRound = [&](auto rC) {
+            constexpr int r = decltype(rC)::value;
+            if constexpr (4 * r < kCLoopSteps)
+            {
+                cStep(std::integral_constant<int, 0>{}, std::integral_constant<int, 4 * r + 0>{});
+                cStep(std::integral_constant<int, 1>{}, std::integral_constant<int, 4 * r + 1>{});
+                cStep(std::integral_constant<int, 2>{}, std::integral_constant<int, 4 * r + 2>{});
+                cStep(std::integral_constant<int, 3>{}, std::integral_constant<int, 4 * r + 3>{});
+            }
+        };
+        static_assert(kCLoopSteps <= 4 * 9, "rounds written out below");
+        cRound(std::integral_constant<int, 0>{});
+        cRound(std::integral_constant<int, 1>{});
+        cRound(std::integral_constant<int, 2>{});
+        cRound(std::integral_constant<int, 3>{});
+        cRound(std::integral_constant<int, 4>{});
+        cRound(std::integral_constant<int, 5>{});
+        cRound(std::integral_constant<int, 6>{});
+        cRound(std::integral_constant<int, 7>{});
+        cRound(std::integral_constant<int, 8>{});
+    }
+    auto regularSteps = [&](uint32_t first) {
+        for (uint32_t kt = first;; kt += 4)
+        {
+            step(std::integral_constant<int, 0>{}, kt, kNoExtra);
+            if (kt + 1 >= steps)
+                break;
+            step(std::integral_constant<int, 1>{}, kt + 1, kNoExtra);
+            if (kt + 2 >= steps)
+                break;
+            step(std::integral_constant<int, 2>{}, kt + 2, kNoExtra);
+            if (kt + 3 >= steps)
+                break;
+            step(std::integral_constant<int, 3>{}, kt + 3, kNoExtra);
+            if (kt + 4 >= steps)
+                break;
+        }
+    };
+    if constexpr (CLOOP)
+    {
+        if (steps > kCLoopSteps)
+            regularSteps(kCLoopSteps);
+    }
+    else
+        regularSteps(0);
+#undef SPH_FENCE
+
+    // ---- epilogue: as in GemmF16Tile256, 64 rows at a time through a private 16 KiB of LDS ----
+    WaitVmem<0>();
+    __syncthreads();
+    {
+        float* stage = reinterpret_cast<float*>(&Lds[0][0][0]) + wave * (64 * 64);
+        const uint32_t rdRow = lane >> 4;        // + 4*t
+        const uint32_t rdChunk = lane & 15;
+        float* outBlock = out + static_cast<size_t>(waveM * 128 + rdRow) * N + waveN * 64 + rdChunk * 4;
+        const size_t rowStep = static_cast<size_t>(4) * N;
+        const uint32_t rowFirst = waveM * 128 + rdRow;
+        const bool colExists = !RAGGED || waveN * 64 + rdChunk * 4 < colsLeft;
+        auto exists = [&](int half, int t) {
+            return !RAGGED || (colExists && rowFirst + 4 * (half * 16 + t) < rowsLeft);
+        };
+        auto stageHalf = [&](int half) {
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    const int i = half * 4 + ii;
+                    const uint32_t row = ii * 16 + l16;
+                    const uint32_t chunk = (j * 4 + g) ^ (row & 15);
+                    *reinterpret_cast<float4*>(&stage[row * 64 + chunk * 4]) =
+                        make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        };
+        auto loadOld = [&](int half, float4 (&old)[16]) {
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
+            {
+                old[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (exists(half, t))
+                    old[t] = NtLoad4(outBlock + (half * 16 + t) * rowStep);
+            }
+        };
+        auto storeHalf = [&](int half, const float4 (&old)[16], auto accumulate) {
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
+            {
+                const uint32_t r = rdRow + 4 * t;
+                float4 v = *reinterpret_cast<const float4*>(
+                    &stage[r * 64 + ((rdChunk ^ (r & 15)) * 4)]);
+                if constexpr (decltype(accumulate)::value)
+                {
+                    v.x += old[t].x;
+                    v.y += old[t].y;
+                    v.z += old[t].z;
+                    v.w += old[t].w;
+                }
+                if (exists(half, t))
+                    *reinterpret_cast<float4*>(outBlock + (half * 16 + t) * rowStep) = v;
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        };
+
+        float4 old[16];
+        if (CLOOP || args.overwrite)
+        {
+            stageHalf(0);
+            storeHalf(0, old, std::false_type{});
+            stageHalf(1);
+            storeHalf(1, old, std::false_type{});
+        }
+        else
+        {
             loadOld(0, old);
             stageHalf(0);
             storeHalf(0, old, std::true_type{});
@@ -1161,13 +1577,24 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
 
     if (tile256)
     {
-        static const bool cloopOff = std::getenv("SPH_F16_NO_CLOOP") != nullptr;
-        if (whole256 && !args.overwrite && K / kTK >= kCLoopSteps && !cloopOff)
-            hipLaunchKernelGGL((GemmF16Tile256<8, false, true>), dim3(grid), dim3(512), 0, stream, args);
+        static const bool m32 = std::getenv("SPH_F16_M32") != nullptr;
+        const bool cloop = whole256 && !args.overwrite && K / kTK >= CLoopSteps(4);
+        const dim3 g(grid), b(512);
+        if (m32)
+        {
+            if (cloop)
+                hipLaunchKernelGGL((GemmF16Tile256<8, false, 4>), g, b, 0, stream, args);
+            else if (whole256)
+                hipLaunchKernelGGL((GemmF16Tile256<8, false, 0>), g, b, 0, stream, args);
+            else
+                hipLaunchKernelGGL((GemmF16Tile256<8, true, 0>), g, b, 0, stream, args);
+        }
+        else if (cloop)
+            hipLaunchKernelGGL((GemmF16Tile256K32<false, 4>), g, b, 0, stream, args);
         else if (whole256)
-            hipLaunchKernelGGL((GemmF16Tile256<8, false, false>), dim3(grid), dim3(512), 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Tile256K32<false, 0>), g, b, 0, stream, args);
         else
-            hipLaunchKernelGGL((GemmF16Tile256<8, true, false>), dim3(grid), dim3(512), 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Tile256K32<true, 0>), g, b, 0, stream, args);
     }
     else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
              (!transA || (M % 8 == 0 && M >= 8)) &&
