@@ -1,6 +1,5 @@
 // fp16-input / fp32-accumulate GEMM  out[u] (+)= A[u] * B[u]  on the CDNA4
-// matrix cores (v_mfma_f32_32x32x16_f16).  This is the tensor-core path the
-// reference only declares (WmmaGemm,
+// matrix cores.  This is the tensor-core path the reference only declares (WmmaGemm,
 // Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50): half
 // inputs, fp32 accumulation, row-major operands, result added into out.
 //
@@ -9,29 +8,27 @@
 //   GemmF16Tile256  K a multiple of 32, N of 8, 16-byte aligned rows, at least three
 //     quarters as many 256 x 256 tiles as compute units and at least three quarters of
 //     the tiled area inside the matrix (a variant with clamped copies and a guarded
-//     epilogue serves M, N that are not multiples of 256).  One
-//     workgroup of 8 wavefronts (2 x 4) owns a 256 x 256 output tile; each
-//     wavefront a 128 x 64 part of it (4 x 2 MFMA tiles, 128 accumulator
-//     registers).  K advances 32 at a time through four LDS stages of 32 KiB
-//     (A 256x32, B 32x256).  Global memory is copied straight into LDS
-//     (global_load_lds, 16 bytes per lane, no VGPR staging), three to four
-//     steps ahead of the MFMAs.  LDS is written lane-linear by those copies,
-//     so bank conflicts are removed by choosing WHICH global chunk each lane
-//     fetches: A rows are XOR-swizzled in 16-byte chunks (chunk ^ (row/2)%8), B
-//     rows in 32-byte chunks (chunk ^ 2*(k%4)); both patterns measured
+//     epilogue serves M, N that are not multiples of 256).  One workgroup of 8 wavefronts
+//     (2 x 4) owns a 256 x 256 output tile; each wavefront a 128 x 64 part of it: 8 x 4
+//     blocks of v_mfma_f32_16x16x32_f16, 128 accumulator registers.  K advances 32 at a
+//     time through four LDS stages of 32 KiB (A 256x32, B 32x256).  Global memory is
+//     copied straight into LDS (global_load_lds, 16 bytes per lane, no VGPR staging),
+//     three to four steps ahead of the MFMAs.  LDS is written lane-linear by those
+//     copies, so bank conflicts are removed by choosing WHICH global chunk each lane
+//     fetches: A rows are XOR-swizzled in 16-byte chunks (chunk ^ (row/2)%8), B k-rows
+//     in 32-byte chunks (chunk ^ (2*(k%4) + (k/8)%2)); both patterns measured
 //     conflict-free for the reads below (4.6 and 2.6 clocks per wavefront read).
-//     A fragments are read with ds_read_b128 (8 consecutive k of one row); B is
-//     stored k-major, so its fragments (8 consecutive k of one column) come
-//     from two ds_read_b64_tr_b16 transposing reads.  The MFMA operands are
-//     swapped (B fragment first) so that every lane ends up with 4 consecutive
-//     columns of one output row and the epilogue moves 16 bytes per access.
-//     Workgroup ids are remapped so that the 32 workgroups that land on one
-//     XCD (ids congruent mod 8) cover a compact 8 x 4 block of tiles and share
-//     their A and B panels through that XCD's L2.
+//     A fragments are read with ds_read_b128 (8 consecutive k of one row); B is stored
+//     k-major, so its fragments (8 consecutive k of one column) come from two
+//     ds_read_b64_tr_b16 transposing reads.  The MFMA operands are swapped (B fragment
+//     first) so that every lane ends up with 4 consecutive columns of one output row
+//     and the epilogue moves 16 bytes per access.  Workgroup ids are remapped so that
+//     the 32 workgroups that land on one XCD (ids congruent mod 8) cover a compact
+//     8 x 4 block of tiles and share their A and B panels through that XCD's L2.
 //
 //   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned, any M: the
-//     same ingredients on 128 x 128 tiles with 4 wavefronts, for shapes with too
-//     few 256-tiles to fill the chip and for operands stored transposed.
+//     same ingredients on 128 x 128 tiles with 4 wavefronts (v_mfma_f32_32x32x16_f16), for
+//     shapes with too few 256-tiles to fill the chip and for operands stored transposed.
 //
 //   GemmF16General  everything else.  128 x 128 tile, 4 wavefronts, K step 32,
 //     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
@@ -41,7 +38,6 @@
 // columns of A and to the general kernel for the rest (two launches).
 #include "sph_internal.h"
 
-#include <cstdlib>
 #include <type_traits>
 
 namespace
@@ -150,7 +146,7 @@ __device__ __forceinline__ bool MapTile(uint32_t id, uint32_t tilesM, uint32_t t
 }
 
 // ---------------------------------------------------------------------------
-// 256 x 256 tile kernel, K step 32, four LDS stages
+// 256 x 256 tile: K step 32, four LDS stages
 // ---------------------------------------------------------------------------
 constexpr int kT = 256;         // tile edge
 constexpr int kTK = 32;         // K step
@@ -158,508 +154,64 @@ constexpr int kTStages = 4;
 constexpr int kStageBytes = kT * kTK * 2;  // per operand per stage (16 KiB)
 constexpr int kStageHalfs = kT * kTK;
 
-// WAVES wavefronts arranged 2 x (WAVES/2): each owns 128 rows and 512/WAVES columns of
-// the tile, i.e. 4 x TJ MFMA tiles with TJ = 16/WAVES.
+// ---------------------------------------------------------------------------
+// 256 x 256 tile kernel, v_mfma_f32_16x16x32_f16
+// ---------------------------------------------------------------------------
+// Why the 16x16x32 instruction: on real (non-zero) operands the chip holds a power limit and
+// the matrix-core rate follows the energy per product, not the issue rate.  The deeper
+// instruction reads and writes every accumulator once per 32 products instead of once per 16:
+// matrix cores fed from LDS only, N(0, 1/64) operands, take 72.8 us for the flops of 4096^3
+// with it against 80.6 us with v_mfma_f32_32x32x16_f16 (on all-zero operands, where nothing
+// is limited by power, 63.6 against 61.1 us).
+//
+// Stage layout.  A stage: 128 LDS rows of 128 bytes; LDS row R holds A[R][k0..k0+31] in its
+// first 64 bytes and A[R+128][k0..k0+31] in the last 64, 16-byte chunks XOR-swizzled with
+// (R/2)%8: the LDS serves a 16-byte read to 16 lanes per clock from 64 banks, and 16
+// consecutive 128-byte rows are 8 even ones on banks 0-31 and 8 odd ones on banks 32-63, so
+// the 8 rows of either parity must take 8 different chunk positions.  B stage: 32 k-rows of
+// 512 bytes, 32-byte chunks XOR-swizzled with 2*(k%4) + (k/8)%2, so that the two 16-lane
+// groups a transposing read serves in one clock (k and k + 8) fall on different banks.
+//
+// Fragments.
+//   A fragment i (rows 16i..16i+15 of the wavefront's 128): lane l holds row l%16, k 8*(l/16)..+7:
+//     one 16-byte LDS read.
+//   B fragment j (columns 16j..16j+15 of its 64): lane l holds column l%16, k 8*(l/16)..+7: two
+//     transposing reads, each 16-lane group g reading the 4 x 16 block at k = 8g + 4h.
+//   With the operands swapped, register v of lane l is row l%16, column 4*(l/16) + v of a block.
+//
+// Pipeline.  LDS holds four K steps.  While step kt is multiplied, the B copies of step kt+3
+// and the A copies of step kt+4 are issued between the MFMAs; a copy has three steps to land.
+// Copies complete in issue order and exactly 2*COPIES_PER_STAGE are issued between the last
+// copy of step kt+1 and the synchronisation point of step kt, so vmcnt <= 2*COPIES_PER_STAGE
+// there means step kt+1 is in LDS.  A step is split by rows: blocks 0-3 before the barrier, 4-7
+// after it.  The A fragments of a step's second half are read during its first half; behind
+// the barrier the first half's A registers take the next step's rows 0-63 and a second set of
+// B registers its B fragments.  The loop body is written out for the four stages so that
+// every LDS address is a register plus an immediate; sched_barrier fences pin the
+// interleaving of MFMAs, LDS reads and copies written here.
+//
 // RAGGED: M and N need not be multiples of 256 (N still a multiple of 8).  Rows past M and
 // 16-byte column chunks past N are clamped to the last valid ones when they are copied (they
 // feed only outputs that are never stored) and the epilogue skips what lies outside.
-// CLOOP (whole tiles, accumulating, at least kCLoopSteps K steps): the old contents of out are
-// not read in the epilogue, when every workgroup would ask for them at once, but during the
-// first K steps: every second step a wavefront has one of its eight 32 x 32 blocks copied
-// straight into a 4 KiB LDS mailbox in accumulator layout and, two steps later, adds it to
-// the accumulators of that block.  The epilogue then only stores.
-// CSP = K steps between two blocks (0 = the epilogue reads out); the prefix that handles the 8
-// blocks is written out step by step and takes CLoopSteps(CSP) steps.
+//
+// CSP != 0 (whole tiles, accumulating, at least CLoopSteps(CSP) K steps): the old contents of
+// out are not read in the epilogue, when every workgroup would ask for them at once, but
+// during the first K steps: every CSP-th step a wavefront has one of its eight 16-row blocks
+// copied straight into a 4 KiB LDS mailbox in accumulator layout and, CSP steps later, adds it
+// to the accumulators of that block.  The epilogue then only stores.  out + A*B is therefore
+// associated as (partial sum + out) + rest of the sum, like a tensor-core kernel that loads
+// the accumulator fragment from C, not as "sum, then one add".
+//
+// Epilogue.  One store instruction in accumulator layout would touch 16 rows with 64 bytes
+// each.  To write (and, without CSP, read) whole 256-byte row segments instead, each
+// wavefront turns its 128 x 64 part round through a private 16 KiB piece of LDS, 64 rows at a
+// time: after that a lane holds 4 consecutive columns and 16 consecutive lanes cover one row.
 constexpr int CLoopSteps(int csp)
 {
     return (8 * csp + 1 + 3) / 4 * 4;
 }
-template <int WAVES, bool RAGGED, int CSP>
-__global__ __launch_bounds__(WAVES * 64) void GemmF16Tile256(const GemmF16Args args)
-{
-    constexpr bool CLOOP = CSP != 0;
-    constexpr int kCLoopSteps = CLoopSteps(CSP);
-    static_assert(!(CLOOP && RAGGED), "old values are added in the loop for whole tiles only");
-    constexpr int WN = WAVES / 2;          // wavefront columns
-    constexpr int TJ = 8 / WN;             // 32-column MFMA blocks per wavefront
-    constexpr int ROUNDS = 16 / WAVES;     // copies per lane per operand per stage
-    constexpr int WAVE_LDS = ROUNDS * 1024;  // bytes of a stage one wavefront fills
-    constexpr int COPIES_PER_STAGE = 2 * ROUNDS;
-    constexpr uint32_t kBias = 4096;       // keeps every lane offset non-negative
-
-    // A stage: 128 LDS rows of 128 bytes; LDS row R holds A[R][k0..k0+31] in its first 64
-    // bytes and A[R+128][k0..k0+31] in the last 64, 16-byte chunks XOR-swizzled with
-    // (R/2)%8: the LDS serves a 16-byte read to 16 lanes per clock from 64 banks, and 16
-    // consecutive 128-byte rows are 8 even ones on banks 0-31 and 8 odd ones on banks 32-63,
-    // so the 8 rows of either parity must take 8 different chunk positions (with R%8 they
-    // take 4, and every fragment read costs 8 clocks instead of 4).
-    // B stage: 32 k-rows of 512 bytes, 32-byte chunks XOR-swizzled with 2*(k%4).
-    __shared__ __attribute__((aligned(1024))) _Float16 Lds[2][kTStages][kStageHalfs];
-    __shared__ __attribute__((aligned(1024))) float CMail[CLOOP ? WAVES * 1024 : 4];
-    auto& As = Lds[0];
-    auto& Bs = Lds[1];
-
-    uint32_t unit, tm, tn;
-    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
-        return;
-
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63;
-    const uint32_t wave = tid >> 6;
-    const uint32_t waveM = wave / WN;  // 0..1 -> 128 rows each
-    const uint32_t waveN = wave % WN;
-
-    const uint32_t K = args.K, N = args.N;
-    // rows and columns of this tile that exist
-    const uint32_t rowsLeft = RAGGED ? min(static_cast<uint32_t>(kT), args.M - tm * kT) : kT;
-    const uint32_t colsLeft = RAGGED ? min(static_cast<uint32_t>(kT), N - tn * kT) : kT;
-    const _Float16* __restrict__ A =
-        args.A + args.strideA * static_cast<int64_t>(unit) + static_cast<size_t>(tm) * kT * args.lda;
-    const _Float16* __restrict__ B =
-        args.B + args.strideB * static_cast<int64_t>(unit) + static_cast<size_t>(tn) * kT;
-    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit) +
-                              static_cast<size_t>(tm) * kT * N + static_cast<size_t>(tn) * kT;
-
-    // ---- global -> LDS copy plan --------------------------------------------
-    // A copy instruction moves 1 KiB per wavefront.  Wavefront w fills the WAVE_LDS bytes
-    // at w*WAVE_LDS of a stage in ROUNDS copies; copy r puts lane i's 16 bytes at
-    // w*WAVE_LDS + r*1024 + i*16.
-    //   A: that is LDS row R = w*8*ROUNDS + r*8 + i/8, physical chunk i%8, which must hold
-    //      logical chunk L = (i%8) ^ ((R/2)%8): matrix row R (L < 4) or R+128 (L >= 4),
-    //      k offset (L%4)*8.
-    //   B: k = w*2*ROUNDS + r*2 + i/32, physical 16-byte chunk i%32, 32-byte chunks
-    //      swizzled with 2*(k%4).
-    // The global address of a copy is a uniform base that advances with the K step plus a
-    // per-lane byte offset that never changes.  The instruction offset r*1024 is added to
-    // both the LDS and the global address, so the lane offsets subtract it again.
-    uint32_t aLane[ROUNDS], bLane[ROUNDS];
-    {
-#pragma unroll
-        for (int r = 0; r < ROUNDS; ++r)
-        {
-            const uint32_t R = wave * (8 * ROUNDS) + 8 * r + (lane >> 3);
-            const uint32_t aL = (lane & 7) ^ ((R >> 1) & 7);
-            const uint32_t row = R + ((aL & 4) ? 128u : 0u);
-            aLane[r] = (min(row, rowsLeft - 1) * args.lda + (aL & 3) * 8) * 2 + kBias - r * 1024;
-        }
-        const uint32_t phys16 = lane & 31;
-#pragma unroll
-        for (int r = 0; r < ROUNDS; ++r)
-        {
-            const uint32_t k = wave * (2 * ROUNDS) + r * 2 + (lane >> 5);
-            const uint32_t logical16 = (((phys16 >> 1) ^ (2 * (k & 3))) << 1) | (phys16 & 1);
-            bLane[r] = (k * N + min(logical16 * 8, colsLeft - 8)) * 2 + kBias - r * 1024;
-        }
-    }
-    const uint32_t waveU = __builtin_amdgcn_readfirstlane(wave);
-    const uint32_t aLds = LdsAddress(&As[0][0]) + waveU * WAVE_LDS;
-    const uint32_t bLds = LdsAddress(&Bs[0][0]) + waveU * WAVE_LDS;
-    const char* aGlobal = reinterpret_cast<const char*>(A) - kBias;
-    const char* bGlobal = reinterpret_cast<const char*>(B) - kBias;
-    const size_t bStepBytes = static_cast<size_t>(kTK) * N * 2;
-
-    // K steps beyond the last are clamped to it: those copies land in buffers that are no
-    // longer read, which keeps the number of copies in flight constant.
-    const uint32_t steps = K / kTK;
-    auto copyA = [&](uint32_t kt, int stage, auto round) {
-        constexpr int r = decltype(round)::value;
-        const uint32_t src = min(kt, steps - 1);
-        DmaToLds16<r * 1024>(aLane[r], aGlobal + static_cast<size_t>(src) * (kTK * 2),
-                             aLds + stage * kStageBytes);
-    };
-    auto copyB = [&](uint32_t kt, int stage, auto round) {
-        constexpr int r = decltype(round)::value;
-        const uint32_t src = min(kt, steps - 1);
-        DmaToLds16<r * 1024>(bLane[r], bGlobal + static_cast<size_t>(src) * bStepBytes,
-                             bLds + stage * kStageBytes);
-    };
-
-    // ---- LDS -> fragment read plan ------------------------------------------
-    // A fragment (row block i, k sub-step ks): lane l reads matrix row
-    //   waveM*128 + i*32 + l%32 = half waveM of LDS row R = i*32 + l%32,
-    //   logical chunk waveM*4 + ks*2 + l/32.
-    const uint32_t l32 = lane & 31;
-    const uint32_t khalf = lane >> 5;
-    const uint32_t aSwz = (l32 >> 1) & 7;
-    const uint32_t aChunkBase = waveM * 4 + khalf;  // + ks*2
-    // B fragment (column block j, sub-step ks): 16-lane group g = l/16, s = l%16;
-    //   columns waveN*(32*TJ) + j*32 + 16*(g%2) + 4*(s%4)..+3,
-    //   k = ks*16 + 8*(g/2) + 4*h + s/4 for the two reads h = 0, 1.
-    const uint32_t g = lane >> 4;
-    const uint32_t s = lane & 15;
-    const uint32_t bKLocal = 8 * (g >> 1) + (s >> 2);          // + ks*16 + 4*h
-    const uint32_t bCol32 = waveN * (2 * TJ) + (g & 1);         // + j*2, logical 32-byte chunk
-    const uint32_t bSwz = 2 * ((s >> 2) & 3);                   // 2*(k%4)
-    const uint32_t bInChunk = (s & 3) * 4;                      // halves inside the chunk
-
-    // element offsets inside a stage, fixed for the whole kernel
-    uint32_t aOff[2], bOff[2][TJ];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-    {
-        aOff[ks] = l32 * 64 + (((aChunkBase + ks * 2) ^ aSwz) * 8);  // + i*32*64
-#pragma unroll
-        for (int j = 0; j < TJ; ++j)
-            bOff[ks][j] =
-                (ks * 16 + bKLocal) * kT + (((bCol32 + j * 2) ^ bSwz) * 16) + bInChunk;
-    }
-
-    auto loadA = [&](int stage, int ks, int i) {
-        return *reinterpret_cast<const halfx8*>(&As[stage][aOff[ks] + i * 32 * 64]);
-    };
-    auto loadB = [&](int stage, int ks, int j) {
-        const _Float16* p = &Bs[stage][bOff[ks][j]];
-        return Join(LdsReadTr(p), LdsReadTr(p + 4 * kT));
-    };
-
-    floatx16 acc[4][TJ];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < TJ; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v)
-                acc[i][j][v] = 0.f;
-
-    // ---- pipeline ---------------------------------------------------------------
-    // LDS holds four K steps.  While step kt is multiplied, the B copies of step kt+3
-    // and the A copies of step kt+4 are issued, spread between the MFMAs so that the
-    // memory pipe sees a steady stream; a copy has three steps to land.  Copies
-    // complete in issue order and exactly 2*COPIES_PER_STAGE are issued between the
-    // last copy of step kt+1 and the synchronisation point of step kt, so
-    // vmcnt <= 2*COPIES_PER_STAGE there means step kt+1 is in LDS.  The barrier sits
-    // in the middle of a step: the MFMAs of the second half need no LDS access of
-    // their own and cover the latency of the first fragment reads of the next step.
-    // The loop body is written out for the four stages so that every LDS address is a
-    // register plus an immediate; sched_barrier fences pin the interleaving of MFMAs,
-    // LDS reads and copies written here (a few non-MFMA instructions after each MFMA).
-#define SPH_FENCE() __builtin_amdgcn_sched_barrier(0)
-
-    // One half step: the 4*TJ MFMAs of fragments (AF, BF), with the reads that fill
-    // (AFN, BFN) from stage `stageN`, sub-step `ksN`, and one operand's copies of K step
-    // ktCopy into stage `stageCopy` slotted between them.
-    auto halfStep = [&](const halfx8 (&AF)[4], const halfx8 (&BF)[TJ], halfx8 (&AFN)[4],
-                        halfx8 (&BFN)[TJ], int stageN, int ksN, uint32_t ktCopy, int stageCopy,
-                        bool copyIsA) {
-        auto copy = [&](auto round) {
-            if (copyIsA)
-                copyA(ktCopy, stageCopy, round);
-            else
-                copyB(ktCopy, stageCopy, round);
-        };
-        auto group = [&](auto iC) {
-            constexpr int i = decltype(iC)::value;
-#pragma unroll
-            for (int j = 0; j < TJ; ++j)
-            {
-                acc[i][j] =
-                    __builtin_amdgcn_mfma_f32_32x32x16_f16(BF[j], AF[i], acc[i][j], 0, 0, 0);
-                SPH_FENCE();
-                if (j == 0)
-                    AFN[i] = loadA(stageN, ksN, i);
-                if constexpr (i < TJ)
-                {
-                    if (j == 1)
-                        BFN[i] = loadB(stageN, ksN, i);
-                }
-                SPH_FENCE();
-            }
-            // copies of this group: rounds [i*ROUNDS/4, (i+1)*ROUNDS/4)
-            if constexpr (ROUNDS == 4)
-                copy(std::integral_constant<int, i>{});
-            else if constexpr (i == 1)
-                copy(std::integral_constant<int, 0>{});
-            else if constexpr (i == 3)
-                copy(std::integral_constant<int, 1>{});
-            SPH_FENCE();
-        };
-        group(std::integral_constant<int, 0>{});
-        group(std::integral_constant<int, 1>{});
-        group(std::integral_constant<int, 2>{});
-        group(std::integral_constant<int, 3>{});
-    };
-
-    auto copyAllA = [&](uint32_t kt, int stage) {
-        copyA(kt, stage, std::integral_constant<int, 0>{});
-        copyA(kt, stage, std::integral_constant<int, 1>{});
-        if constexpr (ROUNDS == 4)
-        {
-            copyA(kt, stage, std::integral_constant<int, 2>{});
-            copyA(kt, stage, std::integral_constant<int, 3>{});
-        }
-    };
-    auto copyAllB = [&](uint32_t kt, int stage) {
-        copyB(kt, stage, std::integral_constant<int, 0>{});
-        copyB(kt, stage, std::integral_constant<int, 1>{});
-        if constexpr (ROUNDS == 4)
-        {
-            copyB(kt, stage, std::integral_constant<int, 2>{});
-            copyB(kt, stage, std::integral_constant<int, 3>{});
-        }
-    };
-
-#pragma unroll
-    for (int st = 0; st < 3; ++st)
-    {
-        copyAllA(st, st);
-        copyAllB(st, st);
-    }
-    copyAllA(3, 3);
-    // stage 0 is followed by 2.5 stages' worth of copies
-    WaitVmem<(5 * COPIES_PER_STAGE) / 2>();
-    __syncthreads();
-
-    halfx8 af0[4], bf0[TJ], af1[4], bf1[TJ];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        af0[i] = loadA(0, 0, i);
-#pragma unroll
-    for (int j = 0; j < TJ; ++j)
-        bf0[j] = loadB(0, 0, j);
-
-    // one K step with its stage index known at compile time; EXTRA = vector memory
-    // operations other than stage copies issued since the first half of the step before
-    auto step = [&](auto stageC, uint32_t kt, auto extraC) {
-        constexpr int cur = decltype(stageC)::value;
-        constexpr int nxt = (cur + 1) % kTStages;
-        constexpr int EXTRA = decltype(extraC)::value;
-        // first half: multiply sub-step 0, fetch sub-step 1, request B of step kt+3
-        halfStep(af0, bf0, af1, bf1, cur, 1, kt + 3, (cur + 3) % kTStages, false);
-        // step kt+1 has landed for every wavefront, and every wavefront is done reading
-        // step kt, whose buffer now takes step kt+4
-        WaitVmem<2 * COPIES_PER_STAGE + EXTRA>();
-        __syncthreads();
-        // second half: multiply sub-step 1, fetch sub-step 0 of step kt+1, request A of kt+4
-        halfStep(af1, bf1, af0, bf0, nxt, 0, kt + 4, cur, true);
-    };
-
-    constexpr std::integral_constant<int, 0> kNoExtra{};
-    if constexpr (CLOOP)
-    {
-        // Block b = 2*i + j of this wavefront: register 4q + r of lane l is row i*32 + l%32,
-        // column j*32 + 8q + 4*(l/32) + r of its 128 x 64 part.  Copy q of a block moves, per
-        // lane, those 4 floats to mailbox + q*1024 + 16*l; the instruction offset 128*j + 32*q
-        // (added to both addresses) selects block column and q, so M0 takes it off again.
-        const uint32_t mail = LdsAddress(&CMail[0]) + waveU * 4096;
-        const uint32_t cLane0 = ((waveM * 128 + l32) * N + waveN * (32 * TJ) + 4 * khalf) * 4;
-        const uint32_t cRowStep = 32 * N * 4;
-        auto issueC = [&](auto bC) {
-            constexpr int b = decltype(bC)::value;
-            constexpr int i = b / TJ, j = b % TJ;
-            const uint32_t laneOff = cLane0 + i * cRowStep;
-            DmaToLds16<j * 128 + 0>(laneOff, out, mail + 0 * 992 - j * 128);
-            DmaToLds16<j * 128 + 32>(laneOff, out, mail + 1 * 992 - j * 128);
-            DmaToLds16<j * 128 + 64>(laneOff, out, mail + 2 * 992 - j * 128);
-            DmaToLds16<j * 128 + 96>(laneOff, out, mail + 3 * 992 - j * 128);
-        };
-        auto addC = [&](auto bC) {
-            constexpr int b = decltype(bC)::value;
-            constexpr int i = b / TJ, j = b % TJ;
-            const float* box = &CMail[wave * 1024 + lane * 4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                const float4 c = *reinterpret_cast<const float4*>(box + q * 256);
-                acc[i][j][4 * q + 0] += c.x;
-                acc[i][j][4 * q + 1] += c.y;
-                acc[i][j][4 * q + 2] += c.z;
-                acc[i][j][4 * q + 3] += c.w;
-            }
-        };
-        // Step s = CSP*b requests block b; step s + CSP adds it.  Ahead of the mid-step wait
-        // of step s lie the stage copies counted there plus the 4 block copies of step s or
-        // s-1, if one of the two requested a block; ahead of the wait for block b at the start
-        // of step CSP*(b+1) lie the stage copies of the CSP steps since its request.
-        constexpr int kBlocks = 4 * TJ;
-        auto cStep = [&](auto stageC, auto sC) {
-            constexpr int st = decltype(sC)::value;
-            constexpr bool requests = st % CSP == 0 && st / CSP < kBlocks;
-            constexpr bool requestedBefore = st >= 1 && (st - 1) % CSP == 0 && (st - 1) / CSP < kBlocks;
-            if constexpr (st % CSP == 0 && st >= CSP && st / CSP <= kBlocks)
-            {
-                WaitVmem<CSP * COPIES_PER_STAGE>();
-                addC(std::integral_constant<int, st / CSP - 1>{});
-            }
-            if constexpr (requests)
-                issueC(std::integral_constant<int, requests ? st / CSP : 0>{});
-            step(stageC, static_cast<uint32_t>(st),
-                 std::integral_constant<int, (requests || requestedBefore) ? 4 : 0>{});
-        };
-        static_assert(CSP * COPIES_PER_STAGE <= 63, "vmcnt holds 6 bits");
-        auto cRound = [&](auto rC) {
-            constexpr int r = decltype(rC)::value;
-            if constexpr (4 * r < kCLoopSteps)
-            {
-                cStep(std::integral_constant<int, 0>{}, std::integral_constant<int, 4 * r + 0>{});
-                cStep(std::integral_constant<int, 1>{}, std::integral_constant<int, 4 * r + 1>{});
-                cStep(std::integral_constant<int, 2>{}, std::integral_constant<int, 4 * r + 2>{});
-                cStep(std::integral_constant<int, 3>{}, std::integral_constant<int, 4 * r + 3>{});
-            }
-        };
-        static_assert(kCLoopSteps <= 4 * 17, "rounds written out below");
-        cRound(std::integral_constant<int, 0>{});
-        cRound(std::integral_constant<int, 1>{});
-        cRound(std::integral_constant<int, 2>{});
-        cRound(std::integral_constant<int, 3>{});
-        cRound(std::integral_constant<int, 4>{});
-        cRound(std::integral_constant<int, 5>{});
-        cRound(std::integral_constant<int, 6>{});
-        cRound(std::integral_constant<int, 7>{});
-        cRound(std::integral_constant<int, 8>{});
-        cRound(std::integral_constant<int, 9>{});
-        cRound(std::integral_constant<int, 10>{});
-        cRound(std::integral_constant<int, 11>{});
-        cRound(std::integral_constant<int, 12>{});
-        cRound(std::integral_constant<int, 13>{});
-        cRound(std::integral_constant<int, 14>{});
-        cRound(std::integral_constant<int, 15>{});
-        cRound(std::integral_constant<int, 16>{});
-    }
-    auto regularSteps = [&](uint32_t first) {
-        for (uint32_t kt = first;; kt += 4)
-        {
-            step(std::integral_constant<int, 0>{}, kt, kNoExtra);
-            if (kt + 1 >= steps)
-                break;
-            step(std::integral_constant<int, 1>{}, kt + 1, kNoExtra);
-            if (kt + 2 >= steps)
-                break;
-            step(std::integral_constant<int, 2>{}, kt + 2, kNoExtra);
-            if (kt + 3 >= steps)
-                break;
-            step(std::integral_constant<int, 3>{}, kt + 3, kNoExtra);
-            if (kt + 4 >= steps)
-                break;
-        }
-    };
-    if constexpr (CLOOP)
-    {
-        if (steps > kCLoopSteps)
-            regularSteps(kCLoopSteps);
-    }
-    else
-        regularSteps(0);
-#undef SPH_FENCE
-
-    // ---- epilogue -------------------------------------------------------------
-    // With the operands swapped the 32x32 result block is indexed [n][m]: register v of
-    // lane l holds column 8*(v/4) + 4*(l/32) + v%4 of row l%32, i.e. registers 4q..4q+3 are
-    // 4 consecutive columns of one row, and one store instruction would touch 32 rows with
-    // 32 bytes each.  To write (and, when accumulating, read) whole 256-byte row segments
-    // instead, each wavefront turns its 128 x (32*TJ) block round through a private 16 KiB
-    // piece of LDS, 64 rows at a time: after that a lane holds 4 consecutive columns and 16
-    // consecutive lanes cover one row of the block.
-    static_assert(TJ == 2, "the staged epilogue is written for 64-column wavefront blocks");
-    WaitVmem<0>();      // clamped copies of the last steps still target LDS
-    __syncthreads();    // ... and every wavefront is done with the stage buffers
-    {
-        // 64 rows x 64 floats per wavefront, 16-byte chunks XOR-swizzled with row % 16 so
-        // that neither the column-wise writes nor the row-wise reads pile up on one bank
-        float* stage = reinterpret_cast<float*>(&Lds[0][0][0]) + wave * (64 * 64);
-        static_assert(WAVES * 64 * 64 * 4 <= static_cast<int>(sizeof(Lds)), "staging fits");
-        const uint32_t rdRow = lane >> 4;        // + 4*t
-        const uint32_t rdChunk = lane & 15;
-        float* outBlock = out + static_cast<size_t>(waveM * 128 + rdRow) * N +
-                          waveN * (32 * TJ) + rdChunk * 4;
-        const size_t rowStep = static_cast<size_t>(4) * N;  // between consecutive t
-        // what of this lane's part exists: rows rowFirst + 4*t of the tile, 4 columns at colFirst
-        const uint32_t rowFirst = waveM * 128 + rdRow;
-        const bool colExists = !RAGGED || waveN * (32 * TJ) + rdChunk * 4 < colsLeft;
-        auto exists = [&](int half, int t) {
-            return !RAGGED || (colExists && rowFirst + 4 * (half * 16 + t) < rowsLeft);
-        };
-
-        auto stageHalf = [&](int half) {
-#pragma unroll
-            for (int ii = 0; ii < 2; ++ii)
-#pragma unroll
-                for (int j = 0; j < TJ; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                    {
-                        const int i = half * 2 + ii;
-                        const uint32_t row = ii * 32 + l32;
-                        const uint32_t chunk = (j * 8 + 2 * q + khalf) ^ (row & 15);
-                        *reinterpret_cast<float4*>(&stage[row * 64 + chunk * 4]) =
-                            make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
-                                        acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-                    }
-            // the block is private to the wavefront: its own LDS writes are visible to it
-            // once they have completed
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        };
-        auto loadOld = [&](int half, float4 (&old)[16]) {
-#pragma unroll
-            for (int t = 0; t < 16; ++t)
-            {
-                old[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (exists(half, t))
-                    old[t] = NtLoad4(outBlock + (half * 16 + t) * rowStep);
-            }
-        };
-        auto storeHalf = [&](int half, const float4 (&old)[16], auto accumulate) {
-#pragma unroll
-            for (int t = 0; t < 16; ++t)
-            {
-                const uint32_t r = rdRow + 4 * t;
-                float4 v = *reinterpret_cast<const float4*>(
-                    &stage[r * 64 + ((rdChunk ^ (r & 15)) * 4)]);
-                if constexpr (decltype(accumulate)::value)
-                {
-                    v.x += old[t].x;
-                    v.y += old[t].y;
-                    v.z += old[t].z;
-                    v.w += old[t].w;
-                }
-                if (exists(half, t))
-                    *reinterpret_cast<float4*>(outBlock + (half * 16 + t) * rowStep) = v;
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        };
-
-        float4 old[16];
-        if (CLOOP || args.overwrite)
-        {
-            stageHalf(0);
-            storeHalf(0, old, std::false_type{});
-            stageHalf(1);
-            storeHalf(1, old, std::false_type{});
-        }
-        else
-        {
-            // the old contents of a half are requested in one batch, in flight while its
-            // accumulators are staged
-            loadOld(0, old);
-            stageHalf(0);
-            storeHalf(0, old, std::true_type{});
-            loadOld(1, old);
-            stageHalf(1);
-            storeHalf(1, old, std::true_type{});
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// 256 x 256 tile on v_mfma_f32_16x16x32_f16
-// ---------------------------------------------------------------------------
-// The same tile, stages, copies and epilogue as GemmF16Tile256, multiplied with the 16x16x32
-// instruction: a wavefront's 128 x 64 part is 8 x 4 blocks of 16 x 16 (4 accumulator registers
-// each) and a K step of 32 is one instruction deep.  Every accumulator is read and written
-// once per 32 products instead of once per 16, and under the power limit that bounds this
-// kernel on real operands the deeper instruction delivers about a tenth more (matrix cores fed
-// from LDS only, N(0, 1/64) operands: 72.8 against 80.6 us for the flops of 4096^3).
-//   A fragment i (rows 16i..16i+15 of the wavefront's 128): lane l holds row l%16, k 8*(l/16)..+7:
-//     one 16-byte LDS read from the A stage layout described above.
-//   B fragment j (columns 16j..16j+15 of its 64): lane l holds column l%16, k 8*(l/16)..+7: two
-//     transposing reads, each 16-lane group g reading the 4 x 16 block at k = 8g + 4h.  The
-//     32-byte chunks of a k-row are XOR-swizzled with 2*(k%4) + (k/8)%2, so that the two groups
-//     served in one clock (k and k + 8) fall on different banks.
-//   With the operands swapped, register v of lane l is row l%16, column 4*(l/16) + v of a block.
-// A step is split by rows: blocks 0-3 before the barrier, 4-7 after it.  The A fragments of a
-// step's second half are read during its first half; behind the barrier the first half's A
-// registers take the next step's rows 0-63 and a second set of B registers its B fragments.
 template <bool RAGGED, int CSP>
-__global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
+__global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 {
     constexpr int WAVES = 8;
     constexpr int ROUNDS = 2;               // copies per lane per operand per stage
@@ -695,7 +247,20 @@ __global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
     float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit) +
                               static_cast<size_t>(tm) * kT * N + static_cast<size_t>(tn) * kT;
 
-    // ---- global -> LDS copy plan (as in GemmF16Tile256; B rows with the swizzle above) ----
+    // ---- global -> LDS copy plan --------------------------------------------
+    // A copy instruction moves 1 KiB per wavefront.  Wavefront w fills the WAVE_LDS bytes
+    // at w*WAVE_LDS of a stage in ROUNDS copies; copy r puts lane i's 16 bytes at
+    // w*WAVE_LDS + r*1024 + i*16.
+    //   A: that is LDS row R = w*8*ROUNDS + r*8 + i/8, physical chunk i%8, which must hold
+    //      logical chunk L = (i%8) ^ ((R/2)%8): matrix row R (L < 4) or R+128 (L >= 4),
+    //      k offset (L%4)*8.
+    //   B: k = w*2*ROUNDS + r*2 + i/32, physical 16-byte chunk i%32, 32-byte chunks
+    //      swizzled as described above.
+    // The global address of a copy is a uniform base that advances with the K step plus a
+    // per-lane byte offset that never changes.  The instruction offset r*1024 is added to
+    // both the LDS and the global address, so the lane offsets subtract it again.  K steps
+    // beyond the last are clamped to it: those copies land in buffers that are no longer
+    // read, which keeps the number of copies in flight constant.
     uint32_t aLane[ROUNDS], bLane[ROUNDS];
     {
 #pragma unroll
@@ -794,7 +359,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
     // receives the next step's.  EXTRA = vector memory operations other than stage copies
     // issued since the first half of the step before.
     auto stepWith = [&](auto stageC, uint32_t kt, auto extraC, const halfx8 (&BF)[4],
-                        halfx8 (&BFN)[4]) {
+                        halfx8 (&BFN)[4], auto&& behindBarrier) {
         constexpr int cur = decltype(stageC)::value;
         constexpr int nxt = (cur + 1) % kTStages;
         constexpr int EXTRA = decltype(extraC)::value;
@@ -821,6 +386,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
         // step kt, whose A buffer now takes step kt+4
         WaitVmem<2 * COPIES_PER_STAGE + EXTRA>();
         __syncthreads();
+        behindBarrier();
         // second half: rows 64-127, fetch the next step's rows 0-63 and B, request A of kt+4
 #pragma unroll
         for (int i = 4; i < 8; ++i)
@@ -846,12 +412,13 @@ __global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
             SPH_FENCE();
         }
     };
-    auto step = [&](auto stageC, uint32_t kt, auto extraC) {
+    auto stepThen = [&](auto stageC, uint32_t kt, auto extraC, auto&& behindBarrier) {
         if constexpr (decltype(stageC)::value % 2 == 0)
-            stepWith(stageC, kt, extraC, bf0, bf1);
+            stepWith(stageC, kt, extraC, bf0, bf1, behindBarrier);
         else
-            stepWith(stageC, kt, extraC, bf1, bf0);
+            stepWith(stageC, kt, extraC, bf1, bf0, behindBarrier);
     };
+    auto step = [&](auto stageC, uint32_t kt, auto extraC) { stepThen(stageC, kt, extraC, [] {}); };
 
     constexpr std::integral_constant<int, 0> kNoExtra{};
     if constexpr (CLOOP)
@@ -887,22 +454,31 @@ __global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
                     SPH_FENCE();
             }
         };
-        // Step s = CSP*b requests row block b; step s + CSP adds it (vmcnt accounting as in
-        // GemmF16Tile256).
+        // Step s = CSP*b requests row block b behind its barrier, where the copies issued
+        // next are the ones needed last (three steps later); step s + CSP adds it at the same
+        // place.  Vector memory operations complete in issue order, so a block that is late
+        // holds back the stage copies behind it (spacing 4 measured 113.6 us on configuration
+        // 3 against 115.3 us with spacing 2).  Ahead of the mid-step wait of step s lie the
+        // stage copies counted there plus the 4 block copies of step s-1 or s-2, if one of them
+        // requested a block; ahead of the wait for block b in step CSP*(b+1) lie the stage
+        // copies of the CSP steps since its request.
         constexpr int kBlocks = 8;
+        static_assert(CSP >= 2, "at most one request among two consecutive steps");
+        auto requestsAt = [](int st) { return st >= 0 && st % CSP == 0 && st / CSP < kBlocks; };
         auto cStep = [&](auto stageC, auto sC) {
             constexpr int st = decltype(sC)::value;
             constexpr bool requests = st % CSP == 0 && st / CSP < kBlocks;
-            constexpr bool requestedBefore = st >= 1 && (st - 1) % CSP == 0 && (st - 1) / CSP < kBlocks;
-            if constexpr (st % CSP == 0 && st >= CSP && st / CSP <= kBlocks)
-            {
-                WaitVmem<CSP * COPIES_PER_STAGE>();
-                addC(std::integral_constant<int, st / CSP - 1>{});
-            }
-            if constexpr (requests)
-                issueC(std::integral_constant<int, requests ? st / CSP : 0>{});
-            step(stageC, static_cast<uint32_t>(st),
-                 std::integral_constant<int, (requests || requestedBefore) ? 4 : 0>{});
+            constexpr bool adds = st % CSP == 0 && st >= CSP && st / CSP <= kBlocks;
+            constexpr int extra = (requestsAt(st - 1) || requestsAt(st - 2)) ? 4 : 0;
+            stepThen(stageC, static_cast<uint32_t>(st), std::integral_constant<int, extra>{}, [&] {
+                if constexpr (adds)
+                {
+                    WaitVmem<CSP * COPIES_PER_STAGE>();
+                    addC(std::integral_constant<int, adds ? st / CSP - 1 : 0>{});
+                }
+                if constexpr (requests)
+                    issueC(std::integral_constant<int, requests ? st / CSP : 0>{});
+            });
         };
         static_assert(CSP * COPIES_PER_STAGE <= 63, "vmcnt holds 6 bits");
         auto cRound = [&](auto rC) {
@@ -952,10 +528,12 @@ __global__ __launch_bounds__(512) void GemmF16Tile256K32(const GemmF16Args args)
         regularSteps(0);
 #undef SPH_FENCE
 
-    // ---- epilogue: as in GemmF16Tile256, 64 rows at a time through a private 16 KiB of LDS ----
-    WaitVmem<0>();
-    __syncthreads();
+    // ---- epilogue ---------------------------------------------------------------
+    WaitVmem<0>();      // clamped copies of the last steps still target LDS
+    __syncthreads();    // ... and every wavefront is done with the stage buffers
     {
+        // 64 rows x 64 floats per wavefront, 16-byte chunks XOR-swizzled with row % 16 so
+        // that neither the column-wise writes nor the row-wise reads pile up on one bank
         float* stage = reinterpret_cast<float*>(&Lds[0][0][0]) + wave * (64 * 64);
         const uint32_t rdRow = lane >> 4;        // + 4*t
         const uint32_t rdChunk = lane & 15;
@@ -1577,24 +1155,18 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
 
     if (tile256)
     {
-        static const bool m32 = std::getenv("SPH_F16_M32") != nullptr;
-        const bool cloop = whole256 && !args.overwrite && K / kTK >= CLoopSteps(4);
+        // old contents of out added inside the loop: spacing 4 from 36 K steps, 2 from 20
+        const bool cloop = whole256 && !args.overwrite;
+        const uint32_t ksteps = K / kTK;
         const dim3 g(grid), b(512);
-        if (m32)
-        {
-            if (cloop)
-                hipLaunchKernelGGL((GemmF16Tile256<8, false, 4>), g, b, 0, stream, args);
-            else if (whole256)
-                hipLaunchKernelGGL((GemmF16Tile256<8, false, 0>), g, b, 0, stream, args);
-            else
-                hipLaunchKernelGGL((GemmF16Tile256<8, true, 0>), g, b, 0, stream, args);
-        }
-        else if (cloop)
-            hipLaunchKernelGGL((GemmF16Tile256K32<false, 4>), g, b, 0, stream, args);
+        if (cloop && ksteps >= CLoopSteps(4))
+            hipLaunchKernelGGL((GemmF16Tile256<false, 4>), g, b, 0, stream, args);
+        else if (cloop && ksteps >= CLoopSteps(2))
+            hipLaunchKernelGGL((GemmF16Tile256<false, 2>), g, b, 0, stream, args);
         else if (whole256)
-            hipLaunchKernelGGL((GemmF16Tile256K32<false, 0>), g, b, 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Tile256<false, 0>), g, b, 0, stream, args);
         else
-            hipLaunchKernelGGL((GemmF16Tile256K32<true, 0>), g, b, 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Tile256<true, 0>), g, b, 0, stream, args);
     }
     else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
              (!transA || (M % 8 == 0 && M >= 8)) &&

@@ -25,12 +25,15 @@ def _oracle(C, A16, B16, M, N, K, batch=1, sa=None, sb=None):
 # the 256-tile kernel is chosen from 192 tiles up (three quarters of the compute units): the
 # batch count brings these small shapes there
 # from 20 K steps up (K >= 640) the accumulating launch adds the old contents of out during the
-# first steps of the loop instead of in the epilogue: K = 640 (no step after the prefix), 672,
-# 704 (one and two steps after it) and longer
+# first steps of the loop instead of in the epilogue, a block every second step (K = 640: no
+# step after the written-out prefix, 672 and 704: one and two steps after it) and from 36 steps
+# up (K >= 1152) every fourth step (1152, 1184, 1216, 1280 likewise); 608 is the last K that
+# reads out in the epilogue
 @pytest.mark.parametrize("shape", [(256, 256, 64, 192), (256, 512, 128, 96), (512, 256, 192, 96),
                                    (768, 1024, 256, 16), (4096, 3072, 32, 1), (256, 256, 640, 192),
                                    (4096, 3072, 672, 1), (512, 256, 704, 96), (1024, 768, 1280, 16),
-                                   (256, 512, 608, 96)])
+                                   (256, 512, 608, 96), (256, 256, 1152, 192), (512, 512, 1184, 48),
+                                   (256, 1024, 1216, 48), (256, 512, 1120, 96)])
 def test_tile256_exact_on_integers(dev, shape):
     M, N, K, batch = shape
     h.announce("sph_gemm_f16f32 tile256 integer exactness", shape)
