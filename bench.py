@@ -61,7 +61,7 @@ def parse():
                    help="also time the neighbouring kernels (backward pass, conversions, CSR x "
                         "CSR, one-pass kernels; reported under 'others')")
     p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
-                                      "csr", "spgemm", "spmm_fast"], default=None,
+                                      "csr", "spgemm"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
     p.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                    help="untimed run-up before each timed leg that lets the clock reach its "
@@ -140,7 +140,7 @@ def bench_gemm_f16(capi, synth, steps, warmup, flags=0, zero_operands=False):
     return event_ms, wall_ms, d
 
 
-def bench_spmm(capi, synth, steps, warmup, fast=False):
+def bench_spmm(capi, synth, steps, warmup):
     d = synth.config5()
     M, K, N = d["M"], d["K"], d["N"]
     dV = capi.DeviceBuffer.from_array(d["V"])
@@ -150,11 +150,7 @@ def bench_spmm(capi, synth, steps, warmup, fast=False):
     dC = capi.DeviceBuffer.from_array(d["C"])
 
     def launch():
-        if fast:
-            capi.call("sph_spmm_csr_f32_ex", dC.ptr, dV.ptr, dCol.ptr, dRow.ptr, M, K, N, dB.ptr,
-                      capi.SPH_SPMM_FAST)
-        else:
-            capi.call("sph_spmm_csr_f32", dC.ptr, dV.ptr, dCol.ptr, dRow.ptr, M, K, N, dB.ptr, 0)
+        capi.call("sph_spmm_csr_f32", dC.ptr, dV.ptr, dCol.ptr, dRow.ptr, M, K, N, dB.ptr, 0)
 
     event_ms, wall_ms = timed_launches(capi, launch, steps, warmup)
     for b in (dV, dCol, dRow, dB, dC):
@@ -614,16 +610,8 @@ def main():
         result["spgemm"] = {"count_plus_fill_ms": ms, "products": products, "nnz_a": nnz_a,
                             "nnz_b": nnz_b, "nnz_c": nnz_c, "algorithmic_bytes": nbytes}
 
-    if args.only == "spmm_fast":
-        sp_event, _, _, nnz, alg_bytes = bench_spmm(capi, synth, max(args.steps * 4, 100),
-                                                    args.warmup, fast=True)
-        result["spmm_fast"] = {"launch_ms": sp_event, "gbs": alg_bytes / (sp_event * 1e-3) / 1e9}
-
     if args.only in (None, "spmm"):
         sp_steps = max(args.steps * 4, 100)
-        fast_event = None
-        if args.only is None:
-            fast_event, _, _, _, _ = bench_spmm(capi, synth, sp_steps, args.warmup, fast=True)
         sp_event, sp_wall, d5, nnz, alg_bytes = bench_spmm(capi, synth, sp_steps, args.warmup)
         gbs = alg_bytes / (sp_event * 1e-3) / 1e9
         spmm = {
@@ -638,16 +626,6 @@ def main():
                          "algorithmic_bytes_per_launch": alg_bytes,
                          "gather_bytes_per_launch": nnz * 256 * 4},
         }
-        if fast_event is not None:
-            fgbs = alg_bytes / (fast_event * 1e-3) / 1e9
-            spmm["fast_mode"] = {
-                "entry_point": "sph_spmm_csr_f32_ex (SPH_SPMM_FAST: values within rounding of "
-                               "the storage-order sum, structure exact)",
-                "launch_ms": fast_event, "value": fgbs, "unit": "GB/s",
-                "roofline": {"bound": "hbm", "kernel": "SpmmLdsSlab", "achieved": fgbs,
-                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": fgbs / PEAK_HBM_GBS,
-                             "traffic": recorded_traffic("spmm_lds_slab_config5.txt"),
-                             "algorithmic_bytes_per_launch": alg_bytes}}
         if not args.no_cpu and args.only is None:
             dt = cpu_spmm_baseline(d5)
             spmm["cpu_baseline"] = {"value": alg_bytes / dt / 1e9, "unit": "GB/s", "cores": 1,

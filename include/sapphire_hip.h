@@ -262,29 +262,15 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M,
  * dense column count.  accumulate == 0 stores (rows without entries become
  * 0), otherwise adds into out.
  * The reference declares no sparse x dense product (Sparse.hpp:20-162 holds
- * sparse x sparse declarations only); this entry fills that slot. */
+ * sparse x sparse declarations only); this entry fills that slot.
+ * The equality with the dense leaf on the densified matrix holds for finite B
+ * only: the dense loop adds 0 * B[k][n] for the absent entries, which is NaN
+ * where B holds Inf or NaN, while the CSR loop never touches those rows of B.
+ * Inf and NaN in V or in the rows of B that are referenced propagate as in the
+ * storage-order CPU loop, element by element. */
 int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL,
                      const uint32_t* ROW, uint32_t M, uint32_t Kdim, uint32_t N,
                      const float* B, int accumulate);
-
-/* sph_spmm_csr_f32 with flags.  SPH_SPMM_FAST drops the bit-for-bit promise for
- * the values: the entries of a row are added with fused multiply-adds in 16
- * interleaved partial sums that are then added up, so an element equals the
- * storage-order sum within rounding (|difference| well below
- * 1e-4 * sum |V[p] * B[COL[p]][n]|), while the structure stays exact: every
- * element of out is written exactly once, rows without entries become 0 (or
- * stay untouched when accumulating), nothing outside out is written.  In
- * exchange the dense operand is gathered from LDS instead of the L2 when its
- * rows fit there (Kdim up to about 10000, N a multiple of 4 from 64 up; other
- * shapes run the exact kernels).  Either way the equality with the dense leaf
- * on the densified matrix holds for finite B only: the dense loop adds
- * 0 * B[k][n] for the absent entries, which is NaN where B holds Inf or NaN,
- * while the CSR loop never touches those rows of B. */
-#define SPH_SPMM_ACCUMULATE 1u
-#define SPH_SPMM_FAST 2u
-int sph_spmm_csr_f32_ex(float* out, const float* V, const uint32_t* COL,
-                        const uint32_t* ROW, uint32_t M, uint32_t Kdim,
-                        uint32_t N, const float* B, uint32_t flags);
 
 /* ---- dense <-> CSR ------------------------------------------------------- */
 

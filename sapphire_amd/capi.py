@@ -21,8 +21,6 @@ SPH_GEMM_OVERWRITE = 1
 SPH_GEMM_TRANS_A = 2
 SPH_GEMM_TRANS_B = 4
 SPH_LINEAR_RELU = 1
-SPH_SPMM_ACCUMULATE = 1
-SPH_SPMM_FAST = 2
 
 
 class SphError(RuntimeError):
@@ -104,7 +102,6 @@ SIGNATURES = {
                                    ctypes.POINTER(ctypes.c_uint32)],
     "sph_spgemm_fill_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
     "sph_spmm_csr_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, ctypes.c_int],
-    "sph_spmm_csr_f32_ex": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32],
 }
 
 

@@ -25,21 +25,8 @@
 // SpmmRowScalar: one wavefront per sparse row, one column per lane (any width, any
 // alignment); the row's (COL, V) pairs are fetched 64 at a time and handed round with
 // v_readlane.
-//
-// A third mapping serves callers that accept values within rounding of that sum instead of
-// its exact bits (SPH_SPMM_FAST).
-//
-// SpmmLdsSlab: a workgroup of 16 wavefronts keeps a slab of 4 dense columns over ALL rows of
-// B in LDS (16 bytes per row of B, 128 KiB at 8192 rows) and gathers from there instead of
-// from the L2: every entry of the sparse matrix then costs one 16-byte LDS read per slab
-// instead of a 256-byte L2 gather per 64-column slab, and what streams through the vector
-// memory path is the (COL, V) arrays, once per slab, in coalesced 64-byte pieces.  16 lanes
-// share a sparse row, lane t taking entries t, t+16, ... with fused multiply-adds; the 16
-// partial sums are added with cross-lane rotations.  The sum of a row is therefore
-// associated differently from the storage-order loop: equal within rounding, not bit for bit.
 #include "sph_internal.h"
 
-#include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
@@ -211,273 +198,6 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
     }
 }
 
-// ---- LDS-resident slab (values within rounding) ------------------------------------------
-#pragma clang fp contract(fast)
-
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
-struct LdsSlabPlan
-{
-    uint32_t slabs;        // N / 4
-    uint32_t slabGroups;   // ceil(slabs / 8)
-    uint32_t parts;        // row partitions per slab
-    uint32_t rowsPerPart;  // multiple of 4
-    uint32_t kSlots;       // rows of B rounded up to 64; slot kSlots holds zeros
-    uint32_t K;            // rows of B
-};
-
-constexpr int kLdsThreads = 1024;
-constexpr int kLdsWaves = kLdsThreads / 64;
-constexpr int kLdsChunks = 3;  // 32-entry chunks of a row fetched ahead: rows of up to 95 entries
-
-// value of lane (l + n) % 16 of the lane's own 16-lane row (DPP row_ror)
-template <int N>
-__device__ __forceinline__ float RowRotate(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
-                                                                 0x120 + N, 0xf, 0xf, false));
-}
-
-__device__ __forceinline__ float RowSum16(float v)
-{
-    v += RowRotate<8>(v);
-    v += RowRotate<4>(v);
-    v += RowRotate<2>(v);
-    v += RowRotate<1>(v);
-    return v;
-}
-
-template <bool ACCUMULATE>
-__global__ __launch_bounds__(kLdsThreads) void SpmmLdsSlab(const SpmmArgs args,
-                                                           const LdsSlabPlan plan)
-{
-    extern __shared__ __attribute__((aligned(16))) float4 slabRows[];  // [kSlots + 1]
-
-    // A unit of work is a group of 8 adjacent slabs (they cut the same 128-byte lines of B)
-    // times one row partition; its 8 workgroups run on one XCD (ids congruent mod 8), so
-    // those lines come from that XCD's L2.  Units are dealt round-robin to the XCDs.
-    const uint32_t xcd = blockIdx.x % 8;
-    const uint32_t local = blockIdx.x / 8;
-    const uint32_t unit = (local / 8) * 8 + xcd;
-    if (unit >= plan.slabGroups * plan.parts)
-        return;
-    const uint32_t slab = (unit % plan.slabGroups) * 8 + local % 8;
-    const uint32_t part = unit / plan.slabGroups;
-    if (slab >= plan.slabs)
-        return;
-
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t N = args.N;
-
-    // ---- the slab: B[k][4*slab .. 4*slab+3] for every k, copied straight into LDS -------
-    // One copy instruction moves 64 rows of B (16 bytes each, N*4 bytes apart) to 64
-    // consecutive slots.  Rows past the last are clamped to it and land in slots nobody
-    // reads.
-    {
-        const char* base = reinterpret_cast<const char*>(args.B + slab * 4);
-        const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
-            (__attribute__((address_space(3))) void*)(slabRows)));
-        for (uint32_t k0 = wave * 64; k0 < plan.kSlots; k0 += kLdsWaves * 64)
-        {
-            const uint32_t k = min(k0 + lane, plan.K - 1);
-            const uint32_t off = k * (N * 4);
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :
-                         : "s"(ldsBase + k0 * 16), "v"(off), "s"(base)
-                         : "memory");
-        }
-        if (threadIdx.x == 0)
-            slabRows[plan.kSlots] = make_float4(0.f, 0.f, 0.f, 0.f);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-    }
-
-    // ---- rows: 16 lanes per row, 4 rows per wavefront and pass ----------------------------
-    const uint32_t t = lane & 15;
-    const uint32_t rowBegin = part * plan.rowsPerPart;
-    const uint32_t rowEnd = min(args.M, rowBegin + plan.rowsPerPart);
-    if (rowBegin >= rowEnd)
-        return;
-    const uint32_t zeroSlot = plan.kSlots;
-    const uint32_t* __restrict__ ROW = args.ROW;
-    const uint32_t* __restrict__ COL = args.COL;
-    const float* __restrict__ V = args.V;
-    constexpr uint32_t kRowsPerRound = kLdsWaves * 4;
-    const uint32_t rows = rowEnd - rowBegin;
-    const uint32_t passes = (rows + kRowsPerRound - 1) / kRowsPerRound;
-
-    // A lane without an entry reads the first entry of this partition instead (it exists
-    // unless the partition is empty, which is settled here) and replaces what it read by the
-    // zero slot, so every load of the loop below is unconditional.
-    const uint32_t partFirst = ROW[rowBegin];
-    const uint32_t partFirstEven = partFirst & ~1u;
-    const uint32_t totalEntries = ROW[args.M];
-    const uint32_t lastPairStart = max(totalEntries, 2u) - 2;
-    if (totalEntries == 1 && ROW[rowEnd] != partFirst)
-    {
-        // a matrix with a single entry has no pair to read: its row is done by one lane group
-        const uint32_t c = COL[0];
-        const float v = V[0];
-        for (uint32_t r = rowBegin + (threadIdx.x >> 4); r < rowEnd; r += kLdsThreads / 16)
-            if (t == 0)
-            {
-                float4* dst = reinterpret_cast<float4*>(args.out + static_cast<size_t>(r) * N + slab * 4);
-                const bool here = ROW[r] == 0 && ROW[r + 1] == 1;
-                const float4 b = slabRows[here ? c : zeroSlot];
-                float4 sum = make_float4(v * b.x, v * b.y, v * b.z, v * b.w);
-                if (!here)
-                    sum = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (ACCUMULATE)
-                {
-                    const float4 old = *dst;
-                    sum = make_float4(old.x + sum.x, old.y + sum.y, old.z + sum.z, old.w + sum.w);
-                }
-                *dst = sum;
-            }
-        return;
-    }
-    if (ROW[rowEnd] == partFirst)
-    {
-        if (!ACCUMULATE)
-            for (uint32_t r = rowBegin + (threadIdx.x >> 4); r < rowEnd; r += kLdsThreads / 16)
-                if (t == 0)
-                    *reinterpret_cast<float4*>(args.out + static_cast<size_t>(r) * N + slab * 4) =
-                        make_float4(0.f, 0.f, 0.f, 0.f);
-        return;
-    }
-
-    // Three passes are in flight per wavefront: the row extents of pass i+2, the entries of
-    // pass i+1 and the gathers of pass i, so that the two dependent global loads of a pass
-    // are hidden behind the LDS work of the passes before it.  Two register sets take turns
-    // (pass i has its entries in set i % 2), so nothing that is still in flight is copied.
-    // Every loaded word also goes into `sink`: a load whose value is only selected under
-    // `valid` is otherwise moved under a branch on `valid`, and with branches in the loop the
-    // wait for a pass's entries becomes a wait for every load in flight.
-    struct Extent
-    {
-        uint32_t p, end;
-    };
-    uint32_t sink = 0;
-    auto rowOf = [&](uint32_t pass) { return rowBegin + pass * kRowsPerRound + wave * 4 + (lane >> 4); };
-    auto loadExtent = [&](uint32_t pass) {
-        const uint32_t row = rowOf(pass);
-        const uint32_t safe = min(row, rowEnd - 1);
-        const uint32_t p = ROW[safe];
-        const uint32_t end = ROW[safe + 1];
-        sink ^= end;
-        return Extent{ p, row < rowEnd ? end : p };
-    };
-    // Lane t of a row's 16 takes the entry pairs 2t, 2t+1 (+ 32 per chunk) counted from the
-    // even index at or below the row's first entry: 8-byte loads, 512 contiguous bytes per
-    // instruction and row group pair, half as many vector memory instructions as with one
-    // entry per lane (the address unit, not the L2, bounds this loop).
-    // A pair that would start at the very last entry of the arrays (odd entry count) is read
-    // one entry earlier instead, so that nothing past the arrays is touched; its entry is then
-    // the second of the pair.
-    auto pairIndex = [&](const Extent& e, int u) { return (e.p & ~1u) + 2 * t + 32 * u; };
-    auto loadEntries = [&](const Extent& e, uint32_t pass, uint2 (&c)[kLdsChunks],
-                           float2 (&v)[kLdsChunks], float4& old) {
-#pragma unroll
-        for (int u = 0; u < kLdsChunks; ++u)
-        {
-            const uint32_t q = pairIndex(e, u);
-            const uint32_t idx = min(q < e.end ? q : partFirstEven, lastPairStart);
-            c[u] = *reinterpret_cast<const uint2*>(COL + idx);
-            v[u] = *reinterpret_cast<const float2*>(V + idx);
-            sink ^= c[u].x ^ c[u].y ^ __builtin_bit_cast(uint32_t, v[u].x) ^
-                    __builtin_bit_cast(uint32_t, v[u].y);
-        }
-        if (ACCUMULATE)
-        {
-            const uint32_t safe = min(rowOf(pass), rowEnd - 1);
-            old = *reinterpret_cast<const float4*>(args.out + static_cast<size_t>(safe) * N + slab * 4);
-        }
-    };
-
-    uint2 c0[kLdsChunks], c1[kLdsChunks];
-    float2 v0[kLdsChunks], v1[kLdsChunks];
-    float4 old0 = make_float4(0.f, 0.f, 0.f, 0.f), old1 = make_float4(0.f, 0.f, 0.f, 0.f);
-    Extent eCur = loadExtent(0);
-    Extent eNext = loadExtent(1);
-    loadEntries(eCur, 0, c0, v0, old0);
-    auto onePass = [&](uint32_t pass, uint2 (&cCur)[kLdsChunks], float2 (&vCur)[kLdsChunks],
-                       float4& oldCur, uint2 (&cNext)[kLdsChunks], float2 (&vNext)[kLdsChunks],
-                       float4& oldNext) {
-        const Extent eAfter = loadExtent(pass + 2);
-        loadEntries(eNext, pass + 1, cNext, vNext, oldNext);
-
-        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int u = 0; u < kLdsChunks; ++u)
-        {
-            const uint32_t q = pairIndex(eCur, u);
-            const bool shifted = q > lastPairStart;      // then q is the last entry of the arrays
-            const bool validX = q >= eCur.p && q < eCur.end;
-            const bool validY = !shifted && q + 1 < eCur.end;  // q + 1 > the even index below p
-            const float4 bx = slabRows[validX ? (shifted ? cCur[u].y : cCur[u].x) : zeroSlot];
-            const float4 by = slabRows[validY ? cCur[u].y : zeroSlot];
-            const float vx = validX ? (shifted ? vCur[u].y : vCur[u].x) : 0.f;
-            const float vy = validY ? vCur[u].y : 0.f;
-            sum.x = fmaf(vx, bx.x, sum.x);
-            sum.y = fmaf(vx, bx.y, sum.y);
-            sum.z = fmaf(vx, bx.z, sum.z);
-            sum.w = fmaf(vx, bx.w, sum.w);
-            sum.x = fmaf(vy, by.x, sum.x);
-            sum.y = fmaf(vy, by.y, sum.y);
-            sum.z = fmaf(vy, by.z, sum.z);
-            sum.w = fmaf(vy, by.w, sum.w);
-        }
-        // rows with more entries than were fetched ahead
-        const uint32_t fetchedEnd = (eCur.p & ~1u) + 32 * kLdsChunks;
-        if (__builtin_amdgcn_ballot_w64(fetchedEnd < eCur.end) != 0)
-        {
-            for (uint32_t q0 = fetchedEnd; __builtin_amdgcn_ballot_w64(q0 < eCur.end) != 0; q0 += 16)
-            {
-                const uint32_t q = q0 + t;
-                const bool valid = q < eCur.end;
-                const uint32_t idx = valid ? q : partFirst;
-                const uint32_t c = valid ? COL[idx] : zeroSlot;
-                const float v = valid ? V[idx] : 0.f;
-                const float4 b = slabRows[c];
-                sum.x = fmaf(v, b.x, sum.x);
-                sum.y = fmaf(v, b.y, sum.y);
-                sum.z = fmaf(v, b.z, sum.z);
-                sum.w = fmaf(v, b.w, sum.w);
-            }
-        }
-        sum.x = RowSum16(sum.x);
-        sum.y = RowSum16(sum.y);
-        sum.z = RowSum16(sum.z);
-        sum.w = RowSum16(sum.w);
-        const uint32_t row = rowOf(pass);
-        if (t == 0 && row < rowEnd)
-        {
-            if (ACCUMULATE)
-            {
-                sum.x += oldCur.x;
-                sum.y += oldCur.y;
-                sum.z += oldCur.z;
-                sum.w += oldCur.w;
-            }
-            *reinterpret_cast<float4*>(args.out + static_cast<size_t>(row) * N + slab * 4) = sum;
-        }
-        eCur = eNext;
-        eNext = eAfter;
-    };
-    for (uint32_t pass = 0; pass < passes; pass += 2)
-    {
-        onePass(pass, c0, v0, old0, c1, v1, old1);
-        if (pass + 1 < passes)
-            onePass(pass + 1, c1, v1, old1, c0, v0, old0);
-    }
-    // never true (the launcher returns before launching for M == 0): keeps `sink` alive
-    if (args.M == 0 && sink == 0x9e3779b9u)
-        args.out[0] = 0.f;
-}
-
-#pragma clang fp contract(off)
-
 // one output column per lane; any N, any alignment
 __global__ __launch_bounds__(kThreads) void SpmmRowScalar(const SpmmArgs args)
 {
@@ -523,52 +243,10 @@ __global__ __launch_bounds__(kThreads) void SpmmRowScalar(const SpmmArgs args)
 }
 }  // namespace
 
-namespace
-{
-// LDS a workgroup may use on this device (cached), for the slab kernel
-size_t LdsLimit()
-{
-    static size_t limit[16] = {};
-    const int d = sph::CurrentDevice();
-    if (d < 0 || d >= 16)
-        return 0;
-    if (limit[d] == 0)
-    {
-        int bytes = 0;
-        if (hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, d) != hipSuccess ||
-            bytes <= 0)
-            bytes = 64 * 1024;
-        limit[d] = static_cast<size_t>(bytes);
-    }
-    return limit[d];
-}
-
-int SpmmCsr(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW, uint32_t M,
-            uint32_t Kdim, uint32_t N, const float* B, bool accumulate, bool fast);
-}  // namespace
-
 extern "C" {
 
 int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW,
                      uint32_t M, uint32_t Kdim, uint32_t N, const float* B, int accumulate)
-{
-    return SpmmCsr(out, V, COL, ROW, M, Kdim, N, B, accumulate != 0, false);
-}
-
-int sph_spmm_csr_f32_ex(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW,
-                        uint32_t M, uint32_t Kdim, uint32_t N, const float* B, uint32_t flags)
-{
-    SPH_REQUIRE((flags & ~(SPH_SPMM_ACCUMULATE | SPH_SPMM_FAST)) == 0, "unknown flag");
-    return SpmmCsr(out, V, COL, ROW, M, Kdim, N, B, (flags & SPH_SPMM_ACCUMULATE) != 0,
-                   (flags & SPH_SPMM_FAST) != 0);
-}
-
-}  // extern "C"
-
-namespace
-{
-int SpmmCsr(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW, uint32_t M,
-            uint32_t Kdim, uint32_t N, const float* B, bool accumulate, bool fast)
 {
     // column indices are trusted to lie below Kdim, as in the dense leaf
     if (M == 0 || N == 0)
@@ -589,48 +267,12 @@ int SpmmCsr(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW
     args.accumulate = accumulate ? 1 : 0;
 
     const uint32_t blocks = (M + kWavesPerBlock - 1) / kWavesPerBlock;
+    // the slab kernel forms 32-bit byte offsets into B with a 24-bit multiply; larger operands
+    // run on the scalar kernel, whose offsets are 64-bit
     const bool vec = (N % 4 == 0) &&
-                     ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(B)) & 15u) == 0;
-    // Slab of 4 columns over all rows of B in LDS: needs the rows to fit, pays from 64 dense
-    // columns up (below that the slab kernel's gathers already stay in the L2 they came from)
-    if (fast && vec && Kdim != 0 && N >= 64 && static_cast<uint64_t>(Kdim) * N * 4 < (1ull << 32))
-    {
-        LdsSlabPlan plan{};
-        plan.K = Kdim;
-        plan.kSlots = (Kdim + 63u) / 64u * 64u;
-        const size_t ldsBytes = (static_cast<size_t>(plan.kSlots) + 1) * 16;
-        if (ldsBytes <= LdsLimit())
-        {
-            plan.slabs = N / 4;
-            const uint32_t cus = static_cast<uint32_t>(sph::ComputeUnits());
-            plan.parts = std::max(1u, std::min((cus + plan.slabs - 1) / plan.slabs, (M + 63u) / 64u));
-            plan.rowsPerPart = ((M + plan.parts - 1) / plan.parts + 3u) / 4u * 4u;
-            plan.slabGroups = (plan.slabs + 7u) / 8u;
-            const uint64_t units = static_cast<uint64_t>(plan.slabGroups) * plan.parts;
-            const uint64_t grid = 8ull * ((units + 7u) / 8u) * 8u;
-            SPH_REQUIRE(grid < (1ull << 31), "too many workgroups for one launch");
-            static bool raised[16] = {};
-            const int d = sph::CurrentDevice();
-            if (ldsBytes > 64 * 1024 && d >= 0 && d < 16 && !raised[d])
-            {
-                SPH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(SpmmLdsSlab<false>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                static_cast<int>(LdsLimit())));
-                SPH_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(SpmmLdsSlab<true>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                static_cast<int>(LdsLimit())));
-                raised[d] = true;
-            }
-            if (accumulate)
-                hipLaunchKernelGGL(SpmmLdsSlab<true>, dim3(static_cast<uint32_t>(grid)),
-                                   dim3(kLdsThreads), ldsBytes, stream, args, plan);
-            else
-                hipLaunchKernelGGL(SpmmLdsSlab<false>, dim3(static_cast<uint32_t>(grid)),
-                                   dim3(kLdsThreads), ldsBytes, stream, args, plan);
-            SPH_CHECK_LAUNCH();
-            return SPH_OK;
-        }
-    }
+                     ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(B)) & 15u) == 0 &&
+                     static_cast<uint64_t>(Kdim) * N * 4 < (1ull << 32) && Kdim < (1u << 24) &&
+                     N < (1u << 22);
     // 16 lanes per row (64-column slabs, 4 rows per wavefront) measured fastest from N = 64
     // up; narrower operands use 8 lanes per row so that fewer lanes idle
     const int lanesPerRow = N <= 32 ? 8 : 16;
@@ -647,9 +289,6 @@ int SpmmCsr(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW
         plan.columnsPerXcd = (plan.slabs * plan.rowParts + 7) / 8;
         const uint64_t grid = 8ull * plan.columnsPerXcd * plan.blocksPerColumn;
         SPH_REQUIRE(grid < (1ull << 31), "too many workgroups for one launch");
-        SPH_REQUIRE(static_cast<uint64_t>(Kdim) * N * 4 < (1ull << 32) && Kdim < (1u << 24) &&
-                        N < (1u << 22),
-                    "dense operand too large for 32-bit gather offsets");
         if (lanesPerRow == 16)
             hipLaunchKernelGGL(SpmmSlabVec4<16>, dim3(static_cast<uint32_t>(grid)),
                                dim3(kThreads), 0, stream, args, plan);
@@ -663,4 +302,4 @@ int SpmmCsr(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW
     return SPH_OK;
 }
 
-}  // namespace
+}  // extern "C"

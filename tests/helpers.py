@@ -59,9 +59,8 @@ def gpu_gemm_grouped(C, A, B, M, N, K, triples):
     return out
 
 
-def gpu_spmm(C, V, COL, ROW, M, Kdim, N, B, accumulate, canary=0, fast=False):
-    """Runs sph_spmm_csr_f32 (sph_spmm_csr_f32_ex with SPH_SPMM_FAST when `fast`) with `canary`
-    guard floats on both sides of out."""
+def gpu_spmm(C, V, COL, ROW, M, Kdim, N, B, accumulate, canary=0):
+    """Runs sph_spmm_csr_f32 with `canary` guard floats on both sides of out."""
     guard = np.full(canary, np.float32(-12345.5), dtype=np.float32)
     padded = np.concatenate([guard, C.ravel(), guard]).astype(np.float32)
     dC = capi.DeviceBuffer.from_array(padded)
@@ -69,13 +68,8 @@ def gpu_spmm(C, V, COL, ROW, M, Kdim, N, B, accumulate, canary=0, fast=False):
     dCol = capi.DeviceBuffer.from_array(COL if COL.size else np.zeros(1, np.uint32))
     dRow = capi.DeviceBuffer.from_array(ROW)
     dB = capi.DeviceBuffer.from_array(B)
-    if fast:
-        flags = capi.SPH_SPMM_FAST | (capi.SPH_SPMM_ACCUMULATE if accumulate else 0)
-        capi.call("sph_spmm_csr_f32_ex", dC.at(4 * canary), dV.ptr, dCol.ptr, dRow.ptr, M, Kdim, N,
-                  dB.ptr, flags)
-    else:
-        capi.call("sph_spmm_csr_f32", dC.at(4 * canary), dV.ptr, dCol.ptr, dRow.ptr, M, Kdim, N,
-                  dB.ptr, 1 if accumulate else 0)
+    capi.call("sph_spmm_csr_f32", dC.at(4 * canary), dV.ptr, dCol.ptr, dRow.ptr, M, Kdim, N,
+              dB.ptr, 1 if accumulate else 0)
     back = dC.download(np.float32, padded.shape)
     for d in (dC, dV, dCol, dRow, dB):
         d.release()
