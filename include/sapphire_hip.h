@@ -91,6 +91,14 @@ int sph_host_free(void* ptr);
 
 /* Wait for everything this thread enqueued on the current device. */
 int sph_stream_sync(void);
+/* Wait for everything any thread enqueued on the current device (what the
+ * reference's cudaFree and cudaDeviceSynchronize did implicitly). */
+int sph_device_sync(void);
+/* Work this thread enqueues from now on waits for everything hipStream holds so
+ * far; no host wait.  NULL or the thread's own stream is a no-op.  For memory
+ * that passes from one thread's stream to another's (the buffer pool behind
+ * Sources/Sapphire/util/ResourceManager.cpp:38-72 hands blocks across threads). */
+int sph_stream_wait_stream(void* hipStream);
 /* The hipStream_t this thread's calls run on (created on first use). */
 int sph_get_stream(void** hipStream);
 /* Run this thread's later calls on a caller-owned hipStream_t; NULL returns
@@ -200,8 +208,11 @@ int sph_gemm_f32(float* out, const float* A, const float* B, uint32_t M,
  * Sources/Sapphire/operations/Backward/LinearBackward.cpp:49-50,70-73 and
  * MathBackward.cpp:46-51.  The K products of an output element are added in
  * the same order with or without the flags, so the result is bit-identical
- * to sph_transpose_f32 followed by sph_gemm_f32.  SPH_GEMM_OVERWRITE stores
- * the product without reading out (K == 0 then stores zeros). */
+ * to sph_transpose_f32 followed by sph_gemm_f32 -- except for a single output
+ * row (M == 1, K >= 64) with SPH_GEMM_TRANS_B: the plain call then runs a
+ * row-reduction kernel that adds in another order, and the two agree within
+ * the fp32 tolerance only.  SPH_GEMM_OVERWRITE stores the product without
+ * reading out (K == 0 then stores zeros). */
 int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M,
                     uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,
                     int64_t strideA, int64_t strideB, uint32_t flags);

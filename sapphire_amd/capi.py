@@ -71,6 +71,8 @@ SIGNATURES = {
     "sph_host_malloc": [ctypes.POINTER(_vp), _sz],
     "sph_host_free": [_vp],
     "sph_stream_sync": [],
+    "sph_device_sync": [],
+    "sph_stream_wait_stream": [_vp],
     "sph_get_stream": [ctypes.POINTER(_vp)],
     "sph_set_stream": [_vp],
     "sph_event_create": [ctypes.POINTER(_vp)],

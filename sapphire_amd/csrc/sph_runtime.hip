@@ -304,6 +304,36 @@ int sph_stream_sync(void)
     return SPH_OK;
 }
 
+int sph_device_sync(void)
+{
+    SPH_REFUSE_WHILE_CAPTURING();
+    SPH_HIP_TRY(hipSetDevice(tlsSlots.device));
+    SPH_HIP_TRY(hipDeviceSynchronize());
+    return SPH_OK;
+}
+
+int sph_stream_wait_stream(void* hipStream)
+{
+    SPH_REFUSE_WHILE_CAPTURING();
+    SPH_STREAM_OR_FAIL(stream);
+    hipStream_t other = static_cast<hipStream_t>(hipStream);
+    if (other == nullptr || other == stream)
+        return SPH_OK;
+    hipEvent_t marker = nullptr;
+    SPH_HIP_TRY(hipEventCreateWithFlags(&marker, hipEventDisableTiming));
+    hipError_t err = hipEventRecord(marker, other);
+    if (err == hipSuccess)
+        err = hipStreamWaitEvent(stream, marker, 0);
+    // the event's resources are released once the wait has been satisfied
+    const hipError_t destroyed = hipEventDestroy(marker);
+    if (err == hipSuccess)
+        err = destroyed;
+    if (err != hipSuccess)
+        return sph::Fail(SPH_ERR_DEVICE, std::string("sph_stream_wait_stream failed with ") +
+                                             hipGetErrorString(err));
+    return SPH_OK;
+}
+
 int sph_get_stream(void** hipStream)
 {
     SPH_REQUIRE(hipStream != nullptr, "hipStream is null");

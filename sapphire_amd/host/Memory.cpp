@@ -99,4 +99,21 @@ void Synchronize()
 {
     Check(sph_stream_sync(), "Synchronize");
 }
+
+void SynchronizeDevice()
+{
+    Check(sph_device_sync(), "SynchronizeDevice");
+}
+
+StreamHandle CurrentStream()
+{
+    void* stream = nullptr;
+    Check(sph_get_stream(&stream), "CurrentStream");
+    return stream;
+}
+
+void StreamWaitStream(StreamHandle stream)
+{
+    Check(sph_stream_wait_stream(stream), "StreamWaitStream");
+}
 }  // namespace Sapphire::Compute::Cuda

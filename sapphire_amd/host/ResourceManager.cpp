@@ -1,122 +1,16 @@
 #include <Sapphire/util/ResourceManager.hpp>
 
 #include <Sapphire/compute/cudaUtil/Memory.hpp>
+#include <Sapphire/util/BlockPool.hpp>
 
 #include <cstdlib>
-#include <map>
 #include <mutex>
 #include <stdexcept>
-#include <string>
-#include <unordered_map>
 
 namespace Sapphire::Util
 {
 namespace
 {
-constexpr std::size_t kGranule = 256;
-
-std::size_t RoundUp(std::size_t bytes)
-{
-    return (bytes + kGranule - 1) / kGranule * kGranule;
-}
-
-// One memory space (host or device): live blocks by address, idle blocks by size.
-class Space
-{
-public:
-    using Allocate = void* (*)(std::size_t);
-    using Release = void (*)(void*);
-
-    Space(Allocate allocate, Release release) : m_allocate(allocate), m_release(release) {}
-
-    void* Get(std::size_t byteSize, bool preserve)
-    {
-        const std::size_t size = RoundUp(byteSize);
-        if (preserve)
-        {
-            void* ptr = m_allocate(size);
-            m_preserved.emplace(ptr, size);
-            return ptr;
-        }
-        void* ptr = nullptr;
-        const auto idle = m_free.find(size);
-        if (idle != m_free.end())
-        {
-            ptr = idle->second;
-            m_free.erase(idle);
-        }
-        else
-            ptr = m_allocate(size);
-        m_volatile.emplace(ptr, size);
-        return ptr;
-    }
-
-    void FreePreserved(void* ptr, const char* who)
-    {
-        const auto it = Find(m_preserved, ptr, who, "Given ptr to free was not found");
-        m_release(ptr);
-        m_preserved.erase(it);
-    }
-
-    void ToPreserved(void* ptr, const char* who)
-    {
-        const auto it = Find(m_volatile, ptr, who, "Cannot find given ptr");
-        m_preserved.insert(*it);
-        m_volatile.erase(it);
-    }
-
-    void ToVolatile(void* ptr, const char* who)
-    {
-        const auto it = Find(m_preserved, ptr, who, "Cannot find given ptr");
-        m_volatile.insert(*it);
-        m_preserved.erase(it);
-    }
-
-    void Clean()
-    {
-        for (const auto& [ptr, size] : m_volatile)
-            m_free.emplace(size, ptr);
-        m_volatile.clear();
-    }
-
-    void ClearPreserved() { ReleaseAll(m_preserved); }
-    void ClearVolatile() { ReleaseAll(m_volatile); }
-    void ClearFree()
-    {
-        for (const auto& [size, ptr] : m_free)
-            m_release(ptr);
-        m_free.clear();
-    }
-
-    std::size_t CountVolatile() const { return m_volatile.size(); }
-    std::size_t CountPreserved() const { return m_preserved.size(); }
-    std::size_t CountFree() const { return m_free.size(); }
-
-private:
-    using Live = std::unordered_map<void*, std::size_t>;
-
-    static Live::iterator Find(Live& pool, void* ptr, const char* who, const char* what)
-    {
-        const auto it = pool.find(ptr);
-        if (it == pool.end())
-            throw std::runtime_error(std::string("ResourceManager::") + who + " - " + what);
-        return it;
-    }
-
-    void ReleaseAll(Live& pool)
-    {
-        for (const auto& [ptr, size] : pool)
-            m_release(ptr);
-        pool.clear();
-    }
-
-    Allocate m_allocate;
-    Release m_release;
-    Live m_volatile;
-    Live m_preserved;
-    std::multimap<std::size_t, void*> m_free;
-};
-
 void* AllocateHost(std::size_t size)
 {
     void* ptr = std::aligned_alloc(64, size);
@@ -145,9 +39,26 @@ void ReleaseCuda(void* ptr)
     Compute::Cuda::CudaFreeAsync(ptr);
 }
 
+void* NoStream()
+{
+    return nullptr;
+}
+
+void NoWait(void*) {}
+
+void* CurrentCudaStream()
+{
+    return Compute::Cuda::CurrentStream();
+}
+
+void WaitForCudaStream(void* stream)
+{
+    Compute::Cuda::StreamWaitStream(stream);
+}
+
 std::mutex gMutex;
-Space gHost(AllocateHost, ReleaseHost);
-Space gCuda(AllocateCuda, ReleaseCuda);
+BlockPool gHost({ AllocateHost, ReleaseHost, NoStream, NoWait });
+BlockPool gCuda({ AllocateCuda, ReleaseCuda, CurrentCudaStream, WaitForCudaStream });
 }  // namespace
 
 void* ResourceManager::GetMemoryCuda(std::size_t byteSize, bool preserve)
@@ -228,14 +139,14 @@ void ResourceManager::ClearFreePool()
 
 void ResourceManager::ClearAll()
 {
-    // device work that may still use the blocks has to finish first
+    // device work that may still use the blocks, on any thread's stream, has to finish first
     bool deviceBlocks = false;
     {
         std::lock_guard<std::mutex> lock(gMutex);
         deviceBlocks = gCuda.CountVolatile() + gCuda.CountPreserved() + gCuda.CountFree() > 0;
     }
     if (deviceBlocks)
-        Compute::Cuda::Synchronize();
+        Compute::Cuda::SynchronizeDevice();
     ClearPreservedPool();
     ClearVolatilePool();
     ClearFreePool();

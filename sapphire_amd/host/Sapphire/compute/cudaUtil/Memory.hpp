@@ -35,6 +35,13 @@ void CopyDeviceToDeviceBroadcast(void* dst, const void* src, std::size_t byteSiz
                                  std::size_t srcStrideByteSize);
 //! Waits for everything the calling thread has enqueued on the current device.
 void Synchronize();
+//! Waits for everything any thread has enqueued on the current device.
+void SynchronizeDevice();
+//! The stream the calling thread's work on the current device is enqueued on.
+StreamHandle CurrentStream();
+//! Work the calling thread enqueues from now on waits for everything `stream` holds so far
+//! (nothing happens when it is the calling thread's own stream).
+void StreamWaitStream(StreamHandle stream);
 }  // namespace Sapphire::Compute::Cuda
 
 #endif

@@ -13,6 +13,7 @@
 #include <Sapphire/operations/Backward/LinearBackward.hpp>
 #include <Sapphire/operations/Backward/MathBackward.hpp>
 #include <Sapphire/operations/Forward/LinearForward.hpp>
+#include <Sapphire/util/BlockPool.hpp>
 #include <Sapphire/util/ResourceManager.hpp>
 
 #include <algorithm>
@@ -20,6 +21,7 @@
 #include <exception>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 using namespace Sapphire;
@@ -111,6 +113,87 @@ int sphh_shape_query(const int* dims, int n, int what, int arg)
         }
     });
     return result;
+}
+
+// The buffer pool's bookkeeping on fake memory and fake streams (no device): `ops` holds
+// triples (code, stream, argument) with code 0 = volatile request of `argument` bytes,
+// 1 = preserved request, 2 = Clean, 3 = FreePreserved(block `argument`), 4 = ClearFree,
+// 5 = ClearVolatile, 6 = ClearPreserved; `stream` (1, 2, ...) is the stream of the thread that
+// makes the call.  The log receives triples (event, a, b): event 0 = block a handed out,
+// 1 = block a allocated, 2 = block a released on stream b, 3 = stream a made to wait for
+// stream b.  Returns the number of log triples written, -1 on an exception.
+namespace
+{
+struct FakeMemory
+{
+    long long* log = nullptr;
+    int cap = 0, used = 0;
+    long long nextBlock = 1;
+    long long stream = 0;
+    void Log(long long e, long long a, long long b)
+    {
+        if (used < cap)
+        {
+            log[3 * used] = e;
+            log[3 * used + 1] = a;
+            log[3 * used + 2] = b;
+        }
+        ++used;
+    }
+};
+FakeMemory* gFake = nullptr;
+void* FakeAllocate(std::size_t)
+{
+    const long long id = gFake->nextBlock++;
+    gFake->Log(1, id, 0);
+    return reinterpret_cast<void*>(static_cast<uintptr_t>(id));
+}
+void FakeRelease(void* ptr)
+{
+    gFake->Log(2, static_cast<long long>(reinterpret_cast<uintptr_t>(ptr)), gFake->stream);
+}
+void* FakeStream()
+{
+    return reinterpret_cast<void*>(static_cast<uintptr_t>(gFake->stream));
+}
+void FakeWait(void* stream)
+{
+    gFake->Log(3, gFake->stream, static_cast<long long>(reinterpret_cast<uintptr_t>(stream)));
+}
+}  // namespace
+
+int sphh_block_pool_run(const int* ops, int count, long long* log, int logCap)
+{
+    int written = -1;
+    Guard([&] {
+        FakeMemory fake;
+        fake.log = log;
+        fake.cap = logCap;
+        gFake = &fake;
+        Util::BlockPool pool({ FakeAllocate, FakeRelease, FakeStream, FakeWait });
+        for (int i = 0; i < count; ++i)
+        {
+            const int code = ops[3 * i], arg = ops[3 * i + 2];
+            fake.stream = ops[3 * i + 1];
+            void* block = reinterpret_cast<void*>(static_cast<uintptr_t>(arg));
+            switch (code)
+            {
+                case 0:
+                case 1:
+                    fake.Log(0, static_cast<long long>(reinterpret_cast<uintptr_t>(
+                                    pool.Get(static_cast<std::size_t>(arg), code == 1))), 0);
+                    break;
+                case 2: pool.Clean(); break;
+                case 3: pool.FreePreserved(block, "FreePreserved"); break;
+                case 4: pool.ClearFree(); break;
+                case 5: pool.ClearVolatile(); break;
+                default: pool.ClearPreserved(); break;
+            }
+        }
+        gFake = nullptr;
+        written = fake.used;
+    });
+    return written;
 }
 
 // leaves: 4 x uint64 per leaf (outOff, aOff, bOff, totalSizeOut); dims7: M N K maxDim sizes;
@@ -611,6 +694,55 @@ int sphh_tensor_lifecycle()
 }
 
 // Host-only checks (no device): pools, TensorData in Host mode, error paths.
+// A device block that passes from one thread's stream to another's through the pool: the
+// first thread keeps its stream busy writing 1 into the block, returns the block with Clean()
+// without waiting, and a second thread takes the block of that size, writes 2 and reads it
+// back.  Every element must read 2: the second stream has to wait for the first one's writes.
+// Returns 0 when that holds, 1 when the block was not reused, 2 when stale values were seen.
+int sphh_pool_handover()
+{
+    int result = -1;
+    Guard([&] {
+        Util::ResourceManager::ClearAll();
+        Compute::Cuda::CudaSetDevice(0);
+        const std::size_t count = std::size_t(16) << 20;  // 64 MiB of floats
+        float* first = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(count * 4));
+        for (int i = 0; i < 40; ++i)
+            Compute::Dense::Cuda::Scalar(first, 1.0f, count);
+        Util::ResourceManager::Clean();  // no wait: the writes above are still in flight
+        int outcome = 0;
+        std::thread second([&] {
+            try
+            {
+                Compute::Cuda::CudaSetDevice(0);
+                float* block = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(count * 4));
+                if (block != first)
+                    outcome = 1;
+                Compute::Dense::Cuda::Scalar(block, 2.0f, count);
+                std::vector<float> host(count);
+                Compute::Cuda::CopyDeviceToHost(host.data(), block, count * 4);
+                Compute::Cuda::Synchronize();
+                // give the first stream time to finish what it still had queued
+                Compute::Cuda::SynchronizeDevice();
+                Compute::Cuda::CopyDeviceToHost(host.data(), block, count * 4);
+                for (float v : host)
+                    if (v != 2.0f && outcome == 0)
+                        outcome = 2;
+            }
+            catch (const std::exception& e)
+            {
+                lastError = e.what();
+                outcome = 3;
+            }
+        });
+        second.join();
+        Compute::Cuda::SynchronizeDevice();
+        Util::ResourceManager::ClearAll();
+        result = outcome;
+    });
+    return result;
+}
+
 int sphh_host_only_lifecycle()
 {
     int failed = 0;

@@ -24,7 +24,8 @@ FLAG_SETS = [capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
 # paths, ragged edges
 SHAPES = [(1, 1, 1), (3, 5, 7), (64, 64, 64), (65, 33, 17), (128, 96, 40), (257, 130, 31),
           (512, 384, 100), (2048, 2048, 64), (4096, 2048, 32), (32, 32, 1024), (40, 24, 515),
-          (8, 200, 4096), (1000, 10, 1000), (256, 256, 96), (640, 600, 72)]
+          (8, 200, 4096), (1000, 10, 1000), (256, 256, 96), (640, 600, 72), (1, 200, 64),
+          (1, 1000, 4096), (1, 64, 63)]
 
 
 def bits(x):
@@ -56,7 +57,12 @@ def test_flags_match_checker_and_materialised_transpose(dev, shape, flags):
     Bd = h.gpu_transpose(Bs, N, K)[0] if flags & capi.SPH_GEMM_TRANS_B else B
     assert np.array_equal(bits(Ad), bits(A)) and np.array_equal(bits(Bd), bits(B))
     plain = h.gpu_gemm_f32(C, Ad, Bd, M, N, K)
-    assert np.array_equal(bits(got), bits(plain))
+    if M == 1 and K >= 64 and flags & capi.SPH_GEMM_TRANS_B:
+        # a single row of plain operands runs the row-reduction kernel (another summation
+        # order than the matrix-core kernels the transposed B goes to): tolerance only
+        assert h.normalised_error(got, plain, np.abs(A), np.abs(B)) <= TOL_F32
+    else:
+        assert np.array_equal(bits(got), bits(plain))
 
 
 @pytest.mark.parametrize("flags", FLAG_SETS)

@@ -163,6 +163,13 @@ def test_tensor_data_life_cycle_on_device(dev):
     assert rc == 0, (rc, lib.sphh_last_error())
 
 
+def test_pool_block_handed_to_another_threads_stream(dev):
+    h.announce("ResourceManager: block reused by a second thread while the first stream still writes")
+    lib = hl.lib()
+    rc = lib.sphh_pool_handover()
+    assert rc == 0, (rc, lib.sphh_last_error())
+
+
 # ---- backward neighbours and the Linear backward pass -------------------------------------------
 
 def _bits(x):

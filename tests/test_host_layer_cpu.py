@@ -96,3 +96,57 @@ def test_matching_dim_agrees_with_checker():
         assert hl.matching_dim(shapes) == po.matching_dim(shapes), shapes
     with pytest.raises(RuntimeError):
         hl.matching_dim([])
+
+
+# ---- buffer pool bookkeeping: blocks are stream-affine ------------------------------------
+def _pool_run(ops):
+    import ctypes
+    flat = (ctypes.c_int * (3 * len(ops)))(*[int(x) for op in ops for x in op])
+    log = (ctypes.c_longlong * (3 * 64))()
+    fn = hl.lib().sphh_block_pool_run
+    fn.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.POINTER(ctypes.c_longlong),
+                   ctypes.c_int]
+    n = fn(flat, len(ops), log, 64)
+    assert 0 <= n <= 64, hl.lib().sphh_last_error()
+    return [tuple(log[3 * i:3 * i + 3]) for i in range(n)]
+
+
+GET, PRESERVE, CLEAN, FREE_PRESERVED, CLEAR_FREE, CLEAR_VOLATILE, CLEAR_PRESERVED = range(7)
+HANDED, ALLOCATED, RELEASED, WAITS = range(4)
+
+
+def test_pool_reuse_on_the_same_stream_needs_no_wait():
+    log = _pool_run([(GET, 1, 1000), (CLEAN, 1, 0), (GET, 1, 1000)])
+    # 1000 bytes round up to 1024; the second request takes the idle block of that size
+    assert log == [(ALLOCATED, 1, 0), (HANDED, 1, 0), (HANDED, 1, 0)]
+
+
+def test_pool_reuse_from_another_stream_waits_for_the_first():
+    log = _pool_run([(GET, 1, 1000), (CLEAN, 1, 0), (GET, 2, 1024), (CLEAN, 2, 0), (GET, 2, 1024),
+                     (GET, 2, 300)])
+    assert log == [(ALLOCATED, 1, 0), (HANDED, 1, 0),
+                   (WAITS, 2, 1), (HANDED, 1, 0),       # stream 2 takes over what stream 1 used
+                   (HANDED, 1, 0),                      # now stream 2's own: no wait
+                   (ALLOCATED, 2, 0), (HANDED, 2, 0)]   # another size: a fresh block
+
+
+def test_pool_release_from_another_stream_waits_for_the_owner():
+    log = _pool_run([(PRESERVE, 1, 512), (FREE_PRESERVED, 2, 1),
+                     (GET, 1, 64), (CLEAN, 2, 0), (CLEAR_FREE, 2, 0),
+                     (GET, 3, 64), (CLEAR_VOLATILE, 3, 0)])
+    assert log == [(ALLOCATED, 1, 0), (HANDED, 1, 0),
+                   (WAITS, 2, 1), (RELEASED, 1, 2),
+                   (ALLOCATED, 2, 0), (HANDED, 2, 0),
+                   (WAITS, 2, 1), (RELEASED, 2, 2),
+                   (ALLOCATED, 3, 0), (HANDED, 3, 0), (RELEASED, 3, 3)]
+
+
+def test_pool_unknown_block_is_refused():
+    import ctypes
+    flat = (ctypes.c_int * 3)(FREE_PRESERVED, 1, 77)
+    log = (ctypes.c_longlong * 3)()
+    fn = hl.lib().sphh_block_pool_run
+    fn.argtypes = [ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.POINTER(ctypes.c_longlong),
+                   ctypes.c_int]
+    assert fn(flat, 1, log, 1) == -1
+    assert b"Given ptr to free was not found" in hl.lib().sphh_last_error()
