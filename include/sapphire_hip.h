@@ -120,8 +120,8 @@ int sph_event_destroy(void* event);
  * into the graph instead of running; entry points that wait for the device,
  * allocate, free, read back or change the stream or device (copies to or from
  * the host, sph_stream_sync, sph_malloc/sph_free, sph_event_elapsed_ms,
- * sph_gemm_f32_grouped, sph_csr_row_offsets_f32 with a host count or more
- * than 65535 rows) return SPH_ERR_UNSUPPORTED and leave the capture intact.
+ * sph_gemm_f32_grouped -- use sph_gemm_f32_grouped_device --,
+ * sph_csr_row_offsets_f32 with a host count or more than 65535 rows) return SPH_ERR_UNSUPPORTED and leave the capture intact.
  * sph_graph_launch enqueues one replay on the thread's stream.  The recorded
  * pointers and sizes are fixed; change inputs by writing into the same
  * buffers.  No counterpart in the reference (its cuBLAS calls are issued one
@@ -236,7 +236,9 @@ int sph_linear_forward_f32(float* y, const float* x, const float* W,
  * is the whole leaf list of BroadcastWith2Inputs
  * (Includes/Sapphire/compute/Broadcast.hpp:83-133) issued as one launch in
  * place of one cuBLAS call per leaf.  Entries whose outOff coincide are
- * applied in entry order. */
+ * applied in entry order.  The table travels through a staging buffer and a
+ * device buffer that belong to the calling thread, so calls from different
+ * threads do not wait for each other. */
 typedef struct
 {
     uint64_t outOff;
@@ -247,6 +249,19 @@ typedef struct
 int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out,
                          const float* A, const float* B, uint32_t M, uint32_t N,
                          uint32_t K);
+
+/* The same launch with the table already in device memory that the caller
+ * owns (and keeps unchanged until the launch has run): nothing is uploaded, so
+ * the call can be recorded into a graph and never waits.  The caller
+ * guarantees that no two entries share an outOff (sph_gemm_f32_grouped cuts
+ * such lists into ordered launches on the host; here one launch applies all
+ * entries at once).  SPH_GROUPED_OFFSETS_MULTIPLE_OF_4 promises that every
+ * offset is a multiple of 4 elements, which lets the kernels use 16-byte
+ * accesses when the bases and M, N, K allow; without it they assume nothing. */
+#define SPH_GROUPED_OFFSETS_MULTIPLE_OF_4 1u
+int sph_gemm_f32_grouped_device(const SphGemmEntry* deviceEntries, uint32_t count,
+                                float* out, const float* A, const float* B,
+                                uint32_t M, uint32_t N, uint32_t K, uint32_t flags);
 
 /* Half-precision inputs, fp32 accumulation, fp32 output: the tensor-core path
  * the reference declares as WmmaGemm

@@ -21,6 +21,7 @@ SPH_GEMM_OVERWRITE = 1
 SPH_GEMM_TRANS_A = 2
 SPH_GEMM_TRANS_B = 4
 SPH_LINEAR_RELU = 1
+SPH_GROUPED_OFFSETS_MULTIPLE_OF_4 = 1
 
 
 class SphError(RuntimeError):
@@ -95,6 +96,7 @@ SIGNATURES = {
     "sph_gemm_f32_ex": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
     "sph_linear_forward_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32],
     "sph_gemm_f32_grouped": [ctypes.POINTER(SphGemmEntry), _u32, _vp, _vp, _vp, _u32, _u32, _u32],
+    "sph_gemm_f32_grouped_device": [_vp, _u32, _vp, _vp, _vp, _u32, _u32, _u32, _u32],
     "sph_gemm_f16f32": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
     "sph_csr_row_offsets_f32": [_vp, _vp, _u32, _u32, _u32, ctypes.POINTER(ctypes.c_uint32)],
     "sph_csr_row_offsets_noalloc_f32": [_vp, _vp, _u32, _u32, _u32],

@@ -30,6 +30,7 @@
 #include <mutex>
 #include <type_traits>
 #include <unordered_set>
+#include <vector>
 
 namespace
 {
@@ -1097,21 +1098,53 @@ __global__ __launch_bounds__(kGemvWaves * 64) void GemvRowKernel(const GemmF32Ar
     out[col] = v;
 }
 
-// Device table for grouped launches: one growing buffer per device with a
-// pinned staging copy.  The table is shared by every caller, so its use is
-// serialised by a mutex and, across streams, by waiting for the stream that
-// used it last.
+// Offset tables of grouped launches: a device buffer the kernels read plus a pinned staging
+// copy, per host thread and device, like the thread's stream -- two threads never wait for
+// each other.  A thread's launches are ordered by its stream, so the only waits are for the
+// thread's own earlier upload (before the staging copy is overwritten) and, when the thread
+// has moved to another stream since (sph_set_stream), an event wait of the new stream for the
+// old one.  Tables of threads that have ended are kept for the next thread.
 struct EntryTable
 {
     SphGemmEntry* dev = nullptr;
     SphGemmEntry* staging = nullptr;  // pinned
     size_t capacity = 0;
     hipEvent_t uploaded = nullptr;    // staging may be overwritten after this
+    hipEvent_t consumed = nullptr;    // the last launch that read dev has finished after this
     bool uploadPending = false;
     hipStream_t lastStream = nullptr;
 };
-std::mutex gTableMutex;
-EntryTable gTables[16];
+std::mutex gIdleTableMutex;
+std::vector<EntryTable> gIdleTables[16];
+
+struct ThreadTables
+{
+    EntryTable table[16];
+    bool have[16] = {};
+    ~ThreadTables()
+    {
+        std::lock_guard<std::mutex> lock(gIdleTableMutex);
+        for (int d = 0; d < 16; ++d)
+            if (have[d])
+                gIdleTables[d].push_back(table[d]);
+    }
+};
+thread_local ThreadTables tlsTables;
+
+EntryTable& ThreadTable(int device)
+{
+    if (!tlsTables.have[device])
+    {
+        std::lock_guard<std::mutex> lock(gIdleTableMutex);
+        if (!gIdleTables[device].empty())
+        {
+            tlsTables.table[device] = gIdleTables[device].back();
+            gIdleTables[device].pop_back();
+        }
+        tlsTables.have[device] = true;
+    }
+    return tlsTables.table[device];
+}
 
 template <int TILE, bool TA, bool TB>
 void LaunchSkinnyTile(const GemmF32Args& args, dim3 grid, bool vec, bool wide, hipStream_t stream)
@@ -1306,7 +1339,7 @@ int GrowTable(EntryTable& t, size_t count)
         return SPH_OK;
     // nothing may still be reading the old buffers
     if (t.lastStream != nullptr)
-        SPH_HIP_TRY(hipStreamSynchronize(t.lastStream));
+        SPH_HIP_TRY(hipEventSynchronize(t.consumed));
     if (t.dev != nullptr)
         SPH_HIP_TRY(hipFree(t.dev));
     if (t.staging != nullptr)
@@ -1323,6 +1356,8 @@ int GrowTable(EntryTable& t, size_t count)
                               hipHostMallocDefault));
     if (t.uploaded == nullptr)
         SPH_HIP_TRY(hipEventCreateWithFlags(&t.uploaded, hipEventDisableTiming));
+    if (t.consumed == nullptr)
+        SPH_HIP_TRY(hipEventCreateWithFlags(&t.consumed, hipEventDisableTiming));
     t.capacity = cap;
     return SPH_OK;
 }
@@ -1403,7 +1438,7 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
                          const float* B, uint32_t M, uint32_t N, uint32_t K)
 {
     SPH_REQUIRE(M != 0 && N != 0, "M and N must be non-zero");
-    SPH_REFUSE_WHILE_CAPTURING();  // the offset table is uploaded from a shared staging buffer
+    SPH_REFUSE_WHILE_CAPTURING();  // the offset table is uploaded from host memory
     if (count == 0 || K == 0)
         return SPH_OK;
     SPH_REQUIRE(entries != nullptr && out != nullptr && A != nullptr && B != nullptr,
@@ -1411,6 +1446,8 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
+    const int device = sph::CurrentDevice();
+    SPH_REQUIRE(device >= 0 && device < 16, "device id out of range");
 
     bool offsetsAligned = true, outAligned = true;
     for (uint32_t i = 0; i < count; ++i)
@@ -1419,15 +1456,16 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
         outAligned = outAligned && (entries[i].outOff % 4) == 0;
     }
 
-    std::lock_guard<std::mutex> lock(gTableMutex);
-    EntryTable& t = gTables[sph::CurrentDevice()];
+    EntryTable& t = ThreadTable(device);
     {
         const int rc = GrowTable(t, count);
         if (rc != SPH_OK)
             return rc;
     }
+    // the thread has moved to another stream since the table was last read: order the new
+    // stream behind that launch (no host wait)
     if (t.lastStream != nullptr && t.lastStream != stream)
-        SPH_HIP_TRY(hipStreamSynchronize(t.lastStream));
+        SPH_HIP_TRY(hipStreamWaitEvent(stream, t.consumed, 0));
     if (t.uploadPending)
         SPH_HIP_TRY(hipEventSynchronize(t.uploaded));
     std::memcpy(t.staging, entries, count * sizeof(SphGemmEntry));
@@ -1441,7 +1479,8 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
     // cut the list into launches inside which every outOff is distinct.
     uint32_t begin = 0;
     std::unordered_set<uint64_t> seen;
-    while (begin < count)
+    int rc = SPH_OK;
+    while (begin < count && rc == SPH_OK)
     {
         seen.clear();
         uint32_t end = begin;
@@ -1456,12 +1495,36 @@ int sph_gemm_f32_grouped(const SphGemmEntry* entries, uint32_t count, float* out
         args.M = M;
         args.N = N;
         args.K = K;
-        const int rc = Launch(args, end - begin, offsetsAligned, outAligned, false, false, stream);
-        if (rc != SPH_OK)
-            return rc;
+        rc = Launch(args, end - begin, offsetsAligned, outAligned, false, false, stream);
         begin = end;
     }
-    return SPH_OK;
+    SPH_HIP_TRY(hipEventRecord(t.consumed, stream));
+    return rc;
+}
+
+int sph_gemm_f32_grouped_device(const SphGemmEntry* deviceEntries, uint32_t count, float* out,
+                                const float* A, const float* B, uint32_t M, uint32_t N,
+                                uint32_t K, uint32_t flags)
+{
+    SPH_REQUIRE(M != 0 && N != 0, "M and N must be non-zero");
+    SPH_REQUIRE((flags & ~SPH_GROUPED_OFFSETS_MULTIPLE_OF_4) == 0, "unknown flag");
+    if (count == 0 || K == 0)
+        return SPH_OK;
+    SPH_REQUIRE(deviceEntries != nullptr && out != nullptr && A != nullptr && B != nullptr,
+                "null pointer");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    const bool aligned = (flags & SPH_GROUPED_OFFSETS_MULTIPLE_OF_4) != 0;
+    GemmF32Args args{};
+    args.out = out;
+    args.A = A;
+    args.B = B;
+    args.entries = deviceEntries;
+    args.M = M;
+    args.N = N;
+    args.K = K;
+    return Launch(args, count, aligned, aligned, false, false, stream);
 }
 
 }  // extern "C"

@@ -152,3 +152,44 @@ def test_blocking_calls_are_refused_during_capture_and_capture_survives(dev):
         capi.call("sph_graph_end_capture", capi.ctypes.byref(handle))   # nothing in progress
     dX.release()
     dY.release()
+
+
+def test_non_affine_broadcast_walk_recorded_into_a_graph(dev):
+    """The leaf list of a broadcast walk whose offsets are not affine (the reference's
+    (chunk % size) * stride rule, here out[u] += A[u % 3] * B[(2 * u) % 5]) kept in a device
+    table the caller owns and launched with sph_gemm_f32_grouped_device inside a recorded
+    graph; every replay equals the eager grouped launch bit for bit."""
+    from oracle import pyoracle as po
+    M, N, K, units = 48, 40, 36, 10
+    h.announce("sph_gemm_f32_grouped_device in a graph", (M, N, K, units))
+    A = synth.uniform(9101, (3, M, K))
+    B = synth.uniform(9102, (5, K, N))
+    C0 = synth.uniform(9103, (units, M, N))
+    triples = [(u * M * N, (u % 3) * M * K, ((2 * u) % 5) * K * N) for u in range(units)]
+    table = np.array(triples, dtype=np.uint64)
+    dTable = capi.DeviceBuffer.from_array(table)
+    dA, dB = capi.DeviceBuffer.from_array(A), capi.DeviceBuffer.from_array(B)
+    dC = capi.DeviceBuffer.from_array(C0)
+    with capi.Graph() as g:
+        with pytest.raises(capi.SphError):          # the uploading form refuses a capture
+            capi.call("sph_gemm_f32_grouped", capi.make_entries(triples), units, dC.ptr, dA.ptr,
+                      dB.ptr, M, N, K)
+        capi.call("sph_gemm_f32_grouped_device", dTable.ptr, units, dC.ptr, dA.ptr, dB.ptr, M, N, K,
+                  capi.SPH_GROUPED_OFFSETS_MULTIPLE_OF_4)
+    ref = C0.copy()
+    for rep in range(3):
+        g.launch()
+        capi.sync()
+        got = dC.download(np.float32, C0.shape)
+        for o, a, b in triples:
+            u = o // (M * N)
+            ref[u] = po.naive_gemm(ref[u], A[a // (M * K)], B[b // (K * N)], M, N, K)
+        den = 1.0 + (rep + 1) * K
+        assert float(np.max(np.abs(got - ref))) <= 1e-4 * den
+        # eager work between the replays: the same walk through the uploading entry point on a copy
+        eager = h.gpu_gemm_grouped(C0, A, B, M, N, K, triples)
+        if rep == 0:
+            assert np.array_equal(bits(eager), bits(got))
+    g.destroy()
+    for d in (dTable, dA, dB, dC):
+        d.release()

@@ -59,3 +59,40 @@ def test_threads_get_distinct_streams_and_independent_results(dev):
         th.join()
     assert not errors, errors
     assert len(set(streams)) == 4 and all(streams), streams
+
+
+def test_concurrent_grouped_launches_with_growing_tables(dev):
+    """Grouped launches from 4 threads at once, each with its own offset tables of growing
+    length (the tables are per thread: no thread waits for another, none sees another's
+    offsets), including lists with repeated output units that are cut into ordered launches."""
+    h.announce("sph_gemm_f32_grouped from 4 threads, tables of 3 .. 3000 entries")
+    M, N, K = 16, 24, 8
+    errors = []
+
+    def worker(t):
+        try:
+            capi.call("sph_set_device", 0)
+            for count in (3, 40, 1500, 3000, 7):
+                units = count
+                A = synth.uniform(700 + t, (units, M, K))
+                B = synth.uniform(800 + t, (5, K, N))
+                C = synth.uniform(900 + t, (max(units // 2, 1), M, N))
+                # unit u: out[u % outs] += A[u] * B[(u * 7 + t) % 5]: non-affine, outputs repeat
+                outs = C.shape[0]
+                triples = [((u % outs) * M * N, u * M * K, ((u * 7 + t) % 5) * K * N)
+                           for u in range(units)]
+                ref = C.copy()
+                for o, a, b in triples:
+                    ref[o // (M * N)] = po.naive_gemm(ref[o // (M * N)], A[a // (M * K)],
+                                                      B[b // (K * N)], M, N, K)
+                got = h.gpu_gemm_grouped(C, A, B, M, N, K, triples)
+                assert np.allclose(got, ref, rtol=1e-4, atol=1e-4), (t, count)
+        except BaseException as exc:  # noqa: BLE001 - reported by the main thread
+            errors.append((t, repr(exc)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
