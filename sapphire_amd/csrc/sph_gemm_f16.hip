@@ -28,7 +28,7 @@
 //
 //   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned, any M: the
 //     same ingredients on 128 x 128 tiles with 4 wavefronts (v_mfma_f32_32x32x16_f16), for
-//     shapes with too few 256-tiles to fill the chip and for operands stored transposed.
+//     shapes with too few 256-tiles to fill the chip.
 //
 //   GemmF16General  everything else.  128 x 128 tile, 4 wavefronts, K step 32,
 //     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
@@ -210,7 +210,7 @@ constexpr int CLoopSteps(int csp)
 {
     return (8 * csp + 1 + 3) / 4 * 4;
 }
-template <bool RAGGED, int CSP>
+template <bool RAGGED, int CSP, bool TA, bool TB>
 __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 {
     constexpr int WAVES = 8;
@@ -240,10 +240,17 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     const uint32_t K = args.K, N = args.N;
     const uint32_t rowsLeft = RAGGED ? min(static_cast<uint32_t>(kT), args.M - tm * kT) : kT;
     const uint32_t colsLeft = RAGGED ? min(static_cast<uint32_t>(kT), N - tn * kT) : kT;
-    const _Float16* __restrict__ A =
-        args.A + args.strideA * static_cast<int64_t>(unit) + static_cast<size_t>(tm) * kT * args.lda;
-    const _Float16* __restrict__ B =
-        args.B + args.strideB * static_cast<int64_t>(unit) + static_cast<size_t>(tn) * kT;
+    // An operand is either K-contiguous (x-rows of K halves: A as given, B stored N x K with
+    // TB) or k-major (k-rows of x halves: B as given, A stored K x M with TA); x is the row of A
+    // or the column of B.  A K-contiguous operand takes the "A stage" layout and the 16-byte
+    // fragment read described above, a k-major one the "B stage" layout and the transposing
+    // read, whichever matrix it is, so the MFMAs and their order do not depend on the flags.
+    const uint32_t pitchA = TA ? args.M : args.lda;  // halves between rows of A as stored
+    const uint32_t pitchB = TB ? K : N;
+    const _Float16* __restrict__ A = args.A + args.strideA * static_cast<int64_t>(unit) +
+                                     static_cast<size_t>(tm) * kT * (TA ? 1u : pitchA);
+    const _Float16* __restrict__ B = args.B + args.strideB * static_cast<int64_t>(unit) +
+                                     static_cast<size_t>(tn) * kT * (TB ? pitchB : 1u);
     float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit) +
                               static_cast<size_t>(tm) * kT * N + static_cast<size_t>(tn) * kT;
 
@@ -251,48 +258,49 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     // A copy instruction moves 1 KiB per wavefront.  Wavefront w fills the WAVE_LDS bytes
     // at w*WAVE_LDS of a stage in ROUNDS copies; copy r puts lane i's 16 bytes at
     // w*WAVE_LDS + r*1024 + i*16.
-    //   A: that is LDS row R = w*8*ROUNDS + r*8 + i/8, physical chunk i%8, which must hold
-    //      logical chunk L = (i%8) ^ ((R/2)%8): matrix row R (L < 4) or R+128 (L >= 4),
+    //   K-contiguous: that is LDS row R = w*8*ROUNDS + r*8 + i/8, physical chunk i%8, which
+    //      must hold logical chunk L = (i%8) ^ ((R/2)%8): x = R (L < 4) or R+128 (L >= 4),
     //      k offset (L%4)*8.
-    //   B: k = w*2*ROUNDS + r*2 + i/32, physical 16-byte chunk i%32, 32-byte chunks
+    //   k-major: k = w*2*ROUNDS + r*2 + i/32, physical 16-byte chunk i%32, 32-byte chunks
     //      swizzled as described above.
     // The global address of a copy is a uniform base that advances with the K step plus a
     // per-lane byte offset that never changes.  The instruction offset r*1024 is added to
     // both the LDS and the global address, so the lane offsets subtract it again.  K steps
     // beyond the last are clamped to it: those copies land in buffers that are no longer
     // read, which keeps the number of copies in flight constant.
-    uint32_t aLane[ROUNDS], bLane[ROUNDS];
-    {
-#pragma unroll
-        for (int r = 0; r < ROUNDS; ++r)
-        {
-            const uint32_t R = wave * (8 * ROUNDS) + 8 * r + (lane >> 3);
-            const uint32_t aL = (lane & 7) ^ ((R >> 1) & 7);
-            const uint32_t row = R + ((aL & 4) ? 128u : 0u);
-            aLane[r] = (min(row, rowsLeft - 1) * args.lda + (aL & 3) * 8) * 2 + kBias - r * 1024;
-        }
+    auto laneKContig = [&](int r, uint32_t xLeft, uint32_t pitch) {
+        const uint32_t R = wave * (8 * ROUNDS) + 8 * r + (lane >> 3);
+        const uint32_t L = (lane & 7) ^ ((R >> 1) & 7);
+        const uint32_t x = R + ((L & 4) ? 128u : 0u);
+        return (min(x, xLeft - 1) * pitch + (L & 3) * 8) * 2 + kBias - r * 1024;
+    };
+    auto laneKMajor = [&](int r, uint32_t xLeft, uint32_t pitch) {
         const uint32_t phys16 = lane & 31;
+        const uint32_t k = wave * (2 * ROUNDS) + r * 2 + (lane >> 5);
+        const uint32_t swz = 2 * (k & 3) + ((k >> 3) & 1);
+        const uint32_t logical16 = (((phys16 >> 1) ^ swz) << 1) | (phys16 & 1);
+        return (k * pitch + min(logical16 * 8, xLeft - 8)) * 2 + kBias - r * 1024;
+    };
+    uint32_t aLane[ROUNDS], bLane[ROUNDS];
 #pragma unroll
-        for (int r = 0; r < ROUNDS; ++r)
-        {
-            const uint32_t k = wave * (2 * ROUNDS) + r * 2 + (lane >> 5);
-            const uint32_t swz = 2 * (k & 3) + ((k >> 3) & 1);
-            const uint32_t logical16 = (((phys16 >> 1) ^ swz) << 1) | (phys16 & 1);
-            bLane[r] = (k * N + min(logical16 * 8, colsLeft - 8)) * 2 + kBias - r * 1024;
-        }
+    for (int r = 0; r < ROUNDS; ++r)
+    {
+        aLane[r] = TA ? laneKMajor(r, rowsLeft, pitchA) : laneKContig(r, rowsLeft, pitchA);
+        bLane[r] = TB ? laneKContig(r, colsLeft, pitchB) : laneKMajor(r, colsLeft, pitchB);
     }
     const uint32_t waveU = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t aLds = LdsAddress(&As[0][0]) + waveU * WAVE_LDS;
     const uint32_t bLds = LdsAddress(&Bs[0][0]) + waveU * WAVE_LDS;
     const char* aGlobal = reinterpret_cast<const char*>(A) - kBias;
     const char* bGlobal = reinterpret_cast<const char*>(B) - kBias;
-    const size_t bStepBytes = static_cast<size_t>(kTK) * N * 2;
+    const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * pitchA * 2 : kTK * 2;
+    const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * pitchB * 2;
 
     const uint32_t steps = K / kTK;
     auto copyA = [&](uint32_t kt, int stage, auto round) {
         constexpr int r = decltype(round)::value;
         const uint32_t src = min(kt, steps - 1);
-        DmaToLds16<r * 1024>(aLane[r], aGlobal + static_cast<size_t>(src) * (kTK * 2),
+        DmaToLds16<r * 1024>(aLane[r], aGlobal + static_cast<size_t>(src) * aStepBytes,
                              aLds + stage * kStageBytes);
     };
     auto copyB = [&](uint32_t kt, int stage, auto round) {
@@ -303,25 +311,45 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     };
 
     // ---- LDS -> fragment read plan ---------------------------------------------------
+    // Block b of an operand = x in [x0 + 16b, x0 + 16b + 16) with x0 the wavefront's first row
+    // (A: waveM*128, 8 blocks) or column (B: waveN*64, 4 blocks); a lane wants x = l16 of the
+    // block and k = 8g .. 8g+7.
+    //   K-contiguous: x is half x/128 of LDS row x%128 = (x0%128) + 16b + l16, logical chunk
+    //      4*(x/128) + g, swizzle (row/2)%8 = (l16/2)%8: one base offset plus 16b rows.
+    //   k-major: k-row 8g + 4h + l16/4, 32-byte chunk x0/16 + b swizzled, halves 4*(l16%4)..+3
+    //      of it: one offset per block.
     const uint32_t l16 = lane & 15;
     const uint32_t g = lane >> 4;
-    // A: LDS row 16i + l16, half waveM of it, logical chunk waveM*4 + g, swizzle (row/2)%8
-    const uint32_t aOff = l16 * 64 + (((waveM * 4 + g) ^ ((l16 >> 1) & 7)) * 8);  // + i*16*64
-    // B: k-row 8g + 4h + l16/4, 32-byte chunk waveN*4 + j swizzled, halves 4*(l16%4)..+3 of it
-    uint32_t bOff[4];
-    {
+    auto offKContig = [&](uint32_t x0) {
+        const uint32_t row = (x0 & 127u) + l16;
+        return row * 64 + ((((x0 >> 7) * 4 + g) ^ ((l16 >> 1) & 7)) * 8);  // + b*16*64
+    };
+    auto offKMajor = [&](uint32_t x0, int b) {
         const uint32_t kRow = 8 * g + (l16 >> 2);
         const uint32_t swz = 2 * ((l16 >> 2) & 3) + (g & 1);
+        return kRow * kT + (((x0 / 16 + b) ^ swz) * 16) + (l16 & 3) * 4;
+    };
+    constexpr int kOffA = TA ? 8 : 1, kOffB = TB ? 1 : 4;
+    uint32_t aOff[kOffA], bOff[kOffB];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            bOff[j] = kRow * kT + (((waveN * 4 + j) ^ swz) * 16) + (l16 & 3) * 4;
-    }
+    for (int b = 0; b < kOffA; ++b)
+        aOff[b] = TA ? offKMajor(waveM * 128, b) : offKContig(waveM * 128);
+#pragma unroll
+    for (int b = 0; b < kOffB; ++b)
+        bOff[b] = TB ? offKContig(waveN * 64) : offKMajor(waveN * 64, b);
+    auto readKContig = [&](const _Float16* p) { return *reinterpret_cast<const halfx8*>(p); };
+    auto readKMajor = [&](const _Float16* p) { return Join(LdsReadTr(p), LdsReadTr(p + 4 * kT)); };
     auto loadA = [&](int stage, int i) {
-        return *reinterpret_cast<const halfx8*>(&As[stage][aOff + i * 16 * 64]);
+        if constexpr (TA)
+            return readKMajor(&As[stage][aOff[i]]);
+        else
+            return readKContig(&As[stage][aOff[0] + i * 16 * 64]);
     };
     auto loadB = [&](int stage, int j) {
-        const _Float16* p = &Bs[stage][bOff[j]];
-        return Join(LdsReadTr(p), LdsReadTr(p + 4 * kT));
+        if constexpr (TB)
+            return readKContig(&Bs[stage][bOff[0] + j * 16 * 64]);
+        else
+            return readKMajor(&Bs[stage][bOff[j]]);
     };
 
     floatx4 acc[8][4];
@@ -1127,12 +1155,28 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
     }
 }
 
+// variant 0: whole tiles, out read in the epilogue; 1 / 2: out added inside the loop with
+// spacing 2 / 4; 3: ragged tiles
+template <bool TA, bool TB>
+void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16Args& args)
+{
+    const dim3 g(grid), b(512);
+    if (variant == 2)
+        hipLaunchKernelGGL((GemmF16Tile256<false, 4, TA, TB>), g, b, 0, stream, args);
+    else if (variant == 1)
+        hipLaunchKernelGGL((GemmF16Tile256<false, 2, TA, TB>), g, b, 0, stream, args);
+    else if (variant == 0)
+        hipLaunchKernelGGL((GemmF16Tile256<false, 0, TA, TB>), g, b, 0, stream, args);
+    else
+        hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB>), g, b, 0, stream, args);
+}
+
 // Picks the kernel for one launch over args.K columns of A (rows args.lda apart).
 int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, bool transB,
               hipStream_t stream)
 {
     const uint32_t M = args.M, N = args.N, K = args.K;
-    const bool plain = !transA && !transB;  // the 256-tile kernel takes plain storage only
+    const bool plain = !transA && !transB;
     // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
     // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
     const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
@@ -1143,8 +1187,14 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
     const bool fills256 =
         static_cast<uint64_t>(M) * N * 4 >=
         static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * kT * kT * 3;
-    const bool tile256 = plain && aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) &&
-                         N >= 8 && tiles256 >= minTiles && fills256;
+    // lane offsets of the copies are 32-bit: 256 rows of a K-contiguous operand, 32 of a
+    // k-major one
+    const uint64_t pitchA = transA ? M : args.lda, pitchB = transB ? K : N;
+    const bool offsetsFit = (transA ? 32 : 256) * pitchA * 2 + 8192 < (1ull << 32) &&
+                            (transB ? 256 : 32) * pitchB * 2 + 8192 < (1ull << 32);
+    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) && N >= 8 &&
+                         (!transA || (M % 8 == 0 && M >= 8)) && tiles256 >= minTiles && fills256 &&
+                         offsetsFit;
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -1158,15 +1208,16 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
         // old contents of out added inside the loop: spacing 4 from 36 K steps, 2 from 20
         const bool cloop = whole256 && !args.overwrite;
         const uint32_t ksteps = K / kTK;
-        const dim3 g(grid), b(512);
-        if (cloop && ksteps >= CLoopSteps(4))
-            hipLaunchKernelGGL((GemmF16Tile256<false, 4>), g, b, 0, stream, args);
-        else if (cloop && ksteps >= CLoopSteps(2))
-            hipLaunchKernelGGL((GemmF16Tile256<false, 2>), g, b, 0, stream, args);
-        else if (whole256)
-            hipLaunchKernelGGL((GemmF16Tile256<false, 0>), g, b, 0, stream, args);
+        const int variant = !whole256 ? 3 : (cloop && ksteps >= CLoopSteps(4)) ? 2
+                                          : (cloop && ksteps >= CLoopSteps(2)) ? 1 : 0;
+        if (transA && transB)
+            LaunchTile256<true, true>(variant, grid, stream, args);
+        else if (transA)
+            LaunchTile256<true, false>(variant, grid, stream, args);
+        else if (transB)
+            LaunchTile256<false, true>(variant, grid, stream, args);
         else
-            hipLaunchKernelGGL((GemmF16Tile256<true, 0>), g, b, 0, stream, args);
+            LaunchTile256<false, false>(variant, grid, stream, args);
     }
     else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
              (!transA || (M % 8 == 0 && M >= 8)) &&

@@ -119,11 +119,15 @@ def test_dma128_exact_on_integers(dev, shape):
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (5, 3, 2, 1), (64, 64, 32, 1), (100, 72, 40, 2),
                                    (130, 254, 96, 1), (257, 255, 63, 1), (256, 512, 128, 3),
                                    (300, 136, 1000, 1), (8, 8, 32, 1), (136, 264, 64, 2),
-                                   (1000, 1000, 992, 1), (512, 384, 2048, 1), (129, 136, 96, 1)])
+                                   (1000, 1000, 992, 1), (512, 384, 2048, 1), (129, 136, 96, 1),
+                                   (256, 256, 64, 192), (512, 256, 1184, 96), (256, 512, 704, 96),
+                                   (248, 256, 96, 192), (4096, 3072, 32, 1), (504, 496, 64, 48)])
 def test_transposed_operands_exact_on_integers(dev, shape, flags):
     """A stored K x M and / or B stored N x K: the same product as with the operands stored
-    plainly, bit for bit on integer-valued inputs: the straight-to-LDS 128-tile kernel when K is
-    a multiple of 32, N of 8 (and M of 8 for a transposed A), the general kernel otherwise."""
+    plainly, bit for bit on integer-valued inputs: the 256-tile kernel (whole and ragged tiles,
+    with the old contents of out added in the loop or in the epilogue) from 192 tiles up, the
+    straight-to-LDS 128-tile kernel below that when K is a multiple of 32, N of 8 (and M of 8
+    for a transposed A), the general kernel otherwise."""
     M, N, K, batch = shape
     h.announce("sph_gemm_f16f32 transposed operands", shape, "flags", flags)
     A = synth.small_integers(41, (batch, M, K), span=3).astype(np.float16)
