@@ -200,6 +200,8 @@ void CreateSparseMatrixWithDenseMatrix(SparseMatrix** dst, const float* src, uin
     auto* array = new SparseMatrix[numMatrices]();
     try
     {
+        // Counting passes of all matrices first, nothing read back: the stream is drained once,
+        // by the first read of an entry count, instead of once per matrix.
         for (uint32_t i = 0; i < numMatrices; ++i)
         {
             const float* dense = src + static_cast<std::size_t>(i) * m * paddedN;
@@ -208,12 +210,21 @@ void CreateSparseMatrixWithDenseMatrix(SparseMatrix** dst, const float* src, uin
             r.N = n;
             r.ROW = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(
                 Bytes(static_cast<std::size_t>(m) + 1), true));
-            uint32_t nnz = 0;
-            Check(sph_csr_row_offsets_f32(r.ROW, dense, m, n, paddedN, &nnz),
+            Check(sph_csr_row_offsets_f32(r.ROW, dense, m, n, paddedN, nullptr),
                   "CreateSparseMatrixWithDenseMatrix");
-            r.NNZ = nnz;
-            r.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(Bytes(nnz), true));
-            r.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(Bytes(nnz), true));
+        }
+        for (uint32_t i = 0; i < numMatrices; ++i)
+        {
+            uint32_t nnz = 0;
+            Cuda::CopyDeviceToHost(&nnz, array[i].ROW + m, sizeof(nnz));
+            array[i].NNZ = nnz;
+        }
+        for (uint32_t i = 0; i < numMatrices; ++i)
+        {
+            const float* dense = src + static_cast<std::size_t>(i) * m * paddedN;
+            SparseMatrix& r = array[i];
+            r.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(Bytes(r.NNZ), true));
+            r.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(Bytes(r.NNZ), true));
             Check(sph_csr_fill_f32(r.V, r.COL, r.ROW, dense, m, n, paddedN),
                   "CreateSparseMatrixWithDenseMatrix");
         }

@@ -78,6 +78,8 @@ void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cu
     };
     try
     {
+        // Counting passes of all matrices first, without reading anything back: the stream is
+        // drained once, by the first read of an entry count, instead of once per matrix.
         for (uint32_t i = 0; i < count; ++i)
         {
             const SparseMatrix& a = cudaA[i];
@@ -89,11 +91,21 @@ void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cu
             c.N = n;
             c.ROW = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(
                 (static_cast<std::size_t>(m) + 1) * 4, true));
-            uint32_t nnz = 0;
             check(sph_spgemm_row_offsets_f32(c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m, a.N,
-                                             n, &nnz));
-            c.NNZ = nnz;
-            const std::size_t bytes = std::max<std::size_t>(nnz, 1) * 4;
+                                             n, nullptr));
+        }
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            uint32_t nnz = 0;
+            Compute::Cuda::CopyDeviceToHost(&nnz, result[i].ROW + m, sizeof(nnz));
+            result[i].NNZ = nnz;
+        }
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            const SparseMatrix& a = cudaA[i];
+            const SparseMatrix& b = cudaB[i];
+            SparseMatrix& c = result[i];
+            const std::size_t bytes = std::max<std::size_t>(c.NNZ, 1) * 4;
             c.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
             c.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
             check(sph_spgemm_fill_f32(c.V, c.COL, c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m,
