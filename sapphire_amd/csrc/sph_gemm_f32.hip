@@ -9,6 +9,8 @@
 // Four kernels, chosen from the shape and the alignment of the operands:
 //   GemmF32DmaKernel     aligned operands with K a multiple of 16: slabs travel global -> LDS
 //                        without staging registers, several K steps ahead (the fast path);
+//                        with more 64-tiles than resident workgroups each workgroup walks
+//                        several tiles and the copy stream runs across the tile boundaries;
 //   GemmF32Kernel        any shape and alignment: register-staged double buffering, 16-byte
 //                        loads when possible, scalar predicated loads otherwise (e.g. the
 //                        reference's random test sizes,
@@ -35,6 +37,7 @@
 namespace
 {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int kBK = 16;
@@ -166,13 +169,9 @@ __device__ __forceinline__ void StashXContig(float* __restrict__ slab, const flo
 // bands of `band` tile rows column by column, which makes a run a compact block of the
 // output whose A rows and B columns the XCD's workgroups share.  Returns false for the
 // surplus workgroups of a grid rounded up to 8 * perXcd.
-__device__ __forceinline__ bool MapTile(const GemmF32Args& args, uint32_t& tm, uint32_t& tn,
-                                        uint32_t& unit)
+__device__ __forceinline__ void MapLogical(const GemmF32Args& args, uint32_t logical, uint32_t& tm,
+                                           uint32_t& tn, uint32_t& unit)
 {
-    const uint32_t id = blockIdx.x;
-    const uint32_t logical = (id & 7u) * args.perXcd + (id >> 3);
-    if (logical >= args.tilesTotal)
-        return false;
     const uint32_t perUnit = args.tilesM * args.tilesN;
     unit = logical / perUnit;
     const uint32_t t = logical - unit * perUnit;
@@ -182,6 +181,16 @@ __device__ __forceinline__ bool MapTile(const GemmF32Args& args, uint32_t& tm, u
     const uint32_t rows = min(args.band, args.tilesM - bandIdx * args.band);
     tm = bandIdx * args.band + within % rows;
     tn = within / rows;
+}
+
+__device__ __forceinline__ bool MapTile(const GemmF32Args& args, uint32_t& tm, uint32_t& tn,
+                                        uint32_t& unit)
+{
+    const uint32_t id = blockIdx.x;
+    const uint32_t logical = (id & 7u) * args.perXcd + (id >> 3);
+    if (logical >= args.tilesTotal)
+        return false;
+    MapLogical(args, logical, tm, tn, unit);
     return true;
 }
 
@@ -492,10 +501,17 @@ struct DmaTile
     }
 };
 
-template <int BM, int BN, int BK, int STAGES, bool TA, bool TB>
+// WALK: a workgroup walks several tiles (every 64th of its XCD's run, 64 = two resident
+// workgroups on each of an XCD's 32 compute units) instead of one.  The copy pipeline runs on
+// across the tile boundary - the last steps of a tile already fetch the first slabs of the
+// next one - and the old values of `out` are requested at a tile's first step and added after
+// its last one, so the matrix pipe does not wait for the first slabs and for `out` once per
+// tile.  The launcher takes this form only for whole tiles, 16-byte output rows and a K
+// that fills the LDS ring a whole number of times, which keeps the number of loads and stores
+// per tile fixed.  Per element the arithmetic is the same as without WALK.
+template <int BM, int BN, int BK, int STAGES, bool TA, bool TB, bool WALK>
 __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args args)
 {
-    static_assert(BM == BN, "square tiles only");
     static_assert(BK == 16 || BK == 32, "K step of 16 or 32");
     constexpr int WM = BM / 2;
     constexpr int WN = BN / 2;
@@ -510,6 +526,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     constexpr uint32_t kCopiesA = TileA::kCopies / 4;  // per wavefront
     constexpr uint32_t kCopiesB = TileB::kCopies / 4;
     constexpr uint32_t kBlocks = BK / 8;  // 8-wide k blocks (4 MFMAs each) per step
+    constexpr int kQuads = TM * TN * 4;   // float4 of `out` per lane
 
     __shared__ __attribute__((aligned(1024))) char lds[STAGES * kStageBytes];
 
@@ -521,35 +538,30 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     const uint32_t l32 = lane & 31;
     const uint32_t khalf = lane >> 5;
 
-    uint32_t tm, tn, unit;
-    if (!MapTile(args, tm, tn, unit))
+    // ---- the tile(s) of this workgroup ------------------------------------------------------
+    uint32_t logical = (blockIdx.x & 7u) * args.perXcd + (blockIdx.x >> 3);
+    uint32_t logicalEnd = args.tilesTotal;
+    uint32_t logicalStride = 0;
+    if constexpr (WALK)
+    {
+        logicalEnd = min((blockIdx.x & 7u) * args.perXcd + args.perXcd, args.tilesTotal);
+        logicalStride = gridDim.x >> 3;
+    }
+    if (logical >= logicalEnd)
         return;
-
-    const float* A;
-    const float* B;
-    float* out;
-    if (args.entries != nullptr)
-    {
-        const SphGemmEntry e = args.entries[unit];
-        A = args.A + e.aOff;
-        B = args.B + e.bOff;
-        out = args.out + e.outOff;
-    }
-    else
-    {
-        A = args.A + args.strideA * static_cast<int64_t>(unit);
-        B = args.B + args.strideB * static_cast<int64_t>(unit);
-        out = args.out + args.strideOut * static_cast<int64_t>(unit);
-    }
     const uint32_t M = args.M, N = args.N, K = args.K;
-    const uint32_t rowBase = tm * BM;
-    const uint32_t colBase = tn * BN;
 
-    // ---- what this lane copies every step -------------------------------------------------
-    // Copy j of an operand is taken by wavefront j % 4.  Lane offsets are bytes from the
-    // operand's base at step 0; the base advances by one K step per step.
-    uint32_t aLane[kCopiesA], bLane[kCopiesB];
-    uint32_t aDst[kCopiesA], bDst[kCopiesB];
+    // Where a tile's operands and output start, and what this lane copies of it every step:
+    // copy j of an operand is taken by wavefront j % 4; lane offsets are bytes from the
+    // operand's base at step 0, the base advances by one K step per step.
+    struct Place
+    {
+        const char* a;
+        const char* b;
+        float* out;
+        uint32_t rowBase, colBase;
+        uint32_t aLane[kCopiesA], bLane[kCopiesB];
+    };
     auto laneOffsetKContig = [&](uint32_t j, uint32_t xBase, uint32_t limit) {
         using T = TileA;  // chunk geometry depends on BK only
         const uint32_t x = j * T::kRowsPerCopyK + lane / T::kChunks;  // row inside the tile
@@ -564,49 +576,75 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         const uint32_t gx = min(xBase + col, limit - 4);
         return (k * limit + gx) * 4u;
     };
+    auto locate = [&](uint32_t logicalTile, Place& p) {
+        uint32_t tm, tn, unit;
+        MapLogical(args, logicalTile, tm, tn, unit);
+        if (args.entries != nullptr)
+        {
+            const SphGemmEntry e = args.entries[unit];
+            p.a = reinterpret_cast<const char*>(args.A + e.aOff);
+            p.b = reinterpret_cast<const char*>(args.B + e.bOff);
+            p.out = args.out + e.outOff;
+        }
+        else
+        {
+            p.a = reinterpret_cast<const char*>(args.A + args.strideA * static_cast<int64_t>(unit));
+            p.b = reinterpret_cast<const char*>(args.B + args.strideB * static_cast<int64_t>(unit));
+            p.out = args.out + args.strideOut * static_cast<int64_t>(unit);
+        }
+        p.rowBase = tm * BM;
+        p.colBase = tn * BN;
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesA; ++i)
+        {
+            const uint32_t j = wave + 4 * i;
+            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, TileA::kRowBytes)
+                            : laneOffsetKContig(j, p.rowBase, M);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesB; ++i)
+        {
+            const uint32_t j = wave + 4 * i;
+            p.bLane[i] = TB ? laneOffsetKContig(j, p.colBase, N)
+                            : laneOffsetXContig(j, p.colBase, N, TileB::kRowBytes);
+        }
+    };
+    // LDS offsets of this wavefront's copies inside a stage
+    uint32_t aDst[kCopiesA], bDst[kCopiesB];
 #pragma unroll
     for (uint32_t i = 0; i < kCopiesA; ++i)
-    {
-        const uint32_t j = wave + 4 * i;
-        if constexpr (TA)
-        {
-            aLane[i] = laneOffsetXContig(j, rowBase, M, TileA::kRowBytes);
-            aDst[i] = TileA::CopyOffsetXContig(j);
-        }
-        else
-        {
-            aLane[i] = laneOffsetKContig(j, rowBase, M);
-            aDst[i] = j * 1024;
-        }
-    }
+        aDst[i] = TA ? TileA::CopyOffsetXContig(wave + 4 * i) : (wave + 4 * i) * 1024;
 #pragma unroll
     for (uint32_t i = 0; i < kCopiesB; ++i)
-    {
-        const uint32_t j = wave + 4 * i;
-        if constexpr (TB)
-        {
-            bLane[i] = laneOffsetKContig(j, colBase, N);
-            bDst[i] = kBytesA + j * 1024;
-        }
-        else
-        {
-            bLane[i] = laneOffsetXContig(j, colBase, N, TileB::kRowBytes);
-            bDst[i] = kBytesA + TileB::CopyOffsetXContig(j);
-        }
-    }
+        bDst[i] = kBytesA +
+                  (TB ? (wave + 4 * i) * 1024 : TileB::CopyOffsetXContig(wave + 4 * i));
+
+    Place cur, nxt;
+    locate(logical, cur);
+
     const size_t aStepBytes = TA ? static_cast<size_t>(BK) * M * 4 : BK * 4;
     const size_t bStepBytes = TB ? BK * 4 : static_cast<size_t>(BK) * N * 4;
     const uint32_t ldsBase =
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsVoidPtr)(lds)));
     const uint32_t steps = K / BK;
 
-    // Copy n (0 .. kCopiesPerWave-1) of this wavefront's share of the next step to fetch, into
-    // stage `stage`.  aSrc / bSrc point at that step's slab; steps past the end fetch the last
-    // one again into a stage nobody reads any more, which keeps the number of outstanding
-    // copies the same in every iteration.
-    const char* aSrc = reinterpret_cast<const char*>(A);
-    const char* bSrc = reinterpret_cast<const char*>(B);
-    uint32_t stepsToAdvance = steps - 1;
+    // ---- the copy stream ------------------------------------------------------------------
+    // Copy n (0 .. kCopiesPerWave-1) of this wavefront's share of the next slab to fetch goes
+    // into stage `stage`; aSrc / bSrc point at that slab.  After a tile's last slab the stream
+    // moves on to the next tile of the walk; when there is none it fetches the last slab again
+    // into a stage nobody reads any more, which keeps the number of outstanding copies the same
+    // in every step.
+    const char* aSrc = cur.a;
+    const char* bSrc = cur.b;
+    uint32_t aLane[kCopiesA], bLane[kCopiesB];
+#pragma unroll
+    for (uint32_t i = 0; i < kCopiesA; ++i)
+        aLane[i] = cur.aLane[i];
+#pragma unroll
+    for (uint32_t i = 0; i < kCopiesB; ++i)
+        bLane[i] = cur.bLane[i];
+    uint32_t slabsLeft = steps;  // of the tile being fetched, the one at aSrc / bSrc included
+    bool haveNext = false;       // `nxt` describes a tile the copy stream has not reached yet
     auto issueOne = [&](uint32_t stage, uint32_t n) {
         const uint32_t base = ldsBase + stage * kStageBytes;
         if (n < kCopiesA)
@@ -615,22 +653,29 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
             DmaToLds16(bLane[n - kCopiesA], bSrc, base + bDst[n - kCopiesA]);
     };
     auto advance = [&]() {
-        if (stepsToAdvance != 0)
+        if (--slabsLeft != 0)
         {
             aSrc += aStepBytes;
             bSrc += bStepBytes;
-            --stepsToAdvance;
         }
+        else if (WALK && haveNext)
+        {
+            aSrc = nxt.a;
+            bSrc = nxt.b;
+#pragma unroll
+            for (uint32_t i = 0; i < kCopiesA; ++i)
+                aLane[i] = nxt.aLane[i];
+#pragma unroll
+            for (uint32_t i = 0; i < kCopiesB; ++i)
+                bLane[i] = nxt.bLane[i];
+            slabsLeft = steps;
+            haveNext = false;
+        }
+        else
+            slabsLeft = 1;
     };
 
     floatx16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v)
-                acc[i][j][v] = 0.f;
 
     // ---- fragment addresses inside a stage -------------------------------------------------
     // K-contiguous operand: byte offset of this lane's row, chunk chosen per 8-wide k block.
@@ -708,12 +753,86 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
                     acc[i][j] =
                         __builtin_amdgcn_mfma_f32_32x32x2f32(b[j][e], a[i][e], acc[i][j], 0, 0, 0);
     };
+
+    // ---- WALK: the values the tile's products are added to ----------------------------------
+    // Register v of lane l holds row l%32 and column 8*(v/4) + 4*(l/32) + v%4 of its 32x32
+    // block, so registers 4q..4q+3 are one float4 of `out`.
+    floatx4 old[WALK ? kQuads : 1];
+    // One straight run of loads per mode, so that none of them is waited for here.
+    auto fetchOld = [&]() {
+        auto where = [&](int idx, uint32_t& r, uint32_t& c) {
+            const int q = idx & 3, j = (idx >> 2) % TN, i = (idx >> 2) / TN;
+            r = cur.rowBase + waveM * WM + i * 32 + l32;
+            c = cur.colBase + waveN * WN + j * 32 + 8 * q + 4 * khalf;
+        };
+        if (args.bias != nullptr)
+        {
+#pragma unroll
+            for (int idx = 0; idx < kQuads; ++idx)
+            {
+                uint32_t r, c;
+                where(idx, r, c);
+                old[idx] = *reinterpret_cast<const floatx4*>(args.bias + c);
+            }
+        }
+        else if (args.overwrite == 0)
+        {
+#pragma unroll
+            for (int idx = 0; idx < kQuads; ++idx)
+            {
+                uint32_t r, c;
+                where(idx, r, c);
+                old[idx] =
+                    *reinterpret_cast<const floatx4*>(cur.out + static_cast<size_t>(r) * N + c);
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int idx = 0; idx < kQuads; ++idx)
+                old[idx] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    // Makes the compiler wait for the values here, where only the copies of one step are in
+    // flight, rather than at their first use after the last step with three steps in flight.
+    auto settleOld = [&]() {
+#pragma unroll
+        for (int i = 0; i < (WALK ? kQuads : 1); ++i)
+            asm volatile("" : "+v"(old[i]));
+    };
+    auto addAndStore = [&]() {
+        const bool relu = args.relu != 0;
+        const bool hasBias = args.bias != nullptr;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                {
+                    const uint32_t r = cur.rowBase + waveM * WM + i * 32 + l32;
+                    const uint32_t c = cur.colBase + waveN * WN + j * 32 + 8 * q + 4 * khalf;
+                    floatx4 v = old[(i * TN + j) * 4 + q];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        // 0 + bias: what the K = 1 product ones x bias leaves in a zero-filled out
+                        if (hasBias)
+                            v[e] = 0.f + v[e];
+                        v[e] += acc[i][j][4 * q + e];
+                        if (relu)
+                            v[e] = v[e] > 0 ? v[e] : 0;
+                    }
+                    *reinterpret_cast<floatx4*>(cur.out + static_cast<size_t>(r) * N + c) = v;
+                }
+    };
+
     // First k block of step s.  The step's housekeeping sits between its MFMAs, where the
     // matrix pipe is already busy: behind the first one the wait for step s+1's copies and the
     // barrier, behind each of the next ones one copy of step s+STAGES-1.
     static_assert(kCopiesPerWave <= 4 * TM * TN, "one copy per MFMA of the first block");
     auto multiplyAndFeed = [&](const float (&a)[TM][4], const float (&b)[TN][4],
-                               uint32_t fillStage) {
+                               uint32_t fillStage, bool tileStart, bool settle) {
 #pragma unroll
         for (uint32_t e = 0; e < 4; ++e)
 #pragma unroll
@@ -727,11 +846,21 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
                     if (n == 0)
                     {
                         // steps up to s+1 have landed once at most the STAGES-3 later ones
-                        // are pending; behind the barrier everybody's copies are visible and
+                        // are pending (loads and stores complete in the order they were issued,
+                        // so the stores and `out` loads of a tile boundary only make this wait
+                        // stricter); behind the barrier everybody's copies are visible and
                         // everybody has read the last fragment of step s-1
                         WaitVmem<(STAGES - 3) * kCopiesPerWave>();
                         __builtin_amdgcn_s_barrier();
                         asm volatile("" ::: "memory");
+                        if constexpr (WALK)
+                        {
+                            // both flags are constants once the ring loop is unrolled
+                            if (tileStart)
+                                fetchOld();
+                            if (settle)
+                                settleOld();
+                        }
                     }
                     if (n < kCopiesPerWave)
                     {
@@ -753,43 +882,96 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     }
 
     // Fragments are read one k block (8 values) ahead of the MFMAs that use them; the first
-    // block of step s+1 is read while the last block of step s is multiplied.  Stage s+1 is
-    // known to be complete from the barrier inside the first block of step s.
+    // block of step s+1 is read while the last block of step s is multiplied (at a tile's last
+    // step that is the first block of the next tile).  Stage s+1 is known to be complete from
+    // the barrier inside the first block of step s.
     float fa[2][TM][4], fb[2][TN][4];
     WaitVmem<(STAGES - 2) * kCopiesPerWave>();
     __syncthreads();
     loadFragments(fa[0], fb[0], lds, 0);
 
-    // The loop is unrolled over the ring so that every stage offset is a constant.
-    for (uint32_t s0 = 0; s0 < steps; s0 += STAGES)
+    for (;;)
     {
-#pragma unroll
-        for (uint32_t u = 0; u < STAGES; ++u)
+        if constexpr (WALK)
         {
-            if (s0 + u >= steps)
-                break;
-            const char* cur = lds + u * kStageBytes;
-            const char* next = lds + ((u + 1) % STAGES) * kStageBytes;
-#pragma unroll
-            for (uint32_t q = 0; q < kBlocks; ++q)
+            // describe the tile after this one before the copy stream gets there
+            const uint32_t after = logical + logicalStride;
+            if (after < logicalEnd)
             {
-                if (q + 1 < kBlocks)
-                    loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], cur, q + 1);
-                else
-                    loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], next, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                if (q == 0)
-                    multiplyAndFeed(fa[0], fb[0], (u + STAGES - 1) % STAGES);
-                else
-                    multiply(fa[q & 1], fb[q & 1]);
-                __builtin_amdgcn_sched_barrier(0);
+                locate(after, nxt);
+                haveNext = true;
             }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    acc[i][j][v] = 0.f;
+
+        // The loop is unrolled over the ring so that every stage offset is a constant.  With
+        // WALK the step count is a positive multiple of STAGES and the first trip round the
+        // ring, which fetches and settles `old`, is written out on its own: the compiler then
+        // sees that no path leads round the place where `old` settles and waits for nothing
+        // when `old` is used after the last step.
+        auto ringCycle = [&](uint32_t s0, auto firstOfTile) {
+            constexpr bool kFirst = decltype(firstOfTile)::value;
+#pragma unroll
+            for (uint32_t u = 0; u < STAGES; ++u)
+            {
+                if (!WALK && s0 + u >= steps)
+                    break;
+                const char* stage = lds + u * kStageBytes;
+                const char* next = lds + ((u + 1) % STAGES) * kStageBytes;
+#pragma unroll
+                for (uint32_t q = 0; q < kBlocks; ++q)
+                {
+                    if (q + 1 < kBlocks)
+                        loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], stage, q + 1);
+                    else
+                        loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], next, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (q == 0)
+                        multiplyAndFeed(fa[0], fb[0], (u + STAGES - 1) % STAGES,
+                                        kFirst && u == 0, kFirst && u == 1);
+                    else
+                        multiply(fa[q & 1], fb[q & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if constexpr (WALK)
+        {
+            ringCycle(0, std::true_type{});
+            for (uint32_t s0 = STAGES; s0 < steps; s0 += STAGES)
+                ringCycle(s0, std::false_type{});
+        }
+        else
+        {
+            for (uint32_t s0 = 0; s0 < steps; s0 += STAGES)
+                ringCycle(s0, std::false_type{});
+        }
+
+        if constexpr (!WALK)
+            break;
+        else
+        {
+            addAndStore();
+            logical += logicalStride;
+            if (logical >= logicalEnd)
+                break;
+            cur.out = nxt.out;
+            cur.rowBase = nxt.rowBase;
+            cur.colBase = nxt.colBase;
         }
     }
     WaitVmem<0>();  // the surplus copies of the last steps still target LDS
 
-    StoreTile<TM, TN>(acc, out, rowBase + waveM * WM, colBase + waveN * WN, M, N, l32, khalf,
-                      args.outVec != 0, args.overwrite == 0, args.bias, args.relu != 0);
+    if constexpr (!WALK)
+        StoreTile<TM, TN>(acc, cur.out, cur.rowBase + waveM * WM, cur.colBase + waveN * WN, M, N,
+                          l32, khalf, args.outVec != 0, args.overwrite == 0, args.bias,
+                          args.relu != 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -810,8 +992,6 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 // unit), which is why the 16-wide tile, a quarter of the work per workgroup on four times as
 // many compute units, is preferred whenever its tiles still fit the chip.
 // ---------------------------------------------------------------------------
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
 template <int TILE, bool VEC, bool TA, bool TB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32Args args)
 {
@@ -1182,24 +1362,26 @@ void LaunchSkinny(const GemmF32Args& args, dim3 grid, uint32_t tile, bool vec, b
         LaunchSkinnyTile<32, TA, TB>(args, grid, vec, wide, stream);
 }
 
+// `walk`: 64-tiles only, each workgroup takes several tiles
 template <bool TA, bool TB>
-void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dma,
+void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dma, bool walk,
                  hipStream_t stream)
 {
     const dim3 block(kThreads);
     if (dma)
     {
         if (big)
-            hipLaunchKernelGGL((GemmF32DmaKernel<128, 128, 16, 4, TA, TB>), grid, block, 0, stream, args);
+            hipLaunchKernelGGL((GemmF32DmaKernel<128, 128, 16, 4, TA, TB, false>), grid, block, 0,
+                               stream, args);
+        else if (walk)
+            hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB, true>), grid, block, 0,
+                               stream, args);
+        else if (args.K % 32 == 0)
+            hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB, false>), grid, block, 0,
+                               stream, args);
         else
-        {
-            if (args.K % 32 == 0)
-                hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB>), grid, block, 0,
-                                   stream, args);
-            else
-                hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 16, 6, TA, TB>), grid, block, 0,
-                                   stream, args);
-        }
+            hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 16, 6, TA, TB, false>), grid, block, 0,
+                               stream, args);
         return;
     }
     if (big)
@@ -1291,6 +1473,11 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // four 64-tiles overlap (measured 6 % slower then); pick the edge with the smaller cost of
     // the busiest compute unit.
     const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
+    // straight-to-LDS pipeline: whole K steps, 16-byte chunks everywhere, at least one chunk
+    // per clamped edge, and lane offsets that fit 32 bits
+    const bool dma = aligned && args.K >= kBK && args.K % kBK == 0 && args.M >= 4 && args.N >= 4 &&
+                     static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
+                     static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
     const uint64_t tiles128 =
         static_cast<uint64_t>((args.M + 127) / 128) * ((args.N + 127) / 128) * units;
     const uint64_t rounds128 = (tiles128 + cus - 1) / cus;
@@ -1315,20 +1502,25 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         args.band = std::min(band, args.tilesM);
     }
 
-    const dim3 grid(args.perXcd * 8);
-    // straight-to-LDS pipeline: whole K steps, 16-byte chunks everywhere, at least one chunk
-    // per clamped edge, and lane offsets that fit 32 bits
-    const bool dma = aligned && args.K >= kBK && args.K % kBK == 0 && args.M >= 4 && args.N >= 4 &&
-                     static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
-                     static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
+    // More 64-tiles than workgroups that can be resident (two per compute unit): each
+    // workgroup walks several tiles with the copy pipeline running across the tile boundaries
+    // (configuration 2: 37.8 -> 35.9 us).  Only for whole tiles, 16-byte output rows and a K
+    // that fills the 4-stage ring of 32-wide steps a whole number of times.  The 128-tile
+    // kernel would need more than 256 registers for it and lose its second resident workgroup
+    // (measured 4096^3: 921 -> 966 us), so it keeps one tile per workgroup.
+    const uint32_t slotsPerXcd = static_cast<uint32_t>(cus / 8 * 2);
+    const bool walk = dma && !big && args.perXcd > slotsPerXcd && args.outVec != 0 &&
+                      args.M % 64 == 0 && args.N % 64 == 0 && args.K % 128 == 0 &&
+                      (reinterpret_cast<uintptr_t>(args.bias) & 15u) == 0;
+    const dim3 grid((walk ? slotsPerXcd : args.perXcd) * 8);
     if (transA && transB)
-        LaunchTiled<true, true>(args, grid, big, aligned, dma, stream);
+        LaunchTiled<true, true>(args, grid, big, aligned, dma, walk, stream);
     else if (transA)
-        LaunchTiled<true, false>(args, grid, big, aligned, dma, stream);
+        LaunchTiled<true, false>(args, grid, big, aligned, dma, walk, stream);
     else if (transB)
-        LaunchTiled<false, true>(args, grid, big, aligned, dma, stream);
+        LaunchTiled<false, true>(args, grid, big, aligned, dma, walk, stream);
     else
-        LaunchTiled<false, false>(args, grid, big, aligned, dma, stream);
+        LaunchTiled<false, false>(args, grid, big, aligned, dma, walk, stream);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
