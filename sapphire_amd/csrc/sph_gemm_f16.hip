@@ -210,7 +210,7 @@ constexpr int CLoopSteps(int csp)
 {
     return (8 * csp + 1 + 3) / 4 * 4;
 }
-template <bool RAGGED, int CSP, bool TA, bool TB>
+template <bool RAGGED, int CSP, bool TA, bool TB, bool TAIL>
 __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 {
     constexpr int WAVES = 8;
@@ -296,18 +296,25 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * pitchA * 2 : kTK * 2;
     const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * pitchB * 2;
 
-    const uint32_t steps = K / kTK;
+    // TAIL: K = 32 q + r with r = 8, 16 or 24.  The last of the q + 1 steps takes the window
+    // [K - 32, K), which lies inside the matrix and needs no other lane offsets (only its
+    // start differs from a whole step's); its first 32 - r values of k were multiplied in
+    // step q - 1 already, so the lanes that hold them (k group g < 4 - r/8, for A and B alike)
+    // feed zeros to the MFMAs of that step instead of what they read from LDS.
+    const uint32_t steps = TAIL ? K / kTK + 1 : K / kTK;
+    const size_t aLastBytes = TAIL ? (TA ? static_cast<size_t>(K - kTK) * pitchA * 2 : (K - kTK) * 2) : 0;
+    const size_t bLastBytes = TAIL ? (TB ? (K - kTK) * 2 : static_cast<size_t>(K - kTK) * pitchB * 2) : 0;
     auto copyA = [&](uint32_t kt, int stage, auto round) {
         constexpr int r = decltype(round)::value;
         const uint32_t src = min(kt, steps - 1);
-        DmaToLds16<r * 1024>(aLane[r], aGlobal + static_cast<size_t>(src) * aStepBytes,
-                             aLds + stage * kStageBytes);
+        const size_t start = (TAIL && src == steps - 1) ? aLastBytes : static_cast<size_t>(src) * aStepBytes;
+        DmaToLds16<r * 1024>(aLane[r], aGlobal + start, aLds + stage * kStageBytes);
     };
     auto copyB = [&](uint32_t kt, int stage, auto round) {
         constexpr int r = decltype(round)::value;
         const uint32_t src = min(kt, steps - 1);
-        DmaToLds16<r * 1024>(bLane[r], bGlobal + static_cast<size_t>(src) * bStepBytes,
-                             bLds + stage * kStageBytes);
+        const size_t start = (TAIL && src == steps - 1) ? bLastBytes : static_cast<size_t>(src) * bStepBytes;
+        DmaToLds16<r * 1024>(bLane[r], bGlobal + start, bLds + stage * kStageBytes);
     };
 
     // ---- LDS -> fragment read plan ---------------------------------------------------
@@ -386,11 +393,20 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     // One K step, stage index known at compile time.  BF holds this step's B fragments, BFN
     // receives the next step's.  EXTRA = vector memory operations other than stage copies
     // issued since the first half of the step before.
-    auto stepWith = [&](auto stageC, uint32_t kt, auto extraC, const halfx8 (&BF)[4],
+    const bool laneRepeats = TAIL && g < 4 - (K % kTK) / 8;  // in the last step's window
+    auto stepWith = [&](auto stageC, uint32_t kt, auto extraC, halfx8 (&BF)[4],
                         halfx8 (&BFN)[4], auto&& behindBarrier) {
         constexpr int cur = decltype(stageC)::value;
         constexpr int nxt = (cur + 1) % kTStages;
         constexpr int EXTRA = decltype(extraC)::value;
+        const bool drop = TAIL && laneRepeats && kt == steps - 1;
+        auto mask = [&](halfx8& f) {
+            if constexpr (TAIL)
+                f = drop ? halfx8{} : f;
+        };
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            mask(BF[j]);
         // first half: rows 0-63, fetch this step's rows 64-127, request B of step kt+3
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -398,6 +414,8 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
+                if (j == 0)
+                    mask(af[i]);
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(BF[j], af[i], acc[i][j], 0, 0, 0);
                 SPH_FENCE();
                 if (i < 2 && (j & 1) == 0)
@@ -422,6 +440,8 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
+                if (j == 0)
+                    mask(af[i]);
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(BF[j], af[i], acc[i][j], 0, 0, 0);
                 SPH_FENCE();
                 if (i < 6)
@@ -655,7 +675,9 @@ constexpr int kDStages = 4;
 constexpr int kDStageBytes = 2 * kD * kTK * 2;  // A + B
 constexpr int kDCopies = 4;                     // per wavefront and step: 2 of A, 2 of B
 
-template <bool TA, bool TB>
+// TAIL: K = 32 q + r, r = 8, 16 or 24, handled as in the 256-tile kernel: a last step over the
+// window [K - 32, K) whose lanes holding the 32 - r values of k already multiplied feed zeros.
+template <bool TA, bool TB, bool TAIL>
 __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
 {
     __shared__ __attribute__((aligned(1024))) char lds[kDStages * kDStageBytes];
@@ -709,7 +731,11 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * M * 2 : kTK * 2;
     const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * N * 2;
     const uint32_t ldsBase = LdsAddress(lds);
-    const uint32_t steps = K / kTK;
+    const uint32_t steps = TAIL ? K / kTK + 1 : K / kTK;
+    // the last window starts K % 32 values of k after the one before it
+    const uint32_t kLast = K % kTK;
+    const size_t aLastBytes = TA ? static_cast<size_t>(kLast) * M * 2 : kLast * 2;
+    const size_t bLastBytes = TB ? kLast * 2 : static_cast<size_t>(kLast) * N * 2;
     // Copy n (0..3: two of A, two of B) of the next step to fetch, into stage `stage`.  aSrc /
     // bSrc point at that step's slabs; surplus steps re-fetch the last one into a stage nobody
     // reads any more, which keeps the number of outstanding copies the same in every iteration.
@@ -726,8 +752,14 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     auto advance = [&]() {
         if (stepsToAdvance != 0)
         {
-            aSrc += aStepBytes;
-            bSrc += bStepBytes;
+            size_t aBytes = aStepBytes, bBytes = bStepBytes;
+            if (TAIL && stepsToAdvance == 1)
+            {
+                aBytes = aLastBytes;
+                bBytes = bLastBytes;
+            }
+            aSrc += aBytes;
+            bSrc += bBytes;
             --stepsToAdvance;
         }
     };
@@ -785,6 +817,21 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
 #pragma unroll
             for (int v = 0; v < 16; ++v)
                 acc[i][j][v] = 0.f;
+    // TAIL: a lane's fragments of half ks hold k group 2 ks + khalf of the step's window; in the
+    // last step the groups below 4 - r/8 repeat values of k the step before has multiplied
+    const uint32_t firstNewGroup = TAIL ? 4 - (K % kTK) / 8 : 0;
+    auto maskRepeated = [&](halfx8 (&af)[2], halfx8 (&bf)[2], int ks, bool lastStep) {
+        if constexpr (TAIL)
+        {
+            const bool drop = lastStep && 2 * ks + khalf < firstNewGroup;
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+            {
+                af[b] = drop ? halfx8{} : af[b];
+                bf[b] = drop ? halfx8{} : bf[b];
+            }
+        }
+    };
     auto multiply = [&](const halfx8 (&af)[2], const halfx8 (&bf)[2]) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -846,12 +893,15 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
                 break;
             const char* cur = lds + u * kDStageBytes;
             const char* next = lds + ((u + 1) % kDStages) * kDStageBytes;
+            const bool lastStep = TAIL && s0 + u == steps - 1;
             loadFragments(af[1], bf[1], cur, 1);
             __builtin_amdgcn_sched_barrier(0);
+            maskRepeated(af[0], bf[0], 0, lastStep);
             multiplyAndFeed(af[0], bf[0], (u + kDStages - 1) % kDStages);
             __builtin_amdgcn_sched_barrier(0);
             loadFragments(af[0], bf[0], next, 0);
             __builtin_amdgcn_sched_barrier(0);
+            maskRepeated(af[1], bf[1], 1, lastStep);
             multiply(af[1], bf[1]);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -1157,21 +1207,21 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
 
 // variant 0: whole tiles, out read in the epilogue; 1 / 2: out added inside the loop with
 // spacing 2 / 4; 3: ragged tiles
-template <bool TA, bool TB>
+template <bool TA, bool TB, bool TAIL>
 void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16Args& args)
 {
     const dim3 g(grid), b(512);
     if (variant == 2)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 4, TA, TB>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 4, TA, TB, TAIL>), g, b, 0, stream, args);
     else if (variant == 1)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 2, TA, TB>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 2, TA, TB, TAIL>), g, b, 0, stream, args);
     else if (variant == 0)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 0, TA, TB>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 0, TA, TB, TAIL>), g, b, 0, stream, args);
     else
-        hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB, TAIL>), g, b, 0, stream, args);
 }
 
-// Picks the kernel for one launch over args.K columns of A (rows args.lda apart).
+// Picks the kernel for one launch.
 int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, bool transB,
               hipStream_t stream)
 {
@@ -1192,9 +1242,13 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
     const uint64_t pitchA = transA ? M : args.lda, pitchB = transB ? K : N;
     const bool offsetsFit = (transA ? 32 : 256) * pitchA * 2 + 8192 < (1ull << 32) &&
                             (transB ? 256 : 32) * pitchB * 2 + 8192 < (1ull << 32);
-    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0) && (N % 8 == 0) && N >= 8 &&
-                         (!transA || (M % 8 == 0 && M >= 8)) && tiles256 >= minTiles && fills256 &&
-                         offsetsFit;
+    // K = 32 q + r, r = 8, 16 or 24: the straight-to-LDS kernels take the r values in a last,
+    // partly masked step (plain storage only; measured 4096 x 4096 x 4080: 229 us on the
+    // general kernel, 175 us with the r values left to a second launch, 128 us this way)
+    const bool tailInKernel = plain && K % kTK != 0 && K % 8 == 0 && K >= 2 * kTK && args.lda == K;
+    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0 || tailInKernel) && (N % 8 == 0) &&
+                         N >= 8 && (!transA || (M % 8 == 0 && M >= 8)) && tiles256 >= minTiles &&
+                         fills256 && offsetsFit;
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -1207,19 +1261,21 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
     {
         // old contents of out added inside the loop: spacing 4 from 36 K steps, 2 from 20
         const bool cloop = whole256 && !args.overwrite;
-        const uint32_t ksteps = K / kTK;
+        const uint32_t ksteps = (K + kTK - 1) / kTK;
         const int variant = !whole256 ? 3 : (cloop && ksteps >= CLoopSteps(4)) ? 2
                                           : (cloop && ksteps >= CLoopSteps(2)) ? 1 : 0;
         if (transA && transB)
-            LaunchTile256<true, true>(variant, grid, stream, args);
+            LaunchTile256<true, true, false>(variant, grid, stream, args);
         else if (transA)
-            LaunchTile256<true, false>(variant, grid, stream, args);
+            LaunchTile256<true, false, false>(variant, grid, stream, args);
         else if (transB)
-            LaunchTile256<false, true>(variant, grid, stream, args);
+            LaunchTile256<false, true, false>(variant, grid, stream, args);
+        else if (K % kTK != 0)
+            LaunchTile256<false, false, true>(variant, grid, stream, args);
         else
-            LaunchTile256<false, false>(variant, grid, stream, args);
+            LaunchTile256<false, false, false>(variant, grid, stream, args);
     }
-    else if (aligned16 && K >= kTK && K % kTK == 0 && N % 8 == 0 && N >= 8 &&
+    else if (aligned16 && K >= kTK && (K % kTK == 0 || tailInKernel) && N % 8 == 0 && N >= 8 &&
              (!transA || (M % 8 == 0 && M >= 8)) &&
              static_cast<uint64_t>(M) * (transA ? kTK : args.lda) < (1ull << 31) &&
              static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31))
@@ -1227,13 +1283,15 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
         // whole K steps and 16-byte chunks everywhere: straight-to-LDS 128-tile kernel
         const dim3 g(grid), b(256);
         if (transA && transB)
-            hipLaunchKernelGGL((GemmF16Dma128<true, true>), g, b, 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Dma128<true, true, false>), g, b, 0, stream, args);
         else if (transA)
-            hipLaunchKernelGGL((GemmF16Dma128<true, false>), g, b, 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Dma128<true, false, false>), g, b, 0, stream, args);
         else if (transB)
-            hipLaunchKernelGGL((GemmF16Dma128<false, true>), g, b, 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Dma128<false, true, false>), g, b, 0, stream, args);
+        else if (K % kTK != 0)
+            hipLaunchKernelGGL((GemmF16Dma128<false, false, true>), g, b, 0, stream, args);
         else
-            hipLaunchKernelGGL((GemmF16Dma128<false, false>), g, b, 0, stream, args);
+            hipLaunchKernelGGL((GemmF16Dma128<false, false, false>), g, b, 0, stream, args);
     }
     else
     {
@@ -1340,22 +1398,6 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.strideB = strideB;
     args.overwrite = (flags & SPH_GEMM_OVERWRITE) ? 1u : 0u;
 
-    // K = 32 q + r with r a multiple of 8: the straight-to-LDS kernels take whole K steps only,
-    // so they multiply the first 32 q columns of A and the general kernel adds the last r
-    // (measured 4096 x 4096 x 4080: 229 us on the general kernel alone, 175 us this way)
-    const uint32_t tail = K % kTK;
-    if (tail != 0 && !transA && !transB && K % 8 == 0 && K >= 2 * kTK && aligned16 && N % 8 == 0)
-    {
-        GemmF16Args head = args;
-        head.K = K - tail;
-        const int rc = LaunchF16(head, batch, aligned16, false, false, stream);
-        if (rc != SPH_OK)
-            return rc;
-        args.A += head.K;
-        args.B += static_cast<size_t>(head.K) * N;
-        args.K = tail;
-        args.overwrite = 0;
-    }
     return LaunchF16(args, batch, aligned16, transA, transB, stream);
 }
 

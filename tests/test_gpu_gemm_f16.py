@@ -65,11 +65,17 @@ def test_tile256_ragged_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref - C)
 
 
-# K = 32 q + r, r in {8, 16, 24}: the straight-to-LDS kernels multiply the first 32 q columns and
-# the general kernel adds the rest (256-tile, ragged 256-tile and 128-tile cases)
+# K = 32 q + r, r in {8, 16, 24}.  The 256-tile kernel takes the window [K - 32, K) as a last
+# step and masks the 32 - r values of k it has already multiplied (shapes with 192 tiles: whole
+# and ragged tiles, old contents added in the epilogue, every second step (20 steps and more:
+# K = 632 ends inside the written-out prefix, 648 after it) and every fourth (36 and more: 1144,
+# 1168, 1176)); the 128-tile kernel multiplies the first 32 q columns and the general kernel adds
+# the rest in a second launch.
 @pytest.mark.parametrize("shape", [(256, 256, 72, 192), (250, 248, 80, 192), (4096, 3072, 88, 1),
+                                   (256, 256, 632, 192), (256, 256, 648, 192), (512, 256, 1144, 96),
+                                   (512, 256, 1168, 96), (256, 512, 1176, 96), (500, 504, 680, 48),
                                    (300, 520, 168, 1), (128, 128, 72, 3), (1000, 1000, 1000, 1)])
-def test_k_tail_split_exact_on_integers(dev, shape):
+def test_k_tail_exact_on_integers(dev, shape):
     M, N, K, batch = shape
     h.announce("sph_gemm_f16f32 K tail integer exactness", shape)
     A = synth.small_integers(31, (batch, M, K), span=3).astype(np.float16)
@@ -80,6 +86,27 @@ def test_k_tail_split_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref)
     got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, flags=capi.SPH_GEMM_OVERWRITE)
     assert np.array_equal(got, ref - C)
+
+
+@pytest.mark.parametrize("K", [72, 80, 88])
+def test_k_tail_window_counts_an_infinity_once(dev, K):
+    """An infinity (and a 0 x Inf) at a k that lies in both of the last two step windows must
+    come out exactly as in the CPU product: +Inf where the partner is positive, NaN where it is
+    zero, and nothing else in the matrix may change."""
+    M, N, batch = 256, 256, 192
+    h.announce("sph_gemm_f16f32 K tail, Inf inside the repeated window", K)
+    A = synth.small_integers(41, (batch, M, K), span=3).astype(np.float16)
+    B = synth.small_integers(42, (batch, K, N), span=3).astype(np.float16)
+    C = synth.small_integers(43, (batch, M, N), span=100)
+    k = K - 20                      # inside [K - 32, 32 q) for r = 8, 16 and 24
+    A[:, 5, k] = np.inf
+    B[:, k, :] = 1
+    B[:, k, 7] = 0                  # Inf x 0
+    with np.errstate(invalid="ignore"):
+        ref = _oracle(C, A, B, M, N, K, batch=batch)
+    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch)
+    assert np.array_equal(got, ref, equal_nan=True)
+    assert np.isnan(got[:, 5, 7]).all() and np.isposinf(got[:, 5, 8]).all()
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1), (5, 3, 2), (31, 33, 17), (64, 64, 32), (100, 72, 40),
