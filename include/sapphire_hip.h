@@ -337,6 +337,27 @@ int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW,
 int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V,
                          const uint32_t* COL, const uint32_t* ROW, uint32_t M,
                          uint32_t N);
+/* sph_csr_from_dense_f32: the conversion of CreateSparseMatrixWithDenseMatrix
+ * (Includes/Sapphire/compute/sparse/Sparse.hpp:153-156) for a caller that can
+ * bound the number of entries beforehand: ROW, V and COL in one call.  V and
+ * COL hold `capacity` entries; ROW (M + 1 entries) is always complete and
+ * ROW[M] is the true count, but only entries with an index below `capacity`
+ * are stored: when the count turns out larger, grow V and COL and call
+ * sph_csr_fill_f32 with the ROW already there.  With nnzHost != NULL the
+ * count is copied to *nnzHost and the call returns after the stream has
+ * drained; with NULL it is asynchronous.
+ * For 16-byte aligned rows of 128 .. 8192 columns and a capacity of at most
+ * about an eighth of the matrix the dense matrix is read once: every row is
+ * compacted into a staging slot of 2 * capacity / M + 32 entries (a
+ * stream-ordered scratch allocation of 8 bytes per slot entry), the counts
+ * are scanned and a small kernel moves the staged entries into place; a row
+ * with more entries than its slot is read a second time.  Other shapes run
+ * the count, scan and fill passes inside the call.  Refused during graph
+ * capture (scratch allocation).  Same ROW, V and COL, bit for bit, as
+ * sph_csr_row_offsets_f32 followed by sph_csr_fill_f32. */
+int sph_csr_from_dense_f32(float* V, uint32_t* COL, uint32_t* ROW,
+                           uint32_t capacity, const float* dense, uint32_t M,
+                           uint32_t N, uint32_t ld, uint32_t* nnzHost);
 
 /* ---- CSR x CSR ------------------------------------------------------------ */
 

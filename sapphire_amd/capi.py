@@ -102,6 +102,8 @@ SIGNATURES = {
     "sph_csr_row_offsets_noalloc_f32": [_vp, _vp, _u32, _u32, _u32],
     "sph_csr_fill_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32],
     "sph_csr_to_dense_f32": [_vp, _u32, _vp, _vp, _vp, _u32, _u32],
+    "sph_csr_from_dense_f32": [_vp, _vp, _vp, _u32, _vp, _u32, _u32, _u32,
+                               ctypes.POINTER(ctypes.c_uint32)],
     "sph_spgemm_row_offsets_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,
                                    ctypes.POINTER(ctypes.c_uint32)],
     "sph_spgemm_fill_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],

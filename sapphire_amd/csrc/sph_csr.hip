@@ -215,7 +215,8 @@ template <int LPR>
 __global__ __launch_bounds__(kThreads) void CsrFillKernel(float* __restrict__ V,
                                                           uint32_t* __restrict__ COL,
                                                           const uint32_t* __restrict__ ROW,
-                                                          const DenseView d)
+                                                          const DenseView d,
+                                                          const uint32_t capacity)
 {
     constexpr uint32_t kGroups = kThreads / LPR;
     const uint32_t lane = threadIdx.x % LPR;
@@ -231,8 +232,9 @@ __global__ __launch_bounds__(kThreads) void CsrFillKernel(float* __restrict__ V,
         const uint32_t row = pass * rowsPerPass + blockIdx.x * kGroups + group;
         const bool rowOk = row < d.M;
         uint32_t slot = rowOk ? ROW[row] : 0u;
-        // a ROW that was not computed from this matrix must not make the stores run past the row
-        const uint32_t rowEnd = rowOk ? ROW[row + 1] : 0u;
+        // a ROW that was not computed from this matrix must not make the stores run past the
+        // row, and nothing is stored past the capacity of V and COL
+        const uint32_t rowEnd = rowOk ? min(ROW[row + 1], capacity) : 0u;
         for (uint32_t col0 = 0; col0 < d.N; col0 += LPR * 4)
         {
             const uint32_t col = col0 + lane * 4;
@@ -258,6 +260,167 @@ __global__ __launch_bounds__(kThreads) void CsrFillKernel(float* __restrict__ V,
                 }
             slot += kept;
         }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Dense -> CSR with one pass over the matrix (rows of 128 .. 8192 columns, 16-byte aligned).
+//
+// A row's place in V / COL depends on the counts of all rows above, which are not known while
+// the row is in registers.  Waiting for them inside the kernel (a decoupled look-back over row
+// tiles) was built and measured on the 8192 x 8192 matrix at 1 %: the pass alone took 42 us,
+// with the look-back 95 us and with ordered tile tickets on top 134 us (8192 device-scope
+// atomics on one address cost 8 ns each, and 2048 resident tiles polling each other's state
+// words slow the loads they are waiting for).  So the pass does not wait: every row writes its
+// entries, in order, into a staging slot of `stage` entries at row * stage, and its count into
+// ROW; the counts are scanned; a second, small kernel moves the staged entries to their final
+// place (8 bytes read and written per entry).  A row with more than `stage` entries (the slot is
+// sized from the caller's capacity, twice the mean plus 32) is rebuilt from the dense matrix by
+// the second kernel instead, so any input converts correctly.
+// ---------------------------------------------------------------------------
+constexpr uint32_t kStageWaves = 4;  // wavefronts per workgroup
+
+// A workgroup holds 4 / WPR rows; WPR wavefronts share a row, each taking QUADS float4 per lane
+// of a contiguous part of it.  Requires d.vec (so N % 4 == 0) and N <= WPR * QUADS * 256.  Few
+// registers per wavefront on purpose: many small workgroups per compute unit, out of step with
+// each other, keep loads in flight while others count and store.
+template <int WPR, int QUADS>
+__global__ __launch_bounds__(kStageWaves * 64) void CsrStageKernel(
+    float* __restrict__ stageV, uint32_t* __restrict__ stageCol, uint32_t* __restrict__ counts,
+    const uint32_t stage, const DenseView d)
+{
+    constexpr uint32_t kRows = kStageWaves / WPR;  // rows per workgroup
+    __shared__ uint32_t sCounts[kStageWaves];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x * kRows + wave / WPR;
+    const uint32_t part = wave % WPR;  // which part of the row
+    const bool rowOk = row < d.M;
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        counts[d.M] = 0;  // the slot the scan turns into the number of entries
+
+    // quad j of lane l of part p holds columns 256 (p QUADS + j) + 4 l .. + 3
+    float4 q[QUADS];
+    const float* rowPtr = d.data + static_cast<size_t>(rowOk ? row : 0) * d.ld;
+#pragma unroll
+    for (int j = 0; j < QUADS; ++j)
+    {
+        const uint32_t col = ((part * QUADS + j) * 64 + lane) * 4;
+        q[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (rowOk && col < d.N)
+            q[j] = *reinterpret_cast<const float4*>(rowPtr + col);
+    }
+    uint32_t total = 0;  // the same in every lane
+#pragma unroll
+    for (int j = 0; j < QUADS; ++j)
+        total += __popcll(__ballot(q[j].x != 0.f)) + __popcll(__ballot(q[j].y != 0.f)) +
+                 __popcll(__ballot(q[j].z != 0.f)) + __popcll(__ballot(q[j].w != 0.f));
+    if (lane == 0)
+        sCounts[wave] = total;
+    __syncthreads();
+    // entries of the parts before this one in the same row
+    uint32_t slot = 0, rowCount = 0;
+#pragma unroll
+    for (uint32_t p = 0; p < WPR; ++p)
+    {
+        const uint32_t c = sCounts[wave - part + p];
+        rowCount += c;
+        if (p < part)
+            slot += c;
+    }
+    if (rowOk && part == 0 && lane == 0)
+        counts[row] = rowCount;
+    if (!rowOk || rowCount > stage)
+        return;  // the second kernel rebuilds an overfull row from the dense matrix
+
+    // inside a part the entries are ordered by (quad, lane, element): ascending columns
+    float* outV = stageV + static_cast<size_t>(row) * stage;
+    uint32_t* outCol = stageCol + static_cast<size_t>(row) * stage;
+    const uint64_t below = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int j = 0; j < QUADS; ++j)
+    {
+        const float v[4] = { q[j].x, q[j].y, q[j].z, q[j].w };
+        uint32_t before = 0, kept = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            const uint64_t m = __ballot(v[e] != 0.f);
+            before += __popcll(m & below);
+            kept += __popcll(m);
+        }
+        if (kept == 0)
+            continue;
+        uint32_t at = slot + before;
+        const uint32_t col = ((part * QUADS + j) * 64 + lane) * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (v[e] != 0.f)
+            {
+                outV[at] = v[e];
+                outCol[at] = col + e;
+                ++at;
+            }
+        slot += kept;
+    }
+}
+
+// One wavefront per row: staged entries move to ROW[row] ..; a row that did not fit its staging
+// slot is read from the dense matrix again.  Nothing is stored at or past `capacity`.
+__global__ __launch_bounds__(256) void CsrUnstageKernel(float* __restrict__ V,
+                                                        uint32_t* __restrict__ COL,
+                                                        const uint32_t* __restrict__ ROW,
+                                                        const float* __restrict__ stageV,
+                                                        const uint32_t* __restrict__ stageCol,
+                                                        const uint32_t stage,
+                                                        const uint32_t capacity, const DenseView d)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= d.M)
+        return;
+    const uint32_t first = ROW[row];
+    const uint32_t count = ROW[row + 1] - first;
+    if (count <= stage)
+    {
+        const float* inV = stageV + static_cast<size_t>(row) * stage;
+        const uint32_t* inCol = stageCol + static_cast<size_t>(row) * stage;
+        for (uint32_t i = lane; i < count; i += 64)
+            if (first + i < capacity)
+            {
+                V[first + i] = inV[i];
+                COL[first + i] = inCol[i];
+            }
+        return;
+    }
+    const uint64_t below = (1ull << lane) - 1ull;
+    uint32_t slot = first;
+    for (uint32_t col0 = 0; col0 < d.N; col0 += 256)
+    {
+        const uint32_t col = col0 + lane * 4;
+        const float4 q = LoadQuad(d, row, col, true);
+        const float v[4] = { q.x, q.y, q.z, q.w };
+        uint32_t before = 0, kept = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            const uint64_t m = __ballot(v[e] != 0.f);
+            before += __popcll(m & below);
+            kept += __popcll(m);
+        }
+        uint32_t at = slot + before;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (v[e] != 0.f)
+            {
+                if (at < capacity)
+                {
+                    V[at] = v[e];
+                    COL[at] = col + e;
+                }
+                ++at;
+            }
+        slot += kept;
     }
 }
 
@@ -355,10 +518,10 @@ template <int LPR>
 struct FillLauncher
 {
     static void Run(uint32_t grid, hipStream_t stream, float* V, uint32_t* COL,
-                    const uint32_t* ROW, const DenseView& d)
+                    const uint32_t* ROW, const DenseView& d, uint32_t capacity)
     {
         hipLaunchKernelGGL(CsrFillKernel<LPR>, dim3(grid), dim3(kThreads), 0, stream, V, COL, ROW,
-                           d);
+                           d, capacity);
     }
 };
 }  // namespace
@@ -480,6 +643,103 @@ int sph_csr_row_offsets_noalloc_f32(uint32_t* ROW, const float* dense, uint32_t 
     return sph::ExclusiveScanInPlace(ROW, M + 1, nullptr, stream, sums);
 }
 
+int sph_csr_from_dense_f32(float* V, uint32_t* COL, uint32_t* ROW, uint32_t capacity,
+                           const float* dense, uint32_t M, uint32_t N, uint32_t ld,
+                           uint32_t* nnzHost)
+{
+    SPH_REQUIRE(ROW != nullptr, "ROW is null");
+    SPH_REQUIRE(ld >= N, "row pitch is shorter than a row");
+    SPH_REQUIRE(M < 0xffffffffu, "too many rows");
+    SPH_REQUIRE(M == 0 || N == 0 || dense != nullptr, "dense is null");
+    SPH_REQUIRE(capacity == 0 || (V != nullptr && COL != nullptr), "V or COL is null");
+    SPH_REFUSE_WHILE_CAPTURING();  // takes a scratch allocation; before anything is enqueued
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    const DenseView d = MakeView(dense, M, N, ld);
+
+    // staging slot per row of the one-pass path: twice the mean the caller's capacity allows
+    // plus 32, a multiple of 4
+    const uint64_t mean = M != 0 ? capacity / M : 0;
+    const uint64_t stage64 = (2 * mean + 32 + 3) / 4 * 4;
+    if (!(d.vec && M != 0 && N >= 128 && N <= 8192 && stage64 * 4 <= N))
+    {
+        // narrow, very wide, unaligned or not very sparse matrices (a staging area of more
+        // than a quarter of the dense matrix): count, scan and fill as separate passes
+        const int lanes = LanesPerRow(N);
+        DispatchLanes<CountLauncher>(lanes, RowGrid(M, lanes), stream, ROW, d);
+        SPH_CHECK_LAUNCH();
+        const int rc = sph::ExclusiveScanInPlace(ROW, M + 1, nullptr, stream);
+        if (rc != SPH_OK)
+            return rc;
+        if (M != 0 && N != 0 && capacity != 0)
+        {
+            DispatchLanes<FillLauncher>(lanes, RowGrid(M, lanes), stream, V, COL, ROW, d, capacity);
+            SPH_CHECK_LAUNCH();
+        }
+        if (nnzHost != nullptr)
+        {
+            SPH_HIP_TRY(hipMemcpyAsync(nnzHost, ROW + M, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                       stream));
+            SPH_HIP_TRY(hipStreamSynchronize(stream));
+        }
+        return SPH_OK;
+    }
+
+    // waves per row and float4 per lane: the narrowest pair that covers a row
+    uint32_t wpr = 1, quads = 1;
+    while (wpr < kStageWaves && wpr * 256 < N)
+        wpr *= 2;
+    while (wpr * quads * 256 < N)
+        quads *= 2;
+    const uint32_t stage = static_cast<uint32_t>(stage64);
+    const size_t stageEntries = static_cast<size_t>(M) * stage;
+    float* stageV = nullptr;
+    SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&stageV), stageEntries * 8, stream));
+    uint32_t* stageCol = reinterpret_cast<uint32_t*>(stageV + stageEntries);
+    const uint32_t rowsPerGroup = kStageWaves / wpr;
+    const dim3 grid((M + rowsPerGroup - 1) / rowsPerGroup), block(kStageWaves * 64);
+#define SPH_STAGE(W, Q)                                                                        \
+    hipLaunchKernelGGL((CsrStageKernel<W, Q>), grid, block, 0, stream, stageV, stageCol, ROW,   \
+                       stage, d)
+    if (wpr == 1)
+        SPH_STAGE(1, 1);
+    else if (wpr == 2)
+        SPH_STAGE(2, 1);
+    else if (quads == 1)
+        SPH_STAGE(4, 1);
+    else if (quads == 2)
+        SPH_STAGE(4, 2);
+    else if (quads == 4)
+        SPH_STAGE(4, 4);
+    else
+        SPH_STAGE(4, 8);
+#undef SPH_STAGE
+    hipError_t launched = hipGetLastError();
+    int rc = SPH_OK;
+    if (launched == hipSuccess)
+        rc = sph::ExclusiveScanInPlace(ROW, M + 1, nullptr, stream);
+    if (launched == hipSuccess && rc == SPH_OK && capacity != 0)
+    {
+        hipLaunchKernelGGL(CsrUnstageKernel, dim3((M + 3) / 4), dim3(256), 0, stream, V, COL, ROW,
+                           stageV, stageCol, stage, capacity, d);
+        launched = hipGetLastError();
+    }
+    SPH_HIP_TRY(hipFreeAsync(stageV, stream));
+    if (launched != hipSuccess)
+        return sph::Fail(SPH_ERR_DEVICE, std::string("sph_csr_from_dense_f32 - launch failed with ") +
+                                             hipGetErrorString(launched));
+    if (rc != SPH_OK)
+        return rc;
+    if (nnzHost != nullptr)
+    {
+        SPH_HIP_TRY(hipMemcpyAsync(nnzHost, ROW + M, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                   stream));
+        SPH_HIP_TRY(hipStreamSynchronize(stream));
+    }
+    return SPH_OK;
+}
+
 int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW, const float* dense, uint32_t M,
                      uint32_t N, uint32_t ld)
 {
@@ -493,7 +753,7 @@ int sph_csr_fill_f32(float* V, uint32_t* COL, const uint32_t* ROW, const float* 
         return SPH_ERR_DEVICE;
     const DenseView d = MakeView(dense, M, N, ld);
     const int lanes = LanesPerRow(N);
-    DispatchLanes<FillLauncher>(lanes, RowGrid(M, lanes), stream, V, COL, ROW, d);
+    DispatchLanes<FillLauncher>(lanes, RowGrid(M, lanes), stream, V, COL, ROW, d, 0xffffffffu);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }

@@ -80,6 +80,88 @@ def test_conversion_matches_checker(dev, case):
     assert np.all(back[:, N:] == 9.0)
 
 
+def gpu_csr_one_call(dense, N, capacity):
+    """(V, COL, ROW, nnz) through sph_csr_from_dense_f32 with room for `capacity` entries; the
+    words past the capacity must come back untouched."""
+    M, ld = dense.shape
+    dD = capi.DeviceBuffer.from_array(dense if dense.size else np.zeros(1, np.float32))
+    dRow = capi.DeviceBuffer.from_array(np.full(M + 1, 0xFFFFFFFF, np.uint32))
+    guard = 8
+    dV = capi.DeviceBuffer.from_array(np.full(capacity + guard, -77.0, np.float32))
+    dCol = capi.DeviceBuffer.from_array(np.full(capacity + guard, 0xABCDEF, np.uint32))
+    nnz = ctypes.c_uint32(0xDEADBEEF)
+    capi.call("sph_csr_from_dense_f32", dV.ptr, dCol.ptr, dRow.ptr, capacity, dD.ptr, M, N, ld,
+              ctypes.byref(nnz))
+    ROW = dRow.download(np.uint32, (M + 1,))
+    V = dV.download(np.float32, (capacity + guard,))
+    COL = dCol.download(np.uint32, (capacity + guard,))
+    assert np.all(V[capacity:] == -77.0) and np.all(COL[capacity:] == 0xABCDEF)
+    for d in (dD, dRow, dV, dCol):
+        d.release()
+    return V[:capacity], COL[:capacity], ROW, nnz.value
+
+
+# shapes of the one-pass path (aligned rows of 128 .. 8192 columns: one, two or four wavefronts
+# per row with 1, 2, 4 or 8 float4 per lane; a last workgroup with fewer rows than it holds;
+# empty matrices; 70000 rows) after the shapes that run as separate passes inside the call
+# (narrow, unaligned, or too dense for a staging area)
+ONE_CALL_CASES = CASES + [(13, 128, 128, 0.3), (1000, 256, 256, 0.1), (4097, 1024, 1028, 0.02),
+                          (70, 8192, 8192, 0.01), (3, 4100, 4100, 0.5), (2500, 520, 520, 1.0),
+                          (5, 132, 136, 0.0), (70000, 128, 128, 0.05), (999, 2048, 2048, 0.003)]
+
+
+@pytest.mark.parametrize("case", ONE_CALL_CASES)
+def test_one_call_conversion_equals_the_two_calls(dev, case):
+    M, N, ld, density = case
+    h.announce("sph_csr_from_dense_f32 M N ld density =", case)
+    dense = sparse_dense(2000 + M + N, (M, ld), density)
+    dense[:, N:] = 5.0
+    wantV, wantCol, wantRow = gpu_csr_from_dense(dense, N)
+    if M * N <= 1 << 22:
+        chkV, chkCol, chkRow = po.csr_from_dense(dense, N=N)
+        assert np.array_equal(wantRow, chkRow) and np.array_equal(wantCol, chkCol)
+        assert np.array_equal(bits(wantV), bits(chkV))
+    total = int(wantRow[M])
+    # room to spare, exactly enough, and too little (the first half of the entries)
+    for capacity in (total + 5, total, total // 2):
+        V, COL, ROW, nnz = gpu_csr_one_call(dense, N, capacity)
+        assert nnz == total and np.array_equal(ROW, wantRow), capacity
+        kept = min(capacity, total)
+        assert np.array_equal(COL[:kept], wantCol[:kept]), capacity
+        assert np.array_equal(bits(V[:kept]), bits(wantV[:kept])), capacity
+        if capacity > total:
+            assert np.all(V[total:] == -77.0)
+
+
+def test_one_call_conversion_with_rows_that_overflow_their_staging_slot(dev):
+    """Mostly empty matrix with three full rows: their entries do not fit the per-row staging
+    slot (sized from the mean), so the second kernel rebuilds them from the dense matrix."""
+    M, N = 1001, 2048
+    h.announce("sph_csr_from_dense_f32 skewed rows", M, N)
+    dense = sparse_dense(4242, (M, N), 0.003)
+    for r in (0, 500, M - 1):
+        dense[r] = synth.uniform(77 + r, (N,)) + np.float32(2.0)      # no zeros
+    wantV, wantCol, wantRow = po.csr_from_dense(dense, N=N)
+    total = int(wantRow[M])
+    for capacity in (total, total - 1000):
+        V, COL, ROW, nnz = gpu_csr_one_call(dense, N, capacity)
+        assert nnz == total and np.array_equal(ROW, wantRow)
+        assert np.array_equal(COL, wantCol[:capacity])
+        assert np.array_equal(bits(V), bits(wantV[:capacity]))
+
+
+def test_one_call_conversion_at_configuration_5_size(dev):
+    d = synth.config5()
+    M, K = d["M"], d["K"]
+    h.announce("sph_csr_from_dense_f32 configuration 5", M, K)
+    dense = synth.densify(d["V"], d["COL"], d["ROW"], M, K)
+    for _ in range(2):                      # the scratch block of the first call is reused
+        V, COL, ROW, nnz = gpu_csr_one_call(dense, K, len(d["V"]))
+        assert nnz == len(d["V"])
+        assert np.array_equal(ROW, d["ROW"]) and np.array_equal(COL, d["COL"])
+        assert np.array_equal(bits(V), bits(d["V"]))
+
+
 def test_special_values_and_unaligned_base(dev):
     h.announce("sph_csr_* -0.0 / NaN / unaligned base")
     dense = np.array([[0.0, -0.0, 2.0, 0.0],
