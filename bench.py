@@ -358,14 +358,19 @@ def bench_spgemm(capi, synth, steps, warmup, n=8192, per_row=8.0):
         capi.call("sph_spgemm_row_offsets_f32", row.ptr, *ptrs, n, n, n, None)
         capi.call("sph_spgemm_fill_f32", val.ptr, col.ptr, row.ptr, *ptrs, n, n, n)
 
+    def one_call():
+        capi.call("sph_spgemm_f32", val.ptr, col.ptr, row.ptr, max(nnz.value, 1), *ptrs, n, n, n,
+                  None)
+
     event_ms, _ = timed_launches(capi, launch, steps, warmup)
+    one_call_ms, _ = timed_launches(capi, one_call, steps, warmup)
     for x in bufs + [row, val, col]:
         x.release()
     # products: for every entry of A, the length of the matching row of B
     lengths = np.diff(b[2].astype(np.int64))
     products = int(lengths[a[1]].sum())
     nbytes = 8 * (a[0].size + b[0].size + nnz.value) + 3 * 4 * (n + 1)
-    return event_ms, products, nnz.value, nbytes, a[0].size, b[0].size
+    return event_ms, products, nnz.value, nbytes, a[0].size, b[0].size, one_call_ms
 
 
 def bench_sparse_linear(capi, synth, steps, warmup, batch=256):
@@ -612,8 +617,10 @@ def main():
                          "csr_bytes": csr_bytes}
 
     if args.only == "spgemm":
-        ms, products, nnz_c, nbytes, nnz_a, nnz_b = bench_spgemm(capi, synth, args.steps, args.warmup)
-        result["spgemm"] = {"count_plus_fill_ms": ms, "products": products, "nnz_a": nnz_a,
+        ms, products, nnz_c, nbytes, nnz_a, nnz_b, one_ms = bench_spgemm(capi, synth, args.steps,
+                                                                         args.warmup)
+        result["spgemm"] = {"count_plus_fill_ms": ms, "one_call_ms": one_ms, "products": products,
+                            "nnz_a": nnz_a,
                             "nnz_b": nnz_b, "nnz_c": nnz_c, "algorithmic_bytes": nbytes}
 
     if args.only in (None, "spmm"):
@@ -705,8 +712,9 @@ def main():
                                            "dense matrix twice (count, then fill)",
             "csr_to_dense_ms": ms_dense,
             "csr_to_dense_gbs": (dense_bytes + csr_bytes) / (ms_dense * 1e-3) / 1e9}
-        ms, products, nnz_c, nbytes, nnz_a, nnz_b = bench_spgemm(capi, synth, 50, 5)
+        ms, products, nnz_c, nbytes, nnz_a, nnz_b, one_ms = bench_spgemm(capi, synth, 50, 5)
         others["spgemm_8192_8_per_row"] = {
+            "one_call_ms": one_ms,
             "workload": "CSR 8192x8192 (nnz %d) x CSR 8192x8192 (nnz %d) -> CSR (nnz %d)"
                         % (nnz_a, nnz_b, nnz_c),
             "count_plus_fill_ms": ms, "products": products,
@@ -714,8 +722,9 @@ def main():
             "algorithmic_gbs": nbytes / (ms * 1e-3) / 1e9,
             "note": "both passes compute every product (the count pass must see which sums "
                     "cancel); products counted once per pass in gproducts_per_s"}
-        ms, products, nnz_c, nbytes, nnz_a, nnz_b = bench_spgemm(capi, synth, 20, 3, n=65536)
+        ms, products, nnz_c, nbytes, nnz_a, nnz_b, one_ms = bench_spgemm(capi, synth, 20, 3, n=65536)
         others["spgemm_65536_8_per_row"] = {
+            "one_call_ms": one_ms,
             "workload": "CSR 65536x65536 (nnz %d) x CSR 65536x65536 (nnz %d) -> CSR (nnz %d)"
                         % (nnz_a, nnz_b, nnz_c),
             "count_plus_fill_ms": ms, "products": products,

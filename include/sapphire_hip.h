@@ -386,6 +386,23 @@ int sph_spgemm_fill_f32(float* VC, uint32_t* COLC, const uint32_t* ROWC,
                         const uint32_t* ROWA, const float* VB,
                         const uint32_t* COLB, const uint32_t* ROWB, uint32_t M,
                         uint32_t K, uint32_t N);
+/* sph_spgemm_f32: the same product in one call for a caller that can bound
+ * the number of entries of C beforehand (VC and COLC hold `capacity` entries).
+ * ROWC is always complete and ROWC[M] the true count; only entries with an
+ * index below `capacity` are stored: when the count turns out larger, grow VC
+ * and COLC and call sph_spgemm_fill_f32 with the ROWC already there.  The
+ * products are computed once instead of twice: the counting pass also writes
+ * every row into a staging slot of 2 * capacity / M + 64 entries (a
+ * stream-ordered scratch allocation of 8 bytes per slot entry), the counts
+ * are scanned, a small kernel moves the staged rows into place and only rows
+ * that did not fit their slot are multiplied again.  nnzHost as in
+ * sph_spgemm_row_offsets_f32.  Refused during graph capture.  Same ROWC, VC
+ * and COLC, bit for bit, as the two calls above. */
+int sph_spgemm_f32(float* VC, uint32_t* COLC, uint32_t* ROWC,
+                   uint32_t capacity, const float* VA, const uint32_t* COLA,
+                   const uint32_t* ROWA, const float* VB, const uint32_t* COLB,
+                   const uint32_t* ROWB, uint32_t M, uint32_t K, uint32_t N,
+                   uint32_t* nnzHost);
 
 #ifdef __cplusplus
 }

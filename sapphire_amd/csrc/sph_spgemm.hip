@@ -65,11 +65,22 @@ struct SpgemmArgs
     uint32_t rowsPerTurn;  // 1 .. kRowsPerTurnMax
     uint32_t heavyOnly;    // strip kernel: leave the rows SpgemmHashKernel takes alone
     // count pass: counts (M + 1 entries, counts[M] = 0).  fill pass: ROWC, VC, COLC.
+    // stage pass: counts as in the count pass, and row r's entries into VC / COLC at
+    // r * slot .. r * slot + slot - 1 (what does not fit is counted and dropped).
     uint32_t* counts;
     const uint32_t* ROWC;
     float* VC;
     uint32_t* COLC;
+    uint32_t slot;      // stage pass: entries per staging slot
+    uint32_t skipUpTo;  // fill pass: rows with at most this many entries are left alone
+    uint32_t capacity;  // fill pass: nothing is stored at or past this index
+    // stage pass: cleared; the move kernel sets it when a row did not fit its slot; a fill
+    // pass that is given it returns at once while it is zero
+    uint32_t* overflow;
 };
+
+// what a pass of the two product kernels does with a row's entries
+constexpr int kCount = 0, kFill = 1, kStage = 2;
 
 __device__ __forceinline__ uint32_t Uniform(uint32_t v, uint32_t lane)
 {
@@ -114,9 +125,13 @@ __device__ __forceinline__ bool LightRow(uint32_t entriesOfA, uint32_t products)
 // the row the listed (column, sum) pairs are sorted by column (bitonic, in LDS), sums that are
 // exactly zero are dropped, and the table is reset through the list.  The cost of a row follows
 // its products, not the width of the matrix.
-template <bool FILL>
+template <int MODE>
 __global__ __launch_bounds__(64) void SpgemmHashKernel(const SpgemmArgs args)
 {
+    constexpr bool FILL = MODE != kCount;    // entries are stored
+    constexpr bool COUNTS = MODE != kFill;   // counts are stored
+    if (MODE == kFill && args.overflow != nullptr && *args.overflow == 0)
+        return;  // every row is in place already
     __shared__ uint32_t keys[kHashSlots];
     __shared__ float sums[kHashSlots];
     __shared__ uint32_t sortKey[kHashProducts];  // first the list of claimed slots, then columns
@@ -144,12 +159,20 @@ __global__ __launch_bounds__(64) void SpgemmHashKernel(const SpgemmArgs args)
         {
             extentBegin = args.ROWA[mine];
             extentEnd = args.ROWA[mine + 1];
-            if (FILL)
+            if (MODE == kFill)
             {
                 outBegin = args.ROWC[mine];
                 outEnd = args.ROWC[mine + 1];
             }
+            if (MODE == kStage)
+            {
+                outBegin = static_cast<uint32_t>(mine) * args.slot;
+                outEnd = outBegin + args.slot;
+            }
         }
+        if (MODE == kFill && args.skipUpTo != 0 &&
+            __ballot(mine < args.M && outEnd - outBegin > args.skipUpTo) == 0)
+            continue;  // all of these rows are in place already
         // stage 1: this lane's entry of A's row i (rows with more than 64 entries are not ours)
         auto loadStage1 = [&](uint32_t i, uint32_t& k, float& value) {
             k = kEmpty;
@@ -192,6 +215,8 @@ __global__ __launch_bounds__(64) void SpgemmHashKernel(const SpgemmArgs args)
         loadStage1(i + 2, k1, value1);
         if (!LightRow(entriesOfA, WaveSum(bEnd - bBegin)))
             continue;  // heavy: the strip kernel's row
+        if (MODE == kFill && Uniform(outEnd, i) - Uniform(outBegin, i) <= args.skipUpTo)
+            continue;  // already in place
 
         uint32_t listed = 0;  // claimed slots so far (uniform)
         for (uint32_t j0 = 0; j0 < entriesOfA; j0 += kAhead)
@@ -267,7 +292,8 @@ __global__ __launch_bounds__(64) void SpgemmHashKernel(const SpgemmArgs args)
 
         uint32_t emitted = 0;
         const uint32_t rowBase = FILL ? Uniform(outBegin, i) : 0u;
-        const uint32_t rowLimit = FILL ? Uniform(outEnd, i) : 0u;
+        const uint32_t rowLimit =
+            MODE == kFill ? min(Uniform(outEnd, i), args.capacity) : FILL ? Uniform(outEnd, i) : 0u;
         if (listed <= 64)
         {
             // one (column, sum) pair per lane: sorted in registers with cross-lane exchanges
@@ -365,23 +391,29 @@ __global__ __launch_bounds__(64) void SpgemmHashKernel(const SpgemmArgs args)
                 emitted += static_cast<uint32_t>(__popcll(m));
             }
         }
-        if (!FILL && lane == 0)
+        if (COUNTS && lane == 0)
             args.counts[row] = emitted;
       }
     }
 }
 
-template <bool FILL>
+template <int MODE>
 __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
 {
+    constexpr bool FILL = MODE != kCount;    // entries are stored
+    constexpr bool COUNTS = MODE != kFill;   // counts are stored
     extern __shared__ float strip[];
     // one bit per column, after the strip; lane l owns words l*wordsPerLane .. +wordsPerLane-1
     uint32_t* bits = reinterpret_cast<uint32_t*>(strip + args.strip);
     const uint32_t wordsInStrip = args.strip / 32;
     const uint32_t wordsPerLane = (wordsInStrip + 63) / 64;  // at most kStripMax / 2048
     const uint32_t lane = threadIdx.x;
-    if (!FILL && blockIdx.x == 0 && lane == 0)
+    if (MODE == kFill && args.overflow != nullptr && *args.overflow == 0)
+        return;  // every row is in place already
+    if (COUNTS && blockIdx.x == 0 && lane == 0)
         args.counts[args.M] = 0;
+    if (MODE == kStage && blockIdx.x == 0 && lane == 0)
+        *args.overflow = 0;
     // cleared once; every block that is touched is cleared again when it is swept
     for (uint32_t x = lane; x < args.strip; x += 64)
         strip[x] = 0.0f;
@@ -400,8 +432,16 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
         if (lane <= rowsHere)
         {
             extentA = args.ROWA[turn + lane];
-            if (FILL)
+            if (MODE == kFill)
                 extentC = args.ROWC[turn + lane];
+            if (MODE == kStage)
+                extentC = (turn + lane) * args.slot;
+        }
+        if (MODE == kFill && args.skipUpTo != 0)
+        {
+            const uint32_t nextC = __shfl_down(extentC, 1, 64);
+            if (__ballot(lane < rowsHere && nextC - extentC > args.skipUpTo) == 0)
+                continue;  // all rows of this turn are in place already
         }
         // stage 1 (columns and values of A's row) and stage 2 (extents in B) of the pipeline
         auto loadStage1 = [&](uint32_t i, uint32_t& k, float& value) {
@@ -438,7 +478,8 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
         const uint32_t aEnd = Uniform(extentA, i + 1);
         uint32_t emitted = 0;  // entries of this row found so far (all strips)
         const uint32_t rowBase = FILL ? Uniform(extentC, i) : 0u;
-        const uint32_t rowLimit = FILL ? Uniform(extentC, i + 1) : 0u;
+        const uint32_t rowEnd = FILL ? Uniform(extentC, i + 1) : 0u;
+        const uint32_t rowLimit = MODE == kFill ? min(rowEnd, args.capacity) : rowEnd;
         // this row's first batch comes out of the pipeline, which then moves on
         const uint32_t firstBegin = nextBegin, firstEnd = nextEnd;
         const float firstValue = value2;
@@ -449,6 +490,8 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
         // in a wide product the light rows belong to SpgemmHashKernel
         if (args.heavyOnly != 0 && LightRow(aEnd - aBegin, WaveSum(firstEnd - firstBegin)))
             continue;
+        if (MODE == kFill && rowEnd - rowBase <= args.skipUpTo)
+            continue;  // already in place
 
         for (uint32_t c0 = 0; c0 < args.N; c0 += args.strip)
         {
@@ -570,7 +613,7 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
                     if (strip[x] != 0.0f)
                         ++kept;
                     if (!FILL)
-                        strip[x] = 0.0f;
+                        strip[x] = 0.0f;  // the storing passes read it once more below
                 }
             }
             // positions: exclusive prefix sum of `kept` over the lanes
@@ -604,10 +647,41 @@ __global__ __launch_bounds__(64) void SpgemmRowKernel(const SpgemmArgs args)
             }
             emitted += Uniform(inclusive, 63);
         }
-        if (!FILL && lane == 0)
+        if (COUNTS && lane == 0)
             args.counts[turn + i] = emitted;
       }
     }
+}
+
+// Staged rows move to their place: row r's ROWC[r + 1] - ROWC[r] entries from r * slot.  Rows
+// that did not fit their slot are left to a fill pass.  One wavefront per row, 4 per workgroup.
+__global__ __launch_bounds__(256) void SpgemmUnstageKernel(float* __restrict__ VC,
+                                                           uint32_t* __restrict__ COLC,
+                                                           const uint32_t* __restrict__ ROWC,
+                                                           const float* __restrict__ stageV,
+                                                           const uint32_t* __restrict__ stageCol,
+                                                           uint32_t M, uint32_t slot,
+                                                           uint32_t capacity, uint32_t* overflow)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M)
+        return;
+    const uint32_t first = ROWC[row];
+    const uint32_t count = ROWC[row + 1] - first;
+    if (count > slot)
+    {
+        if (lane == 0)
+            *overflow = 1;
+        return;
+    }
+    const size_t from = static_cast<size_t>(row) * slot;
+    for (uint32_t i = lane; i < count; i += 64)
+        if (first + i < capacity)
+        {
+            VC[first + i] = stageV[from + i];
+            COLC[first + i] = stageCol[from + i];
+        }
 }
 
 uint32_t StripFor(uint32_t N)
@@ -669,8 +743,8 @@ int sph_spgemm_row_offsets_f32(uint32_t* ROWC, const float* VA, const uint32_t* 
     args.counts = ROWC;
     args.heavyOnly = N > kHashFromWidth ? 1u : 0u;
     if (args.heavyOnly != 0 && M != 0)
-        hipLaunchKernelGGL(SpgemmHashKernel<false>, dim3(HashGridFor(M)), dim3(64), 0, stream, args);
-    hipLaunchKernelGGL(SpgemmRowKernel<false>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
+        hipLaunchKernelGGL(SpgemmHashKernel<kCount>, dim3(HashGridFor(M)), dim3(64), 0, stream, args);
+    hipLaunchKernelGGL(SpgemmRowKernel<kCount>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
                        args.strip * sizeof(float) + args.strip / 8, stream, args);
     SPH_CHECK_LAUNCH();
     return sph::ExclusiveScanInPlace(ROWC, M + 1, nnzHost, stream);
@@ -703,12 +777,108 @@ int sph_spgemm_fill_f32(float* VC, uint32_t* COLC, const uint32_t* ROWC, const f
     args.ROWC = ROWC;
     args.VC = VC;
     args.COLC = COLC;
+    args.capacity = 0xffffffffu;
     args.heavyOnly = N > kHashFromWidth ? 1u : 0u;
     if (args.heavyOnly != 0)
-        hipLaunchKernelGGL(SpgemmHashKernel<true>, dim3(HashGridFor(M)), dim3(64), 0, stream, args);
-    hipLaunchKernelGGL(SpgemmRowKernel<true>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
+        hipLaunchKernelGGL(SpgemmHashKernel<kFill>, dim3(HashGridFor(M)), dim3(64), 0, stream, args);
+    hipLaunchKernelGGL(SpgemmRowKernel<kFill>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
                        args.strip * sizeof(float) + args.strip / 8, stream, args);
     SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int sph_spgemm_f32(float* VC, uint32_t* COLC, uint32_t* ROWC, uint32_t capacity, const float* VA,
+                   const uint32_t* COLA, const uint32_t* ROWA, const float* VB,
+                   const uint32_t* COLB, const uint32_t* ROWB, uint32_t M, uint32_t K, uint32_t N,
+                   uint32_t* nnzHost)
+{
+    SPH_REQUIRE(ROWC != nullptr && ROWA != nullptr, "null pointer");
+    SPH_REQUIRE(M < 0xffffffffu, "too many rows");
+    SPH_REQUIRE(K == 0 || ROWB != nullptr, "null pointer");
+    SPH_REQUIRE(capacity == 0 || (VC != nullptr && COLC != nullptr), "VC or COLC is null");
+    SPH_REFUSE_WHILE_CAPTURING();  // takes a scratch allocation; before anything is enqueued
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    SpgemmArgs args{};
+    args.VA = VA;
+    args.COLA = COLA;
+    args.ROWA = ROWA;
+    args.VB = VB;
+    args.COLB = COLB;
+    args.ROWB = ROWB;
+    args.M = M;
+    args.K = K;
+    args.N = N;
+    args.strip = StripFor(N);
+    args.rowsPerTurn = RowsPerTurnFor(M);
+    args.counts = ROWC;
+    args.heavyOnly = N > kHashFromWidth ? 1u : 0u;
+    const dim3 hashGrid(HashGridFor(M)), rowGrid(GridFor(M, args.rowsPerTurn)), wave(64);
+    const size_t rowLds = args.strip * sizeof(float) + args.strip / 8;
+
+    // staging slot per row: twice the mean the capacity allows plus 64; without room for that
+    // (or without rows) the count, scan and fill passes run one after the other
+    const uint64_t slot = M != 0 ? 2 * static_cast<uint64_t>(capacity / M) + 64 : 0;
+    const bool staged = M != 0 && N != 0 && capacity != 0 && slot * M < (1ull << 31);
+    float* stageV = nullptr;
+    if (staged)
+    {
+        SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&stageV), slot * M * 8 + 4, stream));
+        args.VC = stageV;
+        args.COLC = reinterpret_cast<uint32_t*>(stageV + slot * M);
+        args.overflow = args.COLC + slot * M;
+        args.slot = static_cast<uint32_t>(slot);
+        if (args.heavyOnly != 0)
+            hipLaunchKernelGGL(SpgemmHashKernel<kStage>, hashGrid, wave, 0, stream, args);
+        hipLaunchKernelGGL(SpgemmRowKernel<kStage>, rowGrid, wave, rowLds, stream, args);
+    }
+    else
+    {
+        if (args.heavyOnly != 0 && M != 0)
+            hipLaunchKernelGGL(SpgemmHashKernel<kCount>, hashGrid, wave, 0, stream, args);
+        hipLaunchKernelGGL(SpgemmRowKernel<kCount>, rowGrid, wave, rowLds, stream, args);
+    }
+    hipError_t launched = hipGetLastError();
+    int rc = SPH_OK;
+    if (launched == hipSuccess)
+        rc = sph::ExclusiveScanInPlace(ROWC, M + 1, nullptr, stream);
+    if (launched == hipSuccess && rc == SPH_OK && M != 0 && N != 0 && capacity != 0)
+    {
+        if (staged)
+            hipLaunchKernelGGL(SpgemmUnstageKernel, dim3((M + 3) / 4), dim3(256), 0, stream, VC,
+                               COLC, ROWC, stageV, args.COLC, M, args.slot, capacity,
+                               args.overflow);
+        // rows that did not fit their slot (all rows, without staging) are multiplied again
+        args.ROWC = ROWC;
+        args.VC = VC;
+        args.COLC = COLC;
+        args.capacity = capacity;
+        args.skipUpTo = staged ? args.slot : 0u;
+        // after staging this pass usually finds nothing to do (it returns at once then), so it
+        // is launched with few workgroups, which walk all rows if they must: dispatching the
+        // full grid of empty workgroups alone took 15 us
+        const uint32_t few = static_cast<uint32_t>(sph::ComputeUnits()) * 2;
+        const dim3 fillHashGrid(staged ? std::min(hashGrid.x, few) : hashGrid.x);
+        const dim3 fillRowGrid(staged ? std::min(rowGrid.x, few) : rowGrid.x);
+        if (args.heavyOnly != 0)
+            hipLaunchKernelGGL(SpgemmHashKernel<kFill>, fillHashGrid, wave, 0, stream, args);
+        hipLaunchKernelGGL(SpgemmRowKernel<kFill>, fillRowGrid, wave, rowLds, stream, args);
+        launched = hipGetLastError();
+    }
+    if (stageV != nullptr)
+        SPH_HIP_TRY(hipFreeAsync(stageV, stream));
+    if (launched != hipSuccess)
+        return sph::Fail(SPH_ERR_DEVICE, std::string("sph_spgemm_f32 - launch failed with ") +
+                                             hipGetErrorString(launched));
+    if (rc != SPH_OK)
+        return rc;
+    if (nnzHost != nullptr)
+    {
+        SPH_HIP_TRY(hipMemcpyAsync(nnzHost, ROWC + M, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                   stream));
+        SPH_HIP_TRY(hipStreamSynchronize(stream));
+    }
     return SPH_OK;
 }
 

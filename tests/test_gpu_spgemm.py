@@ -49,6 +49,45 @@ def gpu_spgemm(A, B, M, K, N):
     return V[:nnz.value], COL[:nnz.value], ROW
 
 
+def gpu_spgemm_one_call(A, B, M, K, N, capacity):
+    """(V, COL, ROW, nnz) through sph_spgemm_f32 with room for `capacity` entries; the words past
+    the capacity must come back untouched."""
+    VA, CA, RA = A
+    VB, CB, RB = B
+    bufs = [_dev(VA, np.float32), _dev(CA, np.uint32), _dev(RA, np.uint32),
+            _dev(VB, np.float32), _dev(CB, np.uint32), _dev(RB, np.uint32)]
+    dRow = capi.DeviceBuffer.from_array(np.full(M + 1, 0xFFFFFFFF, np.uint32))
+    guard = 8
+    dV = capi.DeviceBuffer.from_array(np.full(capacity + guard, -77.0, np.float32))
+    dCol = capi.DeviceBuffer.from_array(np.full(capacity + guard, 0xABCDEF, np.uint32))
+    nnz = ctypes.c_uint32(0xDEADBEEF)
+    capi.call("sph_spgemm_f32", dV.ptr, dCol.ptr, dRow.ptr, capacity, *[b.ptr for b in bufs],
+              M, K, N, ctypes.byref(nnz))
+    ROW = dRow.download(np.uint32, (M + 1,))
+    V = dV.download(np.float32, (capacity + guard,))
+    COL = dCol.download(np.uint32, (capacity + guard,))
+    assert np.all(V[capacity:] == -77.0) and np.all(COL[capacity:] == 0xABCDEF)
+    for d in bufs + [dRow, dV, dCol]:
+        d.release()
+    return V[:capacity], COL[:capacity], ROW, nnz.value
+
+
+def check_one_call(A, B, M, K, N, want):
+    """sph_spgemm_f32 against the result of the two calls: with room to spare, exactly enough,
+    half of it (then the first half of the entries), and so little that the staging slots of
+    the longer rows overflow and those rows are multiplied a second time."""
+    wV, wC, wR = want
+    total = int(wR[M])
+    for capacity in (total + 3, total, total // 2, min(total, M)):
+        V, COL, ROW, nnz = gpu_spgemm_one_call(A, B, M, K, N, capacity)
+        assert nnz == total and np.array_equal(ROW, wR), capacity
+        kept = min(capacity, total)
+        assert np.array_equal(COL[:kept], wC[:kept]), capacity
+        assert np.array_equal(bits(V[:kept]), bits(wV[:kept])), capacity
+        if capacity > total:
+            assert np.all(V[total:] == -77.0)
+
+
 # M, K, N, density of A, density of B: single entries, rows of A and of B longer than 64
 # entries, empty operands, a width that needs two strips, widths that are not multiples of 64
 CASES = [(1, 1, 1, 1.0, 1.0), (5, 7, 3, 0.5, 0.5), (40, 60, 33, 0.1, 0.2), (64, 300, 200, 0.05, 0.05),
@@ -68,6 +107,7 @@ def test_product_matches_checker(dev, case):
     assert np.array_equal(ROW, wR)
     assert np.array_equal(COL, wC)
     assert np.array_equal(bits(V), bits(wV))
+    check_one_call(A, B, M, K, N, (wV, wC, wR))
 
 
 def test_cancelling_sums_are_dropped_and_unsorted_b_rows_are_accepted(dev):
@@ -124,6 +164,7 @@ def test_random_shapes_and_densities(dev, block):
         V, COL, ROW = gpu_spgemm(A, B, M, K, N)
         assert np.array_equal(ROW, wR) and np.array_equal(COL, wC)
         assert np.array_equal(bits(V), bits(wV))
+        check_one_call(A, B, M, K, N, (wV, wC, wR))
 
 
 def test_wide_product_mixes_table_rows_and_strip_rows(dev):
@@ -162,3 +203,4 @@ def test_wide_product_mixes_table_rows_and_strip_rows(dev):
     V, COL, ROW = gpu_spgemm(A, B, M, K, N)
     assert np.array_equal(ROW, wR) and np.array_equal(COL, wC)
     assert np.array_equal(bits(V), bits(wV))
+    check_one_call(A, B, M, K, N, (wV, wC, wR))
