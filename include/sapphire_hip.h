@@ -403,6 +403,19 @@ int sph_spgemm_f32(float* VC, uint32_t* COLC, uint32_t* ROWC,
                    const uint32_t* ROWA, const float* VB, const uint32_t* COLB,
                    const uint32_t* ROWB, uint32_t M, uint32_t K, uint32_t N,
                    uint32_t* nnzHost);
+/* sph_spgemm_load_u32: the load-distribution pre-pass the reference declares
+ * (LoadDistKernel, "assigns number of calculation for each element",
+ * Includes/Sapphire/compute/sparse/cuda/SparseGemm.cuh:48-60): load[p] = the
+ * number of entries in the row of B that entry p of A selects, i.e. the
+ * multiplications entry p causes (0 for a column >= K).  `entries` = entries
+ * of A.  With productsHost != NULL the sum of all loads -- the number of
+ * products, an upper bound on the entries of A * B and so a safe `capacity`
+ * for sph_spgemm_f32 -- is copied to *productsHost and the call returns after
+ * the stream has drained (refused during graph capture); load may be NULL
+ * when only that sum is wanted. */
+int sph_spgemm_load_u32(uint32_t* load, const uint32_t* COLA,
+                        const uint32_t* ROWB, uint32_t entries, uint32_t K,
+                        uint64_t* productsHost);
 
 #ifdef __cplusplus
 }

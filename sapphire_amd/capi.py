@@ -107,6 +107,7 @@ SIGNATURES = {
     "sph_spgemm_row_offsets_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,
                                    ctypes.POINTER(ctypes.c_uint32)],
     "sph_spgemm_fill_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
+    "sph_spgemm_load_u32": [_vp, _vp, _vp, _u32, _u32, ctypes.POINTER(ctypes.c_uint64)],
     "sph_spgemm_f32": [_vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,
                        ctypes.POINTER(ctypes.c_uint32)],
     "sph_spmm_csr_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, ctypes.c_int],

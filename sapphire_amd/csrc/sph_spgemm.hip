@@ -684,6 +684,37 @@ __global__ __launch_bounds__(256) void SpgemmUnstageKernel(float* __restrict__ V
         }
 }
 
+// load[p] = entries of the row of B that entry p of A selects (the multiplications entry p
+// causes); *total (when given, zero before the launch) receives their sum.
+__global__ __launch_bounds__(256) void SpgemmLoadKernel(uint32_t* __restrict__ load,
+                                                        const uint32_t* __restrict__ COLA,
+                                                        const uint32_t* __restrict__ ROWB,
+                                                        uint32_t entries, uint32_t K,
+                                                        unsigned long long* total)
+{
+    unsigned long long sum = 0;
+    for (uint64_t p = blockIdx.x * 256ull + threadIdx.x; p < entries; p += 256ull * gridDim.x)
+    {
+        const uint32_t k = COLA[p];
+        const uint32_t n = k < K ? ROWB[k + 1] - ROWB[k] : 0u;
+        if (load != nullptr)
+            load[p] = n;
+        sum += n;
+    }
+    if (total == nullptr)
+        return;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1)
+        sum += __shfl_xor(sum, d, 64);
+    if ((threadIdx.x & 63u) == 0 && sum != 0)
+        atomicAdd(total, sum);
+}
+
+__global__ void ClearTotalKernel(unsigned long long* total)
+{
+    *total = 0;
+}
+
 uint32_t StripFor(uint32_t N)
 {
     const uint32_t padded = (N + 63u) / 64u * 64u;
@@ -784,6 +815,50 @@ int sph_spgemm_fill_f32(float* VC, uint32_t* COLC, const uint32_t* ROWC, const f
     hipLaunchKernelGGL(SpgemmRowKernel<kFill>, dim3(GridFor(M, args.rowsPerTurn)), dim3(64),
                        args.strip * sizeof(float) + args.strip / 8, stream, args);
     SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+int sph_spgemm_load_u32(uint32_t* load, const uint32_t* COLA, const uint32_t* ROWB,
+                        uint32_t entries, uint32_t K, uint64_t* productsHost)
+{
+    SPH_REQUIRE(entries == 0 || COLA != nullptr, "COLA is null");
+    SPH_REQUIRE(entries == 0 || K == 0 || ROWB != nullptr, "ROWB is null");
+    if (productsHost != nullptr)
+        SPH_REFUSE_WHILE_CAPTURING();  // reads back and takes a scratch word
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    if (entries == 0)
+    {
+        if (productsHost != nullptr)
+            *productsHost = 0;
+        return SPH_OK;
+    }
+    unsigned long long* total = nullptr;
+    if (productsHost != nullptr)
+    {
+        SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&total), sizeof(*total), stream));
+        hipLaunchKernelGGL(ClearTotalKernel, dim3(1), dim3(1), 0, stream, total);
+    }
+    const uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>(
+        (static_cast<uint64_t>(entries) + 255) / 256, static_cast<uint64_t>(sph::ComputeUnits()) * 8));
+    hipLaunchKernelGGL(SpgemmLoadKernel, dim3(blocks), dim3(256), 0, stream, load, COLA, ROWB,
+                       entries, K, total);
+    const hipError_t launched = hipGetLastError();
+    hipError_t copied = hipSuccess;
+    if (launched == hipSuccess && productsHost != nullptr)
+    {
+        static_assert(sizeof(unsigned long long) == sizeof(uint64_t), "64-bit total");
+        copied = hipMemcpyAsync(productsHost, total, sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
+        if (copied == hipSuccess)
+            copied = hipStreamSynchronize(stream);
+    }
+    if (total != nullptr)
+        SPH_HIP_TRY(hipFreeAsync(total, stream));
+    if (launched != hipSuccess)
+        return sph::Fail(SPH_ERR_DEVICE, std::string("sph_spgemm_load_u32 - launch failed with ") +
+                                             hipGetErrorString(launched));
+    SPH_HIP_TRY(copied);
     return SPH_OK;
 }
 

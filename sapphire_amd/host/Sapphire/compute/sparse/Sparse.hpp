@@ -4,8 +4,9 @@
 // A "host" record has its V / COL / ROW arrays in host memory; a "device" record is the same
 // 48-byte struct, kept in host memory, whose three arrays are device memory -- the form the
 // kernels behind the C ABI take (they receive the arrays, not the struct).  Arrays come from
-// ResourceManager's preserved pools.  The LoadDistMatrix overloads of the reference belong to
-// its sparse x sparse product and are not provided.
+// ResourceManager's preserved pools.  The LoadDistMatrix overloads (Sparse.hpp:28, 41, 59, 75,
+// 102, 118, 135, 150 of the reference) do the same for the load-distribution records of the
+// sparse x sparse product.
 #ifndef SAPPHIRE_AMD_COMPUTE_SPARSE_SPARSE_HPP
 #define SAPPHIRE_AMD_COMPUTE_SPARSE_SPARSE_HPP
 
@@ -35,6 +36,25 @@ void DeepCopyDeviceToHost(SparseMatrix* hostDstArray, const SparseMatrix* device
 void DeepCopyDeviceToDevice(SparseMatrix* deviceDstArray, const SparseMatrix* deviceSrcArray,
                             uint32_t numMatrices, int deviceId);
 void DeepCopyHostToHost(SparseMatrix* hostDstArray, const SparseMatrix* hostSrcArray,
+                        uint32_t numMatrices);
+
+//! Load-distribution records with the shape and entry counts of the given sparse records
+//! (arrays zero-filled on the host, not initialised on the device).
+void DeepAllocateLoadDistHost(LoadDistMatrix** loadDistArray, SparseMatrix* sparseArray,
+                              uint32_t numMatrices);
+void DeepFreeLoadDistHost(LoadDistMatrix* loadDistArray, uint32_t numMatrices);
+void DeepAllocateLoadDistCuda(LoadDistMatrix** deviceLoadDistArray,
+                              LoadDistMatrix* hostLoadDistArray, uint32_t numMatrices,
+                              int deviceId);
+void DeepFreeLoadDistCuda(LoadDistMatrix* deviceLoadDistArray, uint32_t numMatrices,
+                          int deviceId);
+void DeepCopyDeviceToDevice(LoadDistMatrix* deviceDstArray, LoadDistMatrix* deviceSrcArray,
+                            uint32_t numMatrices, int deviceId);
+void DeepCopyHostToDevice(LoadDistMatrix* deviceDstArray, LoadDistMatrix* hostSrcArray,
+                          uint32_t numMatrices, int deviceId);
+void DeepCopyDeviceToHost(LoadDistMatrix* hostDstArray, LoadDistMatrix* deviceSrcArray,
+                          uint32_t numMatrices, int deviceId);
+void DeepCopyHostToHost(LoadDistMatrix* hostDstArray, LoadDistMatrix* hostSrcArray,
                         uint32_t numMatrices);
 
 //! Builds numMatrices device records from dense matrices in device memory: matrix i starts at

@@ -37,10 +37,28 @@ void FreeSparseMatrix(SparseMatrix& matrix);
 //! (Includes/Sapphire/compute/sparse/cuda/SparseGemm.cuh:38-42).  *cudaOutput receives a new
 //! array of device records (release with Compute::DeepFreeSparseCuda); with copyResultToHost
 //! *hostOutput receives host copies (release with Compute::DeepFreeSparseHost), otherwise
-//! nullptr.  Sums that are exactly zero are not stored; columns ascend within a row.
+//! nullptr.  Sums that are exactly zero are not stored; columns ascend within a row.  The number
+//! of products of a pair (the load-distribution pre-pass) bounds the entries of its result, so
+//! V and COL are allocated for that bound and the products are computed once; a result with
+//! less than half of the bound in use is moved to arrays of its own size.
 void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cudaA,
           SparseMatrix* cudaB, uint32_t m, uint32_t n, std::size_t numMatrices, int deviceId,
           bool copyResultToHost);
+
+//! The load-distribution pre-pass of the sparse x sparse product, with the signatures the
+//! reference declares (Includes/Sapphire/compute/sparse/cuda/SparseGemm.cuh:16-18, 43-46).
+//! CallLoadDist: a, b and loadDist are arrays of device records (loadDist[i] allocated with the
+//! shape and entry count of a[i], e.g. by Compute::DeepAllocateLoadDistCuda); loadDist[i]
+//! receives a[i]'s COL and ROW and, per entry, the number of entries in the row of b[i] it
+//! selects -- the multiplications that entry causes.  nnzArray[i] (host, may be null) receives
+//! the number of products of pair i, which bounds the entries of a[i] * b[i] from above
+//! (saturated at 2^32 - 1).  M is the row count of every a[i].
+void CallLoadDist(SparseMatrix* a, SparseMatrix* b, LoadDistMatrix* loadDist, uint32_t M,
+                  uint32_t* nnzArray, std::size_t numMatrices, int deviceId);
+//! GetLoadDist: the same into host records (allocated like cudaA, e.g. by
+//! Compute::DeepAllocateLoadDistHost); the device records it needs are temporary.
+void GetLoadDist(LoadDistMatrix* hostLoadDist, SparseMatrix* cudaA, SparseMatrix* cudaB,
+                 uint32_t m, std::size_t numMatrices, int deviceId);
 }  // namespace Sapphire::Compute::Sparse::Cuda
 
 namespace Sapphire::Compute

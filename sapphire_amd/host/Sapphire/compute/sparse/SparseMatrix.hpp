@@ -24,4 +24,20 @@ struct alignas(16) SparseMatrix
 
 static_assert(sizeof(SparseMatrix) == 48, "SparseMatrix must stay 48 bytes");
 
+// The companion record of the reference's sparse x sparse product
+// (Includes/Sapphire/compute/sparse/SparseMatrix.hpp:40-50): the shape of a SparseMatrix with,
+// in place of each value, the number of multiplications that entry causes in a product.
+struct alignas(16) LoadDistMatrix
+{
+    uint32_t* Load;  //!< per entry: entries in the row of the right operand it selects
+    uint32_t* COL;
+    uint32_t* ROW;   //!< M + 1 offsets
+    uint32_t NNZ;
+    uint32_t M;
+    uint32_t N;
+    uint32_t Padding[3];
+};
+
+static_assert(sizeof(LoadDistMatrix) == 48, "LoadDistMatrix must stay 48 bytes");
+
 #endif

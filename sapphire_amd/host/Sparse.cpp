@@ -7,6 +7,8 @@
 
 #include <algorithm>
 #include <cstring>
+#include <functional>
+#include <utility>
 #include <stdexcept>
 #include <string>
 
@@ -25,169 +27,266 @@ void Check(int status, const char* function)
         throw std::runtime_error(std::string(function) + " failed with " + sph_last_error());
 }
 
-void RequireRoom(const SparseMatrix& dst, const SparseMatrix& src, const char* function)
+// The two record types differ in the name and element type of their first array only (4-byte
+// elements in both); everything below is written once over "first array, COL, ROW".
+void* First(const SparseMatrix& r)
 {
-    if (dst.V == nullptr || dst.COL == nullptr || dst.ROW == nullptr)
+    return r.V;
+}
+void* First(const LoadDistMatrix& r)
+{
+    return r.Load;
+}
+void SetFirst(SparseMatrix& r, void* p)
+{
+    r.V = static_cast<float*>(p);
+}
+void SetFirst(LoadDistMatrix& r, void* p)
+{
+    r.Load = static_cast<uint32_t*>(p);
+}
+
+template <typename Record>
+void RequireRoom(const Record& dst, const Record& src, const char* function)
+{
+    if (First(dst) == nullptr || dst.COL == nullptr || dst.ROW == nullptr)
         throw std::invalid_argument(std::string(function) + " - destination is not allocated");
     if (dst.NNZ < src.NNZ || dst.M < src.M)
         throw std::invalid_argument(std::string(function) + " - destination is too small");
 }
 
-SparseMatrix AllocateCuda(uint32_t m, uint32_t n, uint32_t nnz)
+template <typename Record>
+Record AllocateCudaRecord(uint32_t m, uint32_t n, uint32_t nnz)
 {
-    SparseMatrix r{};
+    Record r{};
     r.M = m;
     r.N = n;
     r.NNZ = nnz;
-    r.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(Bytes(nnz), true));
+    SetFirst(r, Util::ResourceManager::GetMemoryCuda(Bytes(nnz), true));
     r.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(Bytes(nnz), true));
     r.ROW = static_cast<uint32_t*>(
         Util::ResourceManager::GetMemoryCuda(Bytes(static_cast<std::size_t>(m) + 1), true));
     return r;
 }
 
-void ReleaseCuda(SparseMatrix& r)
+SparseMatrix AllocateCuda(uint32_t m, uint32_t n, uint32_t nnz)
 {
-    if (r.V != nullptr)
-        Util::ResourceManager::FreePreservedCuda(r.V);
+    return AllocateCudaRecord<SparseMatrix>(m, n, nnz);
+}
+
+template <typename Record>
+void ReleaseCudaRecord(Record& r)
+{
+    if (First(r) != nullptr)
+        Util::ResourceManager::FreePreservedCuda(First(r));
     if (r.COL != nullptr)
         Util::ResourceManager::FreePreservedCuda(r.COL);
     if (r.ROW != nullptr)
         Util::ResourceManager::FreePreservedCuda(r.ROW);
-    r = SparseMatrix{};
+    r = Record{};
 }
-}  // namespace
 
-void DeepAllocateSparseHost(SparseMatrix** sparseMatrixArray, uint32_t m, uint32_t n,
-                            const uint32_t nnz[], uint32_t numMatrices)
+void ReleaseCuda(SparseMatrix& r)
 {
-    auto* array = new SparseMatrix[numMatrices]();
+    ReleaseCudaRecord(r);
+}
+
+template <typename Record>
+Record* AllocateHostArray(uint32_t numMatrices, uint32_t m, uint32_t n,
+                          const std::function<uint32_t(uint32_t)>& nnzOf,
+                          const std::function<std::pair<uint32_t, uint32_t>(uint32_t)>& shapeOf)
+{
+    auto* array = new Record[numMatrices]();
     for (uint32_t i = 0; i < numMatrices; ++i)
     {
-        SparseMatrix& r = array[i];
-        r.M = m;
-        r.N = n;
-        r.NNZ = nnz[i];
-        r.V = static_cast<float*>(Util::ResourceManager::GetMemoryHost(Bytes(nnz[i]), true));
-        r.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryHost(Bytes(nnz[i]), true));
+        Record& r = array[i];
+        const auto shape = shapeOf ? shapeOf(i) : std::make_pair(m, n);
+        r.M = shape.first;
+        r.N = shape.second;
+        r.NNZ = nnzOf(i);
+        SetFirst(r, Util::ResourceManager::GetMemoryHost(Bytes(r.NNZ), true));
+        r.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryHost(Bytes(r.NNZ), true));
         r.ROW = static_cast<uint32_t*>(
-            Util::ResourceManager::GetMemoryHost(Bytes(static_cast<std::size_t>(m) + 1), true));
-        std::memset(r.V, 0, Bytes(nnz[i]));
-        std::memset(r.COL, 0, Bytes(nnz[i]));
-        std::memset(r.ROW, 0, Bytes(static_cast<std::size_t>(m) + 1));
+            Util::ResourceManager::GetMemoryHost(Bytes(static_cast<std::size_t>(r.M) + 1), true));
+        std::memset(First(r), 0, Bytes(r.NNZ));
+        std::memset(r.COL, 0, Bytes(r.NNZ));
+        std::memset(r.ROW, 0, Bytes(static_cast<std::size_t>(r.M) + 1));
     }
-    *sparseMatrixArray = array;
+    return array;
 }
 
-void DeepFreeSparseHost(SparseMatrix* sparseMatrixArray, uint32_t numMatrices)
+template <typename Record>
+void FreeHostArray(Record* array, uint32_t numMatrices)
 {
-    if (sparseMatrixArray == nullptr)
+    if (array == nullptr)
         return;
     for (uint32_t i = 0; i < numMatrices; ++i)
     {
-        SparseMatrix& r = sparseMatrixArray[i];
-        if (r.V != nullptr)
-            Util::ResourceManager::FreePreservedHost(r.V);
+        Record& r = array[i];
+        if (First(r) != nullptr)
+            Util::ResourceManager::FreePreservedHost(First(r));
         if (r.COL != nullptr)
             Util::ResourceManager::FreePreservedHost(r.COL);
         if (r.ROW != nullptr)
             Util::ResourceManager::FreePreservedHost(r.ROW);
     }
-    delete[] sparseMatrixArray;
+    delete[] array;
+}
+
+template <typename Record, typename SizesFrom>
+Record* AllocateCudaArray(const SizesFrom* like, uint32_t numMatrices, int deviceId)
+{
+    Cuda::CudaSetDevice(deviceId);
+    auto* array = new Record[numMatrices]();
+    for (uint32_t i = 0; i < numMatrices; ++i)
+        array[i] = AllocateCudaRecord<Record>(like[i].M, like[i].N, like[i].NNZ);
+    return array;
+}
+
+template <typename Record>
+void FreeCudaArray(Record* array, uint32_t numMatrices, int deviceId)
+{
+    if (array == nullptr)
+        return;
+    Cuda::CudaSetDevice(deviceId);
+    Cuda::Synchronize();  // kernels may still be reading the arrays
+    for (uint32_t i = 0; i < numMatrices; ++i)
+        ReleaseCudaRecord(array[i]);
+    delete[] array;
+}
+
+// `copy(dst, src, bytes)` moves one array
+template <typename Record, typename Copy>
+void CopyArray(Record* dstArray, const Record* srcArray, uint32_t numMatrices,
+               const char* function, Copy&& copy)
+{
+    for (uint32_t i = 0; i < numMatrices; ++i)
+    {
+        const Record& s = srcArray[i];
+        Record& d = dstArray[i];
+        RequireRoom(d, s, function);
+        copy(First(d), First(s), static_cast<std::size_t>(s.NNZ) * 4);
+        copy(d.COL, s.COL, static_cast<std::size_t>(s.NNZ) * 4);
+        copy(d.ROW, s.ROW, (static_cast<std::size_t>(s.M) + 1) * 4);
+        d.NNZ = s.NNZ;
+        d.M = s.M;
+        d.N = s.N;
+    }
+}
+
+const auto kHostToDevice = [](void* d, const void* s, std::size_t n) { Cuda::CopyHostToDevice(d, s, n); };
+const auto kDeviceToHost = [](void* d, const void* s, std::size_t n) { Cuda::CopyDeviceToHost(d, s, n); };
+const auto kDeviceToDevice = [](void* d, const void* s, std::size_t n) { Cuda::CopyDeviceToDevice(d, s, n); };
+const auto kHostToHost = [](void* d, const void* s, std::size_t n) { std::memcpy(d, s, n); };
+}  // namespace
+
+void DeepAllocateSparseHost(SparseMatrix** sparseMatrixArray, uint32_t m, uint32_t n,
+                            const uint32_t nnz[], uint32_t numMatrices)
+{
+    *sparseMatrixArray = AllocateHostArray<SparseMatrix>(
+        numMatrices, m, n, [&](uint32_t i) { return nnz[i]; }, nullptr);
+}
+
+void DeepFreeSparseHost(SparseMatrix* sparseMatrixArray, uint32_t numMatrices)
+{
+    FreeHostArray(sparseMatrixArray, numMatrices);
 }
 
 void DeepAllocateSparseCuda(SparseMatrix** deviceSparseArray,
                             const SparseMatrix* hostSparseMatrixArray, uint32_t numMatrices,
                             int deviceId)
 {
-    Cuda::CudaSetDevice(deviceId);
-    auto* array = new SparseMatrix[numMatrices]();
-    for (uint32_t i = 0; i < numMatrices; ++i)
-        array[i] = AllocateCuda(hostSparseMatrixArray[i].M, hostSparseMatrixArray[i].N,
-                                hostSparseMatrixArray[i].NNZ);
-    *deviceSparseArray = array;
+    *deviceSparseArray = AllocateCudaArray<SparseMatrix>(hostSparseMatrixArray, numMatrices, deviceId);
 }
 
 void DeepFreeSparseCuda(SparseMatrix* deviceSparseArray, uint32_t numMatrices, int deviceId)
 {
-    if (deviceSparseArray == nullptr)
-        return;
-    Cuda::CudaSetDevice(deviceId);
-    Cuda::Synchronize();  // kernels may still be reading the arrays
-    for (uint32_t i = 0; i < numMatrices; ++i)
-        ReleaseCuda(deviceSparseArray[i]);
-    delete[] deviceSparseArray;
+    FreeCudaArray(deviceSparseArray, numMatrices, deviceId);
 }
 
 void DeepCopyHostToDevice(SparseMatrix* deviceDstArray, const SparseMatrix* hostSrcArray,
                           uint32_t numMatrices, int deviceId)
 {
     Cuda::CudaSetDevice(deviceId);
-    for (uint32_t i = 0; i < numMatrices; ++i)
-    {
-        const SparseMatrix& s = hostSrcArray[i];
-        SparseMatrix& d = deviceDstArray[i];
-        RequireRoom(d, s, "DeepCopyHostToDevice");
-        Cuda::CopyHostToDevice(d.V, s.V, static_cast<std::size_t>(s.NNZ) * 4);
-        Cuda::CopyHostToDevice(d.COL, s.COL, static_cast<std::size_t>(s.NNZ) * 4);
-        Cuda::CopyHostToDevice(d.ROW, s.ROW, (static_cast<std::size_t>(s.M) + 1) * 4);
-        d.NNZ = s.NNZ;
-        d.M = s.M;
-        d.N = s.N;
-    }
+    CopyArray(deviceDstArray, hostSrcArray, numMatrices, "DeepCopyHostToDevice", kHostToDevice);
 }
 
 void DeepCopyDeviceToHost(SparseMatrix* hostDstArray, const SparseMatrix* deviceSrcArray,
                           uint32_t numMatrices, int deviceId)
 {
     Cuda::CudaSetDevice(deviceId);
-    for (uint32_t i = 0; i < numMatrices; ++i)
-    {
-        const SparseMatrix& s = deviceSrcArray[i];
-        SparseMatrix& d = hostDstArray[i];
-        RequireRoom(d, s, "DeepCopyDeviceToHost");
-        Cuda::CopyDeviceToHost(d.V, s.V, static_cast<std::size_t>(s.NNZ) * 4);
-        Cuda::CopyDeviceToHost(d.COL, s.COL, static_cast<std::size_t>(s.NNZ) * 4);
-        Cuda::CopyDeviceToHost(d.ROW, s.ROW, (static_cast<std::size_t>(s.M) + 1) * 4);
-        d.NNZ = s.NNZ;
-        d.M = s.M;
-        d.N = s.N;
-    }
+    CopyArray(hostDstArray, deviceSrcArray, numMatrices, "DeepCopyDeviceToHost", kDeviceToHost);
 }
 
 void DeepCopyDeviceToDevice(SparseMatrix* deviceDstArray, const SparseMatrix* deviceSrcArray,
                             uint32_t numMatrices, int deviceId)
 {
     Cuda::CudaSetDevice(deviceId);
-    for (uint32_t i = 0; i < numMatrices; ++i)
-    {
-        const SparseMatrix& s = deviceSrcArray[i];
-        SparseMatrix& d = deviceDstArray[i];
-        RequireRoom(d, s, "DeepCopyDeviceToDevice");
-        Cuda::CopyDeviceToDevice(d.V, s.V, static_cast<std::size_t>(s.NNZ) * 4);
-        Cuda::CopyDeviceToDevice(d.COL, s.COL, static_cast<std::size_t>(s.NNZ) * 4);
-        Cuda::CopyDeviceToDevice(d.ROW, s.ROW, (static_cast<std::size_t>(s.M) + 1) * 4);
-        d.NNZ = s.NNZ;
-        d.M = s.M;
-        d.N = s.N;
-    }
+    CopyArray(deviceDstArray, deviceSrcArray, numMatrices, "DeepCopyDeviceToDevice",
+              kDeviceToDevice);
 }
 
 void DeepCopyHostToHost(SparseMatrix* hostDstArray, const SparseMatrix* hostSrcArray,
                         uint32_t numMatrices)
 {
-    for (uint32_t i = 0; i < numMatrices; ++i)
-    {
-        const SparseMatrix& s = hostSrcArray[i];
-        SparseMatrix& d = hostDstArray[i];
-        RequireRoom(d, s, "DeepCopyHostToHost");
-        std::memcpy(d.V, s.V, static_cast<std::size_t>(s.NNZ) * 4);
-        std::memcpy(d.COL, s.COL, static_cast<std::size_t>(s.NNZ) * 4);
-        std::memcpy(d.ROW, s.ROW, (static_cast<std::size_t>(s.M) + 1) * 4);
-        d.NNZ = s.NNZ;
-        d.M = s.M;
-        d.N = s.N;
-    }
+    CopyArray(hostDstArray, hostSrcArray, numMatrices, "DeepCopyHostToHost", kHostToHost);
+}
+
+void DeepAllocateLoadDistHost(LoadDistMatrix** loadDistArray, SparseMatrix* sparseArray,
+                              uint32_t numMatrices)
+{
+    *loadDistArray = AllocateHostArray<LoadDistMatrix>(
+        numMatrices, 0, 0, [&](uint32_t i) { return sparseArray[i].NNZ; },
+        [&](uint32_t i) { return std::make_pair(sparseArray[i].M, sparseArray[i].N); });
+}
+
+void DeepFreeLoadDistHost(LoadDistMatrix* loadDistArray, uint32_t numMatrices)
+{
+    FreeHostArray(loadDistArray, numMatrices);
+}
+
+void DeepAllocateLoadDistCuda(LoadDistMatrix** deviceLoadDistArray,
+                              LoadDistMatrix* hostLoadDistArray, uint32_t numMatrices,
+                              int deviceId)
+{
+    *deviceLoadDistArray =
+        AllocateCudaArray<LoadDistMatrix>(hostLoadDistArray, numMatrices, deviceId);
+}
+
+void DeepFreeLoadDistCuda(LoadDistMatrix* deviceLoadDistArray, uint32_t numMatrices, int deviceId)
+{
+    FreeCudaArray(deviceLoadDistArray, numMatrices, deviceId);
+}
+
+void DeepCopyDeviceToDevice(LoadDistMatrix* deviceDstArray, LoadDistMatrix* deviceSrcArray,
+                            uint32_t numMatrices, int deviceId)
+{
+    Cuda::CudaSetDevice(deviceId);
+    CopyArray(deviceDstArray, static_cast<const LoadDistMatrix*>(deviceSrcArray), numMatrices,
+              "DeepCopyDeviceToDevice", kDeviceToDevice);
+}
+
+void DeepCopyHostToDevice(LoadDistMatrix* deviceDstArray, LoadDistMatrix* hostSrcArray,
+                          uint32_t numMatrices, int deviceId)
+{
+    Cuda::CudaSetDevice(deviceId);
+    CopyArray(deviceDstArray, static_cast<const LoadDistMatrix*>(hostSrcArray), numMatrices,
+              "DeepCopyHostToDevice", kHostToDevice);
+}
+
+void DeepCopyDeviceToHost(LoadDistMatrix* hostDstArray, LoadDistMatrix* deviceSrcArray,
+                          uint32_t numMatrices, int deviceId)
+{
+    Cuda::CudaSetDevice(deviceId);
+    CopyArray(hostDstArray, static_cast<const LoadDistMatrix*>(deviceSrcArray), numMatrices,
+              "DeepCopyDeviceToHost", kDeviceToHost);
+}
+
+void DeepCopyHostToHost(LoadDistMatrix* hostDstArray, LoadDistMatrix* hostSrcArray,
+                        uint32_t numMatrices)
+{
+    CopyArray(hostDstArray, static_cast<const LoadDistMatrix*>(hostSrcArray), numMatrices,
+              "DeepCopyHostToHost", kHostToHost);
 }
 
 void CreateSparseMatrixWithDenseMatrix(SparseMatrix** dst, const float* src, uint32_t m,

@@ -62,6 +62,59 @@ void FreeSparseMatrix(SparseMatrix& matrix)
     matrix = SparseMatrix{};
 }
 
+void CallLoadDist(SparseMatrix* a, SparseMatrix* b, LoadDistMatrix* loadDist, uint32_t M,
+                  uint32_t* nnzArray, std::size_t numMatrices, int deviceId)
+{
+    if (a == nullptr || b == nullptr || loadDist == nullptr)
+        throw std::invalid_argument("Sparse::Cuda::CallLoadDist - null array");
+    Compute::Cuda::CudaSetDevice(deviceId);
+    for (std::size_t i = 0; i < numMatrices; ++i)
+    {
+        const SparseMatrix& left = a[i];
+        const SparseMatrix& right = b[i];
+        LoadDistMatrix& d = loadDist[i];
+        if (left.M != M || left.N != right.M)
+            throw std::invalid_argument("Sparse::Cuda::CallLoadDist - shape mismatch");
+        if (d.Load == nullptr || d.COL == nullptr || d.ROW == nullptr || d.NNZ < left.NNZ ||
+            d.M < left.M)
+            throw std::invalid_argument("Sparse::Cuda::CallLoadDist - record is too small");
+        Compute::Cuda::CopyDeviceToDevice(d.COL, left.COL, static_cast<std::size_t>(left.NNZ) * 4);
+        Compute::Cuda::CopyDeviceToDevice(d.ROW, left.ROW,
+                                          (static_cast<std::size_t>(left.M) + 1) * 4);
+        d.NNZ = left.NNZ;
+        d.M = left.M;
+        d.N = left.N;
+        uint64_t products = 0;
+        if (sph_spgemm_load_u32(d.Load, left.COL, right.ROW, left.NNZ, right.M,
+                                nnzArray != nullptr ? &products : nullptr) != SPH_OK)
+            throw std::runtime_error(std::string("Sparse::Cuda::CallLoadDist failed with ") +
+                                     sph_last_error());
+        if (nnzArray != nullptr)
+            nnzArray[i] = static_cast<uint32_t>(std::min<uint64_t>(products, 0xffffffffull));
+    }
+}
+
+void GetLoadDist(LoadDistMatrix* hostLoadDist, SparseMatrix* cudaA, SparseMatrix* cudaB,
+                 uint32_t m, std::size_t numMatrices, int deviceId)
+{
+    if (hostLoadDist == nullptr)
+        throw std::invalid_argument("Sparse::Cuda::GetLoadDist - null array");
+    const auto count = static_cast<uint32_t>(numMatrices);
+    LoadDistMatrix* device = nullptr;
+    DeepAllocateLoadDistCuda(&device, hostLoadDist, count, deviceId);
+    try
+    {
+        CallLoadDist(cudaA, cudaB, device, m, nullptr, numMatrices, deviceId);
+        DeepCopyDeviceToHost(hostLoadDist, device, count, deviceId);
+    }
+    catch (...)
+    {
+        DeepFreeLoadDistCuda(device, count, deviceId);
+        throw;
+    }
+    DeepFreeLoadDistCuda(device, count, deviceId);
+}
+
 void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cudaA,
           SparseMatrix* cudaB, uint32_t m, uint32_t n, std::size_t numMatrices, int deviceId,
           bool copyResultToHost)
@@ -78,38 +131,56 @@ void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cu
     };
     try
     {
-        // Counting passes of all matrices first, without reading anything back: the stream is
-        // drained once, by the first read of an entry count, instead of once per matrix.
+        // The number of products of a pair bounds the entries of its result; with room for that
+        // many the products are computed once (the counting pass stages every row).  All
+        // products are enqueued before any entry count is read back, so the stream is drained
+        // once for the batch and not once per matrix.
+        std::vector<uint32_t> capacity(count);
         for (uint32_t i = 0; i < count; ++i)
         {
             const SparseMatrix& a = cudaA[i];
             const SparseMatrix& b = cudaB[i];
             if (a.M != m || b.N != n || a.N != b.M)
                 throw std::invalid_argument("Sparse::Cuda::Gemm - shape mismatch");
-            SparseMatrix& c = result[i];
-            c.M = m;
-            c.N = n;
-            c.ROW = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(
-                (static_cast<std::size_t>(m) + 1) * 4, true));
-            check(sph_spgemm_row_offsets_f32(c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m, a.N,
-                                             n, nullptr));
-        }
-        for (uint32_t i = 0; i < count; ++i)
-        {
-            uint32_t nnz = 0;
-            Compute::Cuda::CopyDeviceToHost(&nnz, result[i].ROW + m, sizeof(nnz));
-            result[i].NNZ = nnz;
+            uint64_t products = 0;
+            check(sph_spgemm_load_u32(nullptr, a.COL, b.ROW, a.NNZ, b.M, &products));
+            capacity[i] = static_cast<uint32_t>(std::min<uint64_t>(
+                { products, static_cast<uint64_t>(m) * n, 0xffffffffull }));
         }
         for (uint32_t i = 0; i < count; ++i)
         {
             const SparseMatrix& a = cudaA[i];
             const SparseMatrix& b = cudaB[i];
             SparseMatrix& c = result[i];
-            const std::size_t bytes = std::max<std::size_t>(c.NNZ, 1) * 4;
+            c.M = m;
+            c.N = n;
+            c.ROW = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(
+                (static_cast<std::size_t>(m) + 1) * 4, true));
+            const std::size_t bytes = std::max<std::size_t>(capacity[i], 1) * 4;
             c.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
             c.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
-            check(sph_spgemm_fill_f32(c.V, c.COL, c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m,
-                                      a.N, n));
+            check(sph_spgemm_f32(c.V, c.COL, c.ROW, capacity[i], a.V, a.COL, a.ROW, b.V, b.COL,
+                                 b.ROW, m, a.N, n, nullptr));
+        }
+        for (uint32_t i = 0; i < count; ++i)
+        {
+            SparseMatrix& c = result[i];
+            uint32_t nnz = 0;
+            Compute::Cuda::CopyDeviceToHost(&nnz, c.ROW + m, sizeof(nnz));
+            c.NNZ = nnz;
+            if (static_cast<uint64_t>(nnz) * 2 < capacity[i] && capacity[i] > 1024)
+            {
+                // mostly unused: move the entries to arrays of their own size
+                const std::size_t bytes = std::max<std::size_t>(nnz, 1) * 4;
+                auto* v = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
+                auto* col = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
+                Compute::Cuda::CopyDeviceToDevice(v, c.V, static_cast<std::size_t>(nnz) * 4);
+                Compute::Cuda::CopyDeviceToDevice(col, c.COL, static_cast<std::size_t>(nnz) * 4);
+                Util::ResourceManager::FreePreservedCuda(c.V);
+                Util::ResourceManager::FreePreservedCuda(c.COL);
+                c.V = v;
+                c.COL = col;
+            }
         }
         if (copyResultToHost)
         {

@@ -540,6 +540,66 @@ int sphh_sparse_sparse_gemm(const float* denseA, const float* denseB, unsigned m
     });
 }
 
+// The load-distribution records of the sparse x sparse product for one pair of matrices given
+// dense on the host: GetLoadDist into a host record, then that record through every
+// LoadDistMatrix copy overload (host -> host, host -> device, device -> device, device -> host),
+// and CallLoadDist for the number of products.  load / col hold `capacity` entries, row m + 1.
+int sphh_load_dist(const float* denseA, const float* denseB, unsigned m, unsigned k, unsigned n,
+                   unsigned* nnzA, unsigned* load, unsigned* col, unsigned* row,
+                   unsigned* products, unsigned long capacity)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData A = Upload(Shape({ static_cast<int>(m), static_cast<int>(k) }), denseA, cuda);
+        TensorData B = Upload(Shape({ static_cast<int>(k), static_cast<int>(n) }), denseB, cuda);
+        SparseMatrix* a = nullptr;
+        SparseMatrix* b = nullptr;
+        LoadDistMatrix* host = nullptr;
+        LoadDistMatrix* hostCopy = nullptr;
+        LoadDistMatrix* device = nullptr;
+        LoadDistMatrix* deviceCopy = nullptr;
+        auto release = [&] {
+            Compute::DeepFreeLoadDistCuda(deviceCopy, 1, 0);
+            Compute::DeepFreeLoadDistCuda(device, 1, 0);
+            Compute::DeepFreeLoadDistHost(hostCopy, 1);
+            Compute::DeepFreeLoadDistHost(host, 1);
+            Compute::DeepFreeSparseCuda(b, 1, 0);
+            Compute::DeepFreeSparseCuda(a, 1, 0);
+        };
+        try
+        {
+            Compute::CreateSparseMatrixWithDenseMatrix(&a, A.CudaRawPtr(), m, k, k, 1, 0);
+            Compute::CreateSparseMatrixWithDenseMatrix(&b, B.CudaRawPtr(), k, n, n, 1, 0);
+            *nnzA = a[0].NNZ;
+            if (a[0].NNZ > capacity)
+                throw std::runtime_error("sphh_load_dist - capacity too small");
+            Compute::DeepAllocateLoadDistHost(&host, a, 1);
+            Compute::Sparse::Cuda::GetLoadDist(host, a, b, m, 1, 0);
+            Compute::DeepAllocateLoadDistHost(&hostCopy, a, 1);
+            Compute::DeepCopyHostToHost(hostCopy, host, 1);
+            Compute::DeepAllocateLoadDistCuda(&device, hostCopy, 1, 0);
+            Compute::DeepCopyHostToDevice(device, hostCopy, 1, 0);
+            Compute::DeepAllocateLoadDistCuda(&deviceCopy, hostCopy, 1, 0);
+            Compute::DeepCopyDeviceToDevice(deviceCopy, device, 1, 0);
+            std::memset(hostCopy[0].Load, 0xff, static_cast<std::size_t>(a[0].NNZ) * 4);
+            Compute::DeepCopyDeviceToHost(hostCopy, deviceCopy, 1, 0);
+            std::memcpy(load, hostCopy[0].Load, static_cast<std::size_t>(a[0].NNZ) * 4);
+            std::memcpy(col, hostCopy[0].COL, static_cast<std::size_t>(a[0].NNZ) * 4);
+            std::memcpy(row, hostCopy[0].ROW, (static_cast<std::size_t>(m) + 1) * 4);
+            if (hostCopy[0].M != m || hostCopy[0].N != k || hostCopy[0].NNZ != a[0].NNZ)
+                throw std::runtime_error("sphh_load_dist - record counters were not carried over");
+            Compute::Sparse::Cuda::CallLoadDist(a, b, device, m, products, 1, 0);
+        }
+        catch (...)
+        {
+            release();
+            throw;
+        }
+        release();
+        Util::ResourceManager::Clean();
+    });
+}
+
 // BackProp::MatMulBackward: da and db hold values on entry and are accumulated into.
 int sphh_matmul_backward(float* da, float* db, const float* dy, const float* a, const float* b,
                          const int* aShape, int an, const int* bShape, int bn, const int* yShape,

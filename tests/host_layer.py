@@ -211,6 +211,27 @@ def sparse_sparse_gemm(dA, dB, capacity):
     return V[:nnz.value], COL[:nnz.value], ROW
 
 
+def load_dist(dA, dB):
+    """(load, COL, ROW, products) of the load-distribution pre-pass for two dense-given matrices."""
+    m, k = dA.shape
+    n = dB.shape[1]
+    up = ctypes.POINTER(ctypes.c_uint)
+    h = lib()
+    h.sphh_load_dist.argtypes = [_fp, _fp, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, up, up, up,
+                                 up, up, ctypes.c_ulong]
+    h.sphh_load_dist.restype = ctypes.c_int
+    capacity = max(int(np.count_nonzero(dA)), 1)
+    nnz = ctypes.c_uint(0)
+    products = ctypes.c_uint(0)
+    load = np.zeros(capacity, np.uint32)
+    col = np.zeros(capacity, np.uint32)
+    row = np.zeros(m + 1, np.uint32)
+    _ok(h.sphh_load_dist(_f(np.ascontiguousarray(dA)), _f(np.ascontiguousarray(dB)), m, k, n,
+                         ctypes.byref(nnz), load.ctypes.data_as(up), col.ctypes.data_as(up),
+                         row.ctypes.data_as(up), ctypes.byref(products), capacity))
+    return load[:nnz.value], col[:nnz.value], row, products.value
+
+
 def matmul_backward(da, db, dy, a, b, sequence):
     """Returns the accumulated (da, db)."""
     da, db = np.ascontiguousarray(da.copy()), np.ascontiguousarray(db.copy())

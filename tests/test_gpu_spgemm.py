@@ -144,6 +144,37 @@ def test_host_layer_sparse_sparse_gemm(dev, case):
     assert np.array_equal(ROW, wR) and np.array_equal(COL, wC) and np.array_equal(bits(V), bits(wV))
 
 
+@pytest.mark.parametrize("case", [(7, 9, 5, 0.5, 0.5), (130, 90, 300, 0.05, 0.2),
+                                  (40, 33, 64, 0.0, 0.5), (64, 64, 64, 0.3, 0.0)])
+def test_load_distribution_records(dev, case):
+    """Per entry of A the number of entries in the row of B it selects (the reference's
+    LoadDistMatrix), through GetLoadDist / CallLoadDist and every LoadDistMatrix copy overload of
+    the C++ layer; the C ABI call with and without the load array."""
+    M, K, N, da, db = case
+    h.announce("load distribution M K N dA dB =", case)
+    dA = sparse_dense(7100 + M, (M, K), da)
+    dB = sparse_dense(7200 + N, (K, N), db)
+    VA, CA, RA = po.csr_from_dense(dA)
+    VB, CB, RB = po.csr_from_dense(dB)
+    want = np.diff(RB.astype(np.int64))[CA].astype(np.uint32)
+    load, col, row, products = hl.load_dist(dA, dB)
+    assert np.array_equal(load, want) and np.array_equal(col, CA) and np.array_equal(row, RA)
+    assert products == int(want.sum())
+    # the products bound the entries of the product
+    assert int(po.spgemm_csr((VA, CA, RA), (VB, CB, RB), M, K, N)[2][M]) <= products
+    dCol, dRow = _dev(CA, np.uint32), _dev(RB, np.uint32)
+    dLoad = capi.DeviceBuffer.from_array(np.full(max(len(CA), 1), 0xFFFFFFFF, np.uint32))
+    total = ctypes.c_uint64(123)
+    capi.call("sph_spgemm_load_u32", dLoad.ptr, dCol.ptr, dRow.ptr, len(CA), K, ctypes.byref(total))
+    assert total.value == int(want.sum())
+    assert np.array_equal(dLoad.download(np.uint32, (max(len(CA), 1),))[:len(CA)], want)
+    total = ctypes.c_uint64(123)
+    capi.call("sph_spgemm_load_u32", None, dCol.ptr, dRow.ptr, len(CA), K, ctypes.byref(total))
+    assert total.value == int(want.sum())
+    for d in (dCol, dRow, dLoad):
+        d.release()
+
+
 @pytest.mark.parametrize("block", range(4))
 def test_random_shapes_and_densities(dev, block):
     """Widths on both sides of the bit-map word, run and strip boundaries (32, 64, 4096, several
