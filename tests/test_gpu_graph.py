@@ -129,11 +129,24 @@ def test_blocking_calls_are_refused_during_capture_and_capture_survives(dev):
     dX = capi.DeviceBuffer.from_array(x)
     dY = capi.DeviceBuffer(4 * n)
     host = np.zeros(n, np.float32)
+    words = capi.DeviceBuffer(4 * 64)
     with capi.Graph() as graph:
         capi.call("sph_scale_f32", dY.ptr, dX.ptr, 3.0, n)
         for name, args in [("sph_stream_sync", ()),
                            ("sph_memcpy_d2h", (host.ctypes.data, dY.ptr, 4 * n)),
                            ("sph_memcpy_h2d", (dY.ptr, host.ctypes.data, 4 * n))]:
+            with pytest.raises(capi.SphError) as err:
+                capi.call(name, *args)
+            assert err.value.status == 3 and "captured" in str(err.value)
+        # the one-call conversions and products take a scratch allocation: refused as well,
+        # before anything of theirs is recorded
+        for name, args in [("sph_csr_from_dense_f32", (words.ptr, words.ptr, words.ptr, 8, dX.ptr,
+                                                       4, 128, 128, None)),
+                           ("sph_spgemm_f32", (words.ptr, words.ptr, words.ptr, 8, dX.ptr, words.ptr,
+                                               words.ptr, dX.ptr, words.ptr, words.ptr, 4, 4, 4,
+                                               None)),
+                           ("sph_spgemm_load_u32", (words.ptr, words.ptr, words.ptr, 4, 4,
+                                                    capi.ctypes.byref(capi.ctypes.c_uint64(0))))]:
             with pytest.raises(capi.SphError) as err:
                 capi.call(name, *args)
             assert err.value.status == 3 and "captured" in str(err.value)
@@ -152,6 +165,7 @@ def test_blocking_calls_are_refused_during_capture_and_capture_survives(dev):
         capi.call("sph_graph_end_capture", capi.ctypes.byref(handle))   # nothing in progress
     dX.release()
     dY.release()
+    words.release()
 
 
 def test_non_affine_broadcast_walk_recorded_into_a_graph(dev):
