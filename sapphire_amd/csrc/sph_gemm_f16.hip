@@ -659,10 +659,11 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 // 128 x 128 x 32 kernel with straight-to-LDS copies, ragged M and N
 // ---------------------------------------------------------------------------
 // For shapes the 256-tile kernel does not take (M or N not a multiple of 256) as long as K is a
-// multiple of 32, N of 8 and everything is 16-byte aligned.  Four wavefronts (2 x 2), each
-// 64 x 64 = 2 x 2 MFMA blocks, four LDS stages of 16 KiB (two workgroups per compute unit),
-// copies issued two steps ahead, one barrier per step (placed, with the copies, between the
-// MFMAs of the step's first half), fragments read half a step ahead.
+// multiple of 32 (or 32 q + 8, 16, 24 with plain storage), N of 8 and everything is 16-byte
+// aligned.  Four wavefronts (2 x 2, each 64 x 64 = 2 x 2 MFMA blocks) or eight (2 x 4, each
+// 64 x 32), four LDS stages of 16 KiB (two workgroups per compute unit), copies issued two steps
+// ahead, one barrier per step (placed, with the copies, between the MFMAs of the step's first
+// half), fragments read half a step ahead.
 // A stage: 128 rows of 64 bytes, 16-byte chunk c of row x at position c ^ ((x >> 2) & 3).
 // B stage: 32 k-rows of 256 bytes, 32-byte chunks XOR-swizzled with 2*(k%4), read with the
 // transposing LDS load like the 256-tile kernel.  Rows past M and columns past N are clamped to
@@ -673,13 +674,17 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 constexpr int kD = 128;
 constexpr int kDStages = 4;
 constexpr int kDStageBytes = 2 * kD * kTK * 2;  // A + B
-constexpr int kDCopies = 4;                     // per wavefront and step: 2 of A, 2 of B
 
 // TAIL: K = 32 q + r, r = 8, 16 or 24, handled as in the 256-tile kernel: a last step over the
 // window [K - 32, K) whose lanes holding the 32 - r values of k already multiplied feed zeros.
-template <bool TA, bool TB, bool TAIL>
-__global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
+template <bool TA, bool TB, bool TAIL, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args args)
 {
+    static_assert(WAVES == 4 || WAVES == 8, "2 x 2 or 2 x 4 wavefronts");
+    constexpr int WN = WAVES / 2;          // wavefronts across the tile
+    constexpr int TN = 2 / (WN / 2);       // 32-column blocks per wavefront: 2 or 1
+    constexpr int kCopiesPer = 8 / WAVES;  // 1 KiB copies per operand, step and wavefront
+    constexpr int kDCopies = 2 * kCopiesPer;
     __shared__ __attribute__((aligned(1024))) char lds[kDStages * kDStageBytes];
     constexpr uint32_t kBytesA = kD * kTK * 2;  // 8 KiB
 
@@ -690,8 +695,8 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t waveM = wave >> 1;
-    const uint32_t waveN = wave & 1;
+    const uint32_t waveM = wave / WN;
+    const uint32_t waveN = wave % WN;
     const uint32_t M = args.M, N = args.N, K = args.K;
 
     const _Float16* A = args.A + args.strideA * static_cast<int64_t>(unit);
@@ -718,11 +723,11 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
         const uint32_t gx = min(xBase + logical16 * 8, limit - 8);
         return (k * pitch + gx) * 2u;
     };
-    uint32_t aLane[2], bLane[2], aDst[2], bDst[2];
+    uint32_t aLane[kCopiesPer], bLane[kCopiesPer], aDst[kCopiesPer], bDst[kCopiesPer];
 #pragma unroll
-    for (uint32_t i = 0; i < 2; ++i)
+    for (uint32_t i = 0; i < kCopiesPer; ++i)
     {
-        const uint32_t j = wave + 4 * i;
+        const uint32_t j = wave + WAVES * i;
         aLane[i] = TA ? laneKMajor(j, rowBase, M, M) : laneKContig(j, rowBase, M, args.lda);
         bLane[i] = TB ? laneKContig(j, colBase, N, K) : laneKMajor(j, colBase, N, N);
         aDst[i] = j * 1024;
@@ -744,10 +749,10 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     uint32_t stepsToAdvance = steps - 1;
     auto issueOne = [&](uint32_t stage, uint32_t n) {
         const uint32_t base = ldsBase + stage * kDStageBytes;
-        if (n < 2)
+        if (n < kCopiesPer)
             DmaToLds16<0>(aLane[n], aSrc, base + aDst[n]);
         else
-            DmaToLds16<0>(bLane[n - 2], bSrc, base + bDst[n - 2]);
+            DmaToLds16<0>(bLane[n - kCopiesPer], bSrc, base + bDst[n - kCopiesPer]);
     };
     auto advance = [&]() {
         if (stepsToAdvance != 0)
@@ -778,23 +783,26 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
         const uint32_t chunk32 = (chunkBase + (g & 1)) ^ (2 * ((s >> 2) & 3));
         return k * 256 + chunk32 * 32 + (s & 3) * 8;
     };
-    uint32_t aOff[2][2], bOff[2][2];
+    // a wavefront owns rows waveM*64 .. +63 (two blocks) and columns waveN*32*TN .. (TN blocks)
+    uint32_t aOff[2][2], bOff[2][TN];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
+    {
 #pragma unroll
         for (int b = 0; b < 2; ++b)
-        {
             aOff[ks][b] = TA ? offKMajor(ks, waveM * 4 + b * 2)
                              : offKContig(ks, waveM * 64 + b * 32 + l32);
-            bOff[ks][b] = kBytesA + (TB ? offKContig(ks, waveN * 64 + b * 32 + l32)
-                                        : offKMajor(ks, waveN * 4 + b * 2));
-        }
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+            bOff[ks][b] = kBytesA + (TB ? offKContig(ks, (waveN * TN + b) * 32 + l32)
+                                        : offKMajor(ks, (waveN * TN + b) * 2));
+    }
     auto readKContig = [&](const char* p) { return *reinterpret_cast<const halfx8*>(p); };
     auto readKMajor = [&](const char* p) {
         const _Float16* h = reinterpret_cast<const _Float16*>(p);
         return Join(LdsReadTr(h), LdsReadTr(h + 4 * 128));
     };
-    auto loadFragments = [&](halfx8 (&af)[2], halfx8 (&bf)[2], const char* stage, int ks) {
+    auto loadFragments = [&](halfx8 (&af)[2], halfx8 (&bf)[TN], const char* stage, int ks) {
 #pragma unroll
         for (int b = 0; b < 2; ++b)
         {
@@ -802,6 +810,10 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
                 af[b] = readKMajor(stage + aOff[ks][b]);
             else
                 af[b] = readKContig(stage + aOff[ks][b]);
+        }
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+        {
             if constexpr (TB)
                 bf[b] = readKContig(stage + bOff[ks][b]);
             else
@@ -809,34 +821,34 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
         }
     };
 
-    floatx16 acc[2][2];
+    floatx16 acc[2][TN];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v)
                 acc[i][j][v] = 0.f;
     // TAIL: a lane's fragments of half ks hold k group 2 ks + khalf of the step's window; in the
     // last step the groups below 4 - r/8 repeat values of k the step before has multiplied
     const uint32_t firstNewGroup = TAIL ? 4 - (K % kTK) / 8 : 0;
-    auto maskRepeated = [&](halfx8 (&af)[2], halfx8 (&bf)[2], int ks, bool lastStep) {
+    auto maskRepeated = [&](halfx8 (&af)[2], halfx8 (&bf)[TN], int ks, bool lastStep) {
         if constexpr (TAIL)
         {
             const bool drop = lastStep && 2 * ks + khalf < firstNewGroup;
 #pragma unroll
             for (int b = 0; b < 2; ++b)
-            {
                 af[b] = drop ? halfx8{} : af[b];
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
                 bf[b] = drop ? halfx8{} : bf[b];
-            }
         }
     };
-    auto multiply = [&](const halfx8 (&af)[2], const halfx8 (&bf)[2]) {
+    auto multiply = [&](const halfx8 (&af)[2], const halfx8 (&bf)[TN]) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < TN; ++j)
                 acc[i][j] =
                     __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
     };
@@ -844,11 +856,12 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
     // First half of a step.  The step's housekeeping sits between its MFMAs, where the matrix
     // pipe is already busy: behind the first one the wait for the copies of step st+1 and the
     // barrier, behind every one a copy of step st+3.
-    auto multiplyAndFeed = [&](const halfx8 (&af)[2], const halfx8 (&bf)[2], uint32_t fillStage) {
+    static_assert(kDCopies == 2 * TN, "one copy behind every MFMA of the first half");
+    auto multiplyAndFeed = [&](const halfx8 (&af)[2], const halfx8 (&bf)[TN], uint32_t fillStage) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < TN; ++j)
             {
                 acc[i][j] =
                     __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
@@ -861,8 +874,8 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
                 }
-                issueOne(fillStage, i * 2 + j);
-                if (i == 1 && j == 1)
+                issueOne(fillStage, i * TN + j);
+                if (i == 1 && j == TN - 1)
                     advance();
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -876,7 +889,7 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
             issueOne(p, n);
         advance();
     }
-    halfx8 af[2][2], bf[2][2];
+    halfx8 af[2][2], bf[2][TN];
     WaitVmem<(kDStages - 2) * kDCopies>();
     __syncthreads();
     loadFragments(af[0], bf[0], lds, 0);
@@ -910,33 +923,33 @@ __global__ __launch_bounds__(256) void GemmF16Dma128(const GemmF16Args args)
 
     // ---- epilogue: lane holds row l%32 of a block, columns 8q + 4*(l/32) + 0..3 -----------
     const bool accumulate = args.overwrite == 0;
-    float4 old[16];
+    float4 old[8 * TN];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
             {
                 const uint32_t r = rowBase + waveM * 64 + i * 32 + l32;
-                const uint32_t c = colBase + waveN * 64 + j * 32 + 8 * q + 4 * khalf;
+                const uint32_t c = colBase + (waveN * TN + j) * 32 + 8 * q + 4 * khalf;
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (accumulate && r < M && c < N)  // N % 8 == 0: whole quads only
                     v = *reinterpret_cast<const float4*>(out + static_cast<size_t>(r) * N + c);
-                old[(i * 2 + j) * 4 + q] = v;
+                old[(i * TN + j) * 4 + q] = v;
             }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
             {
                 const uint32_t r = rowBase + waveM * 64 + i * 32 + l32;
-                const uint32_t c = colBase + waveN * 64 + j * 32 + 8 * q + 4 * khalf;
+                const uint32_t c = colBase + (waveN * TN + j) * 32 + 8 * q + 4 * khalf;
                 if (r < M && c < N)
                 {
-                    float4 v = old[(i * 2 + j) * 4 + q];
+                    float4 v = old[(i * TN + j) * 4 + q];
                     v.x += acc[i][j][4 * q + 0];
                     v.y += acc[i][j][4 * q + 1];
                     v.z += acc[i][j][4 * q + 2];
@@ -1281,17 +1294,34 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
              static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31))
     {
         // whole K steps and 16-byte chunks everywhere: straight-to-LDS 128-tile kernel
-        const dim3 g(grid), b(256);
+        // Eight wavefronts per tile (2 x 4, 64 x 32 each) while there is at most one tile per
+        // compute unit: a second wavefront per SIMD covers the LDS latency and the barrier of
+        // the other (1024^3 13.1 -> 10.8 us, 512 x 512 x 4096 28.8 -> 23.6 us).  With more tiles
+        // two workgroups of four share a compute unit anyway and read fewer fragments per
+        // flop (4096 x 2048 x 2048: 50.9 us against 52.5 us on eight).
+        const bool wide = args.totalTiles <= static_cast<uint32_t>(sph::ComputeUnits());
+        const dim3 g(grid);
+#define SPH_DMA128(TA_, TB_, TAIL_)                                                               \
+    do                                                                                            \
+    {                                                                                             \
+        if (wide)                                                                                 \
+            hipLaunchKernelGGL((GemmF16Dma128<TA_, TB_, TAIL_, 8>), g, dim3(512), 0, stream,      \
+                               args);                                                             \
+        else                                                                                      \
+            hipLaunchKernelGGL((GemmF16Dma128<TA_, TB_, TAIL_, 4>), g, dim3(256), 0, stream,      \
+                               args);                                                             \
+    } while (0)
         if (transA && transB)
-            hipLaunchKernelGGL((GemmF16Dma128<true, true, false>), g, b, 0, stream, args);
+            SPH_DMA128(true, true, false);
         else if (transA)
-            hipLaunchKernelGGL((GemmF16Dma128<true, false, false>), g, b, 0, stream, args);
+            SPH_DMA128(true, false, false);
         else if (transB)
-            hipLaunchKernelGGL((GemmF16Dma128<false, true, false>), g, b, 0, stream, args);
+            SPH_DMA128(false, true, false);
         else if (K % kTK != 0)
-            hipLaunchKernelGGL((GemmF16Dma128<false, false, true>), g, b, 0, stream, args);
+            SPH_DMA128(false, false, true);
         else
-            hipLaunchKernelGGL((GemmF16Dma128<false, false, false>), g, b, 0, stream, args);
+            SPH_DMA128(false, false, false);
+#undef SPH_DMA128
     }
     else
     {

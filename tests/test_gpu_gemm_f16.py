@@ -141,6 +141,25 @@ def test_dma128_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref - C)
 
 
+# the 128-tile kernel runs eight wavefronts per tile up to one tile per compute unit (all shapes
+# above) and four beyond that: more than 256 tiles of 128 x 128 that are not 192 whole 256-tiles,
+# plain, with a K tail, and with transposed operands
+@pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
+                                   capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
+@pytest.mark.parametrize("shape", [(128, 128, 64, 300), (200, 136, 96, 80), (120, 256, 72, 160)])
+def test_dma128_four_wavefront_form_exact_on_integers(dev, shape, flags):
+    M, N, K, batch = shape     # (the K tail with transposed operands runs on the general kernel)
+    h.announce("sph_gemm_f16f32 128-tile, many tiles, integer exactness", shape, "flags", flags)
+    A = synth.small_integers(17, (batch, M, K), span=3).astype(np.float16)
+    B = synth.small_integers(18, (batch, K, N), span=3).astype(np.float16)
+    C = synth.small_integers(19, (batch, M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K, batch=batch)
+    As = np.ascontiguousarray(A.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_A else A
+    Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
+    got = h.gpu_gemm_f16(C, As, Bs, M, N, K, batch=batch, flags=flags)
+    assert np.array_equal(got, ref)
+
+
 @pytest.mark.parametrize("flags", [capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
                                    capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (5, 3, 2, 1), (64, 64, 32, 1), (100, 72, 40, 2),
