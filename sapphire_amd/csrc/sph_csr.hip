@@ -424,8 +424,9 @@ __global__ __launch_bounds__(256) void CsrUnstageKernel(float* __restrict__ V,
     }
 }
 
-// One wavefront per row: the row is cleared, then its entries are written over the zeros, in
-// one pass over the dense matrix.  VEC: rows start on 16-byte boundaries and N % 4 == 0.
+// One wavefront per row, one pass over the dense matrix.  A row of at most 128 entries is
+// merged into the zeros in registers; a longer one is cleared first, then its entries are
+// written over the zeros.  VEC: rows start on 16-byte boundaries and N % 4 == 0.
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void CsrToDenseRowKernel(float* __restrict__ dense,
                                                                 uint32_t ld, uint32_t M,
@@ -442,6 +443,57 @@ __global__ __launch_bounds__(kThreads) void CsrToDenseRowKernel(float* __restric
         float* out = dense + static_cast<size_t>(row) * ld;
         const uint32_t begin = ROW[row];
         const uint32_t end = ROW[row + 1];
+        if (VEC && end - begin <= 128)
+        {
+            // A short row is held in registers (two entries per lane) and merged into the
+            // stream of zeros: every 1 KiB piece of the row is stored once, entries included,
+            // so nothing is written twice and no store waits for another.
+            uint32_t c0 = 0xffffffffu, c1 = 0xffffffffu;
+            float v0 = 0.f, v1 = 0.f;
+            if (begin + lane < end)
+            {
+                c0 = COL[begin + lane];
+                v0 = V[begin + lane];
+            }
+            if (begin + 64 + lane < end)
+            {
+                c1 = COL[begin + 64 + lane];
+                v1 = V[begin + 64 + lane];
+            }
+            // an entry outside the matrix is dropped, never written
+            c0 = c0 < N ? c0 : 0xffffffffu;
+            c1 = c1 < N ? c1 : 0xffffffffu;
+            for (uint32_t base = 0; base < N; base += 256)
+            {
+                float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+                auto place = [&](uint64_t hits, uint32_t cols, float vals) {
+                    while (hits != 0)
+                    {
+                        const uint32_t e = static_cast<uint32_t>(__builtin_ctzll(hits));
+                        hits &= hits - 1;
+                        const uint32_t c = static_cast<uint32_t>(__builtin_amdgcn_readlane(
+                                               static_cast<int>(cols), static_cast<int>(e))) - base;
+                        const float v = __builtin_bit_cast(
+                            float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, vals),
+                                                             static_cast<int>(e)));
+                        const bool mine = lane == (c >> 2);
+                        switch (c & 3u)
+                        {
+                            case 0: q.x = mine ? v : q.x; break;
+                            case 1: q.y = mine ? v : q.y; break;
+                            case 2: q.z = mine ? v : q.z; break;
+                            default: q.w = mine ? v : q.w; break;
+                        }
+                    }
+                };
+                // c - base < 256 in unsigned arithmetic: base <= c < base + 256
+                place(__ballot(c0 - base < 256u && c0 != 0xffffffffu), c0, v0);
+                place(__ballot(c1 - base < 256u && c1 != 0xffffffffu), c1, v1);
+                if (base + lane * 4 < N)
+                    *reinterpret_cast<float4*>(out + base + lane * 4) = q;
+            }
+            continue;
+        }
         if (VEC)
         {
             for (uint32_t c = lane * 4; c < N; c += 256)
