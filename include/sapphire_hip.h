@@ -217,6 +217,20 @@ int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M,
                     uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,
                     int64_t strideA, int64_t strideB, uint32_t flags);
 
+/* sph_gemm_f32_sgd: the weight update of Linear's backward pass in one launch,
+ * out = out - ((A * B) * scale) * rate with every operation rounded on its own
+ * (no fused multiply-add), for one M x N matrix.  It replaces, with the same
+ * result bits, the sequence the reference runs
+ * (Sources/Sapphire/operations/Backward/LinearBackward.cpp:55-76 and
+ * Sources/Sapphire/optimizers/SGD.cpp:22-28): Zeros(dw); Gemm(dw, x^T, dy)
+ * [; Scale(dw, dw, scale)]; Scale(temp, dw, rate); Sub(w, w, temp) -- the
+ * gradient is never stored.  scale = 1 for the weights, 1 / batch for the
+ * bias row (A = ones, M = 1).  flags: SPH_GEMM_TRANS_A / SPH_GEMM_TRANS_B as
+ * in sph_gemm_f32_ex.  K = 0 leaves out as it is. */
+int sph_gemm_f32_sgd(float* out, const float* A, const float* B, uint32_t M,
+                     uint32_t N, uint32_t K, float scale, float rate,
+                     uint32_t flags);
+
 /* The forward pass of a fully connected layer in one launch:
  *   y[b][j] = act((0 + bias[j]) + sum_k x[b][k] * W[k][j])
  * x is batch x inputs, W inputs x outputs, bias has outputs entries, y is

@@ -94,6 +94,7 @@ SIGNATURES = {
     "sph_sgd_step_f32": [_vp, _vp, ctypes.c_float, _sz],
     "sph_gemm_f32": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64],
     "sph_gemm_f32_ex": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _i64, _i64, _i64, _u32],
+    "sph_gemm_f32_sgd": [_vp, _vp, _vp, _u32, _u32, _u32, ctypes.c_float, ctypes.c_float, _u32],
     "sph_linear_forward_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32],
     "sph_gemm_f32_grouped": [ctypes.POINTER(SphGemmEntry), _u32, _vp, _vp, _vp, _u32, _u32, _u32],
     "sph_gemm_f32_grouped_device": [_vp, _u32, _vp, _vp, _vp, _u32, _u32, _u32, _u32],

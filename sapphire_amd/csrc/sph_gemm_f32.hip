@@ -57,6 +57,10 @@ struct GemmF32Args
     uint32_t overwrite;  // out = A*B instead of out += A*B
     uint32_t relu;       // out = max(., 0) applied to the value that is stored
     const float* bias;   // when set: out = (0 + bias[column]) + A*B, out is not read
+    // when sgd is set: out = out - ((A*B) * sgdScale) * sgdRate, every operation rounded on its
+    // own -- the update Scale + Sub apply to a gradient that was stored first
+    uint32_t sgd;
+    float sgdScale, sgdRate;
     int64_t strideOut, strideA, strideB;
 };
 
@@ -194,6 +198,21 @@ __device__ __forceinline__ bool MapTile(const GemmF32Args& args, uint32_t& tm, u
     return true;
 }
 
+// What is stored for an element whose old value (or bias term) is `old` and whose product sum
+// is `sum`.  Contraction is off: a fused multiply-add would round once where the separate
+// Scale and Sub of the optimizer round twice.
+__device__ __forceinline__ float Combine(const GemmF32Args& args, float old, float sum)
+{
+#pragma clang fp contract(off)
+    if (args.sgd != 0)
+    {
+        const float scaled = sum * args.sgdScale;
+        const float step = scaled * args.sgdRate;
+        return old - step;
+    }
+    return old + sum;
+}
+
 // k index (inside a 16-wide step) that lane half `khalf` feeds to MFMA instruction t
 __device__ __forceinline__ constexpr uint32_t KOfPair(uint32_t t, uint32_t khalf)
 {
@@ -205,10 +224,13 @@ __device__ __forceinline__ constexpr uint32_t KOfPair(uint32_t t, uint32_t khalf
 template <int TM, int TN>
 __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* __restrict__ out,
                                           uint32_t rowBase, uint32_t colBase, uint32_t M,
-                                          uint32_t N, uint32_t l32, uint32_t khalf, bool wide,
-                                          bool accumulate, const float* __restrict__ bias = nullptr,
-                                          bool relu = false)
+                                          uint32_t N, uint32_t l32, uint32_t khalf,
+                                          const GemmF32Args& args)
 {
+    const bool wide = args.outVec != 0;
+    const bool accumulate = args.overwrite == 0;
+    const float* __restrict__ bias = args.bias;
+    const bool relu = args.relu != 0;
     // ---- out += acc ---------------------------------------------------------
     // With the operands swapped, register v of lane l holds row l%32 and column
     // 8*(v/4) + 4*(l/32) + v%4 of its 32x32 block: registers 4q..4q+3 are 4
@@ -261,10 +283,10 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
                 if (r < M && c < N)
                 {
                     float4 v = old[(i * TN + j) * 4 + q];
-                    v.x += acc[i][j][4 * q + 0];
-                    v.y += acc[i][j][4 * q + 1];
-                    v.z += acc[i][j][4 * q + 2];
-                    v.w += acc[i][j][4 * q + 3];
+                    v.x = Combine(args, v.x, acc[i][j][4 * q + 0]);
+                    v.y = Combine(args, v.y, acc[i][j][4 * q + 1]);
+                    v.z = Combine(args, v.z, acc[i][j][4 * q + 2]);
+                    v.w = Combine(args, v.w, acc[i][j][4 * q + 3]);
                     if (relu)
                     {
                         v.x = v.x > 0 ? v.x : 0;
@@ -428,8 +450,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
         __syncthreads();
     }
 
-    StoreTile<TM, TN>(acc, out, rowBase + waveM * WM, colBase + waveN * WN, M, N, l32, khalf,
-                      args.outVec != 0, args.overwrite == 0, args.bias, args.relu != 0);
+    StoreTile<TM, TN>(acc, out, rowBase + waveM * WM, colBase + waveN * WN, M, N, l32, khalf, args);
 }
 
 // ---------------------------------------------------------------------------
@@ -819,7 +840,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
                         // 0 + bias: what the K = 1 product ones x bias leaves in a zero-filled out
                         if (hasBias)
                             v[e] = 0.f + v[e];
-                        v[e] += acc[i][j][4 * q + e];
+                        v[e] = Combine(args, v[e], acc[i][j][4 * q + e]);
                         if (relu)
                             v[e] = v[e] > 0 ? v[e] : 0;
                     }
@@ -970,8 +991,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 
     if constexpr (!WALK)
         StoreTile<TM, TN>(acc, cur.out, cur.rowBase + waveM * WM, cur.colBase + waveN * WN, M, N,
-                          l32, khalf, args.outVec != 0, args.overwrite == 0, args.bias,
-                          args.relu != 0);
+                          l32, khalf, args);
 }
 
 // ---------------------------------------------------------------------------
@@ -1169,9 +1189,10 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         if (c >= N)
             continue;
         float* p = out + static_cast<size_t>(row) * N + c;
-        if (args.bias != nullptr || args.relu)
+        if (args.bias != nullptr || args.relu || args.sgd)
         {
-            // fused Linear epilogue: (0 + bias) + product, optional ReLU, out not read
+            // fused epilogues: (0 + bias) + product with an optional ReLU (out not read), or the
+            // optimizer step
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 if (c + e < N)
@@ -1181,7 +1202,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
                         old = 0.f + args.bias[c + e];
                     else if (!args.overwrite)
                         old = p[e];
-                    float v = old + acc[4 * q + e];
+                    float v = Combine(args, old, acc[4 * q + e]);
                     if (args.relu)
                         v = v > 0 ? v : 0;
                     p[e] = v;
@@ -1272,7 +1293,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void GemvRowKernel(const GemmF32Ar
         old = 0.f + args.bias[col];
     else if (!args.overwrite)
         old = out[col];
-    float v = old + sum;
+    float v = Combine(args, old, sum);
     if (args.relu)
         v = v > 0 ? v : 0;
     out[col] = v;
@@ -1591,6 +1612,34 @@ int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M, uint
     const bool stridesAligned = (strideA % 4 == 0) && (strideB % 4 == 0);
     return Launch(args, batch, stridesAligned, strideOut % 4 == 0 || batch == 1,
                   (flags & SPH_GEMM_TRANS_A) != 0, (flags & SPH_GEMM_TRANS_B) != 0, stream);
+}
+
+int sph_gemm_f32_sgd(float* out, const float* A, const float* B, uint32_t M, uint32_t N,
+                     uint32_t K, float scale, float rate, uint32_t flags)
+{
+    SPH_REQUIRE(M != 0 && N != 0, "M and N must be non-zero");
+    SPH_REQUIRE((flags & ~(SPH_GEMM_TRANS_A | SPH_GEMM_TRANS_B)) == 0, "unknown flag");
+    SPH_REQUIRE(out != nullptr, "null pointer");
+    SPH_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "null pointer");
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    if (K == 0)
+        return SPH_OK;  // an empty gradient: out - 0 leaves every value as it is
+    GemmF32Args args{};
+    args.out = out;
+    args.A = A;
+    args.B = B;
+    args.entries = nullptr;
+    args.M = M;
+    args.N = N;
+    args.K = K;
+    args.overwrite = 0u;  // the old value of out takes part
+    args.sgd = 1u;
+    args.sgdScale = scale;
+    args.sgdRate = rate;
+    return Launch(args, 1, true, true, (flags & SPH_GEMM_TRANS_A) != 0,
+                  (flags & SPH_GEMM_TRANS_B) != 0, stream);
 }
 
 int sph_linear_forward_f32(float* y, const float* x, const float* W, const float* bias,
