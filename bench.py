@@ -212,12 +212,14 @@ def bench_mlp(capi, synth, steps, warmup, fused=False, graph=False):
     return event_ms, flops
 
 
-def bench_mlp_backward(capi, synth, steps, warmup, direct, graph=False):
+def bench_mlp_backward(capi, synth, steps, warmup, direct, graph=False, fused_update=False):
     """Backward pass + SGD update of configuration 4's three Linear layers through the C ABI
     (the call sequence of LinearBackProp::m_runBackProp per layer, ReLUBackward between
     layers).  direct=False materialises the transposes, zero-fills and uses Scale + Sub like
     the reference; direct=True uses the transposed-read / overwrite flags and the one-pass SGD
-    step.  Parameters drift over the steps; only time is taken here."""
+    step; fused_update (with direct) ends the weight and bias gradient products in the update
+    itself (sph_gemm_f32_sgd), so neither gradient is stored.  Parameters drift over the steps;
+    only time is taken here."""
     d = synth.config4()
     batch = d["x"].shape[0]
     sizes = [d["x"].shape[1]] + [w.shape[1] for w in d["W"]]
@@ -254,6 +256,12 @@ def bench_mlp_backward(capi, synth, steps, warmup, direct, graph=False):
         if direct:
             capi.call("sph_gemm_f32_ex", dx.ptr, dy.ptr, W[l].ptr, batch, n_in, n_out, 1,
                       batch * n_in, batch * n_out, n_in * n_out, TB)
+            if fused_update:
+                capi.call("sph_gemm_f32_sgd", W[l].ptr, x.ptr, dy.ptr, n_in, n_out, batch, 1.0, lr,
+                          TA)
+                capi.call("sph_gemm_f32_sgd", b[l].ptr, ones.ptr, dy.ptr, 1, n_out, batch,
+                          1.0 / batch, lr, 0)
+                return
             capi.call("sph_gemm_f32_ex", dw.ptr, x.ptr, dy.ptr, n_in, n_out, batch, 1,
                       n_in * n_out, n_in * batch, batch * n_out, TA | OV)
         else:
@@ -686,12 +694,17 @@ def main():
         others = {}
         ms_ref, fl = bench_mlp_backward(capi, synth, 100, 10, direct=False)
         ms_dir, _ = bench_mlp_backward(capi, synth, 100, 10, direct=True)
+        ms_fused, _ = bench_mlp_backward(capi, synth, 100, 10, direct=True, fused_update=True)
         others["config4_mlp_backward_sgd"] = {
             "reference_sequence_ms": ms_ref, "direct_ms": ms_dir,
             "direct_tflops": fl / (ms_dir * 1e-3) / 1e12,
+            "direct_update_in_gemm_ms": ms_fused,
+            "direct_update_in_gemm_tflops": fl / (ms_fused * 1e-3) / 1e12,
             "note": "reference sequence: Transpose + Gemm, Zeros, Scale + Sub; direct: "
-                    "transposed-read / overwrite GEMM flags and the one-pass SGD step "
-                    "(bit-identical results)"}
+                    "transposed-read / overwrite GEMM flags and the one-pass SGD step; "
+                    "update in gemm: the weight and bias gradient products end in the SGD "
+                    "step (sph_gemm_f32_sgd), no gradient is stored (bit-identical results "
+                    "in all three)"}
         ms_f, _ = bench_mlp(capi, synth, 100, 10, fused=True, graph=True)
         ms_b, _ = bench_mlp_backward(capi, synth, 100, 10, direct=True, graph=True)
         others["config4_replayed_as_graphs"] = {

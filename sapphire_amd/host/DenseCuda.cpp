@@ -86,6 +86,16 @@ void GemmTransposed(float* out, const float* A, const float* B, unsigned int M, 
           "GemmTransposed");
 }
 
+void GemmSgd(float* out, const float* A, const float* B, unsigned int M, unsigned int N,
+             unsigned int K, bool transposeA, bool transposeB, float scale, float rate,
+             int deviceId)
+{
+    Compute::Cuda::CudaSetDevice(deviceId);
+    const std::uint32_t flags =
+        (transposeA ? SPH_GEMM_TRANS_A : 0u) | (transposeB ? SPH_GEMM_TRANS_B : 0u);
+    Check(sph_gemm_f32_sgd(out, A, B, M, N, K, scale, rate, flags), "GemmSgd");
+}
+
 void LinearForward(float* y, const float* x, const float* W, const float* bias,
                    unsigned int batch, unsigned int inputs, unsigned int outputs, bool relu,
                    int deviceId)

@@ -81,6 +81,26 @@ void RunDirect(TensorData& dx, TensorData& weight, TensorData& bias, const Tenso
                                          weight.CudaRawPtr(), rows, inputs, outputs, 1, false,
                                          true, false, deviceId);
 
+    // dB [1, out] = ones [1, batch] * dy, the ones that Linear's backward pass fills
+    TensorData transposedOnes(Shape({ 1, static_cast<int>(batchSize) }), dy.GetType(),
+                              dy.GetCudaDevice());
+    transposedOnes.SetMode(bias.Mode());
+    Compute::Initialize::Ones(transposedOnes);
+
+    if (optimizer.Fused())
+    {
+        // neither gradient is stored: the products end in the optimizer's step
+        // weight -= ((x^T * dy) * 1) * lr;  bias -= ((ones * dy) * (1 / batch)) * lr
+        Compute::Dense::Cuda::GemmSgd(weight.CudaMutableRawPtr(), x.CudaRawPtr(), dy.CudaRawPtr(),
+                                      inputs, outputs, rows, true, false, 1.0f,
+                                      optimizer.LearningRate(), deviceId);
+        Compute::Dense::Cuda::GemmSgd(bias.CudaMutableRawPtr(), transposedOnes.CudaRawPtr(),
+                                      dy.CudaRawPtr(), 1, outputs, batchSize, false, false,
+                                      1.0f / static_cast<float>(batchSize),
+                                      optimizer.LearningRate(), deviceId);
+        return;
+    }
+
     // dw [in, out] = (x [rows, in])^T * dy [rows, out]
     TensorData dw(weight.GetShape(), weight.GetType(), weight.GetCudaDevice());
     dw.SetMode(weight.Mode());
@@ -88,13 +108,8 @@ void RunDirect(TensorData& dx, TensorData& weight, TensorData& bias, const Tenso
                                          inputs, outputs, rows, 1, true, false, true, deviceId);
     optimizer(weight, dw);
 
-    // dB [1, out] = ones [1, batch] * dy
-    TensorData transposedOnes(Shape({ 1, static_cast<int>(batchSize) }), dy.GetType(),
-                              dy.GetCudaDevice());
     TensorData dB(bias.GetShape(), bias.GetType(), bias.GetCudaDevice());
     dB.SetMode(bias.Mode());
-    transposedOnes.SetMode(bias.Mode());
-    Compute::Initialize::Ones(transposedOnes);
     Compute::Dense::Cuda::GemmTransposed(dB.CudaMutableRawPtr(), transposedOnes.CudaRawPtr(),
                                          dy.CudaRawPtr(), 1, outputs, batchSize, 1, false, false,
                                          true, deviceId);

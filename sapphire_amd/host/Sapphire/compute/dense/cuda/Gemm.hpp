@@ -45,6 +45,13 @@ void GemmTransposed(float* out, const float* A, const float* B, unsigned int M, 
                     unsigned int K, unsigned int batchSize, bool transposeA, bool transposeB,
                     bool overwrite, int deviceId);
 
+//! out -= ((op(A) * op(B)) * scale) * rate for one M x N matrix, every operation rounded on its
+//! own: the gradient product, its optional scaling and the SGD step (Scale + Sub) in one launch,
+//! with the result bits of the separate calls.
+void GemmSgd(float* out, const float* A, const float* B, unsigned int M, unsigned int N,
+             unsigned int K, bool transposeA, bool transposeB, float scale, float rate,
+             int deviceId);
+
 //! y = act((0 + bias) + x * W) in one launch: the two GEMMs of Linear's forward pass on a zero
 //! y, optionally followed by ReLU, with the same result bits.
 void LinearForward(float* y, const float* x, const float* W, const float* bias,

@@ -26,6 +26,8 @@ public:
                     const std::string& name = std::string()) const;
 
     [[nodiscard]] float LearningRate() const { return m_learningRate; }
+    //! One-pass device forms of the update may stand in for Scale + Sub (same result bits).
+    [[nodiscard]] bool Fused() const { return m_fused; }
 
 private:
     float m_learningRate;
