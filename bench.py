@@ -400,7 +400,7 @@ def bench_sparse_linear(capi, synth, steps, warmup, batch=256):
     def product():
         capi.call("sph_spmm_csr_f32", yT.ptr, dV.ptr, dCol.ptr, dRow.ptr, outs, ins, batch, xT.ptr, 1)
 
-    def forward():
+    def forward_unfused():
         capi.call("sph_transpose_f32", xT.ptr, x.ptr, batch, ins, 1, 0)
         capi.call("sph_fill_f32", ones.ptr, 1.0, batch)
         capi.call("sph_fill_f32", yT.ptr, 0.0, outs * batch)
@@ -409,11 +409,18 @@ def bench_sparse_linear(capi, synth, steps, warmup, batch=256):
         product()
         capi.call("sph_transpose_f32", y.ptr, yT.ptr, outs, batch, 1, 0)
 
+    def forward():
+        capi.call("sph_transpose_f32", xT.ptr, x.ptr, batch, ins, 1, 0)
+        capi.call("sph_spmm_csr_bias_f32", yT.ptr, dV.ptr, dCol.ptr, dRow.ptr, outs, ins, batch,
+                  xT.ptr, bias.ptr)
+        capi.call("sph_transpose_f32", y.ptr, yT.ptr, outs, batch, 1, 0)
+
     ms, _ = timed_launches(capi, forward, steps, warmup)
+    ms_unfused, _ = timed_launches(capi, forward_unfused, steps, warmup)
     ms_product, _ = timed_launches(capi, product, steps, warmup)
     for b in (x, bias, dV, dCol, dRow, xT, yT, y, ones):
         b.release()
-    return ms, ms_product, int(d["V"].size)
+    return ms, ms_product, int(d["V"].size), ms_unfused
 
 
 def bench_allocation(capi, nbytes=64 << 20, rounds=200):
@@ -744,13 +751,17 @@ def main():
             "gproducts_per_s": 2 * products / (ms * 1e-3) / 1e9,
             "algorithmic_gbs": nbytes / (ms * 1e-3) / 1e9,
             "note": "16 strips wide: rows with few products go through the hash-table kernel"}
-        ms, ms_product, nnz_w = bench_sparse_linear(capi, synth, 50, 5)
+        ms, ms_product, nnz_w, ms_unfused = bench_sparse_linear(capi, synth, 50, 5)
         others["sparse_linear_forward_8192x8192_batch256"] = {
-            "forward_ms": ms, "csr_x_dense_ms": ms_product, "launches_per_forward": 6,
+            "forward_ms": ms, "csr_x_dense_ms": ms_product, "launches_per_forward": 3,
             "weights_kept": nnz_w,
             "gflops": 2.0 * nnz_w * 256 / (ms * 1e-3) / 1e9,
-            "note": "the NN::SparseLinearForward sequence through the C ABI: transpose x, ones, "
-                    "zero fill, bias x ones (K = 1 GEMM), CSR x dense (accumulating), transpose y"}
+            "note": "the NN::SparseLinearForward sequence through the C ABI: transpose x, CSR x "
+                    "dense with the bias of an output row as the value the product is added to "
+                    "(sph_spmm_csr_bias_f32), transpose y",
+            "six_launch_form_ms": ms_unfused,
+            "six_launch_form_note": "transpose x, ones, zero fill, bias x ones (K = 1 GEMM), CSR "
+                                    "x dense (accumulating), transpose y: same result bits"}
         others["one_pass_kernels_4096x4096"] = bench_elementwise(capi, 50, 5)
         others["device_block_64MiB"] = bench_allocation(capi)
         result["others"] = others

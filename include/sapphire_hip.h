@@ -311,6 +311,15 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M,
 int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL,
                      const uint32_t* ROW, uint32_t M, uint32_t Kdim, uint32_t N,
                      const float* B, int accumulate);
+/* sph_spmm_csr_bias_f32: out[i][j] = (0 + rowBias[i]) + sum_p V[p] * B[COL[p]][j],
+ * out is not read: the bits that sph_spmm_csr_f32 with accumulate leaves in an
+ * out filled by sph_fill_f32(0) and the K = 1 product rowBias x ones -- the
+ * feature-major form of Linear's bias step
+ * (Sources/Sapphire/operations/Forward/Linear.cpp:113-136) for a sparse weight,
+ * without the fill, the ones and the K = 1 launch. */
+int sph_spmm_csr_bias_f32(float* out, const float* V, const uint32_t* COL,
+                          const uint32_t* ROW, uint32_t M, uint32_t Kdim,
+                          uint32_t N, const float* B, const float* rowBias);
 
 /* ---- dense <-> CSR ------------------------------------------------------- */
 

@@ -112,6 +112,7 @@ SIGNATURES = {
     "sph_spgemm_f32": [_vp, _vp, _vp, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,
                        ctypes.POINTER(ctypes.c_uint32)],
     "sph_spmm_csr_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, ctypes.c_int],
+    "sph_spmm_csr_bias_f32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, _vp],
 }
 
 

@@ -48,6 +48,9 @@ struct SpmmArgs
     const float* B;
     uint32_t M, N;
     int accumulate;
+    // when set: out[row][*] = (0 + rowBias[row]) + sum, out is not read -- what accumulating into
+    // an out that the K = 1 product bias x ones has filled gives
+    const float* rowBias;
 };
 
 __device__ __forceinline__ float Bcast(float v, int srcLane)
@@ -186,7 +189,15 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
     if (active)
     {
         float4* dst = reinterpret_cast<float4*>(args.out + static_cast<size_t>(row) * N + col);
-        if (args.accumulate)
+        if (args.rowBias != nullptr)
+        {
+            const float old = 0.f + args.rowBias[row];
+            sum.x = old + sum.x;
+            sum.y = old + sum.y;
+            sum.z = old + sum.z;
+            sum.w = old + sum.w;
+        }
+        else if (args.accumulate)
         {
             const float4 old = *dst;
             sum.x = old.x + sum.x;
@@ -237,16 +248,18 @@ __global__ __launch_bounds__(kThreads) void SpmmRowScalar(const SpmmArgs args)
         if (active)
         {
             float* dst = args.out + static_cast<size_t>(row) * N + n;
-            *dst = args.accumulate ? (*dst + sum) : sum;
+            if (args.rowBias != nullptr)
+                *dst = (0.f + args.rowBias[row]) + sum;
+            else
+                *dst = args.accumulate ? (*dst + sum) : sum;
         }
     }
 }
 }  // namespace
 
-extern "C" {
-
-int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW,
-                     uint32_t M, uint32_t Kdim, uint32_t N, const float* B, int accumulate)
+static int LaunchSpmm(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW,
+                      uint32_t M, uint32_t Kdim, uint32_t N, const float* B, int accumulate,
+                      const float* rowBias)
 {
     // column indices are trusted to lie below Kdim, as in the dense leaf
     if (M == 0 || N == 0)
@@ -265,6 +278,7 @@ int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL, const uint
     args.M = M;
     args.N = N;
     args.accumulate = accumulate ? 1 : 0;
+    args.rowBias = rowBias;
 
     const uint32_t blocks = (M + kWavesPerBlock - 1) / kWavesPerBlock;
     // the slab kernel forms 32-bit byte offsets into B with a 24-bit multiply; larger operands
@@ -300,6 +314,22 @@ int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL, const uint
         hipLaunchKernelGGL(SpmmRowScalar, dim3(blocks), dim3(kThreads), 0, stream, args);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
+}
+
+extern "C" {
+
+int sph_spmm_csr_f32(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW,
+                     uint32_t M, uint32_t Kdim, uint32_t N, const float* B, int accumulate)
+{
+    return LaunchSpmm(out, V, COL, ROW, M, Kdim, N, B, accumulate, nullptr);
+}
+
+int sph_spmm_csr_bias_f32(float* out, const float* V, const uint32_t* COL, const uint32_t* ROW,
+                          uint32_t M, uint32_t Kdim, uint32_t N, const float* B,
+                          const float* rowBias)
+{
+    SPH_REQUIRE(M == 0 || N == 0 || rowBias != nullptr, "rowBias is null");
+    return LaunchSpmm(out, V, COL, ROW, M, Kdim, N, B, 0, rowBias);
 }
 
 }  // extern "C"

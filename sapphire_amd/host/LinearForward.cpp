@@ -78,24 +78,21 @@ void SparseLinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData
         throw std::invalid_argument("NN::Linear - sparse weight shape mismatch");
     const CudaDevice device = x.GetCudaDevice();
 
-    TensorUtil::TensorData x2 = x, y2 = y, biasColumn = bias;
+    TensorUtil::TensorData x2 = x, y2 = y;
     Util::ChangeTensorDataDimension(2, x2);
     Util::ChangeTensorDataDimension(2, y2);
-    biasColumn.Reshape(Shape({ outputs, 1 }));
 
     TensorUtil::TensorData xT(Shape({ inputs, batchSize }), Type::Dense, device);
     TensorUtil::TensorData yT(Shape({ outputs, batchSize }), Type::Dense, device);
-    TensorUtil::TensorData ones(Shape({ 1, batchSize }), Type::Dense, device);
     xT.SetMode(ComputeMode::Cuda);
     yT.SetMode(ComputeMode::Cuda);
-    ones.SetMode(ComputeMode::Cuda);
 
+    // yT = bias x ones + W^T_csr * xT in one launch: the bias of an output row is the value the
+    // product is added to, which is what Zeros(yT); Gemm(yT, bias, ones); accumulate leaves
     Compute::Transpose(xT, x2);
-    Compute::Initialize::Ones(ones);
-    Compute::Initialize::Zeros(yT);  // a pooled buffer may hold an earlier result
-    Compute::Gemm(yT, biasColumn, ones);
-    Compute::Sparse::Cuda::Gemm(yT.CudaMutableRawPtr(), &weightTransposed, xT.CudaRawPtr(),
-                                static_cast<unsigned int>(batchSize), true, device.GetID());
+    Compute::Sparse::Cuda::GemmBias(yT.CudaMutableRawPtr(), &weightTransposed, xT.CudaRawPtr(),
+                                    static_cast<unsigned int>(batchSize), bias.CudaRawPtr(),
+                                    device.GetID());
     Compute::Transpose(y2, yT);
 }
 }  // namespace Sapphire::NN

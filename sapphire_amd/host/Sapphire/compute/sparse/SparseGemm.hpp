@@ -23,6 +23,12 @@ namespace Sapphire::Compute::Sparse::Cuda
 void Gemm(float* out, const SparseMatrix* a, const float* B, unsigned int denseCols,
           bool accumulate, int deviceId);
 
+//! out[a->M x denseCols] = (0 + rowBias[i]) + a * B: the product accumulated into an out that
+//! holds the bias of row i in every column, without reading out (the feature-major bias step of
+//! a sparse Linear layer in the same launch).  rowBias has a->M entries in device memory.
+void GemmBias(float* out, const SparseMatrix* a, const float* B, unsigned int denseCols,
+              const float* rowBias, int deviceId);
+
 //! Builds a record with device arrays from host CSR arrays (rowOffsets has rows + 1
 //! entries, columns ascending inside a row); memory comes from ResourceManager's
 //! preserved device pool.  Release with FreeSparseMatrix.

@@ -25,6 +25,18 @@ void Gemm(float* out, const SparseMatrix* a, const float* B, unsigned int denseC
                                  sph_last_error());
 }
 
+void GemmBias(float* out, const SparseMatrix* a, const float* B, unsigned int denseCols,
+              const float* rowBias, int deviceId)
+{
+    if (a == nullptr)
+        throw std::invalid_argument("Sparse::Cuda::GemmBias - sparse operand is null");
+    Compute::Cuda::CudaSetDevice(deviceId);
+    if (sph_spmm_csr_bias_f32(out, a->V, a->COL, a->ROW, a->M, a->N, denseCols, B, rowBias) !=
+        SPH_OK)
+        throw std::runtime_error(std::string("Sparse::Cuda::GemmBias failed with ") +
+                                 sph_last_error());
+}
+
 SparseMatrix CreateSparseMatrix(const std::vector<float>& values,
                                 const std::vector<uint32_t>& columns,
                                 const std::vector<uint32_t>& rowOffsets, uint32_t rows,

@@ -79,6 +79,27 @@ def gpu_spmm(C, V, COL, ROW, M, Kdim, N, B, accumulate, canary=0):
     return back[canary:canary + C.size].reshape(C.shape)
 
 
+def gpu_spmm_bias(junk, V, COL, ROW, M, Kdim, N, B, row_bias, canary=0):
+    """Runs sph_spmm_csr_bias_f32 over an out that holds `junk`, with guard floats around it."""
+    guard = np.full(canary, np.float32(-12345.5), dtype=np.float32)
+    padded = np.concatenate([guard, junk.ravel(), guard]).astype(np.float32)
+    dC = capi.DeviceBuffer.from_array(padded)
+    dV = capi.DeviceBuffer.from_array(V if V.size else np.zeros(1, np.float32))
+    dCol = capi.DeviceBuffer.from_array(COL if COL.size else np.zeros(1, np.uint32))
+    dRow = capi.DeviceBuffer.from_array(ROW)
+    dB = capi.DeviceBuffer.from_array(B)
+    dBias = capi.DeviceBuffer.from_array(row_bias)
+    capi.call("sph_spmm_csr_bias_f32", dC.at(4 * canary), dV.ptr, dCol.ptr, dRow.ptr, M, Kdim, N,
+              dB.ptr, dBias.ptr)
+    back = dC.download(np.float32, padded.shape)
+    for d in (dC, dV, dCol, dRow, dB, dBias):
+        d.release()
+    if canary:
+        assert np.array_equal(back[:canary], guard), "write before the start of out"
+        assert np.array_equal(back[-canary:], guard), "write past the end of out"
+    return back[canary:canary + junk.size].reshape(junk.shape)
+
+
 def gpu_gemm_f32_ex(C, A, B, M, N, K, flags, batch=1, stride_out=None, stride_a=None,
                     stride_b=None):
     """sph_gemm_f32_ex on numpy operands exactly as stored (A is K x M with SPH_GEMM_TRANS_A,

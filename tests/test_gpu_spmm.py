@@ -64,6 +64,26 @@ def test_equals_dense_product_of_densified_matrix(dev):
     assert np.array_equal(_bits(got), _bits(ref))
 
 
+@pytest.mark.parametrize("N", [1, 3, 64, 100, 256])
+def test_row_bias_form_equals_fill_bias_product_and_accumulate(dev, N):
+    """sph_spmm_csr_bias_f32 against the CPU checker run the long way: out = 0, out += bias x
+    ones (the K = 1 product of Linear's bias step, feature-major), out += A * B.  Rows without
+    entries hold 0 + bias, a bias of -0 becomes +0, out's old contents (NaN) are not read."""
+    h.announce("sph_spmm_csr_bias_f32 N =", N)
+    M, K = 300, 777
+    v, col, row = synth.csr_matrix(950 + N, M, K, 20.0, forced={5: 0, 6: 700, 7: ("cols", [776])})
+    B = synth.uniform(951 + N, (K, N))
+    bias = synth.uniform(952 + N, (M,))
+    bias[5] = -0.0
+    start = po.naive_gemm(np.zeros((M, N), np.float32), bias.reshape(M, 1).copy(),
+                          np.ones((1, N), np.float32), M, N, 1)
+    ref = po.spmm_csr(start, v, col, row, M, N, B)
+    got = h.gpu_spmm_bias(np.full((M, N), np.float32(np.nan)), v, col, row, M, K, N, B, bias,
+                          canary=512)
+    assert np.array_equal(_bits(got), _bits(ref))
+    assert np.array_equal(_bits(got[5]), _bits(np.zeros(N, np.float32)))     # 0 + (-0) = +0
+
+
 def test_all_rows_empty(dev):
     M, K, N = 10, 10, 8
     row = np.zeros(M + 1, np.uint32)
