@@ -3,9 +3,9 @@
 // Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50): half
 // inputs, fp32 accumulation, row-major operands, result added into out.
 //
-// Three kernels:
+// Three kernels (and one for the odd columns, see below):
 //
-//   GemmF16Tile256  K a multiple of 32, N of 8, 16-byte aligned rows, at least three
+//   GemmF16Tile256  K a multiple of 32, N of 8, 16-byte aligned rows of A, at least three
 //     quarters as many 256 x 256 tiles as compute units and at least three quarters of
 //     the tiled area inside the matrix (a variant with clamped copies and a guarded
 //     epilogue serves M, N that are not multiples of 256).  One workgroup of 8 wavefronts
@@ -26,7 +26,7 @@
 //     the 32 workgroups that land on one XCD (ids congruent mod 8) cover a compact
 //     8 x 4 block of tiles and share their A and B panels through that XCD's L2.
 //
-//   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned, any M: the
+//   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned rows of A, any M: the
 //     same ingredients on 128 x 128 tiles with 4 wavefronts (v_mfma_f32_32x32x16_f16), for
 //     shapes with too few 256-tiles to fill the chip.
 //
@@ -34,8 +34,15 @@
 //     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
 //     widest that K, N, the strides and the bases allow), padded LDS rows.
 //
-// K = 32 q + r with r in {8, 16, 24} goes to the first two kernels for the first 32 q
-// columns of A and to the general kernel for the rest (two launches).
+// K = 32 q + r with r in {8, 16, 24} (operands stored plainly) stays on the first two kernels:
+// a last step over [K - 32, K) in which the lanes holding values of k that were multiplied
+// already feed zeros.
+//
+// N = 8 q + r, r != 0: the first 8 q columns go to the first two kernels when they would take
+// that shape (the copies into LDS need no alignment, so rows of B and of out may start
+// anywhere; only a copy's 8 columns have to lie inside the row) and the last r columns to
+// GemmF16Cols, a stream over A with the fragments loaded straight into registers (to the
+// general kernel when A is stored K x M).
 #include "sph_internal.h"
 
 #include <type_traits>
@@ -57,6 +64,9 @@ struct GemmF16Args
     const _Float16* B;
     uint32_t M, N, K;
     uint32_t lda;  // halves between consecutive rows of A (K unless a launch covers part of K)
+    uint32_t ldb;  // halves between consecutive k-rows of a B stored K x N (N unless a launch
+                   // covers some of the columns)
+    uint32_t ldc;  // floats between consecutive rows of out (likewise)
     uint32_t tilesM, tilesN;
     uint32_t totalTiles;  // tilesM * tilesN * batch
     int64_t strideOut, strideA, strideB;
@@ -104,15 +114,28 @@ __device__ __forceinline__ uint32_t LdsAddress(const void* p)
 // it should neither displace the A and B panels in the L2 nor stay there dirty until the end of
 // the kernel.
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+// Four floats that need only be 4-byte aligned: rows of out start anywhere when the row pitch is
+// not a multiple of 4 floats, and a 16-byte vector memory access only asks for dword alignment.
+typedef floatx4 floatx4a4 __attribute__((aligned(4)));
 __device__ __forceinline__ float4 NtLoad4(const float* p)
 {
-    const floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(p));
+    const floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4a4*>(p));
     return make_float4(v[0], v[1], v[2], v[3]);
 }
 __device__ __forceinline__ void NtStore4(float* p, float4 v)
 {
     const floatx4 w = { v.x, v.y, v.z, v.w };
-    __builtin_nontemporal_store(w, reinterpret_cast<floatx4*>(p));
+    __builtin_nontemporal_store(w, reinterpret_cast<floatx4a4*>(p));
+}
+__device__ __forceinline__ float4 Load4(const float* p)
+{
+    const floatx4 v = *reinterpret_cast<const floatx4a4*>(p);
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void Store4(float* p, float4 v)
+{
+    const floatx4 w = { v.x, v.y, v.z, v.w };
+    *reinterpret_cast<floatx4a4*>(p) = w;
 }
 
 __device__ __forceinline__ halfx8 Join(halfx4 lo, halfx4 hi)
@@ -246,13 +269,14 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     // fragment read described above, a k-major one the "B stage" layout and the transposing
     // read, whichever matrix it is, so the MFMAs and their order do not depend on the flags.
     const uint32_t pitchA = TA ? args.M : args.lda;  // halves between rows of A as stored
-    const uint32_t pitchB = TB ? K : N;
+    const uint32_t pitchB = TB ? K : args.ldb;
+    const uint32_t ldc = args.ldc;
     const _Float16* __restrict__ A = args.A + args.strideA * static_cast<int64_t>(unit) +
                                      static_cast<size_t>(tm) * kT * (TA ? 1u : pitchA);
     const _Float16* __restrict__ B = args.B + args.strideB * static_cast<int64_t>(unit) +
                                      static_cast<size_t>(tn) * kT * (TB ? pitchB : 1u);
     float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit) +
-                              static_cast<size_t>(tm) * kT * N + static_cast<size_t>(tn) * kT;
+                              static_cast<size_t>(tm) * kT * ldc + static_cast<size_t>(tn) * kT;
 
     // ---- global -> LDS copy plan --------------------------------------------
     // A copy instruction moves 1 KiB per wavefront.  Wavefront w fills the WAVE_LDS bytes
@@ -476,8 +500,8 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
         // instruction offset 64*j (added to both addresses) selects the block, so M0 takes it
         // off again.
         const uint32_t mail = LdsAddress(&CMail[0]) + waveU * 4096;
-        const uint32_t cLane0 = ((waveM * 128 + l16) * N + waveN * 64 + 4 * g) * 4;
-        const uint32_t cRowStep = 16 * N * 4;
+        const uint32_t cLane0 = ((waveM * 128 + l16) * ldc + waveN * 64 + 4 * g) * 4;
+        const uint32_t cRowStep = 16 * ldc * 4;
         auto issueC = [&](auto bC) {
             constexpr int i = decltype(bC)::value;
             const uint32_t laneOff = cLane0 + i * cRowStep;
@@ -585,8 +609,8 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
         float* stage = reinterpret_cast<float*>(&Lds[0][0][0]) + wave * (64 * 64);
         const uint32_t rdRow = lane >> 4;        // + 4*t
         const uint32_t rdChunk = lane & 15;
-        float* outBlock = out + static_cast<size_t>(waveM * 128 + rdRow) * N + waveN * 64 + rdChunk * 4;
-        const size_t rowStep = static_cast<size_t>(4) * N;
+        float* outBlock = out + static_cast<size_t>(waveM * 128 + rdRow) * ldc + waveN * 64 + rdChunk * 4;
+        const size_t rowStep = static_cast<size_t>(4) * ldc;
         const uint32_t rowFirst = waveM * 128 + rdRow;
         const bool colExists = !RAGGED || waveN * 64 + rdChunk * 4 < colsLeft;
         auto exists = [&](int half, int t) {
@@ -630,7 +654,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
                     v.w += old[t].w;
                 }
                 if (exists(half, t))
-                    *reinterpret_cast<float4*>(outBlock + (half * 16 + t) * rowStep) = v;
+                    Store4(outBlock + (half * 16 + t) * rowStep, v);
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         };
@@ -729,18 +753,18 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
     {
         const uint32_t j = wave + WAVES * i;
         aLane[i] = TA ? laneKMajor(j, rowBase, M, M) : laneKContig(j, rowBase, M, args.lda);
-        bLane[i] = TB ? laneKContig(j, colBase, N, K) : laneKMajor(j, colBase, N, N);
+        bLane[i] = TB ? laneKContig(j, colBase, N, K) : laneKMajor(j, colBase, N, args.ldb);
         aDst[i] = j * 1024;
         bDst[i] = kBytesA + j * 1024;
     }
     const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * M * 2 : kTK * 2;
-    const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * N * 2;
+    const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * args.ldb * 2;
     const uint32_t ldsBase = LdsAddress(lds);
     const uint32_t steps = TAIL ? K / kTK + 1 : K / kTK;
     // the last window starts K % 32 values of k after the one before it
     const uint32_t kLast = K % kTK;
     const size_t aLastBytes = TA ? static_cast<size_t>(kLast) * M * 2 : kLast * 2;
-    const size_t bLastBytes = TB ? kLast * 2 : static_cast<size_t>(kLast) * N * 2;
+    const size_t bLastBytes = TB ? kLast * 2 : static_cast<size_t>(kLast) * args.ldb * 2;
     // Copy n (0..3: two of A, two of B) of the next step to fetch, into stage `stage`.  aSrc /
     // bSrc point at that step's slabs; surplus steps re-fetch the last one into a stage nobody
     // reads any more, which keeps the number of outstanding copies the same in every iteration.
@@ -935,7 +959,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
                 const uint32_t c = colBase + (waveN * TN + j) * 32 + 8 * q + 4 * khalf;
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (accumulate && r < M && c < N)  // N % 8 == 0: whole quads only
-                    v = *reinterpret_cast<const float4*>(out + static_cast<size_t>(r) * N + c);
+                    v = Load4(out + static_cast<size_t>(r) * args.ldc + c);
                 old[(i * TN + j) * 4 + q] = v;
             }
 #pragma unroll
@@ -954,7 +978,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
                     v.y += acc[i][j][4 * q + 1];
                     v.z += acc[i][j][4 * q + 2];
                     v.w += acc[i][j][4 * q + 3];
-                    *reinterpret_cast<float4*>(out + static_cast<size_t>(r) * N + c) = v;
+                    Store4(out + static_cast<size_t>(r) * args.ldc + c, v);
                 }
             }
 }
@@ -1082,7 +1106,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
                 const uint32_t gk = k0 + q / 16;
                 const uint32_t gc = colBase + (q % 16) * 8;
                 if (gk < K)
-                    v = load8(B + static_cast<size_t>(gk) * N + gc, gc, N);
+                    v = load8(B + static_cast<size_t>(gk) * args.ldb + gc, gc, N);
             }
             stageB[i] = v;
         }
@@ -1187,7 +1211,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
             for (int q = 0; q < 4; ++q)
             {
                 const uint32_t c = colBase + waveN * 64 + j * 32 + 8 * q + 4 * khalf;
-                float* p = out + static_cast<size_t>(r) * N + c;
+                float* p = out + static_cast<size_t>(r) * args.ldc + c;
                 if (args.outVec)
                 {
                     if (c < N)
@@ -1218,6 +1242,159 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
     }
 }
 
+// ---------------------------------------------------------------------------
+// the last N % 8 columns of a product whose other columns a straight-to-LDS kernel computes
+// ---------------------------------------------------------------------------
+// out[M x r] (+)= A[M x K] * B[K x r] with r < 8: all of A is read for 2 M r K flops, so this
+// is a stream over A.  A workgroup owns 16 rows; its 8 wavefronts take every 8th K step of
+// 32.  The A fragment of v_mfma_f32_16x16x32_f16 comes straight from global memory: lane l
+// holds k = 8 (l / 16) .. + 7 of row l % 16 (one 16-byte load; K % 8 == 0 and 16-byte aligned
+// rows, which the kernels for the other columns need as well).  The B fragment (column l % 16,
+// the same k; zeros or don't-cares for columns from r on, zeros for k >= K):
+//   B stored N x K: one 16-byte load;
+//   B stored K x N: the r values of a k-row are the last of that row, so the 16 bytes that start
+//     with them end inside the next row (for the last k-row they are read one by one).  The
+//     workgroup first copies these 16 bytes of every k-row of a slab of 4096 into LDS and the
+//     wavefronts pick their fragments up with transposing reads; what lies beyond column r only
+//     reaches outputs that are never stored.
+// The 8 partial products meet in LDS and are added in wavefront order.
+constexpr int kColsWaves = 8;
+constexpr int kColsRows = 16;
+constexpr int kColsSlab = 4096;  // k-rows of B's last columns held in LDS at a time (64 KiB)
+typedef halfx8 halfx8a2 __attribute__((aligned(2)));
+template <bool TB>
+__global__ __launch_bounds__(kColsWaves * 64) void GemmF16Cols(const GemmF16Args args)
+{
+    __shared__ float part[kColsWaves][32][4];
+    __shared__ __attribute__((aligned(16))) _Float16 tailB[TB ? 8 : kColsSlab * 8];
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t M = args.M, r = args.N, K = args.K;
+    const uint32_t unit = blockIdx.x / args.tilesM;
+    const uint32_t rowBase = (blockIdx.x % args.tilesM) * kColsRows;
+    const _Float16* __restrict__ A = args.A + args.strideA * static_cast<int64_t>(unit);
+    const _Float16* __restrict__ B = args.B + args.strideB * static_cast<int64_t>(unit);
+    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit);
+
+    const uint32_t x = lane & 15;          // row of A / column of B
+    const uint32_t kLane = 8 * (lane >> 4);
+    const _Float16* aRow = A + static_cast<size_t>(min(rowBase + x, M - 1)) * args.lda + kLane;
+    const bool colExists = x < r;
+    const _Float16* bCol = B + static_cast<size_t>(colExists ? x : 0) * K + kLane;  // TB only
+    // transposing read: lane x of a 16-lane group addresses k-row x / 4 of a block of four and
+    // columns 4 (x % 4) .. + 3 of it; an LDS k-row holds 8 columns, so lanes that would ask for
+    // columns 8-15 ask for 0-7 again
+    const uint32_t trOffset = (kLane + (x >> 2)) * 8 + 4 * (x & 1);
+    floatx4 acc = { 0.f, 0.f, 0.f, 0.f };
+    auto fetchA = [&](uint32_t step) {
+        halfx8 v = {};
+        if (step * kTK + kLane < K)
+            v = *reinterpret_cast<const halfx8*>(aRow + static_cast<size_t>(step) * kTK);
+        return v;
+    };
+    auto fetchB = [&](uint32_t step, uint32_t slabStart) {
+        halfx8 v = {};
+        if constexpr (TB)
+        {
+            if (colExists && step * kTK + kLane < K)
+                v = *reinterpret_cast<const halfx8*>(bCol + static_cast<size_t>(step) * kTK);
+        }
+        else
+        {
+            const _Float16* p = &tailB[(step * kTK - slabStart) * 8 + trOffset];
+            v = Join(LdsReadTr(p), LdsReadTr(p + 4 * 8));
+        }
+        return v;
+    };
+    for (uint32_t slabStart = 0; slabStart < K; slabStart += kColsSlab)
+    {
+        const uint32_t slabEnd = TB ? K : min(K, slabStart + kColsSlab);
+        if constexpr (!TB)
+        {
+            if (slabStart != 0)
+                __syncthreads();  // everybody is done with the slab before
+            // whole K steps: k-rows from K on are zeros
+            const uint32_t rowsHere = (slabEnd - slabStart + kTK - 1) / kTK * kTK;
+            constexpr int kPerThread = kColsSlab / (kColsWaves * 64);
+            halfx8 rows[kPerThread];
+#pragma unroll
+            for (int i = 0; i < kPerThread; ++i)
+            {
+                const uint32_t gk = slabStart + threadIdx.x + i * kColsWaves * 64;
+                const _Float16* p = B + static_cast<size_t>(gk) * args.ldb;
+                rows[i] = halfx8{};
+                if (gk + 1 < K)
+                    rows[i] = *reinterpret_cast<const halfx8a2*>(p);
+                else if (gk < K)
+                {
+#pragma unroll
+                    for (int e = 0; e < 7; ++e)
+                        if (e < static_cast<int>(r))
+                            rows[i][e] = p[e];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kPerThread; ++i)
+            {
+                const uint32_t k = threadIdx.x + i * kColsWaves * 64;
+                if (k < rowsHere)
+                    *reinterpret_cast<halfx8*>(&tailB[k * 8]) = rows[i];
+            }
+            __syncthreads();
+        }
+        // four steps' loads in flight per wavefront
+        const uint32_t stepEnd = (slabEnd + kTK - 1) / kTK;
+        for (uint32_t step = slabStart / kTK + wave; step < stepEnd; step += 4 * kColsWaves)
+        {
+            halfx8 a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                const uint32_t st = step + u * kColsWaves;
+                a[u] = halfx8{};
+                b[u] = halfx8{};
+                if (st < stepEnd)
+                {
+                    a[u] = fetchA(st);
+                    b[u] = fetchB(st, slabStart);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[u], a[u], acc, 0, 0, 0);
+        }
+        if constexpr (TB)
+            break;
+    }
+    // lane l now holds row l % 16, columns 4 (l / 16) .. + 3: the first 32 lanes hold columns 0-7
+    if (lane < 32)
+        *reinterpret_cast<floatx4*>(&part[wave][lane][0]) = acc;
+    __syncthreads();
+    if (threadIdx.x < 32)
+    {
+        floatx4 sum = *reinterpret_cast<const floatx4*>(&part[0][lane][0]);
+#pragma unroll
+        for (int w = 1; w < kColsWaves; ++w)
+        {
+            const floatx4 p = *reinterpret_cast<const floatx4*>(&part[w][lane][0]);
+            sum[0] += p[0];
+            sum[1] += p[1];
+            sum[2] += p[2];
+            sum[3] += p[3];
+        }
+        const uint32_t row = rowBase + x;
+        const uint32_t col = 4 * (lane >> 4);
+        if (row < M)
+        {
+            float* p = out + static_cast<size_t>(row) * args.ldc + col;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < r)
+                    p[e] = args.overwrite ? sum[e] : p[e] + sum[e];
+        }
+    }
+}
+
 // variant 0: whole tiles, out read in the epilogue; 1 / 2: out added inside the loop with
 // spacing 2 / 4; 3: ragged tiles
 template <bool TA, bool TB, bool TAIL>
@@ -1234,34 +1411,65 @@ void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16
         hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB, TAIL>), g, b, 0, stream, args);
 }
 
-// Picks the kernel for one launch.
-int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, bool transB,
-              hipStream_t stream)
+// What one launch may assume about where its operands lie.
+struct F16Layout
 {
-    const uint32_t M = args.M, N = args.N, K = args.K;
+    bool dmaA;  // A: base and unit stride multiples of 16 bytes
+    bool dmaB;  // B stored N x K: likewise (a B stored K x N is copied from any address)
+    bool transA, transB;
+};
+
+enum class F16Kernel { kTile256, kDma128, kGeneral };
+
+// The kernel that would take M x N x K with these operands.  The straight-to-LDS copies take 16
+// bytes from any 2-byte-aligned address, so the rows of a K x N matrix B may start anywhere
+// (any ldb, any base); N itself has to be a multiple of 8 because a copy is 8 columns wide.
+// out is accessed 16 bytes at a time from 4-byte-aligned addresses.
+F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16Layout& lay)
+{
+    const uint32_t M = args.M, K = args.K;
+    const bool transA = lay.transA, transB = lay.transB;
     const bool plain = !transA && !transB;
     // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
     // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
     const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;
     const uint64_t tiles256 =
         static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * batch;
-    const bool whole256 = (M % kT == 0) && (N % kT == 0);
     // ragged shapes only while at least three quarters of the tiled area is real output
     const bool fills256 =
         static_cast<uint64_t>(M) * N * 4 >=
         static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * kT * kT * 3;
     // lane offsets of the copies are 32-bit: 256 rows of a K-contiguous operand, 32 of a
-    // k-major one
-    const uint64_t pitchA = transA ? M : args.lda, pitchB = transB ? K : N;
+    // k-major one (and 256 rows of out in the kernels that copy it)
+    const uint64_t pitchA = transA ? M : args.lda, pitchB = transB ? K : args.ldb;
     const bool offsetsFit = (transA ? 32 : 256) * pitchA * 2 + 8192 < (1ull << 32) &&
-                            (transB ? 256 : 32) * pitchB * 2 + 8192 < (1ull << 32);
+                            (transB ? 256 : 32) * pitchB * 2 + 8192 < (1ull << 32) &&
+                            256ull * args.ldc * 4 + 8192 < (1ull << 32);
     // K = 32 q + r, r = 8, 16 or 24: the straight-to-LDS kernels take the r values in a last,
     // partly masked step (plain storage only; measured 4096 x 4096 x 4080: 229 us on the
     // general kernel, 175 us with the r values left to a second launch, 128 us this way)
     const bool tailInKernel = plain && K % kTK != 0 && K % 8 == 0 && K >= 2 * kTK && args.lda == K;
-    const bool tile256 = aligned16 && K >= kTK && (K % kTK == 0 || tailInKernel) && (N % 8 == 0) &&
-                         N >= 8 && (!transA || (M % 8 == 0 && M >= 8)) && tiles256 >= minTiles &&
-                         fills256 && offsetsFit;
+    const bool dma = lay.dmaA && (lay.dmaB || !transB) && K >= kTK &&
+                     (K % kTK == 0 || tailInKernel) && N % 8 == 0 && N >= 8 &&
+                     (!transA || (M % 8 == 0 && M >= 8));
+    if (dma && tiles256 >= minTiles && fills256 && offsetsFit)
+        return F16Kernel::kTile256;
+    if (dma && static_cast<uint64_t>(M) * (transA ? kTK : args.lda) < (1ull << 31) &&
+        static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31) &&
+        32ull * args.ldb < (1ull << 30))
+        return F16Kernel::kDma128;
+    return F16Kernel::kGeneral;
+}
+
+// One launch over all of args.N columns with the kernel `kind`.
+int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16Layout& lay,
+                    hipStream_t stream)
+{
+    const uint32_t M = args.M, N = args.N, K = args.K;
+    const bool transA = lay.transA, transB = lay.transB;
+    const bool plain = !transA && !transB;
+    const bool whole256 = (M % kT == 0) && (N % kT == 0);
+    const bool tile256 = kind == F16Kernel::kTile256;
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -1288,10 +1496,7 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
         else
             LaunchTile256<false, false, false>(variant, grid, stream, args);
     }
-    else if (aligned16 && K >= kTK && (K % kTK == 0 || tailInKernel) && N % 8 == 0 && N >= 8 &&
-             (!transA || (M % 8 == 0 && M >= 8)) &&
-             static_cast<uint64_t>(M) * (transA ? kTK : args.lda) < (1ull << 31) &&
-             static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31))
+    else if (kind == F16Kernel::kDma128)
     {
         // whole K steps and 16-byte chunks everywhere: straight-to-LDS 128-tile kernel
         // Eight wavefronts per tile (2 x 4, 64 x 32 each) while there is at most one tile per
@@ -1328,14 +1533,15 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
         // widest load every row start, every row length and every base allows (in halves);
         // an operand is read along its contiguous dimension: K (A), N (B), M (A stored K x M)
         // or K (B stored N x K)
-        const uint64_t mix = static_cast<uint64_t>(K) | (transA ? M : args.lda) | (transB ? K : N) |
+        const uint64_t mix = static_cast<uint64_t>(K) | (transA ? M : args.lda) |
+                             (transB ? K : (args.ldb | N)) |
                              static_cast<uint64_t>(args.strideA) |
                              static_cast<uint64_t>(args.strideB) |
                              (reinterpret_cast<uintptr_t>(args.A) / 2) |
                              (reinterpret_cast<uintptr_t>(args.B) / 2) | 8u;
         const uint32_t vec = static_cast<uint32_t>(mix & (~mix + 1));  // lowest set bit: 1, 2, 4, 8
         args.outVec = ((reinterpret_cast<uintptr_t>(args.out) & 15u) == 0 && args.strideOut % 4 == 0 &&
-                       N % 4 == 0)
+                       N % 4 == 0 && args.ldc % 4 == 0)
                           ? 1u
                           : 0u;
         const dim3 g(grid), b(kGThreads);
@@ -1370,6 +1576,43 @@ int LaunchF16(GemmF16Args args, uint32_t batch, bool aligned16, bool transA, boo
                 hipLaunchKernelGGL((GemmF16General<1, false, true>), g, b, 0, stream, args);
         }
     }
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+// Picks the kernels for one call.  N = 8 q + r with r != 0 and a shape the straight-to-LDS
+// kernels would take at N = 8 q: they compute the first 8 q columns (row pitches of B and out
+// stay N) and the general kernel the last r, each output element still by one kernel
+// (measured 4096 x 4100 x 4096: 270 us on the general kernel alone).
+int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream)
+{
+    const uint32_t N = args.N;
+    const F16Kernel whole = PickF16(args, N, batch, lay);
+    const uint32_t wholeChunks = N & ~7u;
+    if (whole != F16Kernel::kGeneral || N % 8 == 0 || wholeChunks < kG)
+        return LaunchF16Kernel(args, batch, whole, lay, stream);
+    const F16Kernel most = PickF16(args, wholeChunks, batch, lay);
+    if (most == F16Kernel::kGeneral)
+        return LaunchF16Kernel(args, batch, whole, lay, stream);
+    GemmF16Args left = args;
+    left.N = wholeChunks;
+    const int rc = LaunchF16Kernel(left, batch, most, lay, stream);
+    if (rc != SPH_OK)
+        return rc;
+    GemmF16Args right = args;
+    right.N = N - wholeChunks;
+    right.out = args.out + wholeChunks;
+    right.B = args.B + (lay.transB ? static_cast<size_t>(wholeChunks) * args.K : wholeChunks);
+    if (lay.transA)
+        return LaunchF16Kernel(right, batch, F16Kernel::kGeneral, lay, stream);
+    right.tilesM = (args.M + kColsRows - 1) / kColsRows;
+    const uint64_t groups = static_cast<uint64_t>(right.tilesM) * batch;
+    SPH_REQUIRE(groups < (1ull << 31), "too many rows for one launch");
+    const dim3 g(static_cast<uint32_t>(groups)), b(kColsWaves * 64);
+    if (lay.transB)
+        hipLaunchKernelGGL((GemmF16Cols<true>), g, b, 0, stream, right);
+    else
+        hipLaunchKernelGGL((GemmF16Cols<false>), g, b, 0, stream, right);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
@@ -1410,10 +1653,11 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     }
     SPH_REQUIRE(A != nullptr && B != nullptr, "null pointer");
 
-    const bool aligned16 =
-        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) |
-          reinterpret_cast<uintptr_t>(out)) & 15u) == 0 &&
-        (strideA % 8 == 0) && (strideB % 8 == 0) && (strideOut % 4 == 0);
+    F16Layout lay{};
+    lay.transA = transA;
+    lay.transB = transB;
+    lay.dmaA = (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && strideA % 8 == 0;
+    lay.dmaB = (reinterpret_cast<uintptr_t>(B) & 15u) == 0 && strideB % 8 == 0;
 
     GemmF16Args args{};
     args.out = out;
@@ -1423,12 +1667,14 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.N = N;
     args.K = K;
     args.lda = K;
+    args.ldb = N;
+    args.ldc = N;
     args.strideOut = strideOut;
     args.strideA = strideA;
     args.strideB = strideB;
     args.overwrite = (flags & SPH_GEMM_OVERWRITE) ? 1u : 0u;
 
-    return LaunchF16(args, batch, aligned16, transA, transB, stream);
+    return LaunchF16(args, batch, lay, stream);
 }
 
 }  // extern "C"

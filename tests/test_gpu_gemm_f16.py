@@ -188,6 +188,56 @@ def test_transposed_operands_exact_on_integers(dev, shape, flags):
     assert np.array_equal(got, ref - C)
 
 
+# N = 8 q + r, r != 0, with at least 128 whole column chunks' worth of columns: the first 8 q
+# columns on the straight-to-LDS kernels (rows of B and of out start at addresses that are no
+# multiples of 16 bytes), the last r on the general kernel.  (M, N, K, batch): 128-tile kernel
+# with four and with eight wavefronts, ragged and whole 256-tiles (old values of out added in the
+# epilogue, K = 64, or in the loop, K = 640), N % 4 == 0, N % 2 == 0 and odd N, a K tail on top.
+@pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
+                                   capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
+@pytest.mark.parametrize("shape", [(512, 132, 64, 1), (200, 1030, 96, 2), (304, 517, 64, 3),
+                                   (128, 135, 32, 300), (4096, 3076, 64, 1), (256, 257, 64, 192),
+                                   (256, 260, 640, 192), (1000, 999, 992, 1), (248, 250, 72, 3)])
+def test_column_count_not_a_multiple_of_eight(dev, shape, flags):
+    M, N, K, batch = shape
+    h.announce("sph_gemm_f16f32, N % 8 != 0", shape, "flags", flags)
+    span = 4 if K <= 256 else 3
+    A = synth.small_integers(61, (batch, M, K), span=span).astype(np.float16)
+    B = synth.small_integers(62, (batch, K, N), span=span).astype(np.float16)
+    C = synth.small_integers(63, (batch, M, N), span=100)
+    As = np.ascontiguousarray(A.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_A else A
+    Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
+    ref = _oracle(C, A, B, M, N, K, batch=batch)
+    # 37 guard floats after every unit of out: nothing may be written past column N - 1
+    pad = 37
+    padded = np.full((batch, M * N + pad), np.float32(-777.25), np.float32)
+    padded[:, :M * N] = C.reshape(batch, M * N)
+    for extra in (0, capi.SPH_GEMM_OVERWRITE):
+        got = h.gpu_gemm_f16(padded, As, Bs, M, N, K, batch=batch, stride_out=M * N + pad,
+                             flags=flags | extra)
+        assert np.array_equal(got[:, M * N:], padded[:, M * N:]), "guard floats overwritten"
+        want = ref - C if extra else ref
+        assert np.array_equal(got[:, :M * N].reshape(batch, M, N), want)
+
+
+def test_rows_of_b_that_start_anywhere(dev):
+    """A K x N matrix B that begins 2 bytes past a 16-byte boundary (and N % 8 == 0): its rows are
+    copied straight into LDS from addresses that are only 2-byte aligned."""
+    M, N, K = 384, 264, 96
+    h.announce("sph_gemm_f16f32, B at a 2-byte-aligned address", (M, N, K))
+    A = synth.small_integers(71, (M, K)).astype(np.float16)
+    B = synth.small_integers(72, (K, N)).astype(np.float16)
+    C = synth.small_integers(73, (M, N), span=100)
+    ref = _oracle(C, A, B, M, N, K)
+    shifted = np.concatenate([np.zeros(1, np.float16), B.ravel()])
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, shifted, C))
+    capi.call("sph_gemm_f16f32", dC.ptr, dA.ptr, dB.ptr + 2, M, N, K, 1, M * N, M * K, K * N, 0)
+    got = dC.download(np.float32, C.shape)
+    for d in (dA, dB, dC):
+        d.release()
+    assert np.array_equal(got, ref)
+
+
 def test_dma128_batched_with_shared_operand(dev):
     h.announce("sph_gemm_f16f32 128-tile path, batch 3, strideA = 0")
     M, N, K, batch = 200, 136, 96, 3
