@@ -34,7 +34,7 @@
 //     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
 //     widest that K, N, the strides and the bases allow), padded LDS rows.
 //
-// K = 32 q + r with r in {8, 16, 24} (operands stored plainly) stays on the first two kernels:
+// K = 32 q + r with r in {8, 16, 24} stays on the first two kernels:
 // a last step over [K - 32, K) in which the lanes holding values of k that were multiplied
 // already feed zeros.
 //
@@ -683,7 +683,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 // 128 x 128 x 32 kernel with straight-to-LDS copies, ragged M and N
 // ---------------------------------------------------------------------------
 // For shapes the 256-tile kernel does not take (M or N not a multiple of 256) as long as K is a
-// multiple of 32 (or 32 q + 8, 16, 24 with plain storage), N of 8 and everything is 16-byte
+// multiple of 32 (or 32 q + 8, 16, 24), N of 8 and everything is 16-byte
 // aligned.  Four wavefronts (2 x 2, each 64 x 64 = 2 x 2 MFMA blocks) or eight (2 x 4, each
 // 64 x 32), four LDS stages of 16 KiB (two workgroups per compute unit), copies issued two steps
 // ahead, one barrier per step (placed, with the copies, between the MFMAs of the step's first
@@ -1446,9 +1446,9 @@ F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16
                             (transB ? 256 : 32) * pitchB * 2 + 8192 < (1ull << 32) &&
                             256ull * args.ldc * 4 + 8192 < (1ull << 32);
     // K = 32 q + r, r = 8, 16 or 24: the straight-to-LDS kernels take the r values in a last,
-    // partly masked step (plain storage only; measured 4096 x 4096 x 4080: 229 us on the
+    // partly masked step (measured 4096 x 4096 x 4080, operands stored plainly: 229 us on the
     // general kernel, 175 us with the r values left to a second launch, 128 us this way)
-    const bool tailInKernel = plain && K % kTK != 0 && K % 8 == 0 && K >= 2 * kTK && args.lda == K;
+    const bool tailInKernel = K % kTK != 0 && K % 8 == 0 && K >= 2 * kTK && args.lda == K;
     const bool dma = lay.dmaA && (lay.dmaB || !transB) && K >= kTK &&
                      (K % kTK == 0 || tailInKernel) && N % 8 == 0 && N >= 8 &&
                      (!transA || (M % 8 == 0 && M >= 8));
@@ -1485,16 +1485,24 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         const uint32_t ksteps = (K + kTK - 1) / kTK;
         const int variant = !whole256 ? 3 : (cloop && ksteps >= CLoopSteps(4)) ? 2
                                           : (cloop && ksteps >= CLoopSteps(2)) ? 1 : 0;
+        const bool tail = K % kTK != 0;
+#define SPH_TILE256(TA_, TB_)                                                                     \
+    do                                                                                            \
+    {                                                                                             \
+        if (tail)                                                                                 \
+            LaunchTile256<TA_, TB_, true>(variant, grid, stream, args);                           \
+        else                                                                                      \
+            LaunchTile256<TA_, TB_, false>(variant, grid, stream, args);                          \
+    } while (0)
         if (transA && transB)
-            LaunchTile256<true, true, false>(variant, grid, stream, args);
+            SPH_TILE256(true, true);
         else if (transA)
-            LaunchTile256<true, false, false>(variant, grid, stream, args);
+            SPH_TILE256(true, false);
         else if (transB)
-            LaunchTile256<false, true, false>(variant, grid, stream, args);
-        else if (K % kTK != 0)
-            LaunchTile256<false, false, true>(variant, grid, stream, args);
+            SPH_TILE256(false, true);
         else
-            LaunchTile256<false, false, false>(variant, grid, stream, args);
+            SPH_TILE256(false, false);
+#undef SPH_TILE256
     }
     else if (kind == F16Kernel::kDma128)
     {
@@ -1506,7 +1514,8 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         // flop (4096 x 2048 x 2048: 50.9 us against 52.5 us on eight).
         const bool wide = args.totalTiles <= static_cast<uint32_t>(sph::ComputeUnits());
         const dim3 g(grid);
-#define SPH_DMA128(TA_, TB_, TAIL_)                                                               \
+        const bool tail = K % kTK != 0;
+#define SPH_DMA128_(TA_, TB_, TAIL_)                                                              \
     do                                                                                            \
     {                                                                                             \
         if (wide)                                                                                 \
@@ -1516,17 +1525,24 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
             hipLaunchKernelGGL((GemmF16Dma128<TA_, TB_, TAIL_, 4>), g, dim3(256), 0, stream,      \
                                args);                                                             \
     } while (0)
+#define SPH_DMA128(TA_, TB_)                                                                      \
+    do                                                                                            \
+    {                                                                                             \
+        if (tail)                                                                                 \
+            SPH_DMA128_(TA_, TB_, true);                                                          \
+        else                                                                                      \
+            SPH_DMA128_(TA_, TB_, false);                                                         \
+    } while (0)
         if (transA && transB)
-            SPH_DMA128(true, true, false);
+            SPH_DMA128(true, true);
         else if (transA)
-            SPH_DMA128(true, false, false);
+            SPH_DMA128(true, false);
         else if (transB)
-            SPH_DMA128(false, true, false);
-        else if (K % kTK != 0)
-            SPH_DMA128(false, false, true);
+            SPH_DMA128(false, true);
         else
-            SPH_DMA128(false, false, false);
+            SPH_DMA128(false, false);
 #undef SPH_DMA128
+#undef SPH_DMA128_
     }
     else
     {

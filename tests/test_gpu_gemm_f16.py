@@ -69,27 +69,31 @@ def test_tile256_ragged_exact_on_integers(dev, shape):
 # step and masks the 32 - r values of k it has already multiplied (shapes with 192 tiles: whole
 # and ragged tiles, old contents added in the epilogue, every second step (20 steps and more:
 # K = 632 ends inside the written-out prefix, 648 after it) and every fourth (36 and more: 1144,
-# 1168, 1176)); the 128-tile kernel multiplies the first 32 q columns and the general kernel adds
-# the rest in a second launch.
+# 1168, 1176)) and the 128-tile kernel, with the operands stored plainly or the other way round.
 @pytest.mark.parametrize("shape", [(256, 256, 72, 192), (250, 248, 80, 192), (4096, 3072, 88, 1),
                                    (256, 256, 632, 192), (256, 256, 648, 192), (512, 256, 1144, 96),
                                    (512, 256, 1168, 96), (256, 512, 1176, 96), (500, 504, 680, 48),
                                    (300, 520, 168, 1), (128, 128, 72, 3), (1000, 1000, 1000, 1)])
-def test_k_tail_exact_on_integers(dev, shape):
+@pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
+                                   capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
+def test_k_tail_exact_on_integers(dev, shape, flags):
     M, N, K, batch = shape
-    h.announce("sph_gemm_f16f32 K tail integer exactness", shape)
+    h.announce("sph_gemm_f16f32 K tail integer exactness", shape, "flags", flags)
     A = synth.small_integers(31, (batch, M, K), span=3).astype(np.float16)
     B = synth.small_integers(32, (batch, K, N), span=3).astype(np.float16)
     C = synth.small_integers(33, (batch, M, N), span=100)
+    As = np.ascontiguousarray(A.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_A else A
+    Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
     ref = _oracle(C, A, B, M, N, K, batch=batch)
-    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch)
+    got = h.gpu_gemm_f16(C, As, Bs, M, N, K, batch=batch, flags=flags)
     assert np.array_equal(got, ref)
-    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch, flags=capi.SPH_GEMM_OVERWRITE)
+    got = h.gpu_gemm_f16(C, As, Bs, M, N, K, batch=batch, flags=flags | capi.SPH_GEMM_OVERWRITE)
     assert np.array_equal(got, ref - C)
 
 
+@pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
 @pytest.mark.parametrize("K", [72, 80, 88])
-def test_k_tail_window_counts_an_infinity_once(dev, K):
+def test_k_tail_window_counts_an_infinity_once(dev, K, flags):
     """An infinity (and a 0 x Inf) at a k that lies in both of the last two step windows must
     come out exactly as in the CPU product: +Inf where the partner is positive, NaN where it is
     zero, and nothing else in the matrix may change."""
@@ -104,7 +108,9 @@ def test_k_tail_window_counts_an_infinity_once(dev, K):
     B[:, k, 7] = 0                  # Inf x 0
     with np.errstate(invalid="ignore"):
         ref = _oracle(C, A, B, M, N, K, batch=batch)
-    got = h.gpu_gemm_f16(C, A, B, M, N, K, batch=batch)
+    As = np.ascontiguousarray(A.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_A else A
+    Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
+    got = h.gpu_gemm_f16(C, As, Bs, M, N, K, batch=batch, flags=flags)
     assert np.array_equal(got, ref, equal_nan=True)
     assert np.isnan(got[:, 5, 7]).all() and np.isposinf(got[:, 5, 8]).all()
 
