@@ -59,8 +59,6 @@ __device__ __forceinline__ float Bcast(float v, int srcLane)
                               __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), srcLane));
 }
 
-typedef float floatx4v __attribute__((ext_vector_type(4)));
-
 __device__ __forceinline__ uint32_t Bcast(uint32_t v, int srcLane)
 {
     return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), srcLane));
@@ -88,20 +86,45 @@ __device__ __forceinline__ uint32_t GroupBroadcast(uint32_t v)
         __builtin_amdgcn_ds_swizzle(static_cast<int>(v), (J << 5) | (0x1f & ~(LPR - 1))));
 }
 
-// The storage-order sums of one row's entries p .. end - 1 for this lane's 4 columns (colBytes:
-// byte offset of the first of them inside a row of B), gathers into registers.  t: the lane's
-// index among the LPR lanes of its row.
 template <int LPR>
-__device__ __forceinline__ float4 RowSumsInRegisters(const SpmmArgs& args, uint32_t p, uint32_t end,
-                                                     uint32_t t, uint32_t colBytes)
+__global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, const SlabPlan plan)
 {
+    constexpr int kSlabCols = 4 * LPR;
+    constexpr int kLanesPerRow = LPR;
+    constexpr int kRowsPerWave = 64 / LPR;
+    constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlock;
+    // work column w = slab + slabs * part runs on XCD w % 8
+    const uint32_t xcd = blockIdx.x % 8;
+    const uint32_t local = blockIdx.x / 8;
+    const uint32_t w = xcd + 8 * (local / plan.blocksPerColumn);
+    if (w >= plan.slabs * plan.rowParts)
+        return;
+    const uint32_t slab = w % plan.slabs;
+    const uint32_t part = w / plan.slabs;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t t = lane & (kLanesPerRow - 1);
+    const uint32_t rowInPart = (local % plan.blocksPerColumn) * kRowsPerBlock +
+                               (threadIdx.x >> 6) * kRowsPerWave + lane / LPR;
+    const uint32_t row = part * plan.rowsPerPart + rowInPart;
+    const uint32_t N = args.N;
+    const uint32_t col = slab * kSlabCols + t * 4;
+    const bool rowOk = rowInPart < plan.rowsPerPart && row < args.M;
+    const bool active = rowOk && col < N;
+
+    uint32_t p = 0, end = 0;
+    if (rowOk)
+    {
+        p = args.ROW[row];
+        end = args.ROW[row + 1];
+    }
     // Every lane gathers from a valid address on every step, so the loop has no branches:
     // lanes outside the matrix read the slab's first columns, entries past the end of a row
     // read row 0 of B (their COL is 0), and a select keeps such products out of the sum.
     // Byte offsets into B fit 32 bits (checked by the launcher) and are formed with a 24-bit
     // multiply-add.
     const char* __restrict__ Bbytes = reinterpret_cast<const char*>(args.B);
-    const uint32_t rowBytes = args.N * 4;
+    const uint32_t colBytes = (col < N ? col : slab * kSlabCols) * 4;
+    const uint32_t rowBytes = N * 4;
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 
     // all lanes of the wavefront stay in the loop until the longest of its rows is done
@@ -162,269 +185,6 @@ __device__ __forceinline__ float4 RowSumsInRegisters(const SpmmArgs& args, uint3
             eight(std::integral_constant<int, 8>{});
         p = min(p + LPR, end);
     }
-
-    return sum;
-}
-
-template <int LPR>
-__global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, const SlabPlan plan)
-{
-    constexpr int kSlabCols = 4 * LPR;
-    constexpr int kLanesPerRow = LPR;
-    constexpr int kRowsPerWave = 64 / LPR;
-    constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlock;
-    // work column w = slab + slabs * part runs on XCD w % 8
-    const uint32_t xcd = blockIdx.x % 8;
-    const uint32_t local = blockIdx.x / 8;
-    const uint32_t w = xcd + 8 * (local / plan.blocksPerColumn);
-    if (w >= plan.slabs * plan.rowParts)
-        return;
-    const uint32_t slab = w % plan.slabs;
-    const uint32_t part = w / plan.slabs;
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t t = lane & (kLanesPerRow - 1);
-    const uint32_t rowInPart = (local % plan.blocksPerColumn) * kRowsPerBlock +
-                               (threadIdx.x >> 6) * kRowsPerWave + lane / LPR;
-    const uint32_t row = part * plan.rowsPerPart + rowInPart;
-    const uint32_t N = args.N;
-    const uint32_t col = slab * kSlabCols + t * 4;
-    const bool rowOk = rowInPart < plan.rowsPerPart && row < args.M;
-    const bool active = rowOk && col < N;
-
-    uint32_t p = 0, end = 0;
-    if (rowOk)
-    {
-        p = args.ROW[row];
-        end = args.ROW[row + 1];
-    }
-    const uint32_t colBytes = (col < N ? col : slab * kSlabCols) * 4;
-    float4 sum = RowSumsInRegisters<LPR>(args, p, end, t, colBytes);
-
-    if (active)
-    {
-        float4* dst = reinterpret_cast<float4*>(args.out + static_cast<size_t>(row) * N + col);
-        if (args.rowBias != nullptr)
-        {
-            const float old = 0.f + args.rowBias[row];
-            sum.x = old + sum.x;
-            sum.y = old + sum.y;
-            sum.z = old + sum.z;
-            sum.w = old + sum.w;
-        }
-        else if (args.accumulate)
-        {
-            const float4 old = *dst;
-            sum.x = old.x + sum.x;
-            sum.y = old.y + sum.y;
-            sum.z = old.z + sum.z;
-            sum.w = old.w + sum.w;
-        }
-        *dst = sum;
-    }
-}
-
-// ---- slab mapping with the gathers copied straight into LDS ---------------------------------
-// The same work split as SpmmSlabVec4<16> (64-column slabs, 4 rows per wavefront, 16 lanes per
-// row, 4 columns per lane, entries in storage order, product and sum rounded separately), but
-// every vector memory operation is a global_load_lds copy issued by hand: gathers that land in
-// registers reach 25 TB/s chip-wide on L2-resident data with 32 wavefronts per compute unit,
-// gathers that land in LDS 31 TB/s with 8 (measured with 256-byte pieces, 8 in flight per
-// wavefront).  Per wavefront: a ring of SLOTS gather slots of 1 KiB (lane i's 16 bytes at
-// 16 i: its row's piece of B[COL[e]]) and two (COL, V) chunk buffers of 16 entries per row.
-// Order of the copies: CV(0), G(0..7), then per chunk q of 16 entries CV(q+1) followed, for
-// entry e, by "wait for G(e), read it, issue G(e+8)"; copies complete in issue order, so the
-// number of younger copies at each wait is known when the code is written: 7 gathers, and the
-// two chunk copies while e is in the first half of its chunk.  Entries past the end of a row
-// copy a valid (COL, V) pair from further on in the arrays (the index is clamped to the last
-// entry of the matrix), gather that row of B and are kept out of the sum by a select.
-__device__ __forceinline__ void DmaGather16(uint32_t laneByteOffset, const void* uniformBase,
-                                            uint32_t ldsByteAddr)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(ldsByteAddr), "v"(laneByteOffset), "s"(uniformBase)
-                 : "memory");
-}
-// lane i's 4 bytes at `address` land at ldsByteAddr + 4 i
-__device__ __forceinline__ void DmaWord(const void* address, uint32_t ldsByteAddr)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
-                 :
-                 : "s"(ldsByteAddr), "v"(address)
-                 : "memory");
-}
-template <int N>
-__device__ __forceinline__ void WaitCopies()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-
-// The same sums with the gathers copied into LDS.  `mine`: this wavefront's kLdsWaveBytes of
-// LDS; len: entries of this lane's row, starting at p.  Entries are taken 4 at a time, the
-// gathers of entries + 8 issued as soon as a batch's slots are read: 8 slots, two batches in
-// flight.
-constexpr int kLdsSlots = 8;
-constexpr int kLdsWaveBytes = kLdsSlots * 1024 + 1024;
-__device__ __forceinline__ float4 RowSumsThroughLds(const SpmmArgs& args, uint32_t p, uint32_t len,
-                                                    uint32_t lane, uint32_t colBytes,
-                                                    __attribute__((address_space(3))) char* mine)
-{
-    auto lenOf = [&](int l) {
-        return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(len), l));
-    };
-    const uint32_t longest = max(max(lenOf(0), lenOf(16)), max(lenOf(32), lenOf(48)));
-    const uint32_t shortest = min(min(lenOf(0), lenOf(16)), min(lenOf(32), lenOf(48)));
-    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (longest == 0)
-        return sum;
-
-    const uint32_t t = lane & 15;
-    const uint32_t lastEntry = args.ROW[args.M] - 1;  // longest != 0: the matrix has entries
-    const char* Bbytes = reinterpret_cast<const char*>(args.B);
-    const uint32_t rowBytes = args.N * 4;
-    typedef __attribute__((address_space(3))) char LdsChar;
-    typedef __attribute__((address_space(3))) const volatile floatx4v LdsQuad;
-    typedef __attribute__((address_space(3))) const volatile uint32_t LdsWord;
-    typedef __attribute__((address_space(3))) const volatile float LdsFloat;
-    const uint32_t ring = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(mine));
-    const uint32_t cvLds = ring + kLdsSlots * 1024;
-    // this lane's views: its 16 bytes of a slot; entry j of its row in a chunk buffer
-    LdsChar* slotMine = mine + lane * 16;
-    LdsChar* cvMine = mine + kLdsSlots * 1024 + (lane / 16) * 64;
-    const uint32_t chunks = (longest + 15) / 16;
-
-    auto issueChunk = [&](uint32_t q) {
-        const uint32_t idx = min(p + 16 * q + t, lastEntry);
-        DmaWord(args.COL + idx, cvLds + (q & 1) * 512);
-        DmaWord(args.V + idx, cvLds + (q & 1) * 512 + 256);
-    };
-    auto readCol = [&](uint32_t q, int j) { return *(LdsWord*)(cvMine + (q & 1) * 512 + j * 4); };
-    auto readVal = [&](uint32_t q, int j) {
-        return *(LdsFloat*)(cvMine + (q & 1) * 512 + 256 + j * 4);
-    };
-    auto gather = [&](uint32_t c, int slot) {
-        DmaGather16(__umul24(c, rowBytes) + colBytes, Bbytes, ring + slot * 1024);
-    };
-    // entries 16 q + j0 .. + 3; the gathers of entries + 8 are issued
-    auto batch = [&](uint32_t q, auto jC, auto lastC, auto maskedC) {
-        constexpr int j0 = decltype(jC)::value;
-        constexpr bool LAST = decltype(lastC)::value;
-        constexpr bool MASKED = decltype(maskedC)::value;
-        constexpr int firstSlot = j0 % kLdsSlots;
-        // younger copies: the next batch's 4 gathers, and the two chunk copies while this
-        // batch's gathers were issued before them
-        if constexpr (LAST)
-            WaitCopies<(j0 < 12 ? 4 : 0)>();
-        else
-            WaitCopies<(j0 < 8 ? 6 : 4)>();
-        floatx4v b[4];
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            b[i] = *(LdsQuad*)(slotMine + (firstSlot + i) * 1024);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            v[i] = readVal(q, j0 + i);
-        if constexpr (!LAST || j0 < 8)
-        {
-            uint32_t c[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                c[i] = j0 < 8 ? readCol(q, j0 + 8 + i) : readCol(q + 1, j0 - 8 + i);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                gather(c[i], firstSlot + i);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-        {
-            const float x = sum.x + v[i] * b[i][0];
-            const float y = sum.y + v[i] * b[i][1];
-            const float z = sum.z + v[i] * b[i][2];
-            const float ww = sum.w + v[i] * b[i][3];
-            if constexpr (MASKED)
-            {
-                const bool take = 16 * q + j0 + i < len;
-                sum.x = take ? x : sum.x;
-                sum.y = take ? y : sum.y;
-                sum.z = take ? z : sum.z;
-                sum.w = take ? ww : sum.w;
-            }
-            else
-            {
-                sum.x = x;
-                sum.y = y;
-                sum.z = z;
-                sum.w = ww;
-            }
-        }
-    };
-    auto chunk = [&](uint32_t q, auto lastC, auto maskedC) {
-        batch(q, std::integral_constant<int, 0>{}, lastC, maskedC);
-        batch(q, std::integral_constant<int, 4>{}, lastC, maskedC);
-        batch(q, std::integral_constant<int, 8>{}, lastC, maskedC);
-        batch(q, std::integral_constant<int, 12>{}, lastC, maskedC);
-    };
-
-    issueChunk(0);
-    WaitCopies<0>();
-#pragma unroll
-    for (int j = 0; j < kLdsSlots; ++j)
-        gather(readCol(0, j), j);
-    for (uint32_t q = 0; q + 1 < chunks; ++q)
-    {
-        issueChunk(q + 1);
-        if (16 * (q + 1) <= shortest)
-            chunk(q, std::false_type{}, std::false_type{});
-        else
-            chunk(q, std::false_type{}, std::true_type{});
-    }
-    chunk(chunks - 1, std::true_type{}, std::true_type{});
-    return sum;
-}
-
-// 64-column slabs, 4 rows per wavefront (the mapping of SpmmSlabVec4<16>); the first kLdsWaves
-// wavefronts of a workgroup gather through LDS, the others into registers.  A wavefront never
-// mixes the two: the copies into LDS are counted by hand, and a wait the compiler places for a
-// load of its own would take that count for its own.
-template <int kLdsWaves>
-__global__ __launch_bounds__(kThreads) void SpmmSlabSplit(const SpmmArgs args, const SlabPlan plan)
-{
-    constexpr int kSlabCols = 64;
-    constexpr int kRowsPerWave = 4;
-    constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlock;
-    __shared__ __attribute__((aligned(1024))) char lds[kLdsWaves * kLdsWaveBytes];
-    const uint32_t xcd = blockIdx.x % 8;
-    const uint32_t local = blockIdx.x / 8;
-    const uint32_t w = xcd + 8 * (local / plan.blocksPerColumn);
-    if (w >= plan.slabs * plan.rowParts)
-        return;
-    const uint32_t slab = w % plan.slabs;
-    const uint32_t part = w / plan.slabs;
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t t = lane & 15;
-    const uint32_t rowInPart = (local % plan.blocksPerColumn) * kRowsPerBlock +
-                               wave * kRowsPerWave + lane / 16;
-    const uint32_t row = part * plan.rowsPerPart + rowInPart;
-    const uint32_t N = args.N;
-    const uint32_t col = slab * kSlabCols + t * 4;
-    const bool rowOk = rowInPart < plan.rowsPerPart && row < args.M;
-    const bool active = rowOk && col < N;
-
-    uint32_t p = 0, end = 0;
-    if (rowOk)
-    {
-        p = args.ROW[row];
-        end = args.ROW[row + 1];
-    }
-    const uint32_t colBytes = (col < N ? col : slab * kSlabCols) * 4;
-    float4 sum;
-    if (wave < kLdsWaves)
-        sum = RowSumsThroughLds(args, p, end - p, lane, colBytes,
-                                (__attribute__((address_space(3))) char*)lds + wave * kLdsWaveBytes);
-    else
-        sum = RowSumsInRegisters<16>(args, p, end, t, colBytes);
 
     if (active)
     {
@@ -543,18 +303,7 @@ static int LaunchSpmm(float* out, const float* V, const uint32_t* COL, const uin
         plan.columnsPerXcd = (plan.slabs * plan.rowParts + 7) / 8;
         const uint64_t grid = 8ull * plan.columnsPerXcd * plan.blocksPerColumn;
         SPH_REQUIRE(grid < (1ull << 31), "too many workgroups for one launch");
-        const char* var = getenv("SPH_SPMM_VAR");
-        const int variant = var ? atoi(var) : 0;  // 0: gathers into registers in every wavefront
-        const dim3 g(static_cast<uint32_t>(grid)), b(kThreads);
-        if (lanesPerRow == 16 && variant == 1)
-            hipLaunchKernelGGL((SpmmSlabSplit<1>), g, b, 0, stream, args, plan);
-        else if (lanesPerRow == 16 && variant == 2)
-            hipLaunchKernelGGL((SpmmSlabSplit<2>), g, b, 0, stream, args, plan);
-        else if (lanesPerRow == 16 && variant == 3)
-            hipLaunchKernelGGL((SpmmSlabSplit<3>), g, b, 0, stream, args, plan);
-        else if (lanesPerRow == 16 && variant == 4)
-            hipLaunchKernelGGL((SpmmSlabSplit<4>), g, b, 0, stream, args, plan);
-        else if (lanesPerRow == 16)
+        if (lanesPerRow == 16)
             hipLaunchKernelGGL(SpmmSlabVec4<16>, dim3(static_cast<uint32_t>(grid)),
                                dim3(kThreads), 0, stream, args, plan);
         else
