@@ -5,7 +5,7 @@
 //
 // Three kernels (and one for the odd columns, see below):
 //
-//   GemmF16Tile256  K a multiple of 32, N of 8, 16-byte aligned rows of A, at least three
+//   GemmF16Tile256  K >= 32 (a multiple of 32, or any K >= 64), N a multiple of 8, at least three
 //     quarters as many 256 x 256 tiles as compute units and at least three quarters of
 //     the tiled area inside the matrix (a variant with clamped copies and a guarded
 //     epilogue serves M, N that are not multiples of 256).  One workgroup of 8 wavefronts
@@ -26,7 +26,7 @@
 //     the 32 workgroups that land on one XCD (ids congruent mod 8) cover a compact
 //     8 x 4 block of tiles and share their A and B panels through that XCD's L2.
 //
-//   GemmF16Dma128   K a multiple of 32, N of 8, 16-byte aligned rows of A, any M: the
+//   GemmF16Dma128   the same conditions, any M: the
 //     same ingredients on 128 x 128 tiles with 4 wavefronts (v_mfma_f32_32x32x16_f16), for
 //     shapes with too few 256-tiles to fill the chip.
 //
@@ -34,9 +34,8 @@
 //     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
 //     widest that K, N, the strides and the bases allow), padded LDS rows.
 //
-// K = 32 q + r with r in {8, 16, 24} stays on the first two kernels:
-// a last step over [K - 32, K) in which the lanes holding values of k that were multiplied
-// already feed zeros.
+// K = 32 q + r, r != 0, K >= 64 stays on the first two kernels: a last step over [K - 32, K) in
+// which the fragment positions whose k was multiplied already are cleared.
 //
 // N = 8 q + r, r != 0: the first 8 q columns go to the first two kernels when they would take
 // that shape (the copies into LDS need no alignment, so rows of B and of out may start
@@ -63,7 +62,8 @@ struct GemmF16Args
     const _Float16* A;
     const _Float16* B;
     uint32_t M, N, K;
-    uint32_t lda;  // halves between consecutive rows of A (K unless a launch covers part of K)
+    uint32_t lda;  // halves between consecutive rows of A as stored (K; M for an A stored
+                   // K x M, unless a launch covers some of the rows)
     uint32_t ldb;  // halves between consecutive k-rows of a B stored K x N (N unless a launch
                    // covers some of the columns)
     uint32_t ldc;  // floats between consecutive rows of out (likewise)
@@ -72,6 +72,10 @@ struct GemmF16Args
     int64_t strideOut, strideA, strideB;
     uint32_t overwrite;
     uint32_t outVec;  // general kernel: out may be accessed 16 bytes at a time
+    // 128-tile kernel: rows / columns of this launch's out below these are computed but not
+    // stored (a launch over the last 8 rows or columns of a matrix whose other rows or columns
+    // another launch has written)
+    uint32_t rowStoreFrom, colStoreFrom;
 };
 
 // Transposing LDS read: within each group of 16 lanes, lane s supplies the
@@ -141,6 +145,28 @@ __device__ __forceinline__ void Store4(float* p, float4 v)
 __device__ __forceinline__ halfx8 Join(halfx4 lo, halfx4 hi)
 {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// K = 32 q + r, r != 0: the last K step runs over the window [K - 32, K), whose first 32 - r
+// positions the step before has multiplied already.  A fragment register holds 8 consecutive
+// positions (those of group `group`, 8 group .. 8 group + 7); TailMask gives the bits of the
+// ones that are new, KeepNew clears the others.  Both operands are cleared, so that a value
+// that lies in both windows counts once even when it is an infinity.
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uintx4 TailMask(uint32_t group, uint32_t repeated)
+{
+    uintx4 m;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        const uint32_t first = 8 * group + 2 * i;
+        m[i] = (first >= repeated ? 0x0000ffffu : 0u) | (first + 1 >= repeated ? 0xffff0000u : 0u);
+    }
+    return m;
+}
+__device__ __forceinline__ halfx8 KeepNew(halfx8 f, uintx4 m)
+{
+    return __builtin_bit_cast(halfx8, __builtin_bit_cast(uintx4, f) & m);
 }
 
 // Spreads consecutive workgroup ids, which the hardware deals round-robin to
@@ -268,7 +294,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     // or the column of B.  A K-contiguous operand takes the "A stage" layout and the 16-byte
     // fragment read described above, a k-major one the "B stage" layout and the transposing
     // read, whichever matrix it is, so the MFMAs and their order do not depend on the flags.
-    const uint32_t pitchA = TA ? args.M : args.lda;  // halves between rows of A as stored
+    const uint32_t pitchA = args.lda;  // halves between rows of A as stored
     const uint32_t pitchB = TB ? K : args.ldb;
     const uint32_t ldc = args.ldc;
     const _Float16* __restrict__ A = args.A + args.strideA * static_cast<int64_t>(unit) +
@@ -320,11 +346,11 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * pitchA * 2 : kTK * 2;
     const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * pitchB * 2;
 
-    // TAIL: K = 32 q + r with r = 8, 16 or 24.  The last of the q + 1 steps takes the window
+    // TAIL: K = 32 q + r with 0 < r < 32.  The last of the q + 1 steps takes the window
     // [K - 32, K), which lies inside the matrix and needs no other lane offsets (only its
     // start differs from a whole step's); its first 32 - r values of k were multiplied in
-    // step q - 1 already, so the lanes that hold them (k group g < 4 - r/8, for A and B alike)
-    // feed zeros to the MFMAs of that step instead of what they read from LDS.
+    // step q - 1 already, so the fragment positions that hold them (for A and B alike) are
+    // cleared before that step's MFMAs.
     const uint32_t steps = TAIL ? K / kTK + 1 : K / kTK;
     const size_t aLastBytes = TAIL ? (TA ? static_cast<size_t>(K - kTK) * pitchA * 2 : (K - kTK) * 2) : 0;
     const size_t bLastBytes = TAIL ? (TB ? (K - kTK) * 2 : static_cast<size_t>(K - kTK) * pitchB * 2) : 0;
@@ -417,16 +443,17 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     // One K step, stage index known at compile time.  BF holds this step's B fragments, BFN
     // receives the next step's.  EXTRA = vector memory operations other than stage copies
     // issued since the first half of the step before.
-    const bool laneRepeats = TAIL && g < 4 - (K % kTK) / 8;  // in the last step's window
+    const uintx4 tailMask = TailMask(g, kTK - K % kTK);
     auto stepWith = [&](auto stageC, uint32_t kt, auto extraC, halfx8 (&BF)[4],
                         halfx8 (&BFN)[4], auto&& behindBarrier) {
         constexpr int cur = decltype(stageC)::value;
         constexpr int nxt = (cur + 1) % kTStages;
         constexpr int EXTRA = decltype(extraC)::value;
-        const bool drop = TAIL && laneRepeats && kt == steps - 1;
+        const bool last = TAIL && kt == steps - 1;
+        const uintx4 keep = last ? tailMask : uintx4{ ~0u, ~0u, ~0u, ~0u };
         auto mask = [&](halfx8& f) {
             if constexpr (TAIL)
-                f = drop ? halfx8{} : f;
+                f = KeepNew(f, keep);
         };
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -683,8 +710,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 // 128 x 128 x 32 kernel with straight-to-LDS copies, ragged M and N
 // ---------------------------------------------------------------------------
 // For shapes the 256-tile kernel does not take (M or N not a multiple of 256) as long as K is a
-// multiple of 32 (or 32 q + 8, 16, 24), N of 8 and everything is 16-byte
-// aligned.  Four wavefronts (2 x 2, each 64 x 64 = 2 x 2 MFMA blocks) or eight (2 x 4, each
+// multiple of 32 (or any K from 64 up) and N of 8.  Four wavefronts (2 x 2, each 64 x 64 = 2 x 2 MFMA blocks) or eight (2 x 4, each
 // 64 x 32), four LDS stages of 16 KiB (two workgroups per compute unit), copies issued two steps
 // ahead, one barrier per step (placed, with the copies, between the MFMAs of the step's first
 // half), fragments read half a step ahead.
@@ -699,8 +725,8 @@ constexpr int kD = 128;
 constexpr int kDStages = 4;
 constexpr int kDStageBytes = 2 * kD * kTK * 2;  // A + B
 
-// TAIL: K = 32 q + r, r = 8, 16 or 24, handled as in the 256-tile kernel: a last step over the
-// window [K - 32, K) whose lanes holding the 32 - r values of k already multiplied feed zeros.
+// TAIL: K = 32 q + r, 0 < r < 32, handled as in the 256-tile kernel: a last step over the
+// window [K - 32, K) in which the positions of the 32 - r values of k already multiplied are cleared.
 template <bool TA, bool TB, bool TAIL, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args args)
 {
@@ -752,18 +778,18 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
     for (uint32_t i = 0; i < kCopiesPer; ++i)
     {
         const uint32_t j = wave + WAVES * i;
-        aLane[i] = TA ? laneKMajor(j, rowBase, M, M) : laneKContig(j, rowBase, M, args.lda);
+        aLane[i] = TA ? laneKMajor(j, rowBase, M, args.lda) : laneKContig(j, rowBase, M, args.lda);
         bLane[i] = TB ? laneKContig(j, colBase, N, K) : laneKMajor(j, colBase, N, args.ldb);
         aDst[i] = j * 1024;
         bDst[i] = kBytesA + j * 1024;
     }
-    const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * M * 2 : kTK * 2;
+    const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * args.lda * 2 : kTK * 2;
     const size_t bStepBytes = TB ? kTK * 2 : static_cast<size_t>(kTK) * args.ldb * 2;
     const uint32_t ldsBase = LdsAddress(lds);
     const uint32_t steps = TAIL ? K / kTK + 1 : K / kTK;
     // the last window starts K % 32 values of k after the one before it
     const uint32_t kLast = K % kTK;
-    const size_t aLastBytes = TA ? static_cast<size_t>(kLast) * M * 2 : kLast * 2;
+    const size_t aLastBytes = TA ? static_cast<size_t>(kLast) * args.lda * 2 : kLast * 2;
     const size_t bLastBytes = TB ? kLast * 2 : static_cast<size_t>(kLast) * args.ldb * 2;
     // Copy n (0..3: two of A, two of B) of the next step to fetch, into stage `stage`.  aSrc /
     // bSrc point at that step's slabs; surplus steps re-fetch the last one into a stage nobody
@@ -854,18 +880,18 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
             for (int v = 0; v < 16; ++v)
                 acc[i][j][v] = 0.f;
     // TAIL: a lane's fragments of half ks hold k group 2 ks + khalf of the step's window; in the
-    // last step the groups below 4 - r/8 repeat values of k the step before has multiplied
-    const uint32_t firstNewGroup = TAIL ? 4 - (K % kTK) / 8 : 0;
+    // last step the first 32 - r positions repeat values of k the step before has multiplied
+    const uintx4 tailMasks[2] = { TailMask(khalf, kTK - K % kTK), TailMask(2 + khalf, kTK - K % kTK) };
     auto maskRepeated = [&](halfx8 (&af)[2], halfx8 (&bf)[TN], int ks, bool lastStep) {
         if constexpr (TAIL)
         {
-            const bool drop = lastStep && 2 * ks + khalf < firstNewGroup;
+            const uintx4 keep = lastStep ? tailMasks[ks] : uintx4{ ~0u, ~0u, ~0u, ~0u };
 #pragma unroll
             for (int b = 0; b < 2; ++b)
-                af[b] = drop ? halfx8{} : af[b];
+                af[b] = KeepNew(af[b], keep);
 #pragma unroll
             for (int b = 0; b < TN; ++b)
-                bf[b] = drop ? halfx8{} : bf[b];
+                bf[b] = KeepNew(bf[b], keep);
         }
     };
     auto multiply = [&](const halfx8 (&af)[2], const halfx8 (&bf)[TN]) {
@@ -971,14 +997,26 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
             {
                 const uint32_t r = rowBase + waveM * 64 + i * 32 + l32;
                 const uint32_t c = colBase + (waveN * TN + j) * 32 + 8 * q + 4 * khalf;
-                if (r < M && c < N)
+                if (r < M && c < N && r >= args.rowStoreFrom)
                 {
                     float4 v = old[(i * TN + j) * 4 + q];
                     v.x += acc[i][j][4 * q + 0];
                     v.y += acc[i][j][4 * q + 1];
                     v.z += acc[i][j][4 * q + 2];
                     v.w += acc[i][j][4 * q + 3];
-                    Store4(out + static_cast<size_t>(r) * args.ldc + c, v);
+                    float* p = out + static_cast<size_t>(r) * args.ldc + c;
+                    if (c >= args.colStoreFrom)
+                        Store4(p, v);
+                    else
+                    {
+                        // a quad that straddles the first stored column
+                        if (c + 1 >= args.colStoreFrom)
+                            p[1] = v.y;
+                        if (c + 2 >= args.colStoreFrom)
+                            p[2] = v.z;
+                        if (c + 3 >= args.colStoreFrom)
+                            p[3] = v.w;
+                    }
                 }
             }
 }
@@ -1077,7 +1115,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
                 const uint32_t gk = k0 + q / 16;
                 const uint32_t gr = rowBase + (q % 16) * 8;
                 if (gk < K)
-                    v = load8(A + static_cast<size_t>(gk) * M + gr, gr, M);
+                    v = load8(A + static_cast<size_t>(gk) * args.lda + gr, gr, M);
             }
             else
             {
@@ -1248,8 +1286,8 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
 // out[M x r] (+)= A[M x K] * B[K x r] with r < 8: all of A is read for 2 M r K flops, so this
 // is a stream over A.  A workgroup owns 16 rows; its 8 wavefronts take every 8th K step of
 // 32.  The A fragment of v_mfma_f32_16x16x32_f16 comes straight from global memory: lane l
-// holds k = 8 (l / 16) .. + 7 of row l % 16 (one 16-byte load; K % 8 == 0 and 16-byte aligned
-// rows, which the kernels for the other columns need as well).  The B fragment (column l % 16,
+// holds k = 8 (l / 16) .. + 7 of row l % 16 (one 16-byte load from a 2-byte-aligned address; the
+// values of a piece that reaches past K are read one by one).  The B fragment (column l % 16,
 // the same k; zeros or don't-cares for columns from r on, zeros for k >= K):
 //   B stored N x K: one 16-byte load;
 //   B stored K x N: the r values of a k-row are the last of that row, so the 16 bytes that start
@@ -1286,18 +1324,29 @@ __global__ __launch_bounds__(kColsWaves * 64) void GemmF16Cols(const GemmF16Args
     // columns 8-15 ask for 0-7 again
     const uint32_t trOffset = (kLane + (x >> 2)) * 8 + 4 * (x & 1);
     floatx4 acc = { 0.f, 0.f, 0.f, 0.f };
-    auto fetchA = [&](uint32_t step) {
+    // 8 values of k from k0 on, zeros from K on; 16 bytes at once while they lie inside the row
+    auto fetch8 = [&](const _Float16* p, uint32_t k0) {
         halfx8 v = {};
-        if (step * kTK + kLane < K)
-            v = *reinterpret_cast<const halfx8*>(aRow + static_cast<size_t>(step) * kTK);
+        if (k0 + 8 <= K)
+            v = *reinterpret_cast<const halfx8a2*>(p);
+        else
+        {
+#pragma unroll
+            for (int e = 0; e < 7; ++e)
+                if (k0 + e < K)
+                    v[e] = p[e];
+        }
         return v;
+    };
+    auto fetchA = [&](uint32_t step) {
+        return fetch8(aRow + static_cast<size_t>(step) * kTK, step * kTK + kLane);
     };
     auto fetchB = [&](uint32_t step, uint32_t slabStart) {
         halfx8 v = {};
         if constexpr (TB)
         {
-            if (colExists && step * kTK + kLane < K)
-                v = *reinterpret_cast<const halfx8*>(bCol + static_cast<size_t>(step) * kTK);
+            if (colExists)
+                v = fetch8(bCol + static_cast<size_t>(step) * kTK, step * kTK + kLane);
         }
         else
         {
@@ -1414,8 +1463,6 @@ void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16
 // What one launch may assume about where its operands lie.
 struct F16Layout
 {
-    bool dmaA;  // A: base and unit stride multiples of 16 bytes
-    bool dmaB;  // B stored N x K: likewise (a B stored K x N is copied from any address)
     bool transA, transB;
 };
 
@@ -1441,15 +1488,15 @@ F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16
         static_cast<uint64_t>((M + kT - 1) / kT) * ((N + kT - 1) / kT) * kT * kT * 3;
     // lane offsets of the copies are 32-bit: 256 rows of a K-contiguous operand, 32 of a
     // k-major one (and 256 rows of out in the kernels that copy it)
-    const uint64_t pitchA = transA ? M : args.lda, pitchB = transB ? K : args.ldb;
+    const uint64_t pitchA = args.lda, pitchB = transB ? K : args.ldb;
     const bool offsetsFit = (transA ? 32 : 256) * pitchA * 2 + 8192 < (1ull << 32) &&
                             (transB ? 256 : 32) * pitchB * 2 + 8192 < (1ull << 32) &&
                             256ull * args.ldc * 4 + 8192 < (1ull << 32);
-    // K = 32 q + r, r = 8, 16 or 24: the straight-to-LDS kernels take the r values in a last,
+    // K = 32 q + r, 0 < r < 32: the straight-to-LDS kernels take the r values in a last,
     // partly masked step (measured 4096 x 4096 x 4080, operands stored plainly: 229 us on the
     // general kernel, 175 us with the r values left to a second launch, 128 us this way)
-    const bool tailInKernel = K % kTK != 0 && K % 8 == 0 && K >= 2 * kTK && args.lda == K;
-    const bool dma = lay.dmaA && (lay.dmaB || !transB) && K >= kTK &&
+    const bool tailInKernel = K % kTK != 0 && K >= 2 * kTK;
+    const bool dma = K >= kTK &&
                      (K % kTK == 0 || tailInKernel) && N % 8 == 0 && N >= 8 &&
                      (!transA || (M % 8 == 0 && M >= 8));
     if (dma && tiles256 >= minTiles && fills256 && offsetsFit)
@@ -1470,6 +1517,8 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     const bool plain = !transA && !transB;
     const bool whole256 = (M % kT == 0) && (N % kT == 0);
     const bool tile256 = kind == F16Kernel::kTile256;
+    SPH_REQUIRE(kind == F16Kernel::kDma128 || (args.rowStoreFrom == 0 && args.colStoreFrom == 0),
+                "only the 128-tile kernel leaves rows or columns unstored");
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -1549,7 +1598,7 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         // widest load every row start, every row length and every base allows (in halves);
         // an operand is read along its contiguous dimension: K (A), N (B), M (A stored K x M)
         // or K (B stored N x K)
-        const uint64_t mix = static_cast<uint64_t>(K) | (transA ? M : args.lda) |
+        const uint64_t mix = static_cast<uint64_t>(K) | (transA ? (M | args.lda) : args.lda) |
                              (transB ? K : (args.ldb | N)) |
                              static_cast<uint64_t>(args.strideA) |
                              static_cast<uint64_t>(args.strideB) |
@@ -1596,16 +1645,43 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     return SPH_OK;
 }
 
-// Picks the kernels for one call.  N = 8 q + r with r != 0 and a shape the straight-to-LDS
-// kernels would take at N = 8 q: they compute the first 8 q columns (row pitches of B and out
-// stay N) and the general kernel the last r, each output element still by one kernel
-// (measured 4096 x 4100 x 4096: 270 us on the general kernel alone).
+// Picks the kernels for one call.
+//
+// N = 8 q + r with r != 0 and a shape the straight-to-LDS kernels would take at N = 8 q: they
+// compute the first 8 q columns (row pitches of B and out stay N) and GemmF16Cols the last r
+// (measured 4096 x 4100 x 4096: 270 us on the general kernel alone, 130 us this way).
+//
+// An A stored K x M is copied 8 rows of the product at a time, so with it M = 8 q + r is split
+// the same way: the first 8 q rows, then the 128-tile kernel over the LAST 8 rows, which stores
+// only the r rows the first launch has not written.  With such an A the last r columns are
+// served the same way, by the 128-tile kernel over the last 8 columns (GemmF16Cols reads A
+// along K).  Every output element is still computed by one kernel.
 int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream)
 {
-    const uint32_t N = args.N;
+    const uint32_t M = args.M, N = args.N;
     const F16Kernel whole = PickF16(args, N, batch, lay);
+    if (whole != F16Kernel::kGeneral)
+        return LaunchF16Kernel(args, batch, whole, lay, stream);
+
+    if (lay.transA && M % 8 != 0 && M >= kG + 8)
+    {
+        GemmF16Args top = args;
+        top.M = M & ~7u;
+        GemmF16Args bottom = args;
+        bottom.M = 8;
+        bottom.A = args.A + (M - 8);
+        bottom.out = args.out + static_cast<size_t>(M - 8) * args.ldc;
+        bottom.rowStoreFrom = 8 - M % 8;
+        if (PickF16(top, N & ~7u, batch, lay) != F16Kernel::kGeneral &&
+            PickF16(bottom, N & ~7u, batch, lay) == F16Kernel::kDma128)
+        {
+            const int rc = LaunchF16(top, batch, lay, stream);
+            return rc != SPH_OK ? rc : LaunchF16(bottom, batch, lay, stream);
+        }
+    }
+
     const uint32_t wholeChunks = N & ~7u;
-    if (whole != F16Kernel::kGeneral || N % 8 == 0 || wholeChunks < kG)
+    if (N % 8 == 0 || wholeChunks < kG)
         return LaunchF16Kernel(args, batch, whole, lay, stream);
     const F16Kernel most = PickF16(args, wholeChunks, batch, lay);
     if (most == F16Kernel::kGeneral)
@@ -1616,6 +1692,18 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
     if (rc != SPH_OK)
         return rc;
     GemmF16Args right = args;
+    if (lay.transA)
+    {
+        // the last 8 columns, of which the first 8 - r are not stored
+        right.N = 8;
+        right.out = args.out + (N - 8);
+        right.B = args.B + (lay.transB ? static_cast<size_t>(N - 8) * args.K : N - 8);
+        right.colStoreFrom = 8 - N % 8;
+        const F16Kernel thin = PickF16(right, 8, batch, lay);
+        if (thin == F16Kernel::kDma128)
+            return LaunchF16Kernel(right, batch, thin, lay, stream);
+        right = args;
+    }
     right.N = N - wholeChunks;
     right.out = args.out + wholeChunks;
     right.B = args.B + (lay.transB ? static_cast<size_t>(wholeChunks) * args.K : wholeChunks);
@@ -1672,8 +1760,6 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     F16Layout lay{};
     lay.transA = transA;
     lay.transB = transB;
-    lay.dmaA = (reinterpret_cast<uintptr_t>(A) & 15u) == 0 && strideA % 8 == 0;
-    lay.dmaB = (reinterpret_cast<uintptr_t>(B) & 15u) == 0 && strideB % 8 == 0;
 
     GemmF16Args args{};
     args.out = out;
@@ -1682,7 +1768,7 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.M = M;
     args.N = N;
     args.K = K;
-    args.lda = K;
+    args.lda = transA ? M : K;
     args.ldb = N;
     args.ldc = N;
     args.strideOut = strideOut;

@@ -65,7 +65,7 @@ def test_tile256_ragged_exact_on_integers(dev, shape):
     assert np.array_equal(got, ref - C)
 
 
-# K = 32 q + r, r in {8, 16, 24}.  The 256-tile kernel takes the window [K - 32, K) as a last
+# K = 32 q + r, 0 < r < 32.  The 256-tile kernel takes the window [K - 32, K) as a last
 # step and masks the 32 - r values of k it has already multiplied (shapes with 192 tiles: whole
 # and ragged tiles, old contents added in the epilogue, every second step (20 steps and more:
 # K = 632 ends inside the written-out prefix, 648 after it) and every fourth (36 and more: 1144,
@@ -73,7 +73,12 @@ def test_tile256_ragged_exact_on_integers(dev, shape):
 @pytest.mark.parametrize("shape", [(256, 256, 72, 192), (250, 248, 80, 192), (4096, 3072, 88, 1),
                                    (256, 256, 632, 192), (256, 256, 648, 192), (512, 256, 1144, 96),
                                    (512, 256, 1168, 96), (256, 512, 1176, 96), (500, 504, 680, 48),
-                                   (300, 520, 168, 1), (128, 128, 72, 3), (1000, 1000, 1000, 1)])
+                                   (300, 520, 168, 1), (128, 128, 72, 3), (1000, 1000, 1000, 1),
+                                   # K % 8 != 0: rows of A (of a B stored N x K) start at addresses
+                                   # that are no multiples of 16 bytes, positions cleared one by one
+                                   (256, 256, 65, 192), (248, 256, 100, 192), (4096, 3072, 77, 1),
+                                   (512, 256, 1145, 96), (256, 256, 667, 192), (304, 520, 171, 1),
+                                   (128, 128, 95, 3), (1000, 1000, 999, 1), (304, 517, 77, 3)])
 @pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
                                    capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
 def test_k_tail_exact_on_integers(dev, shape, flags):
@@ -92,7 +97,7 @@ def test_k_tail_exact_on_integers(dev, shape, flags):
 
 
 @pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
-@pytest.mark.parametrize("K", [72, 80, 88])
+@pytest.mark.parametrize("K", [72, 80, 88, 73, 83])
 def test_k_tail_window_counts_an_infinity_once(dev, K, flags):
     """An infinity (and a 0 x Inf) at a k that lies in both of the last two step windows must
     come out exactly as in the CPU product: +Inf where the partner is positive, NaN where it is
@@ -102,7 +107,7 @@ def test_k_tail_window_counts_an_infinity_once(dev, K, flags):
     A = synth.small_integers(41, (batch, M, K), span=3).astype(np.float16)
     B = synth.small_integers(42, (batch, K, N), span=3).astype(np.float16)
     C = synth.small_integers(43, (batch, M, N), span=100)
-    k = K - 20                      # inside [K - 32, 32 q) for r = 8, 16 and 24
+    k = K - 20                      # inside [K - 32, 32 q) for r < 20
     A[:, 5, k] = np.inf
     B[:, k, :] = 1
     B[:, k, 7] = 0                  # Inf x 0
@@ -215,6 +220,34 @@ def test_column_count_not_a_multiple_of_eight(dev, shape, flags):
     Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
     ref = _oracle(C, A, B, M, N, K, batch=batch)
     # 37 guard floats after every unit of out: nothing may be written past column N - 1
+    pad = 37
+    padded = np.full((batch, M * N + pad), np.float32(-777.25), np.float32)
+    padded[:, :M * N] = C.reshape(batch, M * N)
+    for extra in (0, capi.SPH_GEMM_OVERWRITE):
+        got = h.gpu_gemm_f16(padded, As, Bs, M, N, K, batch=batch, stride_out=M * N + pad,
+                             flags=flags | extra)
+        assert np.array_equal(got[:, M * N:], padded[:, M * N:]), "guard floats overwritten"
+        want = ref - C if extra else ref
+        assert np.array_equal(got[:, :M * N].reshape(batch, M, N), want)
+
+
+# A stored K x M with M = 8 q + r, r != 0 (and N % 8 != 0 on top): the first 8 q rows as before,
+# the last 8 rows (columns) by a launch of the 128-tile kernel that stores only the r new ones.
+# 257 x 256 x 640 x 192: the whole-tile kernel with the old values added in its loop on top, 8 rows
+# below it; 4095 x 3077: ragged 256-tiles.
+@pytest.mark.parametrize("flags", [capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
+@pytest.mark.parametrize("shape", [(517, 304, 64, 3), (1001, 999, 96, 1), (4095, 3077, 77, 1),
+                                   (143, 143, 64, 5), (257, 256, 640, 192), (137, 136, 32, 1)])
+def test_transposed_a_with_ragged_rows_and_columns(dev, shape, flags):
+    M, N, K, batch = shape
+    h.announce("sph_gemm_f16f32, A stored K x M, M % 8 != 0", shape, "flags", flags)
+    span = 4 if K <= 256 else 3
+    A = synth.small_integers(81, (batch, M, K), span=span).astype(np.float16)
+    B = synth.small_integers(82, (batch, K, N), span=span).astype(np.float16)
+    C = synth.small_integers(83, (batch, M, N), span=100)
+    As = np.ascontiguousarray(A.swapaxes(1, 2))
+    Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
+    ref = _oracle(C, A, B, M, N, K, batch=batch)
     pad = 37
     padded = np.full((batch, M * N + pad), np.float32(-777.25), np.float32)
     padded[:, :M * N] = C.reshape(batch, M * N)
