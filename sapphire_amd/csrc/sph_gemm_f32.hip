@@ -7,8 +7,9 @@
 // which the K products are summed.
 //
 // Four kernels, chosen from the shape and the alignment of the operands:
-//   GemmF32DmaKernel     aligned operands with K a multiple of 16: slabs travel global -> LDS
-//                        without staging registers, several K steps ahead (the fast path);
+//   GemmF32DmaKernel     aligned operands with K a multiple of 4, at least 16: slabs travel
+//                        global -> LDS without staging registers, several K steps ahead (the
+//                        fast path; a K that is no multiple of the step ends in a partial step);
 //                        with more 64-tiles than resident workgroups each workgroup walks
 //                        several tiles and the copy stream runs across the tile boundaries;
 //   GemmF32Kernel        any shape and alignment: register-staged double buffering, 16-byte
@@ -454,7 +455,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
 }
 
 // ---------------------------------------------------------------------------
-// Pipelined variant for aligned operands with K % 16 == 0.
+// Pipelined variant for aligned operands with K % 4 == 0.
 //
 // The tiled kernel above holds a K step in registers between its global load and its LDS
 // store, so only one step can be in flight; with one workgroup per compute unit (mid-size
@@ -530,10 +531,17 @@ struct DmaTile
 // tile.  The launcher takes this form only for whole tiles, 16-byte output rows and a K
 // that fills the LDS ring a whole number of times, which keeps the number of loads and stores
 // per tile fixed.  Per element the arithmetic is the same as without WALK.
-template <int BM, int BN, int BK, int STAGES, bool TA, bool TB, bool WALK>
+//
+// TAIL: K = BK q + r with 0 < r < BK, r a multiple of 4.  The last of the q + 1 steps copies only
+// the r values of k that exist - a lane whose 16-byte chunk (K-contiguous operand) or row
+// (k-major operand) lies past K copies the slab's first chunk or row instead - and the
+// fragments of k >= K are replaced by zeros, for A and B alike, so the step adds what a
+// zero-padded slab would: the same sum, in the same order, as the register-staged kernel.
+template <int BM, int BN, int BK, int STAGES, bool TA, bool TB, bool WALK, bool TAIL = false>
 __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args args)
 {
     static_assert(BK == 16 || BK == 32, "K step of 16 or 32");
+    static_assert(!(WALK && TAIL), "a walk needs whole rings of steps");
     constexpr int WM = BM / 2;
     constexpr int WN = BN / 2;
     constexpr int TM = WM / 32;
@@ -582,17 +590,28 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         float* out;
         uint32_t rowBase, colBase;
         uint32_t aLane[kCopiesA], bLane[kCopiesB];
+        // TAIL: the same for the last, partial slab
+        uint32_t aTail[TAIL ? kCopiesA : 1], bTail[TAIL ? kCopiesB : 1];
     };
-    auto laneOffsetKContig = [&](uint32_t j, uint32_t xBase, uint32_t limit) {
+    const uint32_t steps = TAIL ? (K + BK - 1) / BK : K / BK;
+    const uint32_t lastValid = TAIL ? K - (steps - 1) * BK : BK;  // values of k in the last slab
+    const uint32_t wholeSteps = TAIL ? steps - 1 : steps;          // steps of the pipelined loop
+    // `valid`: values of k the slab holds
+    auto laneOffsetKContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t valid) {
         using T = TileA;  // chunk geometry depends on BK only
         const uint32_t x = j * T::kRowsPerCopyK + lane / T::kChunks;  // row inside the tile
-        const uint32_t c = (lane % T::kChunks) ^ T::Swizzle(x);
+        uint32_t c = (lane % T::kChunks) ^ T::Swizzle(x);
+        if (c * 4 + 4 > valid)
+            c = 0;
         const uint32_t gx = min(xBase + x, limit - 1);
         return (gx * K + c * 4) * 4u;
     };
-    auto laneOffsetXContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t rowBytes) {
+    auto laneOffsetXContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t rowBytes,
+                                 uint32_t valid) {
         const uint32_t b = j * 1024 + lane * 16;  // byte inside the unpadded slab
-        const uint32_t k = b / rowBytes;
+        uint32_t k = b / rowBytes;
+        if (k >= valid)
+            k = 0;
         const uint32_t col = (b % rowBytes) / 4;
         const uint32_t gx = min(xBase + col, limit - 4);
         return (k * limit + gx) * 4u;
@@ -619,15 +638,21 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         for (uint32_t i = 0; i < kCopiesA; ++i)
         {
             const uint32_t j = wave + 4 * i;
-            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, TileA::kRowBytes)
-                            : laneOffsetKContig(j, p.rowBase, M);
+            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, TileA::kRowBytes, BK)
+                            : laneOffsetKContig(j, p.rowBase, M, BK);
+            if constexpr (TAIL)
+                p.aTail[i] = TA ? laneOffsetXContig(j, p.rowBase, M, TileA::kRowBytes, lastValid)
+                                : laneOffsetKContig(j, p.rowBase, M, lastValid);
         }
 #pragma unroll
         for (uint32_t i = 0; i < kCopiesB; ++i)
         {
             const uint32_t j = wave + 4 * i;
-            p.bLane[i] = TB ? laneOffsetKContig(j, p.colBase, N)
-                            : laneOffsetXContig(j, p.colBase, N, TileB::kRowBytes);
+            p.bLane[i] = TB ? laneOffsetKContig(j, p.colBase, N, BK)
+                            : laneOffsetXContig(j, p.colBase, N, TileB::kRowBytes, BK);
+            if constexpr (TAIL)
+                p.bTail[i] = TB ? laneOffsetKContig(j, p.colBase, N, lastValid)
+                                : laneOffsetXContig(j, p.colBase, N, TileB::kRowBytes, lastValid);
         }
     };
     // LDS offsets of this wavefront's copies inside a stage
@@ -647,7 +672,6 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     const size_t bStepBytes = TB ? BK * 4 : static_cast<size_t>(BK) * N * 4;
     const uint32_t ldsBase =
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsVoidPtr)(lds)));
-    const uint32_t steps = K / BK;
 
     // ---- the copy stream ------------------------------------------------------------------
     // Copy n (0 .. kCopiesPerWave-1) of this wavefront's share of the next slab to fetch goes
@@ -664,14 +688,27 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 #pragma unroll
     for (uint32_t i = 0; i < kCopiesB; ++i)
         bLane[i] = cur.bLane[i];
+    uint32_t aLaneLast[TAIL ? kCopiesA : 1], bLaneLast[TAIL ? kCopiesB : 1];
+    if constexpr (TAIL)
+    {
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesA; ++i)
+            aLaneLast[i] = cur.aTail[i];
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesB; ++i)
+            bLaneLast[i] = cur.bTail[i];
+    }
     uint32_t slabsLeft = steps;  // of the tile being fetched, the one at aSrc / bSrc included
     bool haveNext = false;       // `nxt` describes a tile the copy stream has not reached yet
     auto issueOne = [&](uint32_t stage, uint32_t n) {
         const uint32_t base = ldsBase + stage * kStageBytes;
+        // TAIL: the slab at aSrc / bSrc is the tile's last one when slabsLeft is 1
+        const bool partial = TAIL && slabsLeft == 1;
         if (n < kCopiesA)
-            DmaToLds16(aLane[n], aSrc, base + aDst[n]);
+            DmaToLds16(partial ? aLaneLast[TAIL ? n : 0] : aLane[n], aSrc, base + aDst[n]);
         else
-            DmaToLds16(bLane[n - kCopiesA], bSrc, base + bDst[n - kCopiesA]);
+            DmaToLds16(partial ? bLaneLast[TAIL ? n - kCopiesA : 0] : bLane[n - kCopiesA], bSrc,
+                       base + bDst[n - kCopiesA]);
     };
     auto advance = [&]() {
         if (--slabsLeft != 0)
@@ -762,6 +799,27 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
                         stage + bFrag[j] + TileB::RowOffsetXContig(8 * q + e) +
                         khalf * (TileB::RowOffsetXContig(4) - TileB::RowOffsetXContig(0)));
             }
+        }
+    };
+    // TAIL: zeros for the fragments of k >= K, put in where the fragments are used so that the
+    // reads above stay in flight behind the MFMAs of the block before.  The number of valid k
+    // is a multiple of 4: the 4 values of a fragment exist together or not.
+    auto dropMissing = [&](float (&a)[TM][4], float (&b)[TN][4], uint32_t q, uint32_t valid) {
+        if constexpr (TAIL)
+        {
+            const bool exists = 8 * q + 4 * khalf < valid;
+#pragma unroll
+            for (uint32_t e = 0; e < 4; ++e)
+            {
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    a[i][e] = exists ? a[i][e] : 0.f;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    b[j][e] = exists ? b[j][e] : 0.f;
+            }
+            // all of them ahead of the block's MFMAs, which then issue back to back
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto multiply = [&](const float (&a)[TM][4], const float (&b)[TN][4]) {
@@ -941,7 +999,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 #pragma unroll
             for (uint32_t u = 0; u < STAGES; ++u)
             {
-                if (!WALK && s0 + u >= steps)
+                if (!WALK && s0 + u >= wholeSteps)
                     break;
                 const char* stage = lds + u * kStageBytes;
                 const char* next = lds + ((u + 1) % STAGES) * kStageBytes;
@@ -970,8 +1028,26 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         }
         else
         {
-            for (uint32_t s0 = 0; s0 < steps; s0 += STAGES)
+            for (uint32_t s0 = 0; s0 < wholeSteps; s0 += STAGES)
                 ringCycle(s0, std::false_type{});
+        }
+        if constexpr (TAIL)
+        {
+            // The partial step on its own, so that the steps before it carry no selects.  Its
+            // slab has landed (the step before waited for it, or the prologue did) and its
+            // first fragments are in fa[0] / fb[0]; no copy that is still in flight targets its
+            // stage.
+            const char* stage = lds + ((steps - 1) % STAGES) * kStageBytes;
+#pragma unroll
+            for (uint32_t q = 0; q < kBlocks; ++q)
+            {
+                if (q + 1 < kBlocks)
+                    loadFragments(fa[(q + 1) & 1], fb[(q + 1) & 1], stage, q + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                dropMissing(fa[q & 1], fb[q & 1], q, lastValid);
+                multiply(fa[q & 1], fb[q & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
 
         if constexpr (!WALK)
@@ -1391,7 +1467,10 @@ void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dm
     const dim3 block(kThreads);
     if (dma)
     {
-        if (big)
+        if (big && args.K % 16 != 0)
+            hipLaunchKernelGGL((GemmF32DmaKernel<128, 128, 16, 4, TA, TB, false, true>), grid,
+                               block, 0, stream, args);
+        else if (big)
             hipLaunchKernelGGL((GemmF32DmaKernel<128, 128, 16, 4, TA, TB, false>), grid, block, 0,
                                stream, args);
         else if (walk)
@@ -1400,9 +1479,12 @@ void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dm
         else if (args.K % 32 == 0)
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB, false>), grid, block, 0,
                                stream, args);
-        else
+        else if (args.K % 16 == 0)
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 16, 6, TA, TB, false>), grid, block, 0,
                                stream, args);
+        else
+            hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB, false, true>), grid,
+                               block, 0, stream, args);
         return;
     }
     if (big)
@@ -1496,7 +1578,8 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
     // straight-to-LDS pipeline: whole K steps, 16-byte chunks everywhere, at least one chunk
     // per clamped edge, and lane offsets that fit 32 bits
-    const bool dma = aligned && args.K >= kBK && args.K % kBK == 0 && args.M >= 4 && args.N >= 4 &&
+    // (K = 16 q + 4, 8 or 12: a last, partial step)
+    const bool dma = aligned && args.K >= kBK && args.K % 4 == 0 && args.M >= 4 && args.N >= 4 &&
                      static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
                      static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
     const uint64_t tiles128 =

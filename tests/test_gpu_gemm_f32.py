@@ -124,6 +124,39 @@ def test_unaligned_bases(dev):
            "unaligned")
 
 
+# K = 16 q + 4, 8 or 12 on the straight-to-LDS kernel: a last, partial step whose missing values
+# of k count as zeros.  (M, N, K): one step only, 64-tiles with K steps of 32, 128-tiles with K
+# steps of 16, ragged edges.  Bars: the CPU loop within tolerance, and bit for bit the same
+# product from operands that start 4 bytes into their allocation, which the register-staged
+# kernel multiplies (same order of the K products, zero padding included).
+@pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
+                                   capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B,
+                                   capi.SPH_GEMM_OVERWRITE])
+@pytest.mark.parametrize("dims", [(512, 512, 20), (1024, 1024, 1000), (640, 384, 36),
+                                  (2048, 2048, 120), (300, 260, 44), (4096, 2048, 72),
+                                  (1024, 1024, 28)])
+def test_partial_last_k_step(dev, dims, flags):
+    M, N, K = dims
+    h.announce("sph_gemm_f32_ex, K % 16 != 0", dims, "flags", flags)
+    A = synth.uniform(401, (M, K))
+    B = synth.uniform(402, (K, N))
+    C = synth.uniform(403, (M, N))
+    As = np.ascontiguousarray(A.T) if flags & capi.SPH_GEMM_TRANS_A else A
+    Bs = np.ascontiguousarray(B.T) if flags & capi.SPH_GEMM_TRANS_B else B
+    got = h.gpu_gemm_f32_ex(C, As, Bs, M, N, K, flags)
+    start = np.zeros((256, N), np.float32) if flags & capi.SPH_GEMM_OVERWRITE else C[:256].copy()
+    ref = po.gemm_rows(start, A[:256], B, 256, N, K)
+    assert h.normalised_error(got[:256], ref, np.abs(A[:256]), np.abs(B)) <= TOL_F32
+    shifted = [np.concatenate([np.zeros(1, np.float32), x.ravel()]) for x in (As, Bs, C)]
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in shifted)
+    capi.call("sph_gemm_f32_ex", dC.at(4), dA.at(4), dB.at(4), M, N, K, 1, M * N, M * K, K * N,
+              flags)
+    other = dC.download(np.float32, (M * N + 1,))[1:].reshape(M, N)
+    for d in (dA, dB, dC):
+        d.release()
+    assert np.array_equal(got.view(np.uint32), other.view(np.uint32))
+
+
 def test_grouped_plan_with_modulo_quirk(dev):
     """{b,1,M,K} x {b,M,K,N} -> {b,M,M,N} (BroadcastTest.cpp:32-34): the walk picks
     A matrix i % b, which is not NumPy broadcasting; the leaves go out as one launch."""
