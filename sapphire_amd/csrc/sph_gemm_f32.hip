@@ -7,9 +7,10 @@
 // which the K products are summed.
 //
 // Four kernels, chosen from the shape and the alignment of the operands:
-//   GemmF32DmaKernel     aligned operands with K a multiple of 4, at least 16: slabs travel
-//                        global -> LDS without staging registers, several K steps ahead (the
-//                        fast path; a K that is no multiple of the step ends in a partial step);
+//   GemmF32DmaKernel     16-byte aligned bases, K >= 16, an N (an M, for A stored K x M) that
+//                        is a multiple of 4: slabs travel global -> LDS without staging
+//                        registers, several K steps ahead (the fast path; a K that is no
+//                        multiple of the step ends in a partial step);
 //                        with more 64-tiles than resident workgroups each workgroup walks
 //                        several tiles and the copy stream runs across the tile boundaries;
 //   GemmF32Kernel        any shape and alignment: register-staged double buffering, 16-byte
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
 }
 
 // ---------------------------------------------------------------------------
-// Pipelined variant for aligned operands with K % 4 == 0.
+// Pipelined variant.
 //
 // The tiled kernel above holds a K step in registers between its global load and its LDS
 // store, so only one step can be in flight; with one workgroup per compute unit (mid-size
@@ -532,11 +533,12 @@ struct DmaTile
 // that fills the LDS ring a whole number of times, which keeps the number of loads and stores
 // per tile fixed.  Per element the arithmetic is the same as without WALK.
 //
-// TAIL: K = BK q + r with 0 < r < BK, r a multiple of 4.  The last of the q + 1 steps copies only
-// the r values of k that exist - a lane whose 16-byte chunk (K-contiguous operand) or row
-// (k-major operand) lies past K copies the slab's first chunk or row instead - and the
-// fragments of k >= K are replaced by zeros, for A and B alike, so the step adds what a
-// zero-padded slab would: the same sum, in the same order, as the register-staged kernel.
+// TAIL: K = BK q + r with 0 < r < BK.  The last of the q + 1 steps copies only the r values of
+// k that exist - a lane whose 16-byte chunk (K-contiguous operand) or row (k-major operand)
+// lies past K copies the slab's first chunk or row instead, one whose chunk reaches past K the
+// 4 values that end at K - and the fragments are put right where they are used (zeros for
+// k >= K, for A and B alike), so the step adds what a zero-padded slab would: the same sum,
+// in the same order, as the register-staged kernel.
 template <int BM, int BN, int BK, int STAGES, bool TA, bool TB, bool WALK, bool TAIL = false>
 __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args args)
 {
@@ -597,14 +599,21 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     const uint32_t lastValid = TAIL ? K - (steps - 1) * BK : BK;  // values of k in the last slab
     const uint32_t wholeSteps = TAIL ? steps - 1 : steps;          // steps of the pipelined loop
     // `valid`: values of k the slab holds
+    // TAIL: operand bases are moved kTailBias bytes down and lane offsets up, because the chunk
+    // that ends at K may begin before the slab does
+    constexpr uint32_t kTailBias = TAIL ? 16 : 0;
     auto laneOffsetKContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t valid) {
         using T = TileA;  // chunk geometry depends on BK only
         const uint32_t x = j * T::kRowsPerCopyK + lane / T::kChunks;  // row inside the tile
-        uint32_t c = (lane % T::kChunks) ^ T::Swizzle(x);
-        if (c * 4 + 4 > valid)
-            c = 0;
+        const uint32_t c = (lane % T::kChunks) ^ T::Swizzle(x);
+        // float offset of the chunk inside the slab's row, + 4: a chunk that reaches past
+        // `valid` copies the last 4 values of the row (its LDS slot then holds k = valid - 4
+        // .. valid - 1), one that begins past it the row's first chunk
+        uint32_t k4 = c * 4 + 4;
+        if (k4 > valid)
+            k4 = k4 - 4 < valid ? valid : 4;
         const uint32_t gx = min(xBase + x, limit - 1);
-        return (gx * K + c * 4) * 4u;
+        return (gx * K + k4) * 4u - 16u + kTailBias;
     };
     auto laneOffsetXContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t rowBytes,
                                  uint32_t valid) {
@@ -614,7 +623,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
             k = 0;
         const uint32_t col = (b % rowBytes) / 4;
         const uint32_t gx = min(xBase + col, limit - 4);
-        return (k * limit + gx) * 4u;
+        return (k * limit + gx) * 4u + kTailBias;
     };
     auto locate = [&](uint32_t logicalTile, Place& p) {
         uint32_t tm, tn, unit;
@@ -622,14 +631,16 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         if (args.entries != nullptr)
         {
             const SphGemmEntry e = args.entries[unit];
-            p.a = reinterpret_cast<const char*>(args.A + e.aOff);
-            p.b = reinterpret_cast<const char*>(args.B + e.bOff);
+            p.a = reinterpret_cast<const char*>(args.A + e.aOff) - kTailBias;
+            p.b = reinterpret_cast<const char*>(args.B + e.bOff) - kTailBias;
             p.out = args.out + e.outOff;
         }
         else
         {
-            p.a = reinterpret_cast<const char*>(args.A + args.strideA * static_cast<int64_t>(unit));
-            p.b = reinterpret_cast<const char*>(args.B + args.strideB * static_cast<int64_t>(unit));
+            p.a = reinterpret_cast<const char*>(args.A + args.strideA * static_cast<int64_t>(unit)) -
+                  kTailBias;
+            p.b = reinterpret_cast<const char*>(args.B + args.strideB * static_cast<int64_t>(unit)) -
+                  kTailBias;
             p.out = args.out + args.strideOut * static_cast<int64_t>(unit);
         }
         p.rowBase = tm * BM;
@@ -801,22 +812,56 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
             }
         }
     };
-    // TAIL: zeros for the fragments of k >= K, put in where the fragments are used so that the
-    // reads above stay in flight behind the MFMAs of the block before.  The number of valid k
-    // is a multiple of 4: the 4 values of a fragment exist together or not.
+    // TAIL: what the fragments of block q would be if the last slab were zero-padded to a whole
+    // step; `valid` values of k exist.  Put in where the fragments are used so that the reads
+    // above stay in flight behind the MFMAs of the block before.
+    //   k-major operand: zeros for k >= valid.
+    //   K-contiguous operand: chunks that begin at or past `valid` become zeros; the chunk
+    //   that reaches past it was copied from valid - 4 on, so its values are moved down by
+    //   4 - valid % 4 places and followed by zeros.
     auto dropMissing = [&](float (&a)[TM][4], float (&b)[TN][4], uint32_t q, uint32_t valid) {
         if constexpr (TAIL)
         {
-            const bool exists = 8 * q + 4 * khalf < valid;
+            const uint32_t k0 = 8 * q + 4 * khalf;  // k of this lane's fragment element 0
+            const uint32_t shift = (4 - valid % 4) % 4;
+            const bool whole = k0 + 4 <= valid;
+            const bool reaches = !whole && k0 < valid;
+            auto fixKContig = [&](float (&f)[4]) {
+                float g[4];
 #pragma unroll
-            for (uint32_t e = 0; e < 4; ++e)
+                for (uint32_t e = 0; e < 4; ++e)
+                {
+                    // element e + shift of the copied chunk, a zero when that is past its end
+                    float moved = 0.f;
+                    moved = (shift == 1 && e + 1 < 4) ? f[(e + 1) & 3] : moved;
+                    moved = (shift == 2 && e + 2 < 4) ? f[(e + 2) & 3] : moved;
+                    moved = (shift == 3 && e + 3 < 4) ? f[(e + 3) & 3] : moved;
+                    g[e] = whole ? f[e] : (reaches ? moved : 0.f);
+                }
+#pragma unroll
+                for (uint32_t e = 0; e < 4; ++e)
+                    f[e] = g[e];
+            };
+            auto fixKMajor = [&](float (&f)[4]) {
+#pragma unroll
+                for (uint32_t e = 0; e < 4; ++e)
+                    f[e] = k0 + e < valid ? f[e] : 0.f;
+            };
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
             {
+                if constexpr (TA)
+                    fixKMajor(a[i]);
+                else
+                    fixKContig(a[i]);
+            }
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    a[i][e] = exists ? a[i][e] : 0.f;
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    b[j][e] = exists ? b[j][e] : 0.f;
+            for (int j = 0; j < TN; ++j)
+            {
+                if constexpr (TB)
+                    fixKContig(b[j]);
+                else
+                    fixKMajor(b[j]);
             }
             // all of them ahead of the block's MFMAs, which then issue back to back
             __builtin_amdgcn_sched_barrier(0);
@@ -1578,8 +1623,12 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
     // straight-to-LDS pipeline: whole K steps, 16-byte chunks everywhere, at least one chunk
     // per clamped edge, and lane offsets that fit 32 bits
-    // (K = 16 q + 4, 8 or 12: a last, partial step)
-    const bool dma = aligned && args.K >= kBK && args.K % 4 == 0 && args.M >= 4 && args.N >= 4 &&
+    // (a K that is no multiple of the step: a last, partial one).  The copies take 16 bytes from
+    // any 4-byte-aligned address, so only an operand stored k-major, which is copied 4 rows or
+    // columns of the product at a time, needs a row length that is a multiple of 4.
+    const bool dmaLayout = allowVector && basesAligned && (!transA || args.M % 4 == 0) &&
+                           (transB || args.N % 4 == 0);
+    const bool dma = dmaLayout && args.K >= kBK && args.M >= 4 && args.N >= 4 &&
                      static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
                      static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
     const uint64_t tiles128 =

@@ -124,7 +124,7 @@ def test_unaligned_bases(dev):
            "unaligned")
 
 
-# K = 16 q + 4, 8 or 12 on the straight-to-LDS kernel: a last, partial step whose missing values
+# A K that is no multiple of 16 on the straight-to-LDS kernel: a last, partial step whose missing values
 # of k count as zeros.  (M, N, K): one step only, 64-tiles with K steps of 32, 128-tiles with K
 # steps of 16, ragged edges.  Bars: the CPU loop within tolerance, and bit for bit the same
 # product from operands that start 4 bytes into their allocation, which the register-staged
@@ -134,7 +134,12 @@ def test_unaligned_bases(dev):
                                    capi.SPH_GEMM_OVERWRITE])
 @pytest.mark.parametrize("dims", [(512, 512, 20), (1024, 1024, 1000), (640, 384, 36),
                                   (2048, 2048, 120), (300, 260, 44), (4096, 2048, 72),
-                                  (1024, 1024, 28)])
+                                  (1024, 1024, 28),
+                                  # K % 4 != 0: rows of a K-contiguous operand start at 4-byte
+                                  # aligned addresses, the chunk that ends at K is copied shifted
+                                  (512, 512, 17), (1024, 1024, 1001), (640, 384, 35),
+                                  (2048, 2048, 122), (300, 260, 47), (4096, 2048, 65),
+                                  (1024, 1024, 33), (512, 768, 131)])
 def test_partial_last_k_step(dev, dims, flags):
     M, N, K = dims
     h.announce("sph_gemm_f32_ex, K % 16 != 0", dims, "flags", flags)
