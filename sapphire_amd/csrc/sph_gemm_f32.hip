@@ -40,6 +40,9 @@ namespace
 {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+// four floats that need only be 4-byte aligned: the rows of out start anywhere when N is no
+// multiple of 4, and a 16-byte vector memory access only asks for dword alignment
+typedef floatx4 floatx4a4 __attribute__((aligned(4)));
 
 constexpr int kThreads = 256;
 constexpr int kBK = 16;
@@ -222,14 +225,14 @@ __device__ __forceinline__ constexpr uint32_t KOfPair(uint32_t t, uint32_t khalf
 }
 
 // out (+)= acc for the TM x TN blocks of 32 x 32 one wavefront owns; rowBase / colBase are
-// the wavefront's first row and column.  `wide`: N % 4 == 0 and 16-byte aligned output rows.
+// the wavefront's first row and column.  Four consecutive columns that all exist are accessed
+// 16 bytes at a time, whatever the alignment of the row.
 template <int TM, int TN>
 __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* __restrict__ out,
                                           uint32_t rowBase, uint32_t colBase, uint32_t M,
                                           uint32_t N, uint32_t l32, uint32_t khalf,
                                           const GemmF32Args& args)
 {
-    const bool wide = args.outVec != 0;
     const bool accumulate = args.overwrite == 0;
     const float* __restrict__ bias = args.bias;
     const bool relu = args.relu != 0;
@@ -261,8 +264,11 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
                 else if (accumulate && r < M && c < N)
                 {
                     const float* p = out + static_cast<size_t>(r) * N + c;
-                    if (wide)
-                        v = *reinterpret_cast<const float4*>(p);
+                    if (c + 4 <= N)
+                    {
+                        const floatx4 w = *reinterpret_cast<const floatx4a4*>(p);
+                        v = make_float4(w[0], w[1], w[2], w[3]);
+                    }
                     else
                     {
                         v.x = p[0];
@@ -297,8 +303,8 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
                         v.w = v.w > 0 ? v.w : 0;
                     }
                     float* p = out + static_cast<size_t>(r) * N + c;
-                    if (wide)
-                        *reinterpret_cast<float4*>(p) = v;
+                    if (c + 4 <= N)
+                        *reinterpret_cast<floatx4a4*>(p) = floatx4{ v.x, v.y, v.z, v.w };
                     else
                     {
                         p[0] = v.x;
