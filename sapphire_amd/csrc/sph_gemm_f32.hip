@@ -14,12 +14,14 @@
 //                        with more 64-tiles than resident workgroups each workgroup walks
 //                        several tiles and the copy stream runs across the tile boundaries;
 //   GemmF32Kernel        any shape and alignment: register-staged double buffering, 16-byte
-//                        loads when possible, scalar predicated loads otherwise (e.g. the
-//                        reference's random test sizes,
+//                        loads when possible, scalar predicated loads otherwise (small K,
+//                        misaligned bases, e.g. some of the reference's random test sizes,
 //                        Tests/UnitTests/Sources/FunctionTest/GemmTest.cpp:26-33);
 //   GemmF32SkinnyKernel  few output tiles: 16 x 16 or 32 x 32 tiles with K split over the
 //                        wavefronts of a workgroup;
 //   GemvRowKernel        a single output row.
+// An N that is no multiple of 4 is split by the launcher: the first 4 q columns to the kernels
+// above, the last ones to the few-tile kernel.
 // The first two share one decomposition: a workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile
 // of one M x N unit, BM = BN = 128 or 64 (whichever loads the busiest compute unit less),
 // and they add the K products of an element in the same order, so which of them
@@ -54,6 +56,9 @@ struct GemmF32Args
     const float* B;
     const SphGemmEntry* entries;  // device table, or null for stride arithmetic
     uint32_t M, N, K;
+    // floats between consecutive rows of B as stored K x N and of out: N, unless a launch covers
+    // some of the columns of a wider matrix
+    uint32_t ldb, ldc;
     uint32_t tilesM, tilesN;
     uint32_t tilesTotal;  // tilesM * tilesN * units
     uint32_t perXcd;      // ceil(tilesTotal / 8): the grid has 8 * perXcd workgroups
@@ -75,7 +80,7 @@ struct GemmF32Args
 template <int BX, int QUADS, bool VEC>
 __device__ __forceinline__ void FetchKContig(float4 (&stage)[QUADS], const float* __restrict__ src,
                                              uint32_t tid, uint32_t xBase, uint32_t xLimit,
-                                             uint32_t k0, uint32_t K)
+                                             uint32_t k0, uint32_t K)  // rows of K floats
 {
 #pragma unroll
     for (int i = 0; i < QUADS; ++i)
@@ -109,7 +114,7 @@ __device__ __forceinline__ void FetchKContig(float4 (&stage)[QUADS], const float
 template <int BX, int QUADS, bool VEC>
 __device__ __forceinline__ void FetchXContig(float4 (&stage)[QUADS], const float* __restrict__ src,
                                              uint32_t tid, uint32_t xBase, uint32_t xLimit,
-                                             uint32_t k0, uint32_t K)
+                                             uint32_t k0, uint32_t K, uint32_t pitch)
 {
 #pragma unroll
     for (int i = 0; i < QUADS; ++i)
@@ -122,7 +127,7 @@ __device__ __forceinline__ void FetchXContig(float4 (&stage)[QUADS], const float
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (gk < K)
         {
-            const float* p = src + static_cast<size_t>(gk) * xLimit + gx;
+            const float* p = src + static_cast<size_t>(gk) * pitch + gx;
             if (VEC)
             {
                 if (gx < xLimit)
@@ -263,7 +268,7 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
                 }
                 else if (accumulate && r < M && c < N)
                 {
-                    const float* p = out + static_cast<size_t>(r) * N + c;
+                    const float* p = out + static_cast<size_t>(r) * args.ldc + c;
                     if (c + 4 <= N)
                     {
                         const floatx4 w = *reinterpret_cast<const floatx4a4*>(p);
@@ -302,7 +307,7 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
                         v.z = v.z > 0 ? v.z : 0;
                         v.w = v.w > 0 ? v.w : 0;
                     }
-                    float* p = out + static_cast<size_t>(r) * N + c;
+                    float* p = out + static_cast<size_t>(r) * args.ldc + c;
                     if (c + 4 <= N)
                         *reinterpret_cast<floatx4a4*>(p) = floatx4{ v.x, v.y, v.z, v.w };
                     else
@@ -370,13 +375,13 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
 
     auto fetch = [&](uint32_t k0) {
         if constexpr (TA)
-            FetchXContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K);
+            FetchXContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K, M);
         else
             FetchKContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K);
         if constexpr (TB)
             FetchKContig<BN, B_QUADS, VEC>(stageB, B, tid, colBase, N, k0, K);
         else
-            FetchXContig<BN, B_QUADS, VEC>(stageB, B, tid, colBase, N, k0, K);
+            FetchXContig<BN, B_QUADS, VEC>(stageB, B, tid, colBase, N, k0, K, args.ldb);
     };
 
     auto stash = [&](int buf) {
@@ -621,15 +626,15 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         const uint32_t gx = min(xBase + x, limit - 1);
         return (gx * K + k4) * 4u - 16u + kTailBias;
     };
-    auto laneOffsetXContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t rowBytes,
-                                 uint32_t valid) {
+    auto laneOffsetXContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t pitch,
+                                 uint32_t rowBytes, uint32_t valid) {
         const uint32_t b = j * 1024 + lane * 16;  // byte inside the unpadded slab
         uint32_t k = b / rowBytes;
         if (k >= valid)
             k = 0;
         const uint32_t col = (b % rowBytes) / 4;
         const uint32_t gx = min(xBase + col, limit - 4);
-        return (k * limit + gx) * 4u + kTailBias;
+        return (k * pitch + gx) * 4u + kTailBias;
     };
     auto locate = [&](uint32_t logicalTile, Place& p) {
         uint32_t tm, tn, unit;
@@ -655,10 +660,10 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         for (uint32_t i = 0; i < kCopiesA; ++i)
         {
             const uint32_t j = wave + 4 * i;
-            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, TileA::kRowBytes, BK)
+            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, M, TileA::kRowBytes, BK)
                             : laneOffsetKContig(j, p.rowBase, M, BK);
             if constexpr (TAIL)
-                p.aTail[i] = TA ? laneOffsetXContig(j, p.rowBase, M, TileA::kRowBytes, lastValid)
+                p.aTail[i] = TA ? laneOffsetXContig(j, p.rowBase, M, M, TileA::kRowBytes, lastValid)
                                 : laneOffsetKContig(j, p.rowBase, M, lastValid);
         }
 #pragma unroll
@@ -666,10 +671,11 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         {
             const uint32_t j = wave + 4 * i;
             p.bLane[i] = TB ? laneOffsetKContig(j, p.colBase, N, BK)
-                            : laneOffsetXContig(j, p.colBase, N, TileB::kRowBytes, BK);
+                            : laneOffsetXContig(j, p.colBase, N, args.ldb, TileB::kRowBytes, BK);
             if constexpr (TAIL)
                 p.bTail[i] = TB ? laneOffsetKContig(j, p.colBase, N, lastValid)
-                                : laneOffsetXContig(j, p.colBase, N, TileB::kRowBytes, lastValid);
+                                : laneOffsetXContig(j, p.colBase, N, args.ldb, TileB::kRowBytes,
+                                                    lastValid);
         }
     };
     // LDS offsets of this wavefront's copies inside a stage
@@ -686,7 +692,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     locate(logical, cur);
 
     const size_t aStepBytes = TA ? static_cast<size_t>(BK) * M * 4 : BK * 4;
-    const size_t bStepBytes = TB ? BK * 4 : static_cast<size_t>(BK) * N * 4;
+    const size_t bStepBytes = TB ? BK * 4 : static_cast<size_t>(BK) * args.ldb * 4;
     const uint32_t ldsBase =
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsVoidPtr)(lds)));
 
@@ -912,8 +918,8 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
             {
                 uint32_t r, c;
                 where(idx, r, c);
-                old[idx] =
-                    *reinterpret_cast<const floatx4*>(cur.out + static_cast<size_t>(r) * N + c);
+                old[idx] = *reinterpret_cast<const floatx4a4*>(
+                    cur.out + static_cast<size_t>(r) * args.ldc + c);
             }
         }
         else
@@ -953,7 +959,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
                         if (relu)
                             v[e] = v[e] > 0 ? v[e] : 0;
                     }
-                    *reinterpret_cast<floatx4*>(cur.out + static_cast<size_t>(r) * N + c) = v;
+                    *reinterpret_cast<floatx4a4*>(cur.out + static_cast<size_t>(r) * args.ldc + c) = v;
                 }
     };
 
@@ -1244,7 +1250,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         if constexpr (TB)
             return loadAlongK(bPtr, colOk, g);
         else
-            return loadAcrossK(bPtr, N, colOk, g);
+            return loadAcrossK(bPtr, args.ldb, colOk, g);
     };
     // operands swapped: the result block comes out indexed [column][row], which leaves 4
     // consecutive columns of one row in a lane
@@ -1315,7 +1321,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         const uint32_t c = tn * TILE + 4 * kLaneGroups * q + 4 * kh;
         if (c >= N)
             continue;
-        float* p = out + static_cast<size_t>(row) * N + c;
+        float* p = out + static_cast<size_t>(row) * args.ldc + c;
         if (args.bias != nullptr || args.relu || args.sgd)
         {
             // fused epilogues: (0 + bias) + product with an optional ReLU (out not read), or the
@@ -1563,7 +1569,35 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
            bool transA, bool transB, hipStream_t stream)
 {
     GemmF32Args args = base;
-    args.outVec = (outOffsetsAligned && (args.N % 4 == 0) &&
+    const bool part = base.ldc != 0;  // a launch over some of the columns of a wider product
+    if (!part)
+    {
+        args.ldb = args.N;
+        args.ldc = args.N;
+    }
+    // N = 4 q + r, r != 0: the rows of a B stored K x N are copied 4 columns at a time, so the
+    // first 4 q columns go to the kernels below (row pitches stay N) and the last r to the
+    // kernel for narrow products; every output element is still computed by one kernel
+    // (measured 4096 x 4095 x 4096: 1615 us on the register-staged kernel's 4-byte loads).
+    // A B stored N x K would not need this; it is split all the same, so that a product does
+    // not depend on how its operands are stored.
+    if (!part && args.N % 4 != 0 && args.N >= 68 && args.M > 1 && args.K >= kBK)
+    {
+        const uint32_t whole = args.N & ~3u;
+        GemmF32Args left = args;
+        left.N = whole;
+        const int rc = Launch(left, units, allowVector, outOffsetsAligned, transA, transB, stream);
+        if (rc != SPH_OK)
+            return rc;
+        GemmF32Args right = args;
+        right.N = args.N - whole;
+        right.B = args.B + (transB ? static_cast<size_t>(whole) * args.K : whole);
+        right.out = args.out + whole;
+        if (args.bias != nullptr)
+            right.bias = args.bias + whole;
+        return Launch(right, units, allowVector, outOffsetsAligned, transA, transB, stream);
+    }
+    args.outVec = (outOffsetsAligned && (args.N % 4 == 0) && (args.ldc % 4 == 0) &&
                    (reinterpret_cast<uintptr_t>(args.out) & 15u) == 0)
                       ? 1u
                       : 0u;
@@ -1571,11 +1605,12 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         ((reinterpret_cast<uintptr_t>(args.A) | reinterpret_cast<uintptr_t>(args.B)) & 15u) == 0;
     // row lengths of the two operands as stored
     const uint32_t lda = transA ? args.M : args.K;
-    const uint32_t ldb = transB ? args.K : args.N;
+    const uint32_t ldb = transB ? args.K : args.ldb;
     const bool aligned = allowVector && basesAligned && (lda % 4 == 0) && (ldb % 4 == 0);
 
     // a single output row is a reduction over the rows of B, not a matrix-core job
-    if (args.M == 1 && !transB && args.entries == nullptr && args.K >= 64 && units <= 65535)
+    if (args.M == 1 && !transB && args.entries == nullptr && args.K >= 64 && units <= 65535 &&
+        args.ldb == args.N)
     {
         hipLaunchKernelGGL(GemvRowKernel, dim3((args.N + 63) / 64, units), dim3(kGemvWaves * 64),
                            0, stream, args);
@@ -1586,7 +1621,8 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // few 64 x 64 tiles and a long K: split K inside the workgroup instead
     const uint64_t tiles64 =
         static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
-    if (tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) && args.K >= 64)
+    if ((tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) && args.K >= 64) ||
+        (part && args.N < 4))
     {
         // 16 x 16 tiles while there are at most four per compute unit: a quarter of the
         // matrix-core work per workgroup on four times as many compute units, and less of a
@@ -1595,7 +1631,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         const uint64_t blocks16 =
             static_cast<uint64_t>((args.M + 15) / 16) * ((args.N + 15) / 16) * units;
         const uint32_t tile =
-            blocks16 <= static_cast<uint64_t>(sph::ComputeUnits()) * 4 ? 16u : 32u;
+            (blocks16 <= static_cast<uint64_t>(sph::ComputeUnits()) * 4 || args.N < 4) ? 16u : 32u;
         args.tilesM = (args.M + tile - 1) / tile;
         args.tilesN = (args.N + tile - 1) / tile;
         const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
@@ -1632,7 +1668,8 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // (a K that is no multiple of the step: a last, partial one).  The copies take 16 bytes from
     // any 4-byte-aligned address, so only an operand stored k-major, which is copied 4 rows or
     // columns of the product at a time, needs a row length that is a multiple of 4.
-    const bool dmaLayout = allowVector && basesAligned && (!transA || args.M % 4 == 0) &&
+    // (unit strides and table offsets may be anything)
+    const bool dmaLayout = basesAligned && (!transA || args.M % 4 == 0) &&
                            (transB || args.N % 4 == 0);
     const bool dma = dmaLayout && args.K >= kBK && args.M >= 4 && args.N >= 4 &&
                      static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
@@ -1668,7 +1705,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // kernel would need more than 256 registers for it and lose its second resident workgroup
     // (measured 4096^3: 921 -> 966 us), so it keeps one tile per workgroup.
     const uint32_t slotsPerXcd = static_cast<uint32_t>(cus / 8 * 2);
-    const bool walk = dma && !big && args.perXcd > slotsPerXcd && args.outVec != 0 &&
+    const bool walk = dma && !big && args.perXcd > slotsPerXcd &&
                       args.M % 64 == 0 && args.N % 64 == 0 && args.K % 128 == 0 &&
                       (reinterpret_cast<uintptr_t>(args.bias) & 15u) == 0;
     const dim3 grid((walk ? slotsPerXcd : args.perXcd) * 8);
@@ -1747,7 +1784,7 @@ int sph_gemm_f32_ex(float* out, const float* A, const float* B, uint32_t M, uint
     args.strideOut = strideOut;
     args.strideA = strideA;
     args.strideB = strideB;
-    const bool stridesAligned = (strideA % 4 == 0) && (strideB % 4 == 0);
+    const bool stridesAligned = batch == 1 || ((strideA % 4 == 0) && (strideB % 4 == 0));
     return Launch(args, batch, stridesAligned, strideOut % 4 == 0 || batch == 1,
                   (flags & SPH_GEMM_TRANS_A) != 0, (flags & SPH_GEMM_TRANS_B) != 0, stream);
 }

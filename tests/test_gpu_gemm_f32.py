@@ -162,6 +162,42 @@ def test_partial_last_k_step(dev, dims, flags):
     assert np.array_equal(got.view(np.uint32), other.view(np.uint32))
 
 
+# N = 4 q + r, r != 0, from 68 columns up: the first 4 q columns on the tiled kernels with the
+# row pitches left at N, the last r on the kernel for narrow products.  Guard floats behind
+# every unit of out catch a store past column N - 1.
+@pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
+                                   capi.SPH_GEMM_OVERWRITE])
+@pytest.mark.parametrize("dims", [(512, 1026, 64, 1), (1000, 999, 100, 1), (300, 70, 40, 3),
+                                  (64, 69, 16, 5), (2048, 2049, 128, 1), (128, 1031, 2050, 1)])
+def test_column_count_not_a_multiple_of_four(dev, dims, flags):
+    M, N, K, batch = dims
+    h.announce("sph_gemm_f32_ex, N % 4 != 0", dims, "flags", flags)
+    A = synth.uniform(411, (batch, M, K))
+    B = synth.uniform(412, (batch, K, N))
+    C = synth.uniform(413, (batch, M, N))
+    As = np.ascontiguousarray(A.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_A else A
+    Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
+    pad = 29
+    padded = np.full((batch, M * N + pad), np.float32(-777.25), np.float32)
+    padded[:, :M * N] = C.reshape(batch, M * N)
+    got = h.gpu_gemm_f32_ex(padded, As, Bs, M, N, K, flags, batch=batch, stride_out=M * N + pad)
+    assert np.array_equal(got[:, M * N:], padded[:, M * N:]), "guard floats overwritten"
+    got = got[:, :M * N].reshape(batch, M, N)
+    rows = min(M, 128)
+    for b in range(batch):
+        start = (np.zeros((rows, N), np.float32) if flags & capi.SPH_GEMM_OVERWRITE
+                 else C[b, :rows].copy())
+        ref = po.gemm_rows(start, A[b, :rows], B[b], rows, N, K)
+        err = h.normalised_error(got[b, :rows], ref, np.abs(A[b, :rows]), np.abs(B[b]))
+        assert err <= TOL_F32, (b, err)
+        # the last rows too: every row block writes the narrow part
+        start = (np.zeros((rows, N), np.float32) if flags & capi.SPH_GEMM_OVERWRITE
+                 else C[b, M - rows:].copy())
+        ref = po.gemm_rows(start, A[b, M - rows:], B[b], rows, N, K)
+        err = h.normalised_error(got[b, M - rows:], ref, np.abs(A[b, M - rows:]), np.abs(B[b]))
+        assert err <= TOL_F32, (b, err)
+
+
 def test_grouped_plan_with_modulo_quirk(dev):
     """{b,1,M,K} x {b,M,K,N} -> {b,M,M,N} (BroadcastTest.cpp:32-34): the walk picks
     A matrix i % b, which is not NumPy broadcasting; the leaves go out as one launch."""
