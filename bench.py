@@ -61,7 +61,7 @@ def parse():
                    help="also time the neighbouring kernels (backward pass, conversions, CSR x "
                         "CSR, one-pass kernels; reported under 'others')")
     p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
-                                      "csr", "spgemm"], default=None,
+                                      "csr", "spgemm", "shapes"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
     p.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                    help="untimed run-up before each timed leg that lets the clock reach its "
@@ -299,6 +299,46 @@ def bench_mlp_backward(capi, synth, steps, warmup, direct, graph=False, fused_up
         buf.release()
     flops = 2.0 * 2.0 * batch * sum(sizes[l] * sizes[l + 1] for l in range(3))
     return event_ms, flops
+
+
+# Shapes off the kernels' natural grid: a K that is no multiple of the K step, an N (or M) that is
+# no multiple of the copy width, operands stored the other way round.
+OFF_GRID_F16 = [(4096, 4096, 4096), (4096, 4096, 4080), (4096, 4096, 4095), (4096, 4100, 4096),
+                (4096, 4095, 4096), (4095, 4095, 4095), (2048, 2052, 2048), (1024, 1024, 1001)]
+OFF_GRID_F32 = [(1024, 1024, 1024), (1024, 1024, 1000), (1024, 1024, 1001), (1000, 1000, 1000),
+                (1001, 1001, 1001), (1024, 1026, 1024), (2048, 2048, 2047), (2048, 2050, 2048),
+                (4096, 4096, 4096), (4096, 4095, 4096), (4096, 4096, 4100)]
+
+
+def bench_off_grid(capi, synth, steps, warmup):
+    """Event time per launch of one M x N x K product per shape and storage flag set."""
+    rows = []
+
+    def one(entry, M, N, K, flags, A, B):
+        C = np.zeros((M, N), np.float32)
+        dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+
+        def launch():
+            capi.call(entry, dC.ptr, dA.ptr, dB.ptr, M, N, K, 1, M * N, M * K, K * N, flags)
+
+        ms, _ = timed_launches(capi, launch, steps, warmup)
+        for d in (dA, dB, dC):
+            d.release()
+        rows.append({"entry_point": entry, "M": M, "N": N, "K": K, "flags": flags,
+                     "launch_ms": ms, "tflops": 2.0 * M * N * K / (ms * 1e-3) / 1e12})
+
+    for M, N, K in OFF_GRID_F16:
+        A = synth.normal(1, (M, K), 1.0 / np.sqrt(K)).astype(np.float16)
+        B = synth.normal(2, (K, N), 1.0 / np.sqrt(K)).astype(np.float16)
+        for flags in (0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B):
+            # the values only have to be typical; the buffers are read with the other pitch
+            one("sph_gemm_f16f32", M, N, K, flags, A, B)
+    for M, N, K in OFF_GRID_F32:
+        A = synth.uniform(1, (M, K))
+        B = synth.uniform(2, (K, N))
+        for flags in (0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B):
+            one("sph_gemm_f32_ex", M, N, K, flags, A, B)
+    return rows
 
 
 def bench_sgd_step(capi, steps, warmup, mib=64):
@@ -623,6 +663,9 @@ def main():
         result["gemm_f32"] = {"workload": "configuration 2: A[16,512,512] x B[1,512,512] fp32",
                               "launch_ms": ms, "tflops": tf,
                               "frac_fp32_mfma_peak": tf / PEAK_FP32_TFLOPS}
+
+    if args.only == "shapes":
+        result["off_grid_shapes"] = bench_off_grid(capi, synth, min(args.steps, 20), 3)
 
     if args.only == "csr":
         ms_csr, ms_one, ms_dense, dense_bytes, csr_bytes = bench_csr_conversion(
