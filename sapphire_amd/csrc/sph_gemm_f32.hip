@@ -1700,15 +1700,18 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
 
     // More 64-tiles than workgroups that can be resident (two per compute unit): each
     // workgroup walks several tiles with the copy pipeline running across the tile boundaries
-    // (configuration 2: 37.8 -> 35.9 us).  Only for whole tiles, 16-byte output rows and a K
+    // (configuration 2: 37.8 -> 35.9 us).  With fewer tiles every workgroup takes one, and the
+    // form still pays because the old values of out are requested at the tile's first step
+    // instead of after its last (1024^3: 18.7 -> 18.3 us, 1024 x 1024 x 256: 7.9 -> 7.4 us).
+    // Only for whole tiles and a K
     // that fills the 4-stage ring of 32-wide steps a whole number of times.  The 128-tile
     // kernel would need more than 256 registers for it and lose its second resident workgroup
     // (measured 4096^3: 921 -> 966 us), so it keeps one tile per workgroup.
     const uint32_t slotsPerXcd = static_cast<uint32_t>(cus / 8 * 2);
-    const bool walk = dma && !big && args.perXcd > slotsPerXcd &&
+    const bool walk = dma && !big &&
                       args.M % 64 == 0 && args.N % 64 == 0 && args.K % 128 == 0 &&
                       (reinterpret_cast<uintptr_t>(args.bias) & 15u) == 0;
-    const dim3 grid((walk ? slotsPerXcd : args.perXcd) * 8);
+    const dim3 grid((walk ? std::min(slotsPerXcd, args.perXcd) : args.perXcd) * 8);
     if (transA && transB)
         LaunchTiled<true, true>(args, grid, big, aligned, dma, walk, stream);
     else if (transA)
