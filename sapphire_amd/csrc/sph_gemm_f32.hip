@@ -57,8 +57,15 @@ struct GemmF32Args
     const SphGemmEntry* entries;  // device table, or null for stride arithmetic
     uint32_t M, N, K;
     // floats between consecutive rows of B as stored K x N and of out: N, unless a launch covers
-    // some of the columns of a wider matrix
-    uint32_t ldb, ldc;
+    // some of the columns of a wider matrix; likewise of an A stored K x M: M, unless a launch
+    // covers some of the rows
+    uint32_t ldb, ldc, lda;
+    // tiled kernels: rows of this launch's out below this one are computed but not stored (a
+    // launch over the last 4 rows of a product whose other rows another launch has written)
+    uint32_t rowStoreFrom;
+    uint32_t split;      // launcher: 1 = a part of the columns, 2 = a part of the rows, 4 = the
+                         // tiled kernels have been chosen
+    uint32_t basesOk;    // launcher: the caller's A and B start on 16-byte boundaries
     uint32_t tilesM, tilesN;
     uint32_t tilesTotal;  // tilesM * tilesN * units
     uint32_t perXcd;      // ceil(tilesTotal / 8): the grid has 8 * perXcd workgroups
@@ -293,7 +300,7 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
             {
                 const uint32_t r = rowBase + i * 32 + l32;
                 const uint32_t c = colBase + j * 32 + 8 * q + 4 * khalf;
-                if (r < M && c < N)
+                if (r < M && c < N && r >= args.rowStoreFrom)
                 {
                     float4 v = old[(i * TN + j) * 4 + q];
                     v.x = Combine(args, v.x, acc[i][j][4 * q + 0]);
@@ -375,7 +382,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32Kernel(const GemmF32Args args
 
     auto fetch = [&](uint32_t k0) {
         if constexpr (TA)
-            FetchXContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K, M);
+            FetchXContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K, args.lda);
         else
             FetchKContig<BM, A_QUADS, VEC>(stageA, A, tid, rowBase, M, k0, K);
         if constexpr (TB)
@@ -660,10 +667,11 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         for (uint32_t i = 0; i < kCopiesA; ++i)
         {
             const uint32_t j = wave + 4 * i;
-            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, M, TileA::kRowBytes, BK)
+            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, args.lda, TileA::kRowBytes, BK)
                             : laneOffsetKContig(j, p.rowBase, M, BK);
             if constexpr (TAIL)
-                p.aTail[i] = TA ? laneOffsetXContig(j, p.rowBase, M, M, TileA::kRowBytes, lastValid)
+                p.aTail[i] = TA ? laneOffsetXContig(j, p.rowBase, M, args.lda, TileA::kRowBytes,
+                                                    lastValid)
                                 : laneOffsetKContig(j, p.rowBase, M, lastValid);
         }
 #pragma unroll
@@ -691,7 +699,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     Place cur, nxt;
     locate(logical, cur);
 
-    const size_t aStepBytes = TA ? static_cast<size_t>(BK) * M * 4 : BK * 4;
+    const size_t aStepBytes = TA ? static_cast<size_t>(BK) * args.lda * 4 : BK * 4;
     const size_t bStepBytes = TB ? BK * 4 : static_cast<size_t>(BK) * args.ldb * 4;
     const uint32_t ldsBase =
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsVoidPtr)(lds)));
@@ -1242,7 +1250,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
     const float* bPtr = TB ? B + static_cast<size_t>(min(col, N - 1)) * K : B + min(col, N - 1);
     auto loadA = [&](uint32_t g) {
         if constexpr (TA)
-            return loadAcrossK(aPtr, M, rowOk, g);
+            return loadAcrossK(aPtr, args.lda, rowOk, g);
         else
             return loadAlongK(aPtr, rowOk, g);
     };
@@ -1569,27 +1577,34 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
            bool transA, bool transB, hipStream_t stream)
 {
     GemmF32Args args = base;
-    const bool part = base.ldc != 0;  // a launch over some of the columns of a wider product
-    if (!part)
+    if (args.split == 0)
     {
         args.ldb = args.N;
         args.ldc = args.N;
+        args.lda = args.M;
+        args.basesOk =
+            ((reinterpret_cast<uintptr_t>(args.A) | reinterpret_cast<uintptr_t>(args.B)) & 15u) == 0
+                ? 1u
+                : 0u;
     }
+    const bool part = (args.split & 1u) != 0;  // some of the columns of a wider product
     // N = 4 q + r, r != 0: the rows of a B stored K x N are copied 4 columns at a time, so the
     // first 4 q columns go to the kernels below (row pitches stay N) and the last r to the
     // kernel for narrow products; every output element is still computed by one kernel
     // (measured 4096 x 4095 x 4096: 1615 us on the register-staged kernel's 4-byte loads).
     // A B stored N x K would not need this; it is split all the same, so that a product does
     // not depend on how its operands are stored.
-    if (!part && args.N % 4 != 0 && args.N >= 68 && args.M > 1 && args.K >= kBK)
+    if (args.split == 0 && args.N % 4 != 0 && args.N >= 68 && args.M > 1 && args.K >= kBK)
     {
         const uint32_t whole = args.N & ~3u;
         GemmF32Args left = args;
+        left.split = 1;
         left.N = whole;
         const int rc = Launch(left, units, allowVector, outOffsetsAligned, transA, transB, stream);
         if (rc != SPH_OK)
             return rc;
         GemmF32Args right = args;
+        right.split = 1;
         right.N = args.N - whole;
         right.B = args.B + (transB ? static_cast<size_t>(whole) * args.K : whole);
         right.out = args.out + whole;
@@ -1597,20 +1612,52 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
             right.bias = args.bias + whole;
         return Launch(right, units, allowVector, outOffsetsAligned, transA, transB, stream);
     }
+    // M = 4 q + r, r != 0, with A stored K x M: its rows are copied 4 rows of the product at a
+    // time.  The first 4 q rows go to the kernels below; the last 4 rows are launched once more
+    // on their own and store only the r rows the first launch has not written.  Both launches
+    // run the same kernels as an A stored M x K would, so the storage does not change a bit.
+    const bool dmaShape = args.basesOk != 0 && args.K >= kBK && args.N >= 4 &&
+                          (transB || args.N % 4 == 0);
+    // few 64 x 64 tiles and a long K: the kernel that splits K inside the workgroup (decided on
+    // the whole product, so that its parts run the kernels the whole would)
+    const uint64_t tiles64 =
+        static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
+    const bool fewTiles = (args.split & 4u) == 0 &&
+                          ((tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) &&
+                            args.K >= 64) ||
+                           (part && args.N < 4));
+    if ((args.split & 2u) == 0 && transA && args.M % 4 != 0 && args.M >= 68 && dmaShape &&
+        !fewTiles)
+    {
+        GemmF32Args top = args;
+        top.split |= 6u;
+        top.M = args.M & ~3u;
+        const int rc = Launch(top, units, allowVector, outOffsetsAligned, transA, transB, stream);
+        if (rc != SPH_OK)
+            return rc;
+        GemmF32Args bottom = args;
+        bottom.split |= 6u;
+        bottom.M = 4;
+        bottom.A = args.A + (args.M - 4);
+        bottom.out = args.out + static_cast<size_t>(args.M - 4) * args.ldc;
+        bottom.rowStoreFrom = 4 - args.M % 4;
+        return Launch(bottom, units, allowVector, outOffsetsAligned, transA, transB, stream);
+    }
     args.outVec = (outOffsetsAligned && (args.N % 4 == 0) && (args.ldc % 4 == 0) &&
                    (reinterpret_cast<uintptr_t>(args.out) & 15u) == 0)
                       ? 1u
                       : 0u;
+    // (of this launch: a part of a wider product may start anywhere)
     const bool basesAligned =
         ((reinterpret_cast<uintptr_t>(args.A) | reinterpret_cast<uintptr_t>(args.B)) & 15u) == 0;
     // row lengths of the two operands as stored
-    const uint32_t lda = transA ? args.M : args.K;
+    const uint32_t lda = transA ? args.lda : args.K;
     const uint32_t ldb = transB ? args.K : args.ldb;
     const bool aligned = allowVector && basesAligned && (lda % 4 == 0) && (ldb % 4 == 0);
 
     // a single output row is a reduction over the rows of B, not a matrix-core job
     if (args.M == 1 && !transB && args.entries == nullptr && args.K >= 64 && units <= 65535 &&
-        args.ldb == args.N)
+        args.split == 0)
     {
         hipLaunchKernelGGL(GemvRowKernel, dim3((args.N + 63) / 64, units), dim3(kGemvWaves * 64),
                            0, stream, args);
@@ -1618,11 +1665,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         return SPH_OK;
     }
 
-    // few 64 x 64 tiles and a long K: split K inside the workgroup instead
-    const uint64_t tiles64 =
-        static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
-    if ((tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) && args.K >= 64) ||
-        (part && args.N < 4))
+    if (fewTiles)
     {
         // 16 x 16 tiles while there are at most four per compute unit: a quarter of the
         // matrix-core work per workgroup on four times as many compute units, and less of a
@@ -1669,7 +1712,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // any 4-byte-aligned address, so only an operand stored k-major, which is copied 4 rows or
     // columns of the product at a time, needs a row length that is a multiple of 4.
     // (unit strides and table offsets may be anything)
-    const bool dmaLayout = basesAligned && (!transA || args.M % 4 == 0) &&
+    const bool dmaLayout = args.basesOk != 0 && (!transA || args.M % 4 == 0) &&
                            (transB || args.N % 4 == 0);
     const bool dma = dmaLayout && args.K >= kBK && args.M >= 4 && args.N >= 4 &&
                      static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&

@@ -25,7 +25,10 @@ FLAG_SETS = [capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
 SHAPES = [(1, 1, 1), (3, 5, 7), (64, 64, 64), (65, 33, 17), (128, 96, 40), (257, 130, 31),
           (512, 384, 100), (2048, 2048, 64), (4096, 2048, 32), (32, 32, 1024), (40, 24, 515),
           (8, 200, 4096), (1000, 10, 1000), (256, 256, 96), (640, 600, 72), (1, 200, 64),
-          (1, 1000, 4096), (1, 64, 63)]
+          (1, 1000, 4096), (1, 64, 63),
+          # M % 4 != 0 from 68 rows up: an A stored K x M is multiplied in two launches (the last 4
+          # rows once more, of which only the new ones are stored)
+          (1001, 512, 64), (301, 262, 100), (2049, 2048, 96), (69, 4096, 20), (1023, 1001, 1001)]
 
 
 def bits(x):
