@@ -1663,7 +1663,9 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
     if (whole != F16Kernel::kGeneral)
         return LaunchF16Kernel(args, batch, whole, lay, stream);
 
-    if (lay.transA && M % 8 != 0 && M >= kG + 8)
+    // (the parts must not fall back to the general kernel, which stores every row: N has to be
+    // a multiple of 8 or wide enough for the column split below)
+    if (lay.transA && M % 8 != 0 && M >= kG + 8 && (N % 8 == 0 || (N & ~7u) >= kG))
     {
         GemmF16Args top = args;
         top.M = M & ~7u;

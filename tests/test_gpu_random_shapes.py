@@ -15,10 +15,10 @@ from tests import helpers as h
 
 pytestmark = pytest.mark.gpu
 
-DIMS = [1, 2, 7, 10, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 96, 100, 127, 128, 129, 200, 256, 300,
-        511, 512, 640, 1000, 1024]
-DEPTHS = [1, 3, 8, 15, 16, 17, 32, 40, 63, 64, 65, 72, 96, 128, 200, 256, 500, 512, 515, 1024,
-          2048]
+DIMS = [1, 2, 7, 10, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 69, 96, 100, 127, 128, 129, 137, 200,
+        256, 257, 300, 511, 512, 640, 1000, 1001, 1024]
+DEPTHS = [1, 3, 8, 15, 16, 17, 18, 32, 40, 63, 64, 65, 67, 72, 96, 100, 128, 200, 256, 500, 512,
+          515, 1001, 1024, 2048]
 GUARD = 64
 
 
@@ -32,7 +32,7 @@ def _check_guards(back, guard):
     assert np.array_equal(back[-GUARD:], guard), "write past the end of out"
 
 
-@pytest.mark.parametrize("block", range(6))
+@pytest.mark.parametrize("block", range(10))
 def test_fp32_flags_on_random_shapes(dev, block):
     rng = np.random.default_rng(9000 + block)
     for it in range(16):
@@ -57,7 +57,7 @@ def test_fp32_flags_on_random_shapes(dev, block):
         assert err <= 1e-4, (M, N, K, flags, err)
 
 
-@pytest.mark.parametrize("block", range(4))
+@pytest.mark.parametrize("block", range(8))
 def test_fp16_exact_on_random_shapes(dev, block):
     rng = np.random.default_rng(9100 + block)
     for it in range(16):
@@ -65,14 +65,19 @@ def test_fp16_exact_on_random_shapes(dev, block):
         N = int(rng.choice(DIMS + [264, 520, 1004]))
         K = int(rng.choice(DEPTHS + [24, 88, 168, 1000]))
         batch = int(rng.choice([1, 1, 2, 3]))
-        flags = int(rng.choice([0, capi.SPH_GEMM_OVERWRITE]))
+        # the first four blocks as they always were; the others with the operands stored
+        # either way
+        flags = (int(rng.choice([0, capi.SPH_GEMM_OVERWRITE])) if block < 4
+                 else int(rng.integers(0, 8)))
         h.announce("sph_gemm_f16f32 random", (M, N, K, batch), "flags", flags)
         seed = 200000 * (block + 1) + 10 * it
         A = synth.small_integers(seed, (batch, M, K), span=3).astype(np.float16)
         B = synth.small_integers(seed + 1, (batch, K, N), span=3).astype(np.float16)
         C = synth.small_integers(seed + 2, (batch, M, N), span=100)
         guard, padded = _guarded(C)
-        dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, padded))
+        As = np.ascontiguousarray(A.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_A else A
+        Bs = np.ascontiguousarray(B.swapaxes(1, 2)) if flags & capi.SPH_GEMM_TRANS_B else B
+        dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (As, Bs, padded))
         capi.call("sph_gemm_f16f32", dC.at(4 * GUARD), dA.ptr, dB.ptr, M, N, K, batch, M * N,
                   M * K, K * N, flags)
         back = dC.download(np.float32, padded.shape)
@@ -81,5 +86,5 @@ def test_fp16_exact_on_random_shapes(dev, block):
         _check_guards(back, guard)
         ref = po.gemm_rows(C.copy(), A.astype(np.float32), B.astype(np.float32), M, N, K,
                            batch=batch, threads=8)
-        want = ref - C if flags else ref
+        want = ref - C if flags & capi.SPH_GEMM_OVERWRITE else ref
         assert np.array_equal(back[GUARD:-GUARD].reshape(C.shape), want), (M, N, K, batch, flags)
