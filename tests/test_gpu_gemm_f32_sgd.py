@@ -34,7 +34,10 @@ CASES = [(784, 1024, 1024, TA), (1024, 1024, 1024, TA), (1024, 10, 1024, TA),
          (1, 1024, 1024, 0), (1, 10, 1024, 0), (1, 70, 300, 0),
          (2048, 2048, 256, 0), (2048, 2048, 128, TA), (4096, 2048, 64, TB),
          (130, 70, 200, 0), (65, 33, 17, TA | TB), (5, 3, 9, TB), (256, 256, 96, 0),
-         (32, 32, 1024, 0), (40, 24, 515, TA)]
+         (32, 32, 1024, 0), (40, 24, 515, TA),
+         # ragged extents that the launcher splits: N % 4 != 0, M % 4 != 0 with A stored K x M, a
+         # K that ends in a partial step
+         (512, 1026, 100, 0), (301, 262, 1001, TA), (1000, 999, 77, TB), (1001, 130, 64, TA | TB)]
 
 
 @pytest.mark.parametrize("case", CASES)
