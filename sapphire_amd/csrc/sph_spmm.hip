@@ -10,9 +10,9 @@
 // single add into out.  Each output element is owned by exactly one lane which
 // walks the row front to back, so the result is bit-identical to that loop.
 //
-// Two mappings.
+// Three mappings.
 //
-// SpmmSlabVec4 (dense width a multiple of 4, aligned bases): the dense columns are cut
+// SpmmSlabVec4 (the first 4 * (N / 4) dense columns): the dense columns are cut
 // into slabs of 64 (32 for narrow operands); all workgroups that run on one XCD (ids
 // congruent mod 8) work on the same slab, so the part of B an XCD gathers from (K x 64
 // floats, 2 MiB at K = 8192) stays resident in that XCD's L2 instead of being streamed
@@ -22,9 +22,11 @@
 // one 256-byte gather per row, eight of them in flight per lane.  The loop has no branches:
 // entries past the end of a row gather row 0 of B and a select keeps them out of the sum.
 //
-// SpmmRowScalar: one wavefront per sparse row, one column per lane (any width, any
-// alignment); the row's (COL, V) pairs are fetched 64 at a time and handed round with
-// v_readlane.
+// SpmmNarrow (the last N % 4 columns): one lane per (row, column), eight gathers in flight.
+//
+// SpmmRowScalar: one wavefront per sparse row, one column per lane (operands whose byte
+// offsets do not fit 32 bits, N < 4); the row's (COL, V) pairs are fetched 64 at a time and
+// handed round with v_readlane.
 #include "sph_internal.h"
 
 #include <cstdlib>
@@ -47,11 +49,28 @@ struct SpmmArgs
     const uint32_t* ROW;
     const float* B;
     uint32_t M, N;
+    // floats between consecutive rows of B and of out: N, unless a launch covers some of the
+    // columns of a wider operand
+    uint32_t ldB, ldOut;
     int accumulate;
     // when set: out[row][*] = (0 + rowBias[row]) + sum, out is not read -- what accumulating into
     // an out that the K = 1 product bias x ones has filled gives
     const float* rowBias;
 };
+
+// four floats that need only be 4-byte aligned: rows of B and of out start anywhere when their
+// pitch is no multiple of 4, and a 16-byte vector memory access only asks for dword alignment
+typedef float floatx4v __attribute__((ext_vector_type(4)));
+typedef floatx4v floatx4a4 __attribute__((aligned(4)));
+__device__ __forceinline__ float4 Load4(const void* p)
+{
+    const floatx4v v = *reinterpret_cast<const floatx4a4*>(p);
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void Store4(void* p, float4 v)
+{
+    *reinterpret_cast<floatx4a4*>(p) = floatx4v{ v.x, v.y, v.z, v.w };
+}
 
 __device__ __forceinline__ float Bcast(float v, int srcLane)
 {
@@ -124,7 +143,7 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
     // multiply-add.
     const char* __restrict__ Bbytes = reinterpret_cast<const char*>(args.B);
     const uint32_t colBytes = (col < N ? col : slab * kSlabCols) * 4;
-    const uint32_t rowBytes = N * 4;
+    const uint32_t rowBytes = args.ldB * 4;
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 
     // all lanes of the wavefront stay in the loop until the longest of its rows is done
@@ -156,8 +175,7 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
             cj[7] = GroupBroadcast<LPR, base + 7>(c);
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                b[j] = *reinterpret_cast<const float4*>(
-                    Bbytes + (__umul24(cj[j], rowBytes) + colBytes));
+                b[j] = Load4(Bbytes + (__umul24(cj[j], rowBytes) + colBytes));
             vj[0] = __builtin_bit_cast(float, GroupBroadcast<LPR, base + 0>(vbits));
             vj[1] = __builtin_bit_cast(float, GroupBroadcast<LPR, base + 1>(vbits));
             vj[2] = __builtin_bit_cast(float, GroupBroadcast<LPR, base + 2>(vbits));
@@ -188,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
 
     if (active)
     {
-        float4* dst = reinterpret_cast<float4*>(args.out + static_cast<size_t>(row) * N + col);
+        float* dst = args.out + static_cast<size_t>(row) * args.ldOut + col;
         if (args.rowBias != nullptr)
         {
             const float old = 0.f + args.rowBias[row];
@@ -199,14 +217,54 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
         }
         else if (args.accumulate)
         {
-            const float4 old = *dst;
+            const float4 old = Load4(dst);
             sum.x = old.x + sum.x;
             sum.y = old.y + sum.y;
             sum.z = old.z + sum.z;
             sum.w = old.w + sum.w;
         }
-        *dst = sum;
+        Store4(dst, sum);
     }
+}
+
+// Up to 4 output columns (the last N % 4 of a wider operand): one lane per (row, column), 16
+// rows per wavefront; a lane walks its row front to back, eight gathers in flight.
+__global__ __launch_bounds__(kThreads) void SpmmNarrow(const SpmmArgs args)
+{
+    const uint32_t row = (blockIdx.x * kThreads + threadIdx.x) / 4;
+    const uint32_t col = threadIdx.x & 3;
+    if (row >= args.M || col >= args.N)
+        return;
+    const uint32_t begin = args.ROW[row];
+    const uint32_t end = args.ROW[row + 1];
+    const float* __restrict__ B = args.B + col;
+    const size_t ld = args.ldB;
+    float sum = 0.f;
+    uint32_t p = begin;
+    for (; p + 8 <= end; p += 8)
+    {
+        uint32_t c[8];
+        float v[8], b[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+        {
+            c[j] = args.COL[p + j];
+            v[j] = args.V[p + j];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            b[j] = B[c[j] * ld];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            sum = sum + v[j] * b[j];
+    }
+    for (; p < end; ++p)
+        sum = sum + args.V[p] * B[args.COL[p] * ld];
+    float* dst = args.out + static_cast<size_t>(row) * args.ldOut + col;
+    if (args.rowBias != nullptr)
+        *dst = (0.f + args.rowBias[row]) + sum;
+    else
+        *dst = args.accumulate ? (*dst + sum) : sum;
 }
 
 // one output column per lane; any N, any alignment
@@ -242,12 +300,12 @@ __global__ __launch_bounds__(kThreads) void SpmmRowScalar(const SpmmArgs args)
                 const uint32_t cj = Bcast(c, static_cast<int>(j));
                 const float vv = Bcast(v, static_cast<int>(j));
                 if (active)
-                    sum = sum + vv * B[static_cast<size_t>(cj) * N + n];
+                    sum = sum + vv * B[static_cast<size_t>(cj) * args.ldB + n];
             }
         }
         if (active)
         {
-            float* dst = args.out + static_cast<size_t>(row) * N + n;
+            float* dst = args.out + static_cast<size_t>(row) * args.ldOut + n;
             if (args.rowBias != nullptr)
                 *dst = (0.f + args.rowBias[row]) + sum;
             else
@@ -280,22 +338,29 @@ static int LaunchSpmm(float* out, const float* V, const uint32_t* COL, const uin
     args.accumulate = accumulate ? 1 : 0;
     args.rowBias = rowBias;
 
-    const uint32_t blocks = (M + kWavesPerBlock - 1) / kWavesPerBlock;
+    args.ldB = N;
+    args.ldOut = N;
+
     // the slab kernel forms 32-bit byte offsets into B with a 24-bit multiply; larger operands
-    // run on the scalar kernel, whose offsets are 64-bit
-    const bool vec = (N % 4 == 0) &&
-                     ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(B)) & 15u) == 0 &&
-                     static_cast<uint64_t>(Kdim) * N * 4 < (1ull << 32) && Kdim < (1u << 24) &&
-                     N < (1u << 22);
-    // 16 lanes per row (64-column slabs, 4 rows per wavefront) measured fastest from N = 64
-    // up; narrower operands use 8 lanes per row so that fewer lanes idle
-    const int lanesPerRow = N <= 32 ? 8 : 16;
-    if (vec)
+    // run on the scalar kernel, whose offsets are 64-bit.  Its 16-byte accesses need no
+    // alignment beyond 4 bytes, so N = 4 q + r is served by the slab kernel on the first 4 q
+    // columns (row pitches stay N) and by the narrow kernel on the last r: every output
+    // element is still summed by one lane in storage order
+    // (measured on the 8192 x 8192 matrix at 1 %: N = 255 134 us on the scalar kernel).
+    const bool slabFits = static_cast<uint64_t>(Kdim) * N * 4 < (1ull << 32) &&
+                          Kdim < (1u << 24) && N < (1u << 22);
+    const uint32_t whole = N & ~3u;
+    if (slabFits && whole != 0)
     {
+        SpmmArgs left = args;
+        left.N = whole;
+        // 16 lanes per row (64-column slabs, 4 rows per wavefront) measured fastest from N = 64
+        // up; narrower operands use 8 lanes per row so that fewer lanes idle
+        const int lanesPerRow = whole <= 32 ? 8 : 16;
         const uint32_t slabCols = 4u * static_cast<uint32_t>(lanesPerRow);
         const uint32_t rowsPerBlock = (64u / static_cast<uint32_t>(lanesPerRow)) * kWavesPerBlock;
         SlabPlan plan{};
-        plan.slabs = (N + slabCols - 1) / slabCols;
+        plan.slabs = (whole + slabCols - 1) / slabCols;
         plan.rowParts = plan.slabs >= 8 ? 1u : 8u / plan.slabs;
         const uint32_t rowsPerPart = (M + plan.rowParts - 1) / plan.rowParts;
         plan.blocksPerColumn = (rowsPerPart + rowsPerBlock - 1) / rowsPerBlock;
@@ -305,13 +370,28 @@ static int LaunchSpmm(float* out, const float* V, const uint32_t* COL, const uin
         SPH_REQUIRE(grid < (1ull << 31), "too many workgroups for one launch");
         if (lanesPerRow == 16)
             hipLaunchKernelGGL(SpmmSlabVec4<16>, dim3(static_cast<uint32_t>(grid)),
-                               dim3(kThreads), 0, stream, args, plan);
+                               dim3(kThreads), 0, stream, left, plan);
         else
             hipLaunchKernelGGL(SpmmSlabVec4<8>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads),
-                               0, stream, args, plan);
+                               0, stream, left, plan);
+        if (whole != N)
+        {
+            SPH_CHECK_LAUNCH();
+            SpmmArgs right = args;
+            right.N = N - whole;
+            right.B = B + whole;
+            right.out = out + whole;
+            const uint64_t lanes = static_cast<uint64_t>(M) * 4;
+            SPH_REQUIRE(lanes < (1ull << 31), "too many rows for one launch");
+            hipLaunchKernelGGL(SpmmNarrow, dim3(static_cast<uint32_t>((lanes + kThreads - 1) / kThreads)),
+                               dim3(kThreads), 0, stream, right);
+        }
     }
     else
+    {
+        const uint32_t blocks = (M + kWavesPerBlock - 1) / kWavesPerBlock;
         hipLaunchKernelGGL(SpmmRowScalar, dim3(blocks), dim3(kThreads), 0, stream, args);
+    }
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }

@@ -40,7 +40,7 @@ def test_config5_full_size_bit_exact(dev):
     assert np.array_equal(got2[0], C[0])
 
 
-@pytest.mark.parametrize("N", [1, 3, 4, 10, 64, 100, 256, 260, 512, 1000])
+@pytest.mark.parametrize("N", [1, 3, 4, 5, 7, 10, 33, 64, 65, 67, 100, 255, 256, 260, 512, 1000, 1001])
 def test_ragged_dense_widths(dev, N):
     h.announce("sph_spmm_csr_f32 N =", N)
     M, K = 300, 777
@@ -48,6 +48,11 @@ def test_ragged_dense_widths(dev, N):
     B = synth.uniform(901 + N, (K, N))
     ref = po.spmm_csr(np.zeros((M, N), np.float32), v, col, row, M, N, B)
     got = h.gpu_spmm(np.ones((M, N), np.float32), v, col, row, M, K, N, B, False, canary=512)
+    assert np.array_equal(_bits(got), _bits(ref))
+    # and added to what out holds
+    C = synth.uniform(902 + N, (M, N))
+    ref = po.spmm_csr(C.copy(), v, col, row, M, N, B)
+    got = h.gpu_spmm(C, v, col, row, M, K, N, B, True, canary=512)
     assert np.array_equal(_bits(got), _bits(ref))
 
 
@@ -64,7 +69,7 @@ def test_equals_dense_product_of_densified_matrix(dev):
     assert np.array_equal(_bits(got), _bits(ref))
 
 
-@pytest.mark.parametrize("N", [1, 3, 64, 100, 256])
+@pytest.mark.parametrize("N", [1, 3, 6, 64, 65, 100, 255, 256])
 def test_row_bias_form_equals_fill_bias_product_and_accumulate(dev, N):
     """sph_spmm_csr_bias_f32 against the CPU checker run the long way: out = 0, out += bias x
     ones (the K = 1 product of Linear's bias step, feature-major), out += A * B.  Rows without
