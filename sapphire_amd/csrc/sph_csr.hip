@@ -38,7 +38,6 @@ struct DenseView
 {
     const float* data;
     uint32_t M, N, ld;
-    int vec;  // rows start 16-byte aligned and N % 4 == 0
 };
 
 // 4 consecutive columns of one row; columns past N read as 0
@@ -49,8 +48,14 @@ __device__ __forceinline__ float4 LoadQuad(const DenseView& d, uint32_t row, uin
     if (rowOk && col < d.N)
     {
         const float* p = d.data + static_cast<size_t>(row) * d.ld + col;
-        if (d.vec)
-            v = *reinterpret_cast<const float4*>(p);
+        // four columns that all exist: one 16-byte access, which only asks for 4-byte alignment
+        if (col + 4 <= d.N)
+        {
+            typedef float floatx4 __attribute__((ext_vector_type(4)));
+            typedef floatx4 floatx4a4 __attribute__((aligned(4)));
+            const floatx4 w = *reinterpret_cast<const floatx4a4*>(p);
+            v = make_float4(w[0], w[1], w[2], w[3]);
+        }
         else
         {
             v.x = p[0];
@@ -281,7 +286,7 @@ __global__ __launch_bounds__(kThreads) void CsrFillKernel(float* __restrict__ V,
 constexpr uint32_t kStageWaves = 4;  // wavefronts per workgroup
 
 // A workgroup holds 4 / WPR rows; WPR wavefronts share a row, each taking QUADS float4 per lane
-// of a contiguous part of it.  Requires d.vec (so N % 4 == 0) and N <= WPR * QUADS * 256.  Few
+// of a contiguous part of it.  Requires N <= WPR * QUADS * 256.  Few
 // registers per wavefront on purpose: many small workgroups per compute unit, out of step with
 // each other, keep loads in flight while others count and store.
 template <int WPR, int QUADS>
@@ -301,14 +306,11 @@ __global__ __launch_bounds__(kStageWaves * 64) void CsrStageKernel(
 
     // quad j of lane l of part p holds columns 256 (p QUADS + j) + 4 l .. + 3
     float4 q[QUADS];
-    const float* rowPtr = d.data + static_cast<size_t>(rowOk ? row : 0) * d.ld;
 #pragma unroll
     for (int j = 0; j < QUADS; ++j)
     {
         const uint32_t col = ((part * QUADS + j) * 64 + lane) * 4;
-        q[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (rowOk && col < d.N)
-            q[j] = *reinterpret_cast<const float4*>(rowPtr + col);
+        q[j] = LoadQuad(d, row, col, rowOk);
     }
     uint32_t total = 0;  // the same in every lane
 #pragma unroll
@@ -426,8 +428,24 @@ __global__ __launch_bounds__(256) void CsrUnstageKernel(float* __restrict__ V,
 
 // One wavefront per row, one pass over the dense matrix.  A row of at most 128 entries is
 // merged into the zeros in registers; a longer one is cleared first, then its entries are
-// written over the zeros.  VEC: rows start on 16-byte boundaries and N % 4 == 0.
-template <bool VEC>
+// written over the zeros.  Four columns that all exist are stored 16 bytes at a time, whatever
+// the alignment of the row (a vector store only asks for 4-byte alignment).
+__device__ __forceinline__ void StoreQuad(float* p, float4 q, uint32_t col, uint32_t N)
+{
+    if (col + 4 <= N)
+    {
+        typedef float floatx4 __attribute__((ext_vector_type(4)));
+        typedef floatx4 floatx4a4 __attribute__((aligned(4)));
+        *reinterpret_cast<floatx4a4*>(p) = floatx4{ q.x, q.y, q.z, q.w };
+    }
+    else
+    {
+        if (col + 0 < N) p[0] = q.x;
+        if (col + 1 < N) p[1] = q.y;
+        if (col + 2 < N) p[2] = q.z;
+    }
+}
+
 __global__ __launch_bounds__(kThreads) void CsrToDenseRowKernel(float* __restrict__ dense,
                                                                 uint32_t ld, uint32_t M,
                                                                 uint32_t N,
@@ -443,7 +461,7 @@ __global__ __launch_bounds__(kThreads) void CsrToDenseRowKernel(float* __restric
         float* out = dense + static_cast<size_t>(row) * ld;
         const uint32_t begin = ROW[row];
         const uint32_t end = ROW[row + 1];
-        if (VEC && end - begin <= 128)
+        if (end - begin <= 128)
         {
             // A short row is held in registers (two entries per lane) and merged into the
             // stream of zeros: every 1 KiB piece of the row is stored once, entries included,
@@ -489,21 +507,12 @@ __global__ __launch_bounds__(kThreads) void CsrToDenseRowKernel(float* __restric
                 // c - base < 256 in unsigned arithmetic: base <= c < base + 256
                 place(__ballot(c0 - base < 256u && c0 != 0xffffffffu), c0, v0);
                 place(__ballot(c1 - base < 256u && c1 != 0xffffffffu), c1, v1);
-                if (base + lane * 4 < N)
-                    *reinterpret_cast<float4*>(out + base + lane * 4) = q;
+                StoreQuad(out + base + lane * 4, q, base + lane * 4, N);
             }
             continue;
         }
-        if (VEC)
-        {
-            for (uint32_t c = lane * 4; c < N; c += 256)
-                *reinterpret_cast<float4*>(out + c) = make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-        else
-        {
-            for (uint32_t c = lane; c < N; c += 64)
-                out[c] = 0.f;
-        }
+        for (uint32_t c = lane * 4; c < N; c += 256)
+            StoreQuad(out + c, make_float4(0.f, 0.f, 0.f, 0.f), c, N);
         // An entry is written by another lane than the one that cleared its place: the zeros
         // have to be acknowledged by the cache before the entries follow them.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -540,7 +549,6 @@ DenseView MakeView(const float* dense, uint32_t M, uint32_t N, uint32_t ld)
     d.M = M;
     d.N = N;
     d.ld = ld;
-    d.vec = (N % 4 == 0) && (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(dense) & 15u) == 0;
     return d;
 }
 
@@ -714,9 +722,12 @@ int sph_csr_from_dense_f32(float* V, uint32_t* COL, uint32_t* ROW, uint32_t capa
     // plus 32, a multiple of 4
     const uint64_t mean = M != 0 ? capacity / M : 0;
     const uint64_t stage64 = (2 * mean + 32 + 3) / 4 * 4;
-    if (!(d.vec && M != 0 && N >= 128 && N <= 8192 && stage64 * 4 <= N))
+    // (below 16 Mi elements the three launches of the one-pass path cost more than the second
+    // pass over the matrix they save: 8192 x 1000 18 us against 26 us, equal at 8192 x 2048)
+    if (!(M != 0 && N >= 128 && N <= 8192 && stage64 * 4 <= N &&
+          static_cast<uint64_t>(M) * N >= (1ull << 24)))
     {
-        // narrow, very wide, unaligned or not very sparse matrices (a staging area of more
+        // narrow, very wide, small or not very sparse matrices (a staging area of more
         // than a quarter of the dense matrix): count, scan and fill as separate passes
         const int lanes = LanesPerRow(N);
         DispatchLanes<CountLauncher>(lanes, RowGrid(M, lanes), stream, ROW, d);
@@ -820,15 +831,9 @@ int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V, const uint32
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
-    const bool vec = (N % 4 == 0) && (ld % 4 == 0) &&
-                     (reinterpret_cast<uintptr_t>(dense) & 15u) == 0;
     const uint32_t grid = RowGrid(M, 64);
-    if (vec)
-        hipLaunchKernelGGL(CsrToDenseRowKernel<true>, dim3(grid), dim3(kThreads), 0, stream, dense,
-                           ld, M, N, V, COL, ROW);
-    else
-        hipLaunchKernelGGL(CsrToDenseRowKernel<false>, dim3(grid), dim3(kThreads), 0, stream, dense,
-                           ld, M, N, V, COL, ROW);
+    hipLaunchKernelGGL(CsrToDenseRowKernel, dim3(grid), dim3(kThreads), 0, stream, dense, ld, M, N,
+                       V, COL, ROW);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }

@@ -107,7 +107,15 @@ def gpu_csr_one_call(dense, N, capacity):
 # (narrow, unaligned, or too dense for a staging area)
 ONE_CALL_CASES = CASES + [(13, 128, 128, 0.3), (1000, 256, 256, 0.1), (4097, 1024, 1028, 0.02),
                           (70, 8192, 8192, 0.01), (3, 4100, 4100, 0.5), (2500, 520, 520, 1.0),
-                          (5, 132, 136, 0.0), (70000, 128, 128, 0.05), (999, 2048, 2048, 0.003)]
+                          (5, 132, 136, 0.0), (70000, 128, 128, 0.05), (999, 2048, 2048, 0.003),
+                          # from 16 Mi elements up the one-pass path itself runs (below, the
+                          # separate passes are faster): every row layout of it, rows that are
+                          # no multiples of 4 floats long or apart, a last workgroup with
+                          # fewer rows than it holds
+                          (131101, 128, 128, 0.05), (65601, 256, 260, 0.02), (32301, 520, 520, 0.02),
+                          (16401, 1024, 1028, 0.02), (16390, 1027, 1027, 0.02),
+                          (8201, 2048, 2048, 0.003), (4101, 4100, 4100, 0.01),
+                          (2101, 8190, 8191, 0.01), (2049, 8192, 8192, 0.01)]
 
 
 @pytest.mark.parametrize("case", ONE_CALL_CASES)
@@ -136,7 +144,7 @@ def test_one_call_conversion_equals_the_two_calls(dev, case):
 def test_one_call_conversion_with_rows_that_overflow_their_staging_slot(dev):
     """Mostly empty matrix with three full rows: their entries do not fit the per-row staging
     slot (sized from the mean), so the second kernel rebuilds them from the dense matrix."""
-    M, N = 1001, 2048
+    M, N = 8201, 2048
     h.announce("sph_csr_from_dense_f32 skewed rows", M, N)
     dense = sparse_dense(4242, (M, N), 0.003)
     for r in (0, 500, M - 1):
