@@ -369,8 +369,8 @@ int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V,
  * sph_csr_fill_f32 with the ROW already there.  With nnzHost != NULL the
  * count is copied to *nnzHost and the call returns after the stream has
  * drained; with NULL it is asynchronous.
- * For 16-byte aligned rows of 128 .. 8192 columns and a capacity of at most
- * about an eighth of the matrix the dense matrix is read once: every row is
+ * For rows of 128 .. 8192 columns, at least 16 Mi elements and a capacity of at
+ * most about an eighth of the matrix the dense matrix is read once: every row is
  * compacted into a staging slot of 2 * capacity / M + 32 entries (a
  * stream-ordered scratch allocation of 8 bytes per slot entry), the counts
  * are scanned and a small kernel moves the staged entries into place; a row
