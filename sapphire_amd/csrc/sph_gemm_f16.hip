@@ -725,8 +725,8 @@ constexpr int kD = 128;
 constexpr int kDStages = 4;
 constexpr int kDStageBytes = 2 * kD * kTK * 2;  // A + B
 
-// TAIL: K = 32 q + r, 0 < r < 32, handled as in the 256-tile kernel: a last step over the
-// window [K - 32, K) in which the positions of the 32 - r values of k already multiplied are cleared.
+// TAIL: K = 32 q + r, 0 < r < 32: a last step over the window [K - 32, K) whose slab has the
+// positions of the 32 - r values of k already multiplied cleared in LDS.
 template <bool TA, bool TB, bool TAIL, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args args)
 {
@@ -879,19 +879,26 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
 #pragma unroll
             for (int v = 0; v < 16; ++v)
                 acc[i][j][v] = 0.f;
-    // TAIL: a lane's fragments of half ks hold k group 2 ks + khalf of the step's window; in the
-    // last step the first 32 - r positions repeat values of k the step before has multiplied
-    const uintx4 tailMasks[2] = { TailMask(khalf, kTK - K % kTK), TailMask(2 + khalf, kTK - K % kTK) };
-    auto maskRepeated = [&](halfx8 (&af)[2], halfx8 (&bf)[TN], int ks, bool lastStep) {
-        if constexpr (TAIL)
+    // TAIL: the positions of the last slab whose k the step before has multiplied are cleared
+    // in LDS, by the lane that copied them, once the copies have landed and before the barrier
+    // that publishes the stage, so the steps themselves carry no masks (1024 x 1024 x 784:
+    // 13.6 -> 11.4 us against masks on the fragments of every step; the 256-tile kernel keeps
+    // those, it has no registers to spare for this and measured 134 -> 143 us).
+    auto clearRepeated = [&](char* stage) {
+        const uint32_t repeated = kTK - K % kTK;
+        const uint32_t c = (lane & 3) ^ ((lane >> 4) & 3);  // chunk of a K-contiguous row
+        const uintx4 contig = TailMask(c, repeated);
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesPer; ++i)
         {
-            const uintx4 keep = lastStep ? tailMasks[ks] : uintx4{ ~0u, ~0u, ~0u, ~0u };
-#pragma unroll
-            for (int b = 0; b < 2; ++b)
-                af[b] = KeepNew(af[b], keep);
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-                bf[b] = KeepNew(bf[b], keep);
+            const uint32_t j = wave + WAVES * i;
+            const uint32_t k = j * 4 + (lane >> 4);  // row of a k-major slab
+            const uint32_t keepAll = k < repeated ? 0u : ~0u;
+            const uintx4 major = { keepAll, keepAll, keepAll, keepAll };
+            uintx4* a = reinterpret_cast<uintx4*>(stage + j * 1024 + lane * 16);
+            uintx4* b = reinterpret_cast<uintx4*>(stage + kBytesA + j * 1024 + lane * 16);
+            *a = *a & (TA ? major : contig);
+            *b = *b & (TB ? contig : major);
         }
     };
     auto multiply = [&](const halfx8 (&af)[2], const halfx8 (&bf)[TN]) {
@@ -907,7 +914,8 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
     // pipe is already busy: behind the first one the wait for the copies of step st+1 and the
     // barrier, behind every one a copy of step st+3.
     static_assert(kDCopies == 2 * TN, "one copy behind every MFMA of the first half");
-    auto multiplyAndFeed = [&](const halfx8 (&af)[2], const halfx8 (&bf)[TN], uint32_t fillStage) {
+    auto multiplyAndFeed = [&](const halfx8 (&af)[2], const halfx8 (&bf)[TN], uint32_t fillStage,
+                               bool nextIsLast, char* next) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -921,6 +929,14 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
                     // behind the barrier everybody's copies are visible and everybody has
                     // read the last fragment of step st-1
                     WaitVmem<(kDStages - 3) * kDCopies>();
+                    if constexpr (TAIL)
+                    {
+                        if (nextIsLast)
+                        {
+                            clearRepeated(next);
+                            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        }
+                    }
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
                 }
@@ -955,16 +971,14 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
             if (s0 + u >= steps)
                 break;
             const char* cur = lds + u * kDStageBytes;
-            const char* next = lds + ((u + 1) % kDStages) * kDStageBytes;
-            const bool lastStep = TAIL && s0 + u == steps - 1;
+            char* next = lds + ((u + 1) % kDStages) * kDStageBytes;
             loadFragments(af[1], bf[1], cur, 1);
             __builtin_amdgcn_sched_barrier(0);
-            maskRepeated(af[0], bf[0], 0, lastStep);
-            multiplyAndFeed(af[0], bf[0], (u + kDStages - 1) % kDStages);
+            multiplyAndFeed(af[0], bf[0], (u + kDStages - 1) % kDStages,
+                            TAIL && s0 + u + 2 == steps, next);
             __builtin_amdgcn_sched_barrier(0);
             loadFragments(af[0], bf[0], next, 0);
             __builtin_amdgcn_sched_barrier(0);
-            maskRepeated(af[1], bf[1], 1, lastStep);
             multiply(af[1], bf[1]);
             __builtin_amdgcn_sched_barrier(0);
         }
