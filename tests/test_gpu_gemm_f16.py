@@ -199,7 +199,7 @@ def test_transposed_operands_exact_on_integers(dev, shape, flags):
     assert np.array_equal(got, ref - C)
 
 
-# N = 8 q + r, r != 0, with at least 128 whole column chunks' worth of columns: the first 8 q
+# N = 8 q + r, r != 0: the first 8 q
 # columns on the straight-to-LDS kernels (rows of B and of out start at addresses that are no
 # multiples of 16 bytes), the last r on the general kernel.  (M, N, K, batch): 128-tile kernel
 # with four and with eight wavefronts, ragged and whole 256-tiles (old values of out added in the
@@ -208,7 +208,11 @@ def test_transposed_operands_exact_on_integers(dev, shape, flags):
                                    capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
 @pytest.mark.parametrize("shape", [(512, 132, 64, 1), (200, 1030, 96, 2), (304, 517, 64, 3),
                                    (128, 135, 32, 300), (4096, 3076, 64, 1), (256, 257, 64, 192),
-                                   (256, 260, 640, 192), (1000, 999, 992, 1), (248, 250, 72, 3)])
+                                   (256, 260, 640, 192), (1000, 999, 992, 1), (248, 250, 72, 3),
+                                   # narrow products: 8 or 96 columns on the 128-tile kernel and the
+                                   # rest, or all of fewer than 8 columns, on the last-columns kernel
+                                   (1024, 10, 1024, 1), (304, 100, 96, 2), (512, 5, 64, 3),
+                                   (1000, 7, 1001, 1), (40, 3, 32, 1)])
 def test_column_count_not_a_multiple_of_eight(dev, shape, flags):
     M, N, K, batch = shape
     h.announce("sph_gemm_f16f32, N % 8 != 0", shape, "flags", flags)
