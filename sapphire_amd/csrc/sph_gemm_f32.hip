@@ -1594,7 +1594,13 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // (measured 4096 x 4095 x 4096: 1615 us on the register-staged kernel's 4-byte loads).
     // A B stored N x K would not need this; it is split all the same, so that a product does
     // not depend on how its operands are stored.
-    if (args.split == 0 && args.N % 4 != 0 && args.N >= 68 && args.M > 1 && args.K >= kBK)
+    // (not when the whole product goes to the few-tile kernel, which takes any N as it is)
+    const uint64_t wholeTiles64 =
+        static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
+    const bool wholeIsFewTiles =
+        wholeTiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) && args.K >= 64;
+    if (args.split == 0 && args.N % 4 != 0 && args.N > 4 && args.M > 1 && args.K >= kBK &&
+        !wholeIsFewTiles)
     {
         const uint32_t whole = args.N & ~3u;
         GemmF32Args left = args;

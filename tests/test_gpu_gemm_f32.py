@@ -162,13 +162,15 @@ def test_partial_last_k_step(dev, dims, flags):
     assert np.array_equal(got.view(np.uint32), other.view(np.uint32))
 
 
-# N = 4 q + r, r != 0, from 68 columns up: the first 4 q columns on the tiled kernels with the
+# N = 4 q + r, r != 0: the first 4 q columns on the tiled kernels with the
 # row pitches left at N, the last r on the kernel for narrow products.  Guard floats behind
 # every unit of out catch a store past column N - 1.
 @pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
                                    capi.SPH_GEMM_OVERWRITE])
 @pytest.mark.parametrize("dims", [(512, 1026, 64, 1), (1000, 999, 100, 1), (300, 70, 40, 3),
-                                  (64, 69, 16, 5), (2048, 2049, 128, 1), (128, 1031, 2050, 1)])
+                                  (64, 69, 16, 5), (2048, 2049, 128, 1), (128, 1031, 2050, 1),
+                                  # narrow products with enough rows for the tiled kernels
+                                  (16384, 10, 64, 1), (9000, 5, 32, 1), (4096, 30, 100, 2)])
 def test_column_count_not_a_multiple_of_four(dev, dims, flags):
     M, N, K, batch = dims
     h.announce("sph_gemm_f32_ex, N % 4 != 0", dims, "flags", flags)
