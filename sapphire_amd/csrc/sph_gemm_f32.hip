@@ -1223,6 +1223,12 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
                 if (k < K)
                     v = *reinterpret_cast<const float4*>(rowPtr + k);
             }
+            else if (k + 4 <= K)
+            {
+                // a row that starts anywhere (K % 4 != 0): still one 16-byte load
+                const floatx4a4 w = *reinterpret_cast<const floatx4a4*>(rowPtr + k);
+                v = make_float4(w[0], w[1], w[2], w[3]);
+            }
             else
             {
                 if (k + 0 < K) v.x = rowPtr[k + 0];
