@@ -1153,7 +1153,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 // unit), which is why the 16-wide tile, a quarter of the work per workgroup on four times as
 // many compute units, is preferred whenever its tiles still fit the chip.
 // ---------------------------------------------------------------------------
-template <int TILE, bool VEC, bool TA, bool TB, int WAVES>
+template <int TILE, bool TA, bool TB, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32Args args)
 {
     static_assert(TILE == 32 || TILE == 16, "MFMA shapes 32x32x2 and 16x16x4");
@@ -1211,60 +1211,46 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         acc[v] = 0.f;
 
     // Lane group h holds k = kGroupK*g + 4*h + e for e = 0..3.  An operand stored with K
-    // contiguous (A as given, B passed transposed) is read as one 16-byte segment of its row;
-    // one stored k-major (B as given, A passed transposed) as 4 elements `ld` apart.
-    auto loadAlongK = [&](const float* rowPtr, bool ok, uint32_t g) {
-        const uint32_t k = g * kGroupK + kh * 4;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok)
-        {
-            if (VEC)
-            {
-                if (k < K)
-                    v = *reinterpret_cast<const float4*>(rowPtr + k);
-            }
-            else if (k + 4 <= K)
-            {
-                // a row that starts anywhere (K % 4 != 0): still one 16-byte load
-                const floatx4a4 w = *reinterpret_cast<const floatx4a4*>(rowPtr + k);
-                v = make_float4(w[0], w[1], w[2], w[3]);
-            }
-            else
-            {
-                if (k + 0 < K) v.x = rowPtr[k + 0];
-                if (k + 1 < K) v.y = rowPtr[k + 1];
-                if (k + 2 < K) v.z = rowPtr[k + 2];
-                if (k + 3 < K) v.w = rowPtr[k + 3];
-            }
-        }
-        return v;
-    };
-    auto loadAcrossK = [&](const float* colPtr, size_t ld, bool ok, uint32_t g) {
-        const uint32_t k = g * kGroupK + kh * 4;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (ok)
-        {
-            const float* p = colPtr + static_cast<size_t>(k) * ld;
-            if (k + 0 < K) v.x = p[0];
-            if (k + 1 < K) v.y = p[ld];
-            if (k + 2 < K) v.z = p[2 * ld];
-            if (k + 3 < K) v.w = p[3 * ld];
-        }
-        return v;
-    };
+    // contiguous (A as given, B passed transposed) is read as one 16-byte segment of its row
+    // (from any 4-byte-aligned address); one stored k-major (B as given, A passed transposed) as
+    // 4 elements `ld` apart.  Rows and columns past the edge read the last valid one: what they
+    // produce is never stored.
     const float* aPtr = TA ? A + min(row, M - 1) : A + static_cast<size_t>(min(row, M - 1)) * K;
     const float* bPtr = TB ? B + static_cast<size_t>(min(col, N - 1)) * K : B + min(col, N - 1);
+    // whole groups (every k below K): no conditions anywhere, so the loads of several groups
+    // stay in flight behind the matrix instructions (a load inside a branch makes the compiler
+    // wait for all of them)
+    auto loadAlongK = [&](const float* rowPtr, uint32_t g) {
+        const floatx4a4 w =
+            *reinterpret_cast<const floatx4a4*>(rowPtr + (g * kGroupK + kh * 4));
+        return make_float4(w[0], w[1], w[2], w[3]);
+    };
+    auto loadAcrossK = [&](const float* colPtr, size_t ld, uint32_t g) {
+        const float* p = colPtr + static_cast<size_t>(g * kGroupK + kh * 4) * ld;
+        return make_float4(p[0], p[ld], p[2 * ld], p[3 * ld]);
+    };
     auto loadA = [&](uint32_t g) {
         if constexpr (TA)
-            return loadAcrossK(aPtr, args.lda, rowOk, g);
+            return loadAcrossK(aPtr, args.lda, g);
         else
-            return loadAlongK(aPtr, rowOk, g);
+            return loadAlongK(aPtr, g);
     };
     auto loadB = [&](uint32_t g) {
         if constexpr (TB)
-            return loadAlongK(bPtr, colOk, g);
+            return loadAlongK(bPtr, g);
         else
-            return loadAcrossK(bPtr, args.ldb, colOk, g);
+            return loadAcrossK(bPtr, args.ldb, g);
+    };
+    // the last group when K is no multiple of kGroupK: element by element, zeros past K
+    auto loadPartial = [&](const float* base, size_t step, uint32_t g) {
+        const uint32_t k = g * kGroupK + kh * 4;
+        const float* p = base + static_cast<size_t>(k) * step;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k + 0 < K) v.x = p[0];
+        if (k + 1 < K) v.y = p[step];
+        if (k + 2 < K) v.z = p[2 * step];
+        if (k + 3 < K) v.w = p[3 * step];
+        return v;
     };
     // operands swapped: the result block comes out indexed [column][row], which leaves 4
     // consecutive columns of one row in a lane
@@ -1274,31 +1260,58 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         else
             acc = __builtin_amdgcn_mfma_f32_16x16x4f32(b, a, acc, 0, 0, 0);
     };
+    auto multiplyGroup = [&](const float4& a, const float4& b) {
+        multiply(b.x, a.x);
+        multiply(b.y, a.y);
+        multiply(b.z, a.z);
+        multiply(b.w, a.w);
+    };
 
-    constexpr int kDepth = 4;  // groups in flight
-    float4 fa[kDepth], fb[kDepth];
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d)
+    // groups in flight; 8, or twice the wavefronts per tile, are slower: the loop is bound by
+    // what the caches deliver, not by the latency of a load
+    constexpr int kDepth = 4;
+    const uint32_t whole = K / kGroupK;        // groups with every k below K
+    const uint32_t wholeEnd = min(gEnd, whole);  // this wavefront's whole groups end here
+    if (gBegin < wholeEnd)
     {
-        fa[d] = gBegin + d < gEnd ? loadA(gBegin + d) : make_float4(0.f, 0.f, 0.f, 0.f);
-        fb[d] = gBegin + d < gEnd ? loadB(gBegin + d) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-    for (uint32_t g = gBegin; g < gEnd; g += kDepth)
-    {
+        const uint32_t lastWhole = wholeEnd - 1;
+        const uint32_t roundsEnd = gBegin + (wholeEnd - gBegin) / kDepth * kDepth;
+        float4 fa[kDepth], fb[kDepth];
 #pragma unroll
         for (int d = 0; d < kDepth; ++d)
         {
-            const float4 a = fa[d];
-            const float4 b = fb[d];
-            const uint32_t next = g + kDepth + d;
-            fa[d] = next < gEnd ? loadA(next) : make_float4(0.f, 0.f, 0.f, 0.f);
-            fb[d] = next < gEnd ? loadB(next) : make_float4(0.f, 0.f, 0.f, 0.f);
-            // groups past gEnd carry zeros and add nothing
-            multiply(b.x, a.x);
-            multiply(b.y, a.y);
-            multiply(b.z, a.z);
-            multiply(b.w, a.w);
+            // past the last whole group: that group once more, loaded and not used
+            fa[d] = loadA(min(gBegin + d, lastWhole));
+            fb[d] = loadB(min(gBegin + d, lastWhole));
         }
+        for (uint32_t g = gBegin; g < roundsEnd; g += kDepth)
+        {
+#pragma unroll
+            for (int d = 0; d < kDepth; ++d)
+            {
+                // multiply, then load the group kDepth further on into the same registers
+                // (loading first needs a second set and a copy, behind a wait for every load,
+                // at the end of each round); the fences keep that order
+                multiplyGroup(fa[d], fb[d]);
+                __builtin_amdgcn_sched_barrier(0);
+                const uint32_t next = min(g + kDepth + d, lastWhole);
+                fa[d] = loadA(next);
+                fb[d] = loadB(next);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // fewer than kDepth whole groups left: already in registers
+#pragma unroll
+        for (int d = 0; d < kDepth - 1; ++d)
+            if (roundsEnd + d < wholeEnd)
+                multiplyGroup(fa[d], fb[d]);
+    }
+    if (gBegin <= whole && whole < gEnd)
+    {
+        // at most one group, and only in the wavefront that holds the end of K
+        const float4 a = TA ? loadPartial(aPtr, args.lda, whole) : loadPartial(aPtr, 1, whole);
+        const float4 b = TB ? loadPartial(bPtr, 1, whole) : loadPartial(bPtr, args.ldb, whole);
+        multiplyGroup(a, b);
     }
 
     // lane l holds row l % TILE, columns 4*kLaneGroups*q + 4*(l / TILE) + 0..3 of the tile;
@@ -1495,7 +1508,7 @@ EntryTable& ThreadTable(int device)
 }
 
 template <int TILE, bool TA, bool TB>
-void LaunchSkinnyTile(const GemmF32Args& args, dim3 grid, bool vec, bool wide, hipStream_t stream)
+void LaunchSkinnyTile(const GemmF32Args& args, dim3 grid, bool wide, hipStream_t stream)
 {
     // `wide` (16 x 16 tiles only): 16 wavefronts per tile instead of 4 when K is long enough to
     // give each wavefront a few steps
@@ -1503,31 +1516,21 @@ void LaunchSkinnyTile(const GemmF32Args& args, dim3 grid, bool vec, bool wide, h
     {
         if (wide)
         {
-            if (vec)
-                hipLaunchKernelGGL((GemmF32SkinnyKernel<16, true, TA, TB, 16>), grid, dim3(1024),
-                                   0, stream, args);
-            else
-                hipLaunchKernelGGL((GemmF32SkinnyKernel<16, false, TA, TB, 16>), grid, dim3(1024),
-                                   0, stream, args);
+            hipLaunchKernelGGL((GemmF32SkinnyKernel<16, TA, TB, 16>), grid, dim3(1024), 0, stream,
+                               args);
             return;
         }
     }
-    if (vec)
-        hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, true, TA, TB, 4>), grid, dim3(256), 0,
-                           stream, args);
-    else
-        hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, false, TA, TB, 4>), grid, dim3(256), 0,
-                           stream, args);
+    hipLaunchKernelGGL((GemmF32SkinnyKernel<TILE, TA, TB, 4>), grid, dim3(256), 0, stream, args);
 }
 
 template <bool TA, bool TB>
-void LaunchSkinny(const GemmF32Args& args, dim3 grid, uint32_t tile, bool vec, bool wide,
-                  hipStream_t stream)
+void LaunchSkinny(const GemmF32Args& args, dim3 grid, uint32_t tile, bool wide, hipStream_t stream)
 {
     if (tile == 16)
-        LaunchSkinnyTile<16, TA, TB>(args, grid, vec, wide, stream);
+        LaunchSkinnyTile<16, TA, TB>(args, grid, wide, stream);
     else
-        LaunchSkinnyTile<32, TA, TB>(args, grid, vec, wide, stream);
+        LaunchSkinnyTile<32, TA, TB>(args, grid, wide, stream);
 }
 
 // `walk`: 64-tiles only, each workgroup takes several tiles
@@ -1691,22 +1694,16 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         args.tilesN = (args.N + tile - 1) / tile;
         const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
         const dim3 gridSkinny(static_cast<uint32_t>(blocks));
-        // 16-byte loads are used only for operands stored with K contiguous
-        bool kVec = allowVector && (args.K % 4 == 0);
-        if (!transA)
-            kVec = kVec && (reinterpret_cast<uintptr_t>(args.A) & 15u) == 0;
-        if (transB)
-            kVec = kVec && (reinterpret_cast<uintptr_t>(args.B) & 15u) == 0;
         const bool wide = tile == 16 && blocks <= static_cast<uint64_t>(sph::ComputeUnits()) &&
                           args.K >= 512;
         if (transA && transB)
-            LaunchSkinny<true, true>(args, gridSkinny, tile, kVec, wide, stream);
+            LaunchSkinny<true, true>(args, gridSkinny, tile, wide, stream);
         else if (transA)
-            LaunchSkinny<true, false>(args, gridSkinny, tile, false, wide, stream);
+            LaunchSkinny<true, false>(args, gridSkinny, tile, wide, stream);
         else if (transB)
-            LaunchSkinny<false, true>(args, gridSkinny, tile, kVec, wide, stream);
+            LaunchSkinny<false, true>(args, gridSkinny, tile, wide, stream);
         else
-            LaunchSkinny<false, false>(args, gridSkinny, tile, kVec, wide, stream);
+            LaunchSkinny<false, false>(args, gridSkinny, tile, wide, stream);
         SPH_CHECK_LAUNCH();
         return SPH_OK;
     }
