@@ -3,7 +3,13 @@
 // Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50): half
 // inputs, fp32 accumulation, row-major operands, result added into out.
 //
-// Three kernels (and one for the odd columns, see below):
+// Four kernels (and one for the odd columns, see below):
+//
+//   GemmF16Few      products with at most one 32 x 32 output tile per compute unit (or at most 16
+//     rows or columns), whatever K, the storage flags and the alignment: one 32 x 32 or 16 x 16
+//     tile per workgroup, K split over its wavefronts, fragments loaded straight from global
+//     memory in MFMA layout.  The tiled kernels below would use a few compute units for these
+//     and wait out a memory latency per K step on each.
 //
 //   GemmF16Tile256  K >= 32 (a multiple of 32, or any K >= 64), N a multiple of 8, at least three
 //     quarters as many 256 x 256 tiles as compute units and at least three quarters of
@@ -44,6 +50,7 @@
 // general kernel when A is stored K x M).
 #include "sph_internal.h"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace
@@ -1474,6 +1481,239 @@ void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16
         hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB, TAIL>), g, b, 0, stream, args);
 }
 
+// ---------------------------------------------------------------------------
+// Few output tiles: one 32 x 32 (v_mfma_f32_32x32x16_f16) or 16 x 16 (16x16x32) tile per
+// workgroup, K split across its WAVES wavefronts
+// ---------------------------------------------------------------------------
+// A product whose output covers only a few 128-tiles leaves most of the chip idle on the tiled
+// kernels, and each of their workgroups then waits out a memory latency per K step (128 x 1024
+// x 1024: 10.6 us on 8 compute units).  Here every wavefront reads its fragments straight from
+// global memory in MFMA layout - lane l holds row (column) l % TILE and the 8 values
+// k = kGroupK g + 8 (l / TILE) .. + 7 of group g: one 16-byte load from an operand stored with K
+// contiguous (any 2-byte-aligned address), eight 2-byte loads `ld` apart from one stored
+// k-major - keeps the loads of several groups in flight, and accumulates a private TILE x TILE
+// partial over its share of K.  The partials are added in wavefront order through LDS, so the
+// result does not depend on timing, and the k assignment is the same for every storage order,
+// so it does not depend on the flags either.  Any M, N, K, pitch and alignment.
+template <int TILE, bool TA, bool TB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
+{
+    static_assert(TILE == 32 || TILE == 16, "MFMA shapes 32x32x16 and 16x16x32");
+    constexpr uint32_t kLaneGroups = 64 / TILE;     // groups of TILE lanes
+    constexpr uint32_t kGroupK = 8 * kLaneGroups;   // k per MFMA: 16 or 32
+    constexpr int kAcc = TILE * TILE / 64;          // accumulator registers: 16 or 4
+    constexpr int kQuads = kAcc / 4;
+    using Acc = typename std::conditional<TILE == 32, floatx16, floatx4>::type;
+
+    __shared__ float partial[WAVES - 1][TILE * TILE];
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t lt = lane % TILE;  // row of A / column of B this lane feeds
+    const uint32_t kh = lane / TILE;  // which 8 values of k of an MFMA
+
+    uint32_t id = blockIdx.x;
+    const uint32_t tn = id % args.tilesN;
+    id /= args.tilesN;
+    const uint32_t tm = id % args.tilesM;
+    const uint32_t unit = id / args.tilesM;
+
+    const _Float16* __restrict__ A = args.A + args.strideA * static_cast<int64_t>(unit);
+    const _Float16* __restrict__ B = args.B + args.strideB * static_cast<int64_t>(unit);
+    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit);
+    const uint32_t M = args.M, N = args.N, K = args.K;
+    const uint32_t row = tm * TILE + lt;
+    const uint32_t col = tn * TILE + lt;
+
+    // this wavefront's K range, in groups of kGroupK
+    const uint32_t groups = (K + kGroupK - 1) / kGroupK;
+    const uint32_t perWave = (groups + WAVES - 1) / WAVES;
+    const uint32_t gBegin = min(wave * perWave, groups);
+    const uint32_t gEnd = min(gBegin + perWave, groups);
+
+    Acc acc;
+#pragma unroll
+    for (int v = 0; v < kAcc; ++v)
+        acc[v] = 0.f;
+
+    // rows and columns past the edge read the last valid one: what they produce is never stored
+    const _Float16* aPtr = TA ? A + min(row, M - 1) : A + static_cast<size_t>(min(row, M - 1)) * args.lda;
+    const _Float16* bPtr = TB ? B + static_cast<size_t>(min(col, N - 1)) * K : B + min(col, N - 1);
+    // whole groups (every k below K): no conditions anywhere, so that the compiler can count
+    // the loads in flight instead of waiting for all of them.  The eight 2-byte values of an
+    // operand stored k-major stay in a register each while they are in flight and are packed
+    // where they are used: packed where they are loaded, every round would end with a wait for
+    // its last load.
+    struct AlongK
+    {
+        halfx8 v;
+        __device__ __forceinline__ halfx8 get() const { return v; }
+    };
+    struct AcrossK
+    {
+        uint32_t r[8];
+        __device__ __forceinline__ halfx8 get() const
+        {
+            uintx4 w;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = r[2 * i] | (r[2 * i + 1] << 16);
+            return __builtin_bit_cast(halfx8, w);
+        }
+    };
+    using FragA = typename std::conditional<TA, AcrossK, AlongK>::type;
+    using FragB = typename std::conditional<TB, AlongK, AcrossK>::type;
+    auto loadAlongK = [&](const _Float16* rowPtr, uint32_t g) {
+        AlongK f;
+        f.v = *reinterpret_cast<const halfx8a2*>(rowPtr + (g * kGroupK + kh * 8));
+        return f;
+    };
+    auto loadAcrossK = [&](const _Float16* colPtr, size_t ld, uint32_t g) {
+        const uint16_t* p =
+            reinterpret_cast<const uint16_t*>(colPtr + static_cast<size_t>(g * kGroupK + kh * 8) * ld);
+        AcrossK f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            f.r[e] = p[e * ld];
+        return f;
+    };
+    auto loadA = [&](uint32_t g) -> FragA {
+        if constexpr (TA)
+            return loadAcrossK(aPtr, args.lda, g);
+        else
+            return loadAlongK(aPtr, g);
+    };
+    auto loadB = [&](uint32_t g) -> FragB {
+        if constexpr (TB)
+            return loadAlongK(bPtr, g);
+        else
+            return loadAcrossK(bPtr, args.ldb, g);
+    };
+    // the last group when K is no multiple of kGroupK: element by element, zeros past K
+    auto loadPartial = [&](const _Float16* base, size_t step, uint32_t g) -> halfx8 {
+        const uint32_t k = g * kGroupK + kh * 8;
+        const _Float16* p = base + static_cast<size_t>(k) * step;
+        halfx8 v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+        {
+            v[e] = static_cast<_Float16>(0.f);
+            if (k + e < K)
+                v[e] = p[e * step];
+        }
+        return v;
+    };
+    // operands swapped: the result block comes out indexed [column][row], which leaves 4
+    // consecutive columns of one row in a lane
+    auto multiply = [&](const halfx8& a, const halfx8& b) {
+        if constexpr (TILE == 32)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(b, a, acc, 0, 0, 0);
+        else
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(b, a, acc, 0, 0, 0);
+    };
+
+    constexpr int kDepth = 4;  // groups in flight
+    const uint32_t whole = K / kGroupK;          // groups with every k below K
+    const uint32_t wholeEnd = min(gEnd, whole);  // this wavefront's whole groups end here
+    if (gBegin < wholeEnd)
+    {
+        const uint32_t lastWhole = wholeEnd - 1;
+        const uint32_t roundsEnd = gBegin + (wholeEnd - gBegin) / kDepth * kDepth;
+        FragA fa[kDepth];
+        FragB fb[kDepth];
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d)
+        {
+            // past the last whole group: that group once more, loaded and not used
+            fa[d] = loadA(min(gBegin + d, lastWhole));
+            fb[d] = loadB(min(gBegin + d, lastWhole));
+        }
+        for (uint32_t g = gBegin; g < roundsEnd; g += kDepth)
+        {
+#pragma unroll
+            for (int d = 0; d < kDepth; ++d)
+            {
+                // multiply, then load the group kDepth further on into the same registers
+                // (loading first needs a second set and a copy, behind a wait for every load,
+                // at the end of each round); the fences keep that order
+                multiply(fa[d].get(), fb[d].get());
+                __builtin_amdgcn_sched_barrier(0);
+                const uint32_t next = min(g + kDepth + d, lastWhole);
+                fa[d] = loadA(next);
+                fb[d] = loadB(next);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // fewer than kDepth whole groups left: already in registers
+#pragma unroll
+        for (int d = 0; d < kDepth - 1; ++d)
+            if (roundsEnd + d < wholeEnd)
+                multiply(fa[d].get(), fb[d].get());
+    }
+    if (gBegin <= whole && whole < gEnd)
+    {
+        // at most one group, and only in the wavefront that holds the end of K
+        const halfx8 a = TA ? loadPartial(aPtr, args.lda, whole) : loadPartial(aPtr, 1, whole);
+        const halfx8 b = TB ? loadPartial(bPtr, 1, whole) : loadPartial(bPtr, args.ldb, whole);
+        multiply(a, b);
+    }
+
+    // lane l holds row l % TILE, columns 4*kLaneGroups*q + 4*(l / TILE) + 0..3 of the tile;
+    // partial sums of the other wavefronts go through LDS, wavefront 0 adds them in order
+    if (wave != 0)
+    {
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q)
+            *reinterpret_cast<float4*>(
+                &partial[wave - 1][lt * TILE + 4 * kLaneGroups * q + 4 * kh]) =
+                make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+    }
+    __syncthreads();
+    if (wave != 0)
+        return;
+#pragma unroll
+    for (int w = 0; w < WAVES - 1; ++w)
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q)
+        {
+            const float4 p = *reinterpret_cast<const float4*>(
+                &partial[w][lt * TILE + 4 * kLaneGroups * q + 4 * kh]);
+            acc[4 * q + 0] += p.x;
+            acc[4 * q + 1] += p.y;
+            acc[4 * q + 2] += p.z;
+            acc[4 * q + 3] += p.w;
+        }
+    if (row >= M)
+        return;
+#pragma unroll
+    for (int q = 0; q < kQuads; ++q)
+    {
+        const uint32_t c = tn * TILE + 4 * kLaneGroups * q + 4 * kh;
+        if (c >= N)
+            continue;
+        float* p = out + static_cast<size_t>(row) * args.ldc + c;
+        if (c + 4 <= N)
+        {
+            floatx4 v = floatx4{acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+            if (!args.overwrite)
+            {
+                const floatx4 old = *reinterpret_cast<const floatx4a4*>(p);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    v[e] = old[e] + v[e];
+            }
+            *reinterpret_cast<floatx4a4*>(p) = v;
+        }
+        else
+        {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (c + e < N)
+                    p[e] = args.overwrite ? acc[4 * q + e] : p[e] + acc[4 * q + e];
+        }
+    }
+}
+
 // What one launch may assume about where its operands lie.
 struct F16Layout
 {
@@ -1746,6 +1986,62 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
+template <bool TA, bool TB>
+void LaunchFew(const GemmF16Args& args, uint32_t blocks, uint32_t tile, bool wide,
+               hipStream_t stream)
+{
+    const dim3 g(blocks);
+    if (tile == 16 && wide)
+        hipLaunchKernelGGL((GemmF16Few<16, TA, TB, 16>), g, dim3(1024), 0, stream, args);
+    else if (tile == 16)
+        hipLaunchKernelGGL((GemmF16Few<16, TA, TB, 4>), g, dim3(256), 0, stream, args);
+    else
+        hipLaunchKernelGGL((GemmF16Few<32, TA, TB, 4>), g, dim3(256), 0, stream, args);
+}
+
+// Products with at most one 32 x 32 output tile per compute unit, and narrow ones (16 rows or
+// columns at most) with up to four 16 x 16 tiles per compute unit, run on the few-tile kernel,
+// whatever their storage flags and alignment: the decision looks at M, N and the batch only, so
+// one product always takes the same kernel and sums in the same order.  Measured against the
+// 128-tile kernel (us, plain / A stored K x M / B stored N x K): 256 x 1024 x 1024 6.5 / 7.0 /
+// 7.3 against 10.6 / 11.7 / 10.3, 512^3 5.2 against 8.5, 100 x 1024 x 784 5.4 against 10.4,
+// 1024 x 10 x 1024 4.5 against 12.5, 16384 x 10 x 256 4.6 against 11.9; with two tiles per
+// compute unit (512 x 1024 x 1024) the two are level, with four the tiled kernel wins.
+bool TakesFewTiles(uint32_t M, uint32_t N, uint32_t batch)
+{
+    const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
+    const uint64_t blocks32 = static_cast<uint64_t>((M + 31) / 32) * ((N + 31) / 32) * batch;
+    const uint64_t blocks16 = static_cast<uint64_t>((M + 15) / 16) * ((N + 15) / 16) * batch;
+    return blocks32 <= cus || (std::min(M, N) <= 16 && blocks16 <= 4 * cus);
+}
+
+int LaunchFewTiles(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream)
+{
+    // 16 x 16 tiles while there are at most one and a half per compute unit, or for a narrow
+    // matrix (less of a tile outside it): a quarter of the matrix-core work per workgroup on
+    // four times as many compute units, but twice the operand bytes per flop (64 x 1024 x 1024:
+    // 4.9 us against 6.3 on 32 x 32; 128 x 1024 x 1024: 6.9 against 6.4); 16 wavefronts per tile
+    // when the tiles fit the chip once and K is long (128 x 128 x 4096: 10.4 us against 14.2)
+    const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
+    const uint64_t blocks16 =
+        static_cast<uint64_t>((args.M + 15) / 16) * ((args.N + 15) / 16) * batch;
+    const uint32_t tile =
+        (2 * blocks16 <= 3 * cus || std::min(args.M, args.N) <= 16) ? 16u : 32u;
+    args.tilesM = (args.M + tile - 1) / tile;
+    args.tilesN = (args.N + tile - 1) / tile;
+    const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
+    const bool wide = tile == 16 && blocks <= cus && args.K >= 1024;
+    if (lay.transA && lay.transB)
+        LaunchFew<true, true>(args, static_cast<uint32_t>(blocks), tile, wide, stream);
+    else if (lay.transA)
+        LaunchFew<true, false>(args, static_cast<uint32_t>(blocks), tile, wide, stream);
+    else if (lay.transB)
+        LaunchFew<false, true>(args, static_cast<uint32_t>(blocks), tile, wide, stream);
+    else
+        LaunchFew<false, false>(args, static_cast<uint32_t>(blocks), tile, wide, stream);
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
 }  // namespace
 
 extern "C" {
@@ -1802,6 +2098,8 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.strideB = strideB;
     args.overwrite = (flags & SPH_GEMM_OVERWRITE) ? 1u : 0u;
 
+    if (TakesFewTiles(M, N, batch))
+        return LaunchFewTiles(args, batch, lay, stream);
     return LaunchF16(args, batch, lay, stream);
 }
 

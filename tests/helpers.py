@@ -123,3 +123,31 @@ def gpu_transpose(x, rows, cols, batch=1):
     dX.release()
     dY.release()
     return out
+
+
+# Small products run on the few-tile kernel: at most one 32 x 32 output tile per compute unit
+# (256 of them), or a matrix of at most 16 rows or columns with at most four 16 x 16 tiles per
+# compute unit.  The tests of the tiled kernels' edges use small matrices, so each of those shapes
+# is run twice: as given (few-tile kernel, where it qualifies) and with the batch raised until
+# the tiled kernels take it.
+F16_FEW_TILE_CUS = 256
+
+
+def f16_few_tiles(M, N, batch):
+    b32 = -(-M // 32) * -(-N // 32) * batch
+    b16 = -(-M // 16) * -(-N // 16) * batch
+    return b32 <= F16_FEW_TILE_CUS or (min(M, N) <= 16 and b16 <= 4 * F16_FEW_TILE_CUS)
+
+
+def f16_both_kernel_families(shapes):
+    out = []
+    for shape in shapes:
+        M, N, K = shape[:3]
+        batch = shape[3] if len(shape) > 3 else 1
+        out.append((M, N, K, batch))
+        if f16_few_tiles(M, N, batch):
+            tiled = batch
+            while f16_few_tiles(M, N, tiled):
+                tiled += 1
+            out.append((M, N, K, tiled))
+    return out

@@ -31,9 +31,10 @@ def same_specials(got, ref, tol, den):
 
 # ---- subnormals -----------------------------------------------------------------------------
 
-# every kernel of the fp16 entry: 256-tiles with and without the in-loop accumulate, 128-tiles,
-# general
-F16_SHAPES = [(256, 256, 64, 192), (256, 256, 1152, 192), (128, 136, 96, 1), (70, 50, 44, 1)]
+# every kernel of the fp16 entry: 256-tiles with and without the in-loop accumulate, few-tile
+# (32- and 16-wide tiles), 128-tiles, general
+F16_SHAPES = [(256, 256, 64, 192), (256, 256, 1152, 192), (128, 136, 96, 1), (70, 50, 44, 1),
+              (128, 136, 96, 20), (70, 50, 44, 50), (300, 200, 1100, 1)]
 
 
 @pytest.mark.parametrize("shape", F16_SHAPES)
