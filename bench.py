@@ -303,11 +303,14 @@ def bench_mlp_backward(capi, synth, steps, warmup, direct, graph=False, fused_up
 
 # Shapes off the kernels' natural grid: a K that is no multiple of the K step, an N (or M) that is
 # no multiple of the copy width, operands stored the other way round.
+# small products (few output tiles: a layer of a small network on a small batch) ride along
+SMALL = [(256, 1024, 1024), (100, 1024, 784), (1024, 10, 1024), (128, 128, 4096), (512, 1024, 1024)]
 OFF_GRID_F16 = [(4096, 4096, 4096), (4096, 4096, 4080), (4096, 4096, 4095), (4096, 4100, 4096),
-                (4096, 4095, 4096), (4095, 4095, 4095), (2048, 2052, 2048), (1024, 1024, 1001)]
+                (4096, 4095, 4096), (4095, 4095, 4095), (2048, 2052, 2048), (1024, 1024, 1001),
+                (1024, 1024, 1024)] + SMALL
 OFF_GRID_F32 = [(1024, 1024, 1024), (1024, 1024, 1000), (1024, 1024, 1001), (1000, 1000, 1000),
                 (1001, 1001, 1001), (1024, 1026, 1024), (2048, 2048, 2047), (2048, 2050, 2048),
-                (4096, 4096, 4096), (4096, 4095, 4096), (4096, 4096, 4100)]
+                (4096, 4096, 4096), (4096, 4095, 4096), (4096, 4096, 4100)] + SMALL
 
 
 def bench_off_grid(capi, synth, steps, warmup):
