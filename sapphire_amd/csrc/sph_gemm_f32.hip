@@ -1682,14 +1682,19 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
 
     if (fewTiles)
     {
-        // 16 x 16 tiles while there are at most four per compute unit: a quarter of the
-        // matrix-core work per workgroup on four times as many compute units, and less of a
-        // tile outside a narrow matrix (measured: 256^3 6.5 -> 4.1 us, 1024 x 10 x 1024
-        // 13.3 -> 6.1 us, 256 x 256 x 4096 40 -> 16.5 us; 640^3 is better off on 32 x 32)
+        // 16 x 16 tiles while there are at most two per compute unit, or for a matrix of at most
+        // 16 rows or columns: a quarter of the matrix-core work per workgroup on four times as
+        // many compute units and less of a tile outside a narrow matrix, but twice the operand
+        // bytes per flop (measured, 16-wide against 32-wide tiles: 256^3 3.7 / 5.2 us,
+        // 1024 x 10 x 1024 7.2 / 8.9, 128 x 128 x 4096 13.8 / 23.4, 128 x 1024 x 1024 8.4 / 8.8;
+        // 192 x 1024 x 1024 11.0 / 9.3, 256 x 1024 x 1024 14.0 / 9.0, 512^3 9.6 / 6.6,
+        // 256 x 1024 x 4096 51.5 / 25.3)
         const uint64_t blocks16 =
             static_cast<uint64_t>((args.M + 15) / 16) * ((args.N + 15) / 16) * units;
-        const uint32_t tile =
-            (blocks16 <= static_cast<uint64_t>(sph::ComputeUnits()) * 4 || args.N < 4) ? 16u : 32u;
+        const uint32_t tile = (blocks16 <= static_cast<uint64_t>(sph::ComputeUnits()) * 2 ||
+                               std::min(args.M, args.N) <= 16)
+                                  ? 16u
+                                  : 32u;
         args.tilesM = (args.M + tile - 1) / tile;
         args.tilesN = (args.N + tile - 1) / tile;
         const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
