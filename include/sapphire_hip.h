@@ -284,7 +284,12 @@ int sph_gemm_f32_grouped_device(const SphGemmEntry* deviceEntries, uint32_t coun
  * flags: SPH_GEMM_OVERWRITE stores A*B without reading out (for callers that
  * know out holds zeros); default accumulates like the reference.
  * SPH_GEMM_TRANS_A / SPH_GEMM_TRANS_B read an operand stored transposed
- * (A as K x M, B as N x K), as in sph_gemm_f32_ex. */
+ * (A as K x M, B as N x K), as in sph_gemm_f32_ex.  The order in which the K
+ * products of an output element are added depends on the shape and, on the
+ * last M % 8 rows and N % 8 columns, on the storage order: results agree with
+ * the CPU loop within the fp16 path's 1e-2 tolerance, and exactly whenever
+ * every partial sum is exactly representable (the products themselves are
+ * exact in fp32, subnormal inputs included). */
 
 int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M,
                     uint32_t N, uint32_t K, uint32_t batch, int64_t strideOut,

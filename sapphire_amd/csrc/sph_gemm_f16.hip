@@ -47,7 +47,7 @@
 // that shape (the copies into LDS need no alignment, so rows of B and of out may start
 // anywhere; only a copy's 8 columns have to lie inside the row) and the last r columns to
 // GemmF16Cols, a stream over A with the fragments loaded straight into registers (to the
-// general kernel when A is stored K x M).
+// few-tile kernel when A is stored K x M, as are the last M % 8 rows of such an A).
 #include "sph_internal.h"
 
 #include <algorithm>
@@ -79,10 +79,6 @@ struct GemmF16Args
     int64_t strideOut, strideA, strideB;
     uint32_t overwrite;
     uint32_t outVec;  // general kernel: out may be accessed 16 bytes at a time
-    // 128-tile kernel: rows / columns of this launch's out below these are computed but not
-    // stored (a launch over the last 8 rows or columns of a matrix whose other rows or columns
-    // another launch has written)
-    uint32_t rowStoreFrom, colStoreFrom;
 };
 
 // Transposing LDS read: within each group of 16 lanes, lane s supplies the
@@ -1018,26 +1014,14 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
             {
                 const uint32_t r = rowBase + waveM * 64 + i * 32 + l32;
                 const uint32_t c = colBase + (waveN * TN + j) * 32 + 8 * q + 4 * khalf;
-                if (r < M && c < N && r >= args.rowStoreFrom)
+                if (r < M && c < N)
                 {
                     float4 v = old[(i * TN + j) * 4 + q];
                     v.x += acc[i][j][4 * q + 0];
                     v.y += acc[i][j][4 * q + 1];
                     v.z += acc[i][j][4 * q + 2];
                     v.w += acc[i][j][4 * q + 3];
-                    float* p = out + static_cast<size_t>(r) * args.ldc + c;
-                    if (c >= args.colStoreFrom)
-                        Store4(p, v);
-                    else
-                    {
-                        // a quad that straddles the first stored column
-                        if (c + 1 >= args.colStoreFrom)
-                            p[1] = v.y;
-                        if (c + 2 >= args.colStoreFrom)
-                            p[2] = v.z;
-                        if (c + 3 >= args.colStoreFrom)
-                            p[3] = v.w;
-                    }
+                    Store4(out + static_cast<size_t>(r) * args.ldc + c, v);
                 }
             }
 }
@@ -1771,8 +1755,6 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     const bool plain = !transA && !transB;
     const bool whole256 = (M % kT == 0) && (N % kT == 0);
     const bool tile256 = kind == F16Kernel::kTile256;
-    SPH_REQUIRE(kind == F16Kernel::kDma128 || (args.rowStoreFrom == 0 && args.colStoreFrom == 0),
-                "only the 128-tile kernel leaves rows or columns unstored");
     const uint32_t edge = tile256 ? kT : kG;
     args.tilesM = (M + edge - 1) / edge;
     args.tilesN = (N + edge - 1) / edge;
@@ -1910,6 +1892,8 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
 // only the r rows the first launch has not written.  With such an A the last r columns are
 // served the same way, by the 128-tile kernel over the last 8 columns (GemmF16Cols reads A
 // along K).  Every output element is still computed by one kernel.
+int LaunchFewTiles(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream);
+
 int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream)
 {
     const uint32_t M = args.M, N = args.N;
@@ -1917,22 +1901,21 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
     if (whole != F16Kernel::kGeneral)
         return LaunchF16Kernel(args, batch, whole, lay, stream);
 
-    // (the parts must not fall back to the general kernel, which stores every row: N has to be
-    // a multiple of 8 or wide enough for the column split below)
-    if (lay.transA && M % 8 != 0 && M >= 16 && (N % 8 == 0 || (N & ~7u) >= 8))
+    // A stored K x M with M = 8 q + r, r != 0: the first 8 q rows as a product of their own (if
+    // a straight-to-LDS kernel then takes them), the last r rows on the few-tile kernel, which
+    // reads any rows from anywhere
+    if (lay.transA && M % 8 != 0 && M >= 16 && (N & ~7u) >= 8)
     {
         GemmF16Args top = args;
         top.M = M & ~7u;
-        GemmF16Args bottom = args;
-        bottom.M = 8;
-        bottom.A = args.A + (M - 8);
-        bottom.out = args.out + static_cast<size_t>(M - 8) * args.ldc;
-        bottom.rowStoreFrom = 8 - M % 8;
-        if (PickF16(top, N & ~7u, batch, lay) != F16Kernel::kGeneral &&
-            PickF16(bottom, N & ~7u, batch, lay) == F16Kernel::kDma128)
+        if (PickF16(top, N & ~7u, batch, lay) != F16Kernel::kGeneral)
         {
+            GemmF16Args bottom = args;
+            bottom.M = M % 8;
+            bottom.A = args.A + top.M;
+            bottom.out = args.out + static_cast<size_t>(top.M) * args.ldc;
             const int rc = LaunchF16(top, batch, lay, stream);
-            return rc != SPH_OK ? rc : LaunchF16(bottom, batch, lay, stream);
+            return rc != SPH_OK ? rc : LaunchFewTiles(bottom, batch, lay, stream);
         }
     }
 
@@ -1942,12 +1925,11 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
     // fewer than 8 columns: the kernel for the last columns computes all of them (it streams A
     // along K, so not for an A stored K x M; measured 1024 x 10 x 1024: 53 us on the general
     // kernel's 2-byte loads)
-    const bool colsAlone = wholeChunks == 0 && !lay.transA && args.K >= kTK &&
-                           args.rowStoreFrom == 0 && args.colStoreFrom == 0;
+    const bool colsAlone = wholeChunks == 0 && !lay.transA && args.K >= kTK;
     if (!colsAlone)
     {
-        if (wholeChunks == 0)
-            return LaunchF16Kernel(args, batch, whole, lay, stream);
+        if (wholeChunks == 0)  // fewer than 8 columns of an A stored K x M, or K < 32
+            return LaunchFewTiles(args, batch, lay, stream);
         const F16Kernel most = PickF16(args, wholeChunks, batch, lay);
         if (most == F16Kernel::kGeneral)
             return LaunchF16Kernel(args, batch, whole, lay, stream);
@@ -1958,23 +1940,13 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
             return rc;
     }
     GemmF16Args right = args;
-    if (lay.transA)
-    {
-        // the last 8 columns, of which the first 8 - r are not stored
-        right.N = 8;
-        right.out = args.out + (N - 8);
-        right.B = args.B + (lay.transB ? static_cast<size_t>(N - 8) * args.K : N - 8);
-        right.colStoreFrom = 8 - N % 8;
-        const F16Kernel thin = PickF16(right, 8, batch, lay);
-        if (thin == F16Kernel::kDma128)
-            return LaunchF16Kernel(right, batch, thin, lay, stream);
-        right = args;
-    }
     right.N = N - wholeChunks;
     right.out = args.out + wholeChunks;
     right.B = args.B + (lay.transB ? static_cast<size_t>(wholeChunks) * args.K : wholeChunks);
+    // the last-columns kernel streams A along K; with A stored K x M the few-tile kernel takes
+    // the columns
     if (lay.transA)
-        return LaunchF16Kernel(right, batch, F16Kernel::kGeneral, lay, stream);
+        return LaunchFewTiles(right, batch, lay, stream);
     right.tilesM = (args.M + kColsRows - 1) / kColsRows;
     const uint64_t groups = static_cast<uint64_t>(right.tilesM) * batch;
     SPH_REQUIRE(groups < (1ull << 31), "too many rows for one launch");

@@ -204,7 +204,8 @@ def test_transposed_operands_exact_on_integers(dev, shape, flags):
 
 # N = 8 q + r, r != 0: the first 8 q
 # columns on the straight-to-LDS kernels (rows of B and of out start at addresses that are no
-# multiples of 16 bytes), the last r on the general kernel.  (M, N, K, batch): 128-tile kernel
+# multiples of 16 bytes), the last r on the last-columns kernel (the few-tile kernel when A is
+# stored K x M).  (M, N, K, batch): 128-tile kernel
 # with four and with eight wavefronts, ragged and whole 256-tiles (old values of out added in the
 # epilogue, K = 64, or in the loop, K = 640), N % 4 == 0, N % 2 == 0 and odd N, a K tail on top.
 @pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
@@ -239,7 +240,7 @@ def test_column_count_not_a_multiple_of_eight(dev, shape, flags):
 
 
 # A stored K x M with M = 8 q + r, r != 0 (and N % 8 != 0 on top): the first 8 q rows as before,
-# the last 8 rows (columns) by a launch of the 128-tile kernel that stores only the r new ones.
+# the last r rows (columns) by a launch of the few-tile kernel over that strip.
 # 257 x 256 x 640 x 192: the whole-tile kernel with the old values added in its loop on top, 8 rows
 # below it; 4095 x 3077: ragged 256-tiles.
 @pytest.mark.parametrize("flags", [capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
