@@ -2002,6 +2002,7 @@ int LaunchFewTiles(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipSt
     args.tilesM = (args.M + tile - 1) / tile;
     args.tilesN = (args.N + tile - 1) / tile;
     const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
+    SPH_REQUIRE(blocks < (1ull << 31), "too many tiles for one launch");
     const bool wide = tile == 16 && blocks <= cus && args.K >= 1024;
     if (lay.transA && lay.transB)
         LaunchFew<true, true>(args, static_cast<uint32_t>(blocks), tile, wide, stream);
