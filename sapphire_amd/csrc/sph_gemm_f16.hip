@@ -3,7 +3,7 @@
 // Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50): half
 // inputs, fp32 accumulation, row-major operands, result added into out.
 //
-// Four kernels (and one for the odd columns, see below):
+// Four kernels:
 //
 //   GemmF16Few      products with at most one 32 x 32 output tile per compute unit (or at most 16
 //     rows or columns), whatever K, the storage flags and the alignment: one 32 x 32 or 16 x 16
@@ -43,11 +43,10 @@
 // K = 32 q + r, r != 0, K >= 64 stays on the first two kernels: a last step over [K - 32, K) in
 // which the fragment positions whose k was multiplied already are cleared.
 //
-// N = 8 q + r, r != 0: the first 8 q columns go to the first two kernels when they would take
-// that shape (the copies into LDS need no alignment, so rows of B and of out may start
+// N = 8 q + r, r != 0: the first 8 q columns go to the tiled straight-to-LDS kernels when they
+// would take that shape (the copies into LDS need no alignment, so rows of B and of out may start
 // anywhere; only a copy's 8 columns have to lie inside the row) and the last r columns to
-// GemmF16Cols, a stream over A with the fragments loaded straight into registers (to the
-// few-tile kernel when A is stored K x M, as are the last M % 8 rows of such an A).
+// GemmF16Few, as do the last M % 8 rows of an A stored K x M.
 #include "sph_internal.h"
 
 #include <algorithm>
@@ -1285,169 +1284,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
     }
 }
 
-// ---------------------------------------------------------------------------
-// the last N % 8 columns of a product whose other columns a straight-to-LDS kernel computes
-// ---------------------------------------------------------------------------
-// out[M x r] (+)= A[M x K] * B[K x r] with r < 8: all of A is read for 2 M r K flops, so this
-// is a stream over A.  A workgroup owns 16 rows; its 8 wavefronts take every 8th K step of
-// 32.  The A fragment of v_mfma_f32_16x16x32_f16 comes straight from global memory: lane l
-// holds k = 8 (l / 16) .. + 7 of row l % 16 (one 16-byte load from a 2-byte-aligned address; the
-// values of a piece that reaches past K are read one by one).  The B fragment (column l % 16,
-// the same k; zeros or don't-cares for columns from r on, zeros for k >= K):
-//   B stored N x K: one 16-byte load;
-//   B stored K x N: the r values of a k-row are the last of that row, so the 16 bytes that start
-//     with them end inside the next row (for the last k-row they are read one by one).  The
-//     workgroup first copies these 16 bytes of every k-row of a slab of 4096 into LDS and the
-//     wavefronts pick their fragments up with transposing reads; what lies beyond column r only
-//     reaches outputs that are never stored.
-// The 8 partial products meet in LDS and are added in wavefront order.
-constexpr int kColsWaves = 8;
-constexpr int kColsRows = 16;
-constexpr int kColsSlab = 4096;  // k-rows of B's last columns held in LDS at a time (64 KiB)
 typedef halfx8 halfx8a2 __attribute__((aligned(2)));
-template <bool TB>
-__global__ __launch_bounds__(kColsWaves * 64) void GemmF16Cols(const GemmF16Args args)
-{
-    __shared__ float part[kColsWaves][32][4];
-    __shared__ __attribute__((aligned(16))) _Float16 tailB[TB ? 8 : kColsSlab * 8];
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t M = args.M, r = args.N, K = args.K;
-    const uint32_t unit = blockIdx.x / args.tilesM;
-    const uint32_t rowBase = (blockIdx.x % args.tilesM) * kColsRows;
-    const _Float16* __restrict__ A = args.A + args.strideA * static_cast<int64_t>(unit);
-    const _Float16* __restrict__ B = args.B + args.strideB * static_cast<int64_t>(unit);
-    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit);
-
-    const uint32_t x = lane & 15;          // row of A / column of B
-    const uint32_t kLane = 8 * (lane >> 4);
-    const _Float16* aRow = A + static_cast<size_t>(min(rowBase + x, M - 1)) * args.lda + kLane;
-    const bool colExists = x < r;
-    const _Float16* bCol = B + static_cast<size_t>(colExists ? x : 0) * K + kLane;  // TB only
-    // transposing read: lane x of a 16-lane group addresses k-row x / 4 of a block of four and
-    // columns 4 (x % 4) .. + 3 of it; an LDS k-row holds 8 columns, so lanes that would ask for
-    // columns 8-15 ask for 0-7 again
-    const uint32_t trOffset = (kLane + (x >> 2)) * 8 + 4 * (x & 1);
-    floatx4 acc = { 0.f, 0.f, 0.f, 0.f };
-    // 8 values of k from k0 on, zeros from K on; 16 bytes at once while they lie inside the row
-    auto fetch8 = [&](const _Float16* p, uint32_t k0) {
-        halfx8 v = {};
-        if (k0 + 8 <= K)
-            v = *reinterpret_cast<const halfx8a2*>(p);
-        else
-        {
-#pragma unroll
-            for (int e = 0; e < 7; ++e)
-                if (k0 + e < K)
-                    v[e] = p[e];
-        }
-        return v;
-    };
-    auto fetchA = [&](uint32_t step) {
-        return fetch8(aRow + static_cast<size_t>(step) * kTK, step * kTK + kLane);
-    };
-    auto fetchB = [&](uint32_t step, uint32_t slabStart) {
-        halfx8 v = {};
-        if constexpr (TB)
-        {
-            if (colExists)
-                v = fetch8(bCol + static_cast<size_t>(step) * kTK, step * kTK + kLane);
-        }
-        else
-        {
-            const _Float16* p = &tailB[(step * kTK - slabStart) * 8 + trOffset];
-            v = Join(LdsReadTr(p), LdsReadTr(p + 4 * 8));
-        }
-        return v;
-    };
-    for (uint32_t slabStart = 0; slabStart < K; slabStart += kColsSlab)
-    {
-        const uint32_t slabEnd = TB ? K : min(K, slabStart + kColsSlab);
-        if constexpr (!TB)
-        {
-            if (slabStart != 0)
-                __syncthreads();  // everybody is done with the slab before
-            // whole K steps: k-rows from K on are zeros
-            const uint32_t rowsHere = (slabEnd - slabStart + kTK - 1) / kTK * kTK;
-            constexpr int kPerThread = kColsSlab / (kColsWaves * 64);
-            halfx8 rows[kPerThread];
-#pragma unroll
-            for (int i = 0; i < kPerThread; ++i)
-            {
-                const uint32_t gk = slabStart + threadIdx.x + i * kColsWaves * 64;
-                const _Float16* p = B + static_cast<size_t>(gk) * args.ldb;
-                rows[i] = halfx8{};
-                if (gk + 1 < K)
-                    rows[i] = *reinterpret_cast<const halfx8a2*>(p);
-                else if (gk < K)
-                {
-#pragma unroll
-                    for (int e = 0; e < 7; ++e)
-                        if (e < static_cast<int>(r))
-                            rows[i][e] = p[e];
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < kPerThread; ++i)
-            {
-                const uint32_t k = threadIdx.x + i * kColsWaves * 64;
-                if (k < rowsHere)
-                    *reinterpret_cast<halfx8*>(&tailB[k * 8]) = rows[i];
-            }
-            __syncthreads();
-        }
-        // four steps' loads in flight per wavefront
-        const uint32_t stepEnd = (slabEnd + kTK - 1) / kTK;
-        for (uint32_t step = slabStart / kTK + wave; step < stepEnd; step += 4 * kColsWaves)
-        {
-            halfx8 a[4], b[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-            {
-                const uint32_t st = step + u * kColsWaves;
-                a[u] = halfx8{};
-                b[u] = halfx8{};
-                if (st < stepEnd)
-                {
-                    a[u] = fetchA(st);
-                    b[u] = fetchB(st, slabStart);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[u], a[u], acc, 0, 0, 0);
-        }
-        if constexpr (TB)
-            break;
-    }
-    // lane l now holds row l % 16, columns 4 (l / 16) .. + 3: the first 32 lanes hold columns 0-7
-    if (lane < 32)
-        *reinterpret_cast<floatx4*>(&part[wave][lane][0]) = acc;
-    __syncthreads();
-    if (threadIdx.x < 32)
-    {
-        floatx4 sum = *reinterpret_cast<const floatx4*>(&part[0][lane][0]);
-#pragma unroll
-        for (int w = 1; w < kColsWaves; ++w)
-        {
-            const floatx4 p = *reinterpret_cast<const floatx4*>(&part[w][lane][0]);
-            sum[0] += p[0];
-            sum[1] += p[1];
-            sum[2] += p[2];
-            sum[3] += p[3];
-        }
-        const uint32_t row = rowBase + x;
-        const uint32_t col = 4 * (lane >> 4);
-        if (row < M)
-        {
-            float* p = out + static_cast<size_t>(row) * args.ldc + col;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (col + e < r)
-                    p[e] = args.overwrite ? sum[e] : p[e] + sum[e];
-        }
-    }
-}
 
 // variant 0: whole tiles, out read in the epilogue; 1 / 2: out added inside the loop with
 // spacing 2 / 4; 3: ragged tiles
@@ -1884,14 +1721,13 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
 // Picks the kernels for one call.
 //
 // N = 8 q + r with r != 0 and a shape the straight-to-LDS kernels would take at N = 8 q: they
-// compute the first 8 q columns (row pitches of B and out stay N) and GemmF16Cols the last r
-// (measured 4096 x 4100 x 4096: 270 us on the general kernel alone, 130 us this way).
+// compute the first 8 q columns (row pitches of B and out stay N) and the few-tile kernel, which
+// reads any rows and columns from anywhere, the last r (measured 4096 x 4100 x 4096: 270 us on
+// the general kernel alone, 129 us this way).
 //
 // An A stored K x M is copied 8 rows of the product at a time, so with it M = 8 q + r is split
-// the same way: the first 8 q rows, then the 128-tile kernel over the LAST 8 rows, which stores
-// only the r rows the first launch has not written.  With such an A the last r columns are
-// served the same way, by the 128-tile kernel over the last 8 columns (GemmF16Cols reads A
-// along K).  Every output element is still computed by one kernel.
+// the same way: the first 8 q rows, then the few-tile kernel over the last r rows.  Every output
+// element is still computed by one kernel.
 int LaunchFewTiles(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream);
 
 int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream)
@@ -1922,42 +1758,24 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
     const uint32_t wholeChunks = N & ~7u;
     if (N % 8 == 0)
         return LaunchF16Kernel(args, batch, whole, lay, stream);
-    // fewer than 8 columns: the kernel for the last columns computes all of them (it streams A
-    // along K, so not for an A stored K x M; measured 1024 x 10 x 1024: 53 us on the general
-    // kernel's 2-byte loads)
-    const bool colsAlone = wholeChunks == 0 && !lay.transA && args.K >= kTK;
-    if (!colsAlone)
-    {
-        if (wholeChunks == 0)  // fewer than 8 columns of an A stored K x M, or K < 32
-            return LaunchFewTiles(args, batch, lay, stream);
-        const F16Kernel most = PickF16(args, wholeChunks, batch, lay);
-        if (most == F16Kernel::kGeneral)
-            return LaunchF16Kernel(args, batch, whole, lay, stream);
-        GemmF16Args left = args;
-        left.N = wholeChunks;
-        const int rc = LaunchF16Kernel(left, batch, most, lay, stream);
-        if (rc != SPH_OK)
-            return rc;
-    }
+    // fewer than 8 columns, or no straight-to-LDS kernel for the first 8 q: one kernel for all
+    if (wholeChunks == 0)
+        return LaunchFewTiles(args, batch, lay, stream);
+    const F16Kernel most = PickF16(args, wholeChunks, batch, lay);
+    if (most == F16Kernel::kGeneral)
+        return LaunchF16Kernel(args, batch, whole, lay, stream);
+    GemmF16Args left = args;
+    left.N = wholeChunks;
+    const int rc = LaunchF16Kernel(left, batch, most, lay, stream);
+    if (rc != SPH_OK)
+        return rc;
     GemmF16Args right = args;
     right.N = N - wholeChunks;
     right.out = args.out + wholeChunks;
     right.B = args.B + (lay.transB ? static_cast<size_t>(wholeChunks) * args.K : wholeChunks);
-    // the last-columns kernel streams A along K; with A stored K x M the few-tile kernel takes
-    // the columns
-    if (lay.transA)
-        return LaunchFewTiles(right, batch, lay, stream);
-    right.tilesM = (args.M + kColsRows - 1) / kColsRows;
-    const uint64_t groups = static_cast<uint64_t>(right.tilesM) * batch;
-    SPH_REQUIRE(groups < (1ull << 31), "too many rows for one launch");
-    const dim3 g(static_cast<uint32_t>(groups)), b(kColsWaves * 64);
-    if (lay.transB)
-        hipLaunchKernelGGL((GemmF16Cols<true>), g, b, 0, stream, right);
-    else
-        hipLaunchKernelGGL((GemmF16Cols<false>), g, b, 0, stream, right);
-    SPH_CHECK_LAUNCH();
-    return SPH_OK;
+    return LaunchFewTiles(right, batch, lay, stream);
 }
+
 template <bool TA, bool TB>
 void LaunchFew(const GemmF16Args& args, uint32_t blocks, uint32_t tile, bool wide,
                hipStream_t stream)

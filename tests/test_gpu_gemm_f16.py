@@ -204,8 +204,7 @@ def test_transposed_operands_exact_on_integers(dev, shape, flags):
 
 # N = 8 q + r, r != 0: the first 8 q
 # columns on the straight-to-LDS kernels (rows of B and of out start at addresses that are no
-# multiples of 16 bytes), the last r on the last-columns kernel (the few-tile kernel when A is
-# stored K x M).  (M, N, K, batch): 128-tile kernel
+# multiples of 16 bytes), the last r on the few-tile kernel.  (M, N, K, batch): 128-tile kernel
 # with four and with eight wavefronts, ragged and whole 256-tiles (old values of out added in the
 # epilogue, K = 64, or in the loop, K = 640), N % 4 == 0, N % 2 == 0 and odd N, a K tail on top.
 @pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
@@ -215,7 +214,7 @@ def test_transposed_operands_exact_on_integers(dev, shape, flags):
      (4096, 3076, 64, 1), (256, 257, 64, 192), (256, 260, 640, 192), (1000, 999, 992, 1),
      (248, 250, 72, 3),
      # narrow products: 8 or 96 columns on the 128-tile kernel and the rest, or all of fewer than
-     # 8 columns, on the last-columns kernel
+     # 8 columns, on the few-tile kernel
      (1024, 10, 1024, 1), (304, 100, 96, 2), (512, 5, 64, 3), (1000, 7, 1001, 1), (40, 3, 32, 1)]))
 def test_column_count_not_a_multiple_of_eight(dev, shape, flags):
     M, N, K, batch = shape
