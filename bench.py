@@ -130,6 +130,7 @@ def bench_gemm_f16(capi, synth, steps, warmup, flags=0, zero_operands=False):
     dA = capi.DeviceBuffer.from_array(d["A"])
     dB = capi.DeviceBuffer.from_array(d["B"])
     dC = capi.DeviceBuffer.from_array(d["C"])
+    capi.require_gemm_extents(dC, dA, dB, n, n, n, 1, n * n, n * n, n * n, operand_bytes=2)
 
     def launch():
         capi.call("sph_gemm_f16f32", dC.ptr, dA.ptr, dB.ptr, n, n, n, 1, n * n, n * n, n * n, flags)
@@ -148,6 +149,8 @@ def bench_spmm(capi, synth, steps, warmup):
     dRow = capi.DeviceBuffer.from_array(d["ROW"])
     dB = capi.DeviceBuffer.from_array(d["B"])
     dC = capi.DeviceBuffer.from_array(d["C"])
+    capi.require_csr_extents(dC, dV, dCol, dRow, dB, M, K, N, int(d["V"].size))
+    capi.validate_csr(dCol, dRow, M, K, int(d["V"].size))
 
     def launch():
         capi.call("sph_spmm_csr_f32", dC.ptr, dV.ptr, dCol.ptr, dRow.ptr, M, K, N, dB.ptr, 0)
@@ -163,6 +166,7 @@ def bench_spmm(capi, synth, steps, warmup):
 
 def bench_f32(capi, A, B, C, M, N, K, batch, sb, steps, warmup):
     dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    capi.require_gemm_extents(dC, dA, dB, M, N, K, batch, M * N, M * K, sb)
 
     def launch():
         capi.call("sph_gemm_f32", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, M * N, M * K, sb)
@@ -320,6 +324,8 @@ def bench_off_grid(capi, synth, steps, warmup):
     def one(entry, M, N, K, flags, A, B):
         C = np.zeros((M, N), np.float32)
         dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+        capi.require_gemm_extents(dC, dA, dB, M, N, K, 1, M * N, M * K, K * N,
+                                  operand_bytes=2 if entry == "sph_gemm_f16f32" else 4)
 
         def launch():
             capi.call(entry, dC.ptr, dA.ptr, dB.ptr, M, N, K, 1, M * N, M * K, K * N, flags)

@@ -387,6 +387,21 @@ int sph_csr_from_dense_f32(float* V, uint32_t* COL, uint32_t* ROW,
                            uint32_t capacity, const float* dense, uint32_t M,
                            uint32_t N, uint32_t ld, uint32_t* nnzHost);
 
+/* sph_csr_validate_u32: checks a CSR record before a product that trusts it.
+ * The reference's SparseMatrix (Includes/Sapphire/compute/sparse/SparseMatrix.hpp:28-38)
+ * carries no invariant checks, and neither do the products here: they read
+ * B[COL[p]] and the entries ROW[i] .. ROW[i + 1] as given, so an index outside
+ * the operand is a device memory fault.  This call reads only ROW[0 .. M] and
+ * COL[0 .. nnz) and reports, after the stream has drained (refused during
+ * graph capture): ROW[0] == 0, ROW non-decreasing, ROW[M] == nnz, every
+ * COL[p] < Kdim.  Any violation is SPH_ERR_INVALID with the violated rules
+ * named in sph_last_error(); when problemsHost is not NULL it receives a bit
+ * mask (1 ROW[0] != 0, 2 ROW decreasing, 4 ROW[M] != nnz, 8 column out of
+ * range, 16 a row whose columns are not strictly ascending -- the last one is
+ * reported but is no error: the products do not need sorted rows). */
+int sph_csr_validate_u32(const uint32_t* COL, const uint32_t* ROW, uint32_t M,
+                         uint32_t Kdim, uint32_t nnz, uint32_t* problemsHost);
+
 /* ---- CSR x CSR ------------------------------------------------------------ */
 
 /* C = A * B with all three in CSR (A is M x K, B is K x N).  The reference

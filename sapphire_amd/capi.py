@@ -105,6 +105,7 @@ SIGNATURES = {
     "sph_csr_to_dense_f32": [_vp, _u32, _vp, _vp, _vp, _u32, _u32],
     "sph_csr_from_dense_f32": [_vp, _vp, _vp, _u32, _vp, _u32, _u32, _u32,
                                ctypes.POINTER(ctypes.c_uint32)],
+    "sph_csr_validate_u32": [_vp, _vp, _u32, _u32, _u32, ctypes.POINTER(ctypes.c_uint32)],
     "sph_spgemm_row_offsets_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32,
                                    ctypes.POINTER(ctypes.c_uint32)],
     "sph_spgemm_fill_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],
@@ -194,6 +195,40 @@ class DeviceBuffer:
             self.release()
         except Exception:
             pass
+
+
+def require_gemm_extents(d_out, d_a, d_b, M, N, K, batch, stride_out, stride_a, stride_b,
+                         operand_bytes=4):
+    """Raises unless the three device buffers hold what a strided-batched product of this shape
+    reads and writes.  The C ABI takes raw pointers and trusts the extents; a caller that owns
+    DeviceBuffers checks them here before every such call, because an operand that is smaller
+    than its stated shape is a device memory fault, not an error code."""
+    last = max(int(batch), 1) - 1
+    need = (("out", d_out, (last * stride_out + M * N) * 4),
+            ("A", d_a, (last * stride_a + M * K) * operand_bytes),
+            ("B", d_b, (last * stride_b + K * N) * operand_bytes))
+    for name, buf, nbytes in need:
+        if buf.nbytes < nbytes:
+            raise ValueError("%s holds %d bytes, the %dx%dx%d x%d product needs %d"
+                             % (name, buf.nbytes, M, N, K, batch, nbytes))
+
+
+def require_csr_extents(d_out, d_v, d_col, d_row, d_b, M, Kdim, N, nnz):
+    """The same for a CSR x dense product: V and COL of nnz entries, ROW of M + 1, B Kdim x N,
+    out M x N."""
+    need = (("out", d_out, M * N * 4), ("V", d_v, nnz * 4), ("COL", d_col, nnz * 4),
+            ("ROW", d_row, (M + 1) * 4), ("B", d_b, Kdim * N * 4))
+    for name, buf, nbytes in need:
+        if buf.nbytes < nbytes:
+            raise ValueError("%s holds %d bytes, the %dx%d CSR x %dx%d product needs %d"
+                             % (name, buf.nbytes, M, Kdim, Kdim, N, nbytes))
+
+
+def validate_csr(d_col, d_row, M, Kdim, nnz):
+    """sph_csr_validate_u32 on device arrays; raises SphError when the record is unsafe."""
+    problems = ctypes.c_uint32(0)
+    call("sph_csr_validate_u32", d_col.ptr, d_row.ptr, M, Kdim, nnz, ctypes.byref(problems))
+    return problems.value
 
 
 def device_count():

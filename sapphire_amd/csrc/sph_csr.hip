@@ -839,3 +839,112 @@ int sph_csr_to_dense_f32(float* dense, uint32_t ld, const float* V, const uint32
 }
 
 }  // extern "C"
+
+// ---------------------------------------------------------------------------
+// Validation of a CSR record before it is handed to a kernel that trusts it.
+//
+// The products (sph_spmm_csr_f32, sph_spgemm_*) read B[COL[p]] and V[ROW[i] .. ROW[i + 1])
+// without checking: an index past the operand is a memory fault that can take the device
+// down for every process on it.  A caller that builds the arrays itself checks them here
+// first; the check only reads ROW[0 .. M] and COL[0 .. nnz), so it is safe on any contents.
+// ---------------------------------------------------------------------------
+namespace
+{
+enum : uint32_t
+{
+    kCsrRowStart = 1u,       // ROW[0] != 0
+    kCsrRowOrder = 2u,       // ROW[i] > ROW[i + 1]
+    kCsrRowTotal = 4u,       // ROW[M] != nnz
+    kCsrColRange = 8u,       // COL[p] >= Kdim
+    kCsrColUnsorted = 16u,   // a row's columns are not strictly ascending (not an error)
+};
+
+__global__ __launch_bounds__(256) void CsrValidateKernel(const uint32_t* __restrict__ COL,
+                                                         const uint32_t* __restrict__ ROW,
+                                                         uint32_t M, uint32_t Kdim, uint32_t nnz,
+                                                         uint32_t* __restrict__ problems)
+{
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+    const uint64_t first = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint32_t found = 0;
+    if (first == 0)
+    {
+        if (ROW[0] != 0)
+            found |= kCsrRowStart;
+        if (ROW[M] != nnz)
+            found |= kCsrRowTotal;
+    }
+    for (uint64_t i = first; i < M; i += stride)
+    {
+        const uint32_t begin = ROW[i], end = ROW[i + 1];
+        if (begin > end)
+            found |= kCsrRowOrder;
+        else if (end <= nnz)
+        {
+            // ascending columns inside the row; every index read lies below nnz
+            for (uint32_t p = begin; p + 1 < end; ++p)
+                if (COL[p] >= COL[p + 1])
+                {
+                    found |= kCsrColUnsorted;
+                    break;
+                }
+        }
+    }
+    for (uint64_t p = first; p < nnz; p += stride)
+        if (COL[p] >= Kdim)
+            found |= kCsrColRange;
+    if (found != 0)
+        atomicOr(problems, found);
+}
+}  // namespace
+
+extern "C" {
+
+int sph_csr_validate_u32(const uint32_t* COL, const uint32_t* ROW, uint32_t M, uint32_t Kdim,
+                         uint32_t nnz, uint32_t* problemsHost)
+{
+    if (problemsHost != nullptr)
+        *problemsHost = 0;
+    SPH_REQUIRE(ROW != nullptr, "ROW is null");
+    SPH_REQUIRE(nnz == 0 || COL != nullptr, "COL is null");
+    SPH_REQUIRE(M < 0xffffffffu, "too many rows");
+    SPH_REFUSE_WHILE_CAPTURING();  // reads the verdict back
+    hipStream_t stream = sph::CurrentStream();
+    if (stream == nullptr)
+        return SPH_ERR_DEVICE;
+    uint32_t* problems = nullptr;
+    SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&problems), sizeof(uint32_t), stream));
+    SPH_HIP_TRY(hipMemsetAsync(problems, 0, sizeof(uint32_t), stream));
+    const uint64_t items = std::max<uint64_t>(std::max<uint64_t>(M, nnz), 1);
+    const uint32_t grid = static_cast<uint32_t>(std::min<uint64_t>((items + 255) / 256, 4096));
+    hipLaunchKernelGGL(CsrValidateKernel, dim3(grid), dim3(256), 0, stream, COL, ROW, M, Kdim, nnz,
+                       problems);
+    const hipError_t launched = hipGetLastError();
+    uint32_t found = 0;
+    hipError_t copied = hipSuccess;
+    if (launched == hipSuccess)
+    {
+        copied = hipMemcpyAsync(&found, problems, sizeof(uint32_t), hipMemcpyDeviceToHost, stream);
+        if (copied == hipSuccess)
+            copied = hipStreamSynchronize(stream);
+    }
+    SPH_HIP_TRY(hipFreeAsync(problems, stream));
+    if (launched != hipSuccess)
+        return sph::Fail(SPH_ERR_DEVICE, std::string("sph_csr_validate_u32 launch failed with ") +
+                                             hipGetErrorString(launched));
+    SPH_HIP_TRY(copied);
+    if (problemsHost != nullptr)
+        *problemsHost = found;
+    if ((found & (kCsrRowStart | kCsrRowOrder | kCsrRowTotal | kCsrColRange)) != 0)
+    {
+        std::string what;
+        if (found & kCsrRowStart) what += " ROW[0] is not 0;";
+        if (found & kCsrRowOrder) what += " ROW is not non-decreasing;";
+        if (found & kCsrRowTotal) what += " ROW[M] differs from the entry count;";
+        if (found & kCsrColRange) what += " a column index is not below the column count;";
+        return sph::Fail(SPH_ERR_INVALID, "sph_csr_validate_u32 -" + what);
+    }
+    return SPH_OK;
+}
+
+}  // extern "C"

@@ -28,6 +28,7 @@ def gpu_gemm_f32(C, A, B, M, N, K, batch=1, stride_out=None, stride_a=None, stri
     sa = M * K if stride_a is None else stride_a
     sb = K * N if stride_b is None else stride_b
     dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    capi.require_gemm_extents(dC, dA, dB, M, N, K, batch, so, sa, sb)
     capi.call("sph_gemm_f32", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, so, sa, sb)
     out = dC.download(np.float32, C.shape)
     for d in (dA, dB, dC):
@@ -42,6 +43,7 @@ def gpu_gemm_f16(C, A16, B16, M, N, K, batch=1, stride_out=None, stride_a=None, 
     sb = K * N if stride_b is None else stride_b
     assert A16.dtype == np.float16 and B16.dtype == np.float16
     dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A16, B16, C))
+    capi.require_gemm_extents(dC, dA, dB, M, N, K, batch, so, sa, sb, operand_bytes=2)
     capi.call("sph_gemm_f16f32", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, so, sa, sb, flags)
     out = dC.download(np.float32, C.shape)
     for d in (dA, dB, dC):
@@ -52,6 +54,9 @@ def gpu_gemm_f16(C, A16, B16, M, N, K, batch=1, stride_out=None, stride_a=None, 
 def gpu_gemm_grouped(C, A, B, M, N, K, triples):
     dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
     entries = capi.make_entries(triples)
+    for o, a, b in triples:
+        assert (o + M * N) * 4 <= dC.nbytes and (a + M * K) * 4 <= dA.nbytes \
+            and (b + K * N) * 4 <= dB.nbytes, "a grouped unit lies outside its buffer"
     capi.call("sph_gemm_f32_grouped", entries, len(triples), dC.ptr, dA.ptr, dB.ptr, M, N, K)
     out = dC.download(np.float32, C.shape)
     for d in (dA, dB, dC):
@@ -68,6 +73,9 @@ def gpu_spmm(C, V, COL, ROW, M, Kdim, N, B, accumulate, canary=0):
     dCol = capi.DeviceBuffer.from_array(COL if COL.size else np.zeros(1, np.uint32))
     dRow = capi.DeviceBuffer.from_array(ROW)
     dB = capi.DeviceBuffer.from_array(B)
+    assert padded.nbytes >= 4 * (2 * canary + M * N)
+    capi.require_csr_extents(dC, dV, dCol, dRow, dB, M, Kdim, N, int(V.size))
+    capi.validate_csr(dCol, dRow, M, Kdim, int(V.size))
     capi.call("sph_spmm_csr_f32", dC.at(4 * canary), dV.ptr, dCol.ptr, dRow.ptr, M, Kdim, N,
               dB.ptr, 1 if accumulate else 0)
     back = dC.download(np.float32, padded.shape)
@@ -89,6 +97,9 @@ def gpu_spmm_bias(junk, V, COL, ROW, M, Kdim, N, B, row_bias, canary=0):
     dRow = capi.DeviceBuffer.from_array(ROW)
     dB = capi.DeviceBuffer.from_array(B)
     dBias = capi.DeviceBuffer.from_array(row_bias)
+    assert padded.nbytes >= 4 * (2 * canary + M * N) and dBias.nbytes >= 4 * M
+    capi.require_csr_extents(dC, dV, dCol, dRow, dB, M, Kdim, N, int(V.size))
+    capi.validate_csr(dCol, dRow, M, Kdim, int(V.size))
     capi.call("sph_spmm_csr_bias_f32", dC.at(4 * canary), dV.ptr, dCol.ptr, dRow.ptr, M, Kdim, N,
               dB.ptr, dBias.ptr)
     back = dC.download(np.float32, padded.shape)
@@ -108,6 +119,7 @@ def gpu_gemm_f32_ex(C, A, B, M, N, K, flags, batch=1, stride_out=None, stride_a=
     sa = M * K if stride_a is None else stride_a
     sb = K * N if stride_b is None else stride_b
     dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    capi.require_gemm_extents(dC, dA, dB, M, N, K, batch, so, sa, sb)
     capi.call("sph_gemm_f32_ex", dC.ptr, dA.ptr, dB.ptr, M, N, K, batch, so, sa, sb, flags)
     out = dC.download(np.float32, C.shape)
     for d in (dA, dB, dC):
