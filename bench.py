@@ -3,14 +3,18 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
 
-A step is one pass of the hot path over one batch of synthetic input: one launch of the
-fp16-input / fp32-accumulate GEMM at M = N = K = 4096 (configuration 3), out += A*B with the
-inputs already resident in HBM.  The script does W untimed steps, then times exactly K steps
-between two synchronisation points and prints ONE JSON line.  `value` is TFLOP/s of those K
-steps (2*4096^3 flop each).  The same line carries
+A step is one pass of the hot path over one batch of synthetic input: the fp16-input /
+fp32-accumulate GEMM at M = N = K = 4096 (configuration 3: y zeros, y += A*B) with the inputs
+already resident in HBM, issued the way the operator layer issues it -- a fresh TensorData y
+from the buffer pool, Compute::GemmHalf(y, A, B), ResourceManager::Clean() -- which is one
+kernel launch per step.  The script does W untimed steps, then times exactly K steps between
+two synchronisation points and prints ONE JSON line.  `value` is TFLOP/s of those K steps
+(2*4096^3 flop each).  The same line carries
 
   roofline      the GEMM kernel against the dense fp16 MFMA peak, from HIP events recorded on
-                the stream the kernel runs on;
+                the stream the kernel runs on, with the shader clock polled beside the leg;
+  gemm_accumulate_into_used_out_variant   the raw C-ABI call adding into an out that is in use;
+  gemm_zero_operands_variant              the headline leg on all-zero operands (clock beside it);
   spmm          the CSR x dense product of configuration 5 (8192 x 8192 at 1 % times
                 8192 x 256), timed the same way, against the HBM peak on algorithmic bytes;
   configs       configurations 1, 2 and 4 (fp32 GEMM, batched fp32 GEMM with a shared B, the
@@ -60,14 +64,14 @@ def parse():
     p.add_argument("--all", action="store_true",
                    help="also time the neighbouring kernels (backward pass, conversions, CSR x "
                         "CSR, one-pass kernels; reported under 'others')")
-    p.add_argument("--only", choices=["gemm", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
-                                      "csr", "spgemm", "shapes"], default=None,
+    p.add_argument("--only", choices=["gemm", "gemm_operator", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
+                                      "csr", "spgemm", "shapes", "mfma_ceiling"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
     p.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                    help="untimed run-up before each timed leg that lets the clock reach its "
                         "working frequency (0 = none)")
     p.add_argument("--zero-operands", action="store_true",
-                   help="with --only gemm: all-zero A and B, to see how far the clock (and the "
+                   help="with --only gemm / gemm_operator: all-zero A and B, to see how far the clock (and the "
                         "rate) depends on operand values; the line says data = zeros")
     return p.parse_args()
 
@@ -89,9 +93,102 @@ def settle(capi, launch):
         capi.sync()
 
 
-def timed_launches(capi, launch, steps, warmup):
+class ClockSampler:
+    """Polls the shader clock (sclk) in a thread beside a leg, so that the line shows at what
+    clock a figure was taken.  One visible card with a readable pp_dpm_sclk: that file, every
+    20 ms; otherwise `rocm-smi --showclocks` as fast as it returns."""
+
+    def __init__(self):
+        import glob
+        import threading
+        self.samples = []      # (seconds since start, MHz)
+        self.source = None
+        self._stop = threading.Event()
+        self._t0 = time.perf_counter()
+        files = [f for f in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
+                 if os.access(f, os.R_OK)]
+        self._file = files[0] if len(files) == 1 else None
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    @staticmethod
+    def _current_from_levels(text):
+        # "1: 1679Mhz *": the starred level is the current clock
+        for line in text.splitlines():
+            if "*" in line:
+                digits = "".join(ch if ch.isdigit() else " " for ch in line.split(":", 1)[-1])
+                return float(digits.split()[0])
+        return None
+
+    def _read(self):
+        if self._file is not None:
+            try:
+                mhz = self._current_from_levels(open(self._file).read())
+                if mhz is not None:
+                    self.source = "pp_dpm_sclk"
+                    time.sleep(0.02)
+                    return mhz
+            except OSError:
+                pass
+            self._file = None
+        import re
+        import subprocess
+        try:
+            text = subprocess.run(["rocm-smi", "--showclocks"], stdout=subprocess.PIPE,
+                                  stderr=subprocess.DEVNULL, text=True, timeout=5).stdout
+        except (OSError, subprocess.SubprocessError):
+            return None
+        best = None
+        for line in text.splitlines():
+            if "sclk" in line:
+                m = re.search(r"\((\d+)\s*Mhz\)", line, re.I)
+                if m:
+                    best = max(best or 0.0, float(m.group(1)))   # the card under load
+        if best is not None:
+            self.source = "rocm-smi --showclocks"
+        return best
+
+    def _run(self):
+        while not self._stop.is_set():
+            mhz = self._read()
+            if mhz is None:
+                if self._file is None and self.source is None:
+                    return      # no way to read the clock here
+                continue
+            self.samples.append((time.perf_counter() - self._t0, mhz))
+
+    def start(self):
+        self._thread.start()
+        return self
+
+    def stop(self, window_s=0.35):
+        """Stops polling; summary of the samples of the last `window_s` seconds of the leg."""
+        t_end = time.perf_counter() - self._t0
+        self._stop.set()
+        self._thread.join(timeout=6)
+        mhz = [m for t, m in self.samples if t >= t_end - window_s and t <= t_end]
+        if not mhz:
+            mhz = [m for _, m in self.samples[-2:]]
+        out = {"source": self.source, "samples_mhz": [int(m) for _, m in self.samples][-40:],
+               "window_s": window_s}
+        if mhz:
+            out["sclk_mhz_under_load"] = float(np.median(mhz))
+            out["samples_in_window"] = len(mhz)
+        return out
+
+
+def timed_launches(capi, launch, steps, warmup, clock=None):
     """Average milliseconds per launch from HIP events on the launch stream, and the wall-clock
-    milliseconds per step between two stream synchronisations."""
+    milliseconds per step between two stream synchronisations.  With `clock` (a dict) the
+    shader clock is polled beside the leg and its summary is put there."""
+    sampler = ClockSampler().start() if clock is not None else None
+    try:
+        return _timed_launches(capi, launch, steps, warmup)
+    finally:
+        if sampler is not None:
+            clock.update(sampler.stop())
+
+
+def _timed_launches(capi, launch, steps, warmup):
     settle(capi, launch)
     for _ in range(warmup):
         launch()
@@ -121,7 +218,7 @@ def timed_maybe_graph(capi, launch, steps, warmup, graph):
     return event_ms
 
 
-def bench_gemm_f16(capi, synth, steps, warmup, flags=0, zero_operands=False):
+def bench_gemm_f16(capi, synth, steps, warmup, flags=0, zero_operands=False, clock=None):
     n = 4096
     d = synth.config3(n)
     if zero_operands:
@@ -135,9 +232,35 @@ def bench_gemm_f16(capi, synth, steps, warmup, flags=0, zero_operands=False):
     def launch():
         capi.call("sph_gemm_f16f32", dC.ptr, dA.ptr, dB.ptr, n, n, n, 1, n * n, n * n, n * n, flags)
 
-    event_ms, wall_ms = timed_launches(capi, launch, steps, warmup)
+    event_ms, wall_ms = timed_launches(capi, launch, steps, warmup, clock=clock)
     for b in (dA, dB, dC):
         b.release()
+    return event_ms, wall_ms, d
+
+
+def bench_gemm_f16_operator(capi, synth, steps, warmup, zero_operands=False, clock=None):
+    """Configuration 3 as the operator layer runs it: per step a fresh y [4096, 4096] is taken
+    from the buffer pool (it reads as zeros, the fill is deferred), Compute::GemmHalf(y, A, B)
+    adds the product to it -- seeing the fresh state, it stores the product instead of filling,
+    reading and adding -- and ResourceManager::Clean() hands the step's blocks back.  Driven
+    through the C view of the C++ layer that the parity tests use."""
+    from tests import host_layer as hl
+    n = 4096
+    d = synth.config3(n)
+    if zero_operands:
+        d["A"][...] = 0
+        d["B"][...] = 0
+    dA = capi.DeviceBuffer.from_array(d["A"])
+    dB = capi.DeviceBuffer.from_array(d["B"])
+    assert dA.nbytes >= 2 * n * n and dB.nbytes >= 2 * n * n
+    sampler = ClockSampler().start() if clock is not None else None
+    try:
+        event_ms, wall_ms = hl.bench_gemm_half_fresh_y(dA.ptr, dB.ptr, n, steps, warmup, SETTLE_MS)
+    finally:
+        if sampler is not None:
+            clock.update(sampler.stop())
+    dA.release()
+    dB.release()
     return event_ms, wall_ms, d
 
 
@@ -537,6 +660,45 @@ def bench_copy(capi, steps, warmup, mib=64):
     return event_ms, 4 * n
 
 
+MFMA_CEILING_VARIANTS = [
+    "v_mfma_f32_32x32x16_f16 fed from LDS (12 fragment reads per 16 MFMAs)",
+    "v_mfma_f32_16x16x32_f16 fed from LDS (12 fragment reads per 32 MFMAs)",
+    "32x32x16 + one workgroup barrier per half step",
+    "32x32x16 + 32 KiB per K step of global_load_lds from L2",
+    "32x32x16, 8 fragment reads per 16 MFMAs (ratio of a 128 x 128 wavefront part)",
+    "16x16x32 + 32 KiB per K step of global_load_lds from L2",
+]
+
+
+def bench_mfma_ceiling(settle_ms, timed):
+    """What the matrix cores deliver on N(0, 1/64) operands and on zeros with the 256-tile
+    kernel's loop stripped to its parts (sapphire_amd/probe/mfma_ceiling.hip): every variant
+    issues the matrix instructions of a 4096^3 product from 256 workgroups of 8 wavefronts."""
+    import ctypes
+    path = os.path.join(ROOT, "sapphire_amd", "libsapphire_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError("%s is missing: build it with `python -m sapphire_amd.build probe`" % path)
+    probe = ctypes.CDLL(path)
+    probe.sph_probe_flop_per_launch.restype = ctypes.c_double
+    probe.sph_probe_mfma_run.argtypes = [ctypes.c_int, ctypes.c_double, ctypes.c_double,
+                                         ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    flop = probe.sph_probe_flop_per_launch()
+    rows = []
+    for variant in range(probe.sph_probe_variants()):
+        row = {"variant": variant, "loop": MFMA_CEILING_VARIANTS[variant]}
+        for tag, sigma in (("normal_1_64", 1.0 / 64), ("zeros", 0.0)):
+            us = ctypes.c_double(0)
+            sampler = ClockSampler().start()
+            rc = probe.sph_probe_mfma_run(variant, sigma, settle_ms, timed, ctypes.byref(us))
+            clock = sampler.stop()
+            if rc != 0:
+                raise RuntimeError("sph_probe_mfma_run(%d) failed with hipError %d" % (variant, rc))
+            row[tag] = {"us_per_launch": us.value, "tflops": flop / (us.value * 1e-6) / 1e12,
+                        "sclk_mhz_under_load": clock.get("sclk_mhz_under_load")}
+        rows.append(row)
+    return {"flop_per_launch": flop, "settle_ms": settle_ms, "timed_launches": timed, "rows": rows}
+
+
 def f32_roofline(workload, entry, kernel, ms, flops, alg_bytes):
     tf = flops / (ms * 1e-3) / 1e12
     return {"workload": workload, "entry_point": entry, "launch_ms": ms, "value": tf,
@@ -546,6 +708,27 @@ def f32_roofline(workload, entry, kernel, ms, flops, alg_bytes):
                          "frac": tf / PEAK_FP32_TFLOPS, "flop_per_step": flops,
                          "algorithmic_bytes_per_step": alg_bytes,
                          "hbm_gbs_on_algorithmic_bytes": alg_bytes / (ms * 1e-3) / 1e9}}
+
+
+def spmm_gather_path(nnz, n, launch_ms, info):
+    """The bound the CSR x dense kernel actually runs against.  Every stored entry gathers one
+    row of B (n floats), far more bytes than the algorithmic ones, and they come from L2, not
+    HBM: bytes gathered per second, and the L2 requests they take against the rate at which the
+    L2 can look requests up (128 channels, one 128-byte line request per channel and clock)."""
+    gathered = nnz * n * 4
+    line_requests = gathered // 128            # minimum: every 128-byte line asked for once
+    channels = 128
+    clock_hz = info.clockMHz * 1e6
+    ceiling_requests_per_s = channels * clock_hz
+    floor_ms = line_requests / ceiling_requests_per_s * 1e3
+    return {"gathered_bytes_per_launch": gathered,
+            "gathered_tb_per_s": gathered / (launch_ms * 1e-3) / 1e12,
+            "min_l2_line_requests_per_launch": line_requests,
+            "l2_request_ceiling_per_s": ceiling_requests_per_s,
+            "l2_request_ceiling_note": "%d L2 channels x one tag look-up per clock x %d MHz"
+                                       % (channels, info.clockMHz),
+            "launch_ms_at_l2_request_ceiling": floor_ms,
+            "frac_of_l2_request_ceiling": floor_ms / launch_ms}
 
 
 def cpu_gemm_baseline(d, rows=32):
@@ -616,12 +799,25 @@ def main():
     result = {}
     n = 4096
     flops = 2.0 * n ** 3
-    if args.only in (None, "gemm"):
-        zeros = args.zero_operands and args.only == "gemm"
-        event_ms, wall_ms, d3 = bench_gemm_f16(capi, synth, args.steps, args.warmup,
-                                               zero_operands=zeros)
+    if args.only in (None, "gemm", "gemm_operator"):
+        zeros = args.zero_operands and args.only is not None
+        operator_leg = args.only in (None, "gemm_operator")
+        clock = {}
+        leg = bench_gemm_f16_operator if operator_leg else bench_gemm_f16
+        event_ms, wall_ms, d3 = leg(capi, synth, args.steps, args.warmup, zero_operands=zeros,
+                                    clock=clock)
         tflops = flops / (wall_ms * 1e-3) / 1e12
         kernel_tflops = flops / (event_ms * 1e-3) / 1e12
+        if operator_leg:
+            entry = ("Compute::GemmHalf(y, A, B) on a fresh TensorData y (accumulate contract "
+                     "y += A*B; the operator sees that y's zero fill is still deferred and runs "
+                     "sph_gemm_f16f32 with SPH_GEMM_OVERWRITE), ResourceManager::Clean() per step")
+            alg_bytes = 2 * 64 * (1 << 20)    # A, B read, y written; the zeros are never read
+            profile = "gemm_f16_tile256_config3_fresh_y.txt"
+        else:
+            entry = "sph_gemm_f16f32 (accumulate into a given out)"
+            alg_bytes = 3 * 64 * (1 << 20)
+            profile = "gemm_f16_tile256_config3.txt"
         result.update({
             "metric": "GEMM TFLOP/s + % MFMA peak (4096^3 fp16->fp32); SpMM GB/s + % HBM peak",
             "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
@@ -629,29 +825,52 @@ def main():
             "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "f16 in / f32 accumulate",
             "data": "zeros" if zeros else "synthetic",
-            "config": {"workload": "configuration 3: out[4096,4096] f32 += A[4096,4096] f16 * "
+            "config": {"workload": "configuration 3: y[4096,4096] f32 (zeros) += A[4096,4096] f16 * "
                                    "B[4096,4096] f16, N(0,1/sqrt(K)) inputs, row-major, one launch "
                                    "per step, inputs resident in HBM",
-                       "entry_point": "sph_gemm_f16f32 (accumulate)"},
+                       "entry_point": entry},
             "roofline": {"bound": "mfma", "kernel": "GemmF16Tile256",
                          "achieved": kernel_tflops, "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                          "frac": kernel_tflops / PEAK_FP16_TFLOPS,
-                         "traffic": recorded_traffic("gemm_f16_tile256_config3.txt"),
-                         "traffic_unit": "bytes per launch (profiles/gemm_f16_tile256_config3.txt)",
-                         "algorithmic_bytes_per_launch": 3 * 64 * (1 << 20),
+                         "traffic": recorded_traffic(profile),
+                         "traffic_unit": "bytes per launch (profiles/%s)" % profile,
+                         "algorithmic_bytes_per_launch": alg_bytes,
                          "launch_ms": event_ms, "flop_per_launch": flops,
                          "peak_from_device": device_peak,
                          "peak_from_device_note": "%d CUs x 4096 flop/clk x %d MHz"
-                                                  % (info.computeUnits, info.clockMHz)},
+                                                  % (info.computeUnits, info.clockMHz),
+                         "clock": clock},
             "device": {"name": info.name.decode(), "arch": info.arch.decode(),
                        "compute_units": info.computeUnits, "clock_mhz": info.clockMHz},
         })
         if args.only is None:
-            ev_over, _, _ = bench_gemm_f16(capi, synth, args.steps, args.warmup,
-                                           flags=capi.SPH_GEMM_OVERWRITE)
-            result["gemm_overwrite_variant"] = {
-                "note": "same launch with SPH_GEMM_OVERWRITE (out is not read)",
-                "launch_ms": ev_over, "tflops": flops / (ev_over * 1e-3) / 1e12}
+            ev_acc, _, _ = bench_gemm_f16(capi, synth, args.steps, args.warmup)
+            result["gemm_accumulate_into_used_out_variant"] = {
+                "note": "sph_gemm_f16f32 through the C ABI adding into an out that holds earlier "
+                        "results (out is read inside the K loop and written): what a caller "
+                        "pays when y is not fresh",
+                "launch_ms": ev_acc, "tflops": flops / (ev_acc * 1e-3) / 1e12,
+                "frac": flops / (ev_acc * 1e-3) / 1e12 / PEAK_FP16_TFLOPS}
+            zclock = {}
+            ev_zero, _, _ = bench_gemm_f16_operator(capi, synth, args.steps, args.warmup,
+                                                    zero_operands=True, clock=zclock)
+            tf_zero = flops / (ev_zero * 1e-3) / 1e12
+            result["gemm_zero_operands_variant"] = {
+                "note": "the headline leg again (same call, same kernel, same instruction "
+                        "stream) on all-zero A and B: the chip holds a power limit, and on "
+                        "operands that do not toggle the matrix cores it keeps its full clock; "
+                        "compare clock.sclk_mhz_under_load here with roofline.clock",
+                "data": "zeros", "launch_ms": ev_zero, "tflops": tf_zero,
+                "frac": tf_zero / PEAK_FP16_TFLOPS, "clock": zclock}
+            mhz, zmhz = clock.get("sclk_mhz_under_load"), zclock.get("sclk_mhz_under_load")
+            if mhz and zmhz:
+                result["roofline"]["frac_of_peak_at_measured_clock"] = kernel_tflops / (
+                    info.computeUnits * 4096 * mhz * 1e6 / 1e12)
+                result["gemm_zero_operands_variant"]["frac_of_peak_at_measured_clock"] = tf_zero / (
+                    info.computeUnits * 4096 * zmhz * 1e6 / 1e12)
+
+    if args.only == "mfma_ceiling":
+        result["mfma_ceiling"] = bench_mfma_ceiling(args.settle_ms, max(args.steps, 100))
 
     if args.only == "copy":
         ms, nbytes = bench_copy(capi, args.steps, args.warmup)
@@ -704,7 +923,8 @@ def main():
                          "traffic": recorded_traffic("spmm_slab_config5.txt"),
                          "traffic_unit": "bytes per launch (profiles/spmm_slab_config5.txt)",
                          "algorithmic_bytes_per_launch": alg_bytes,
-                         "gather_bytes_per_launch": nnz * 256 * 4},
+                         "gather_bytes_per_launch": nnz * 256 * 4,
+                         "gather_path": spmm_gather_path(nnz, 256, sp_event, info)},
         }
         if not args.no_cpu and args.only is None:
             dt = cpu_spmm_baseline(d5)

@@ -7,6 +7,8 @@ Outputs (git-ignored, next to the package so that they travel with the tree):
     sapphire_amd/libsapphire_hip.so    C ABI of include/sapphire_hip.h
     sapphire_amd/libsapphire_host.so   C++ operator layer (Sapphire:: namespace)
     tests/host_harness/libhost_harness.so   C view of that layer for the Python tests
+    sapphire_amd/libsapphire_probe.so  measurement aid for bench.py --only mfma_ceiling (not
+                                       part of the C ABI, not loaded by anything else)
 """
 import concurrent.futures
 import os
@@ -80,6 +82,17 @@ def build_hip():
     return HIP_LIB
 
 
+PROBE_DIR = os.path.join(PKG, "probe")
+PROBE_LIB = os.path.join(PKG, "libsapphire_probe.so")
+
+
+def build_probe():
+    """The matrix-core ceiling probe behind `bench.py --only mfma_ceiling`."""
+    objs = _compile_all(_sources(PROBE_DIR, {".hip"}), HIP_FLAGS, "probe")
+    _run([_hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", PROBE_LIB] + objs)
+    return PROBE_LIB
+
+
 def build_host():
     """C++17 operator layer, linked against the C ABI library beside it."""
     flags = ["-O2", "-std=c++17", "-fPIC", "-x", "c++",
@@ -112,6 +125,7 @@ def build_oracle():
 
 def build_all():
     build_hip()
+    build_probe()
     build_host()
     build_harness()
     build_oracle()
@@ -120,6 +134,6 @@ def build_all():
 if __name__ == "__main__":
     parts = sys.argv[1:] or ["all"]
     for part in parts:
-        {"hip": build_hip, "host": build_host, "harness": build_harness,
+        {"hip": build_hip, "probe": build_probe, "host": build_host, "harness": build_harness,
          "oracle": build_oracle, "all": build_all}[part]()
         print("built", part)

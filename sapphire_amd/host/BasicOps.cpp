@@ -33,7 +33,6 @@ void Gemm(TensorData& y, const TensorData& a, const TensorData& b)
 
     const GemmPlan plan = PlanGemm(y.GetShape(), a.GetShape(), b.GetShape());
     const int deviceId = y.GetCudaDevice().GetID();
-    float* out = y.CudaMutableRawPtr();
     const float* A = a.CudaRawPtr();
     const float* B = b.CudaRawPtr();
 
@@ -41,7 +40,22 @@ void Gemm(TensorData& y, const TensorData& a, const TensorData& b)
     // common cases: no batch, equal batches, one operand shared by the batch) ...
     std::uint32_t count = 0;
     std::int64_t strideOut = 0, strideA = 0, strideB = 0;
-    if (AsStridedBatch(plan, count, strideOut, strideA, strideB))
+    const bool strided = AsStridedBatch(plan, count, strideOut, strideA, strideB);
+    // A fresh y whose zero fill is still deferred, written exactly once everywhere by this
+    // walk: y += a*b on zeros is y = a*b, so the product is stored and neither the fill nor
+    // the read of the zeros happens (same result bits: 0 + s == s for every sum the kernels
+    // produce, none of which is -0).
+    if (strided && strideOut == static_cast<std::int64_t>(plan.M) * plan.N &&
+        static_cast<std::uint64_t>(count) * plan.M * plan.N ==
+            static_cast<std::uint64_t>(y.Size()) &&
+        y.TakeDeferredZero())
+    {
+        Dense::Cuda::GemmStrided(y.CudaOverwriteRawPtr(), A, B, plan.M, plan.N, plan.K, count,
+                                 strideOut, strideA, strideB, true, deviceId);
+        return;
+    }
+    float* out = y.CudaMutableRawPtr();
+    if (strided)
     {
         if (strideOut == static_cast<std::int64_t>(plan.M) * plan.N &&
             strideA == static_cast<std::int64_t>(plan.M) * plan.K &&
@@ -74,6 +88,22 @@ void Gemm(TensorData& y, const TensorData& a, const TensorData& b)
     Dense::Cuda::GemmGrouped(units, out, A, B, plan.M, plan.N, plan.K, deviceId);
 }
 
+void GemmHalf(TensorData& y, const std::uint16_t* a, const std::uint16_t* b, unsigned int K)
+{
+    RequireDeviceMode(y, "GemmHalf");
+    if (a == nullptr || b == nullptr)
+        throw std::invalid_argument("Compute::GemmHalf - null operand");
+    const auto M = static_cast<unsigned int>(y.Rows());
+    const auto N = static_cast<unsigned int>(y.Cols());
+    const auto batch = static_cast<unsigned int>(y.GetNumUnits(2));
+    const int deviceId = y.GetCudaDevice().GetID();
+    const std::size_t mn = static_cast<std::size_t>(M) * N;
+    const bool freshZero = y.TakeDeferredZero();
+    float* out = freshZero ? y.CudaOverwriteRawPtr() : y.CudaMutableRawPtr();
+    Dense::Cuda::GemmHalf(out, a, b, M, N, K, batch, mn, static_cast<std::size_t>(M) * K,
+                          static_cast<std::size_t>(K) * N, freshZero, deviceId);
+}
+
 void Transpose(TensorData& y, const TensorData& x)
 {
     RequireSameMode(y, x, "Transpose");
@@ -82,7 +112,10 @@ void Transpose(TensorData& y, const TensorData& x)
     const int cols = x.Cols();
     const bool broadcast = x.GetNumUnits(2) == 1;
     const int matrices = y.GetShape().Size() / (rows * cols);
-    Dense::Cuda::Transpose(y.CudaMutableRawPtr(), x.CudaRawPtr(), static_cast<unsigned int>(rows),
+    // writes every element of y (matrices * rows * cols of them)
+    float* out = static_cast<long long>(matrices) * rows * cols == y.Size() ? y.CudaOverwriteRawPtr()
+                                                                           : y.CudaMutableRawPtr();
+    Dense::Cuda::Transpose(out, x.CudaRawPtr(), static_cast<unsigned int>(rows),
                            static_cast<unsigned int>(cols), static_cast<unsigned int>(matrices),
                            broadcast);
 }
@@ -91,7 +124,7 @@ void ReLU(TensorData& y, const TensorData& x)
 {
     RequireSameMode(y, x, "ReLU");
     RequireDeviceMode(y, "ReLU");
-    Dense::Cuda::ReLU(y.CudaMutableRawPtr(), x.CudaRawPtr(), static_cast<unsigned int>(y.Size()));
+    Dense::Cuda::ReLU(y.CudaOverwriteRawPtr(), x.CudaRawPtr(), static_cast<unsigned int>(y.Size()));
 }
 
 void ReLUBackward(TensorData& dx, const TensorData& dy, const TensorData& x)
@@ -107,7 +140,9 @@ void Scale(TensorData& y, const TensorData& x, const float factor)
 {
     RequireSameMode(y, x, "Scale");
     RequireDeviceMode(y, "Scale");
-    Dense::Cuda::Scale(y.CudaMutableRawPtr(), x.CudaRawPtr(), factor,
+    // y may be x (in place): settle x first, then y has no deferred fill left to drop
+    const float* in = x.CudaRawPtr();
+    Dense::Cuda::Scale(y.CudaOverwriteRawPtr(), in, factor,
                        static_cast<unsigned int>(y.GetShape().Size()));
 }
 

@@ -49,6 +49,16 @@ void GemmMatrixWiseBroadcast(float* out, const float* A, const float* B, unsigne
           "GemmMatrixWiseBroadcast");
 }
 
+void GemmStrided(float* out, const float* A, const float* B, unsigned int M, unsigned int N,
+                 unsigned int K, unsigned int batchSize, std::int64_t strideOut,
+                 std::int64_t strideA, std::int64_t strideB, bool overwrite, int deviceId)
+{
+    Compute::Cuda::CudaSetDevice(deviceId);
+    Check(sph_gemm_f32_ex(out, A, B, M, N, K, batchSize, strideOut, strideA, strideB,
+                          overwrite ? SPH_GEMM_OVERWRITE : SPH_GEMM_ACCUMULATE),
+          "GemmStrided");
+}
+
 void GemmGrouped(const std::vector<GemmUnit>& units, float* out, const float* A, const float* B,
                  unsigned int M, unsigned int N, unsigned int K, int deviceId)
 {
@@ -152,7 +162,7 @@ namespace Sapphire::Compute::Initialize
 void Scalar(TensorUtil::TensorData& data, float value)
 {
     if (data.Mode() == ComputeMode::Cuda)
-        Dense::Cuda::Scalar(data.CudaMutableRawPtr(), value, data.DenseTotalLengthCuda);
+        Dense::Cuda::Scalar(data.CudaOverwriteRawPtr(), value, data.DenseTotalLengthCuda);
     else
         std::fill_n(data.HostMutableRawPtr(), data.HostTotalSize, value);
 }

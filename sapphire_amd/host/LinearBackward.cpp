@@ -77,9 +77,13 @@ void RunDirect(TensorData& dx, TensorData& weight, TensorData& bias, const Tenso
     const unsigned int rows = static_cast<unsigned int>(dy.Size()) / outputs;
 
     // dx [rows, in] += dy [rows, out] * (weight [in, out])^T
-    Compute::Dense::Cuda::GemmTransposed(dx.CudaMutableRawPtr(), dy.CudaRawPtr(),
-                                         weight.CudaRawPtr(), rows, inputs, outputs, 1, false,
-                                         true, false, deviceId);
+    // (a fresh dx is stored into instead of filled, read and added to)
+    const bool dxFresh = static_cast<std::size_t>(dx.Size()) ==
+                             static_cast<std::size_t>(rows) * inputs &&
+                         dx.TakeDeferredZero();
+    Compute::Dense::Cuda::GemmTransposed(dxFresh ? dx.CudaOverwriteRawPtr() : dx.CudaMutableRawPtr(),
+                                         dy.CudaRawPtr(), weight.CudaRawPtr(), rows, inputs,
+                                         outputs, 1, false, true, dxFresh, deviceId);
 
     // dB [1, out] = ones [1, batch] * dy, the ones that Linear's backward pass fills
     TensorData transposedOnes(Shape({ 1, static_cast<int>(batchSize) }), dy.GetType(),
@@ -104,13 +108,13 @@ void RunDirect(TensorData& dx, TensorData& weight, TensorData& bias, const Tenso
     // dw [in, out] = (x [rows, in])^T * dy [rows, out]
     TensorData dw(weight.GetShape(), weight.GetType(), weight.GetCudaDevice());
     dw.SetMode(weight.Mode());
-    Compute::Dense::Cuda::GemmTransposed(dw.CudaMutableRawPtr(), x.CudaRawPtr(), dy.CudaRawPtr(),
+    Compute::Dense::Cuda::GemmTransposed(dw.CudaOverwriteRawPtr(), x.CudaRawPtr(), dy.CudaRawPtr(),
                                          inputs, outputs, rows, 1, true, false, true, deviceId);
     optimizer(weight, dw);
 
     TensorData dB(bias.GetShape(), bias.GetType(), bias.GetCudaDevice());
     dB.SetMode(bias.Mode());
-    Compute::Dense::Cuda::GemmTransposed(dB.CudaMutableRawPtr(), transposedOnes.CudaRawPtr(),
+    Compute::Dense::Cuda::GemmTransposed(dB.CudaOverwriteRawPtr(), transposedOnes.CudaRawPtr(),
                                          dy.CudaRawPtr(), 1, outputs, batchSize, 1, false, false,
                                          true, deviceId);
     Compute::Scale(dB, dB, 1.0f / static_cast<float>(batchSize));

@@ -55,8 +55,9 @@ void LinearForwardFused(TensorUtil::TensorData& y, const TensorUtil::TensorData&
     if (x.Size() != batchSize * inputs || y.Size() != batchSize * outputs ||
         bias.Size() != outputs)
         throw std::invalid_argument("NN::Linear - shape mismatch");
+    // y is written everywhere and not read
     Compute::Dense::Cuda::LinearForward(
-        y.CudaMutableRawPtr(), x.CudaRawPtr(), weight.CudaRawPtr(), bias.CudaRawPtr(),
+        y.CudaOverwriteRawPtr(), x.CudaRawPtr(), weight.CudaRawPtr(), bias.CudaRawPtr(),
         static_cast<unsigned int>(batchSize), static_cast<unsigned int>(inputs),
         static_cast<unsigned int>(outputs), relu, y.GetCudaDevice().GetID());
 }
@@ -90,7 +91,7 @@ void SparseLinearForward(TensorUtil::TensorData& y, const TensorUtil::TensorData
     // yT = bias x ones + W^T_csr * xT in one launch: the bias of an output row is the value the
     // product is added to, which is what Zeros(yT); Gemm(yT, bias, ones); accumulate leaves
     Compute::Transpose(xT, x2);
-    Compute::Sparse::Cuda::GemmBias(yT.CudaMutableRawPtr(), &weightTransposed, xT.CudaRawPtr(),
+    Compute::Sparse::Cuda::GemmBias(yT.CudaOverwriteRawPtr(), &weightTransposed, xT.CudaRawPtr(),
                                     static_cast<unsigned int>(batchSize), bias.CudaRawPtr(),
                                     device.GetID());
     Compute::Transpose(y2, yT);

@@ -109,6 +109,18 @@ void ResourceManager::MoveToVolatileCuda(void* ptr)
     gCuda.ToVolatile(ptr, "MoveToVolatileCuda");
 }
 
+void ResourceManager::MarkZeroPendingCuda(void* ptr)
+{
+    std::lock_guard<std::mutex> lock(gMutex);
+    gCuda.MarkZeroPending(ptr);
+}
+
+bool ResourceManager::TakeZeroPendingCuda(void* ptr)
+{
+    std::lock_guard<std::mutex> lock(gMutex);
+    return gCuda.TakeZeroPending(ptr);
+}
+
 void ResourceManager::Clean()
 {
     std::lock_guard<std::mutex> lock(gMutex);

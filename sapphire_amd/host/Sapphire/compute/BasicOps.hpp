@@ -9,6 +9,8 @@
 
 #include <Sapphire/tensor/TensorData.hpp>
 
+#include <cstdint>
+
 namespace Sapphire::Compute
 {
 using TensorUtil::TensorData;
@@ -17,6 +19,14 @@ using TensorUtil::TensorData;
 //! BroadcastWith2Inputs.  No shape validation, as documented for the reference
 //! (Includes/Sapphire/compute/BasicOps.hpp:16-19).  All three must be in the same mode.
 void Gemm(TensorData& y, const TensorData& a, const TensorData& b);
+
+//! y += a * b with half-precision operands and fp32 accumulation, the operand form of the
+//! tensor-core product the reference declares (WmmaGemm,
+//! Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50).  TensorData holds fp32
+//! only, so a and b are device arrays of IEEE binary16 bit patterns: a is [batch, M, K], b is
+//! [batch, K, N] with M, N the trailing dimensions of y and batch its leading ones, packed back
+//! to back.  A fresh y (zero fill still deferred) receives the product without being read.
+void GemmHalf(TensorData& y, const std::uint16_t* a, const std::uint16_t* b, unsigned int K);
 
 //! y = transpose of the trailing two dimensions of x; a 2-D x is repeated for every matrix
 //! of y (Sources/Sapphire/compute/BasicOps.cpp:269-290).

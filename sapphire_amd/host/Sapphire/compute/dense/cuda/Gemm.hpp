@@ -20,6 +20,13 @@ void GemmMatrixWiseBroadcast(float* out, const float* A, const float* B, unsigne
                              unsigned int N, unsigned int K, unsigned int batchSize,
                              bool broadcastA, bool broadcastB, int deviceId);
 
+//! out[c] (+)= A[c] * B[c] for c < batchSize with the three element strides given (0 repeats an
+//! operand): the general form behind the two calls above.  `overwrite` stores the product
+//! without reading out.
+void GemmStrided(float* out, const float* A, const float* B, unsigned int M, unsigned int N,
+                 unsigned int K, unsigned int batchSize, std::int64_t strideOut,
+                 std::int64_t strideA, std::int64_t strideB, bool overwrite, int deviceId);
+
 //! Element offsets of one M x N unit product.
 struct GemmUnit
 {

@@ -78,9 +78,21 @@ public:
     static void DeepCopy(TensorData& dst, const TensorData& src);
 
     [[nodiscard]] const float* HostRawPtr() const { return m_denseHost; }
-    [[nodiscard]] const float* CudaRawPtr() const { return m_denseCuda; }
     [[nodiscard]] float* HostMutableRawPtr() const { return m_denseHost; }
-    [[nodiscard]] float* CudaMutableRawPtr() const { return m_denseCuda; }
+    //! The device buffer.  A fresh device buffer reads as zeros
+    //! (Sources/Sapphire/tensor/TensorData.cpp:330,354 of the reference fill it at allocation);
+    //! here the fill is deferred until the buffer is first asked for through these two, which
+    //! enqueue it on the calling thread's stream before they return the pointer.
+    [[nodiscard]] const float* CudaRawPtr() const;
+    [[nodiscard]] float* CudaMutableRawPtr() const;
+    //! For an operator that is about to write every element of the device buffer without
+    //! reading any: the pointer, with a deferred fill dropped instead of run.
+    [[nodiscard]] float* CudaOverwriteRawPtr() const;
+    //! True when the device buffer is fresh and its zero fill still deferred; the state is
+    //! cleared and nothing is filled.  For an accumulating operator that covers the whole
+    //! buffer: y += f(..) on known zeros is y = f(..), so it may store instead of add and
+    //! must then take the pointer from CudaOverwriteRawPtr().
+    [[nodiscard]] bool TakeDeferredZero() const;
 
     //! CSR record with host arrays / with device arrays, for Type::Sparse operands of the
     //! sparse x dense product (owned by the caller).

@@ -49,7 +49,7 @@ public:
         if (preserve)
         {
             void* ptr = m_hooks.allocate(size);
-            m_preserved.emplace(ptr, Block{ size, stream });
+            m_preserved.emplace(ptr, Block{ size, stream, false });
             return ptr;
         }
         void* ptr = nullptr;
@@ -62,7 +62,7 @@ public:
         }
         else
             ptr = m_hooks.allocate(size);
-        m_volatile.emplace(ptr, Block{ size, stream });
+        m_volatile.emplace(ptr, Block{ size, stream, false });
         return ptr;
     }
 
@@ -103,6 +103,25 @@ public:
         m_free.clear();
     }
 
+    //! Deferred zero fill.  A block handed out by Get() may be marked "holds zeros that have not
+    //! been written yet"; whoever uses the block first takes the mark and either fills the
+    //! block or, when it is about to write every byte anyway, does nothing.  The mark dies
+    //! with the block's live entry (Clean, release), so a reused block starts unmarked.
+    void MarkZeroPending(void* ptr)
+    {
+        if (Block* b = FindLive(ptr))
+            b->zeroPending = true;
+    }
+    //! True when the mark was set; clears it.
+    bool TakeZeroPending(void* ptr)
+    {
+        Block* b = FindLive(ptr);
+        if (b == nullptr || !b->zeroPending)
+            return false;
+        b->zeroPending = false;
+        return true;
+    }
+
     std::size_t CountVolatile() const { return m_volatile.size(); }
     std::size_t CountPreserved() const { return m_preserved.size(); }
     std::size_t CountFree() const { return m_free.size(); }
@@ -112,8 +131,18 @@ private:
     {
         std::size_t size;
         void* stream;
+        bool zeroPending = false;
     };
     using Live = std::unordered_map<void*, Block>;
+
+    Block* FindLive(void* ptr)
+    {
+        auto it = m_volatile.find(ptr);
+        if (it != m_volatile.end())
+            return &it->second;
+        it = m_preserved.find(ptr);
+        return it != m_preserved.end() ? &it->second : nullptr;
+    }
 
     static Live::iterator Find(Live& pool, void* ptr, const char* who, const char* what)
     {

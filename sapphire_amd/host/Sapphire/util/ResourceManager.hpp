@@ -35,6 +35,15 @@ public:
     static void MoveToVolatileHost(void* ptr);
     static void MoveToVolatileCuda(void* ptr);
 
+    //! Deferred zero fill of a device block obtained from GetMemoryCuda: Mark says "this block
+    //! is to be read as zeros, the fill has not been enqueued"; Take returns whether the mark
+    //! was set and clears it (the caller then fills the block, or overwrites all of it).  The
+    //! reference fills every fresh device buffer at once
+    //! (Sources/Sapphire/tensor/TensorData.cpp:354); deferring it lets an operator whose first
+    //! act is to write the whole buffer skip both the fill and the read of the zeros.
+    static void MarkZeroPendingCuda(void* ptr);
+    static bool TakeZeroPendingCuda(void* ptr);
+
     //! Volatile blocks become reusable; nothing is released.
     static void Clean();
     static void ClearPreservedPool();

@@ -93,6 +93,33 @@ TensorData& TensorData::operator=(TensorData&& other) noexcept
     return *this;
 }
 
+const float* TensorData::CudaRawPtr() const
+{
+    return CudaMutableRawPtr();
+}
+
+float* TensorData::CudaMutableRawPtr() const
+{
+    if (m_denseCuda != nullptr && Util::ResourceManager::TakeZeroPendingCuda(m_denseCuda))
+    {
+        Compute::Cuda::CudaSetDevice(m_device.GetID());
+        Compute::Dense::Cuda::Scalar(m_denseCuda, 0.0f, DenseTotalLengthCuda);
+    }
+    return m_denseCuda;
+}
+
+float* TensorData::CudaOverwriteRawPtr() const
+{
+    if (m_denseCuda != nullptr)
+        (void)Util::ResourceManager::TakeZeroPendingCuda(m_denseCuda);
+    return m_denseCuda;
+}
+
+bool TensorData::TakeDeferredZero() const
+{
+    return m_denseCuda != nullptr && Util::ResourceManager::TakeZeroPendingCuda(m_denseCuda);
+}
+
 void TensorData::Reshape(const Shape& shape)
 {
     if (shape.Size() != m_shape.Size())
@@ -118,7 +145,8 @@ void TensorData::SetData(std::vector<float> data)
                                     std::to_string(data.size()) + ") expected size : (" +
                                     std::to_string(expected) + ")");
     if (m_mode == ComputeMode::Cuda)
-        Compute::Cuda::CopyHostToDevice(m_denseCuda, data.data(), sizeof(float) * data.size());
+        Compute::Cuda::CopyHostToDevice(CudaOverwriteRawPtr(), data.data(),
+                                        sizeof(float) * data.size());
     else
         std::copy(data.begin(), data.end(), m_denseHost);
 }
@@ -192,7 +220,7 @@ void TensorData::DeepCopy(TensorData& dst, const TensorData& src)
     const std::size_t unit = static_cast<std::size_t>(src.Size());
     const std::size_t repeats = static_cast<std::size_t>(dst.Size()) / unit;
     if (dst.Mode() == ComputeMode::Cuda)
-        Compute::Cuda::CopyDeviceToDeviceBroadcast(dst.m_denseCuda, src.m_denseCuda,
+        Compute::Cuda::CopyDeviceToDeviceBroadcast(dst.CudaOverwriteRawPtr(), src.CudaRawPtr(),
                                                    repeats * unit * sizeof(float),
                                                    unit * sizeof(float));
     else
@@ -205,7 +233,9 @@ void TensorData::UploadDense()
     RequireDense(m_type, "TensorData::m_toCuda");
     if (m_denseCuda == nullptr)
         AllocateCuda();
-    Compute::Cuda::CopyHostToDevice(m_denseCuda, m_denseHost, HostTotalSize * sizeof(float));
+    // the whole device buffer when the two sides have the same length (they always do here)
+    float* dst = HostTotalSize == DenseTotalLengthCuda ? CudaOverwriteRawPtr() : CudaMutableRawPtr();
+    Compute::Cuda::CopyHostToDevice(dst, m_denseHost, HostTotalSize * sizeof(float));
 }
 
 void TensorData::DownloadDense()
@@ -213,7 +243,7 @@ void TensorData::DownloadDense()
     RequireDense(m_type, "TensorData::m_toHost");
     if (m_denseHost == nullptr)
         AllocateHost();
-    Compute::Cuda::CopyDeviceToHost(m_denseHost, m_denseCuda, HostTotalSize * sizeof(float));
+    Compute::Cuda::CopyDeviceToHost(m_denseHost, CudaRawPtr(), HostTotalSize * sizeof(float));
 }
 
 void TensorData::AllocateHost()
@@ -232,7 +262,9 @@ void TensorData::AllocateCuda()
     Compute::Cuda::CudaSetDevice(m_device.GetID());
     m_denseCuda = static_cast<float*>(
         Util::ResourceManager::GetMemoryCuda(DenseTotalLengthCuda * sizeof(float), m_preserve));
-    // every fresh device buffer starts at zero (TensorData.cpp:354 of the reference)
-    Compute::Dense::Cuda::Scalar(m_denseCuda, 0.0f, DenseTotalLengthCuda);
+    // Every fresh device buffer reads as zeros (TensorData.cpp:354 of the reference fills it
+    // here).  The fill is deferred to the first use of the buffer: CudaRawPtr() /
+    // CudaMutableRawPtr() enqueue it, an operator that writes the whole buffer drops it.
+    Util::ResourceManager::MarkZeroPendingCuda(m_denseCuda);
 }
 }  // namespace Sapphire::TensorUtil

@@ -16,7 +16,11 @@
 #include <Sapphire/util/BlockPool.hpp>
 #include <Sapphire/util/ResourceManager.hpp>
 
+#include <sapphire_hip.h>
+
 #include <algorithm>
+#include <chrono>
+#include <cstdint>
 #include <cstring>
 #include <exception>
 #include <stdexcept>
@@ -248,6 +252,91 @@ int sphh_compute_gemm(float* yData, const int* y, int yn, const float* aData, co
         Compute::Gemm(Out, A, B);
         Download(Out, yData);
         Util::ResourceManager::Clean();
+    });
+}
+
+// Compute::Gemm into a FRESH y (never filled, never read): the operator sees the deferred zero
+// state of the new buffer and stores the product.  yOut receives the result.
+int sphh_compute_gemm_fresh_y(float* yOut, const int* y, int yn, const float* aData, const int* a,
+                              int an, const float* bData, const int* b, int bn)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData A = Upload(MakeShape(a, an), aData, cuda);
+        TensorData B = Upload(MakeShape(b, bn), bData, cuda);
+        TensorData Out(MakeShape(y, yn), Type::Dense, cuda);
+        Compute::Gemm(Out, A, B);
+        Download(Out, yOut);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// Compute::GemmHalf on device arrays of binary16 bit patterns.  freshY != 0: y is a new
+// TensorData (deferred zero fill, the product is stored); otherwise y holds yData and the
+// product is added to it.  yData receives the result.
+int sphh_gemm_half(float* yData, const int* y, int yn, const std::uint16_t* aDev,
+                   const std::uint16_t* bDev, unsigned int K, int freshY)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        TensorData Out = freshY ? TensorData(MakeShape(y, yn), Type::Dense, cuda)
+                                : Upload(MakeShape(y, yn), yData, cuda);
+        Compute::GemmHalf(Out, aDev, bDev, K);
+        Download(Out, yData);
+        Util::ResourceManager::Clean();
+    });
+}
+
+// Times `steps` passes of: take a fresh y [n, n] from the pool, y += a * b through
+// Compute::GemmHalf, hand the pass's blocks back (ResourceManager::Clean(), what a model does at
+// the end of a pass).  settleMs of the same passes run untimed first.  eventMs: per pass from
+// events on the thread's stream; wallMs: per pass between two stream synchronisations.
+int sphh_bench_gemm_half_fresh_y(const std::uint16_t* aDev, const std::uint16_t* bDev, int n,
+                                 int steps, int warmup, double settleMs, float* eventMs,
+                                 double* wallMs)
+{
+    return Guard([&] {
+        const CudaDevice cuda(0, "device0");
+        Compute::Cuda::CudaSetDevice(0);
+        auto pass = [&] {
+            TensorData y(Shape({ n, n }), Type::Dense, cuda);
+            Compute::GemmHalf(y, aDev, bDev, static_cast<unsigned int>(n));
+            Util::ResourceManager::Clean();
+        };
+        auto require = [](int rc, const char* what) {
+            if (rc != SPH_OK)
+                throw std::runtime_error(std::string(what) + " failed with " + sph_last_error());
+        };
+        const auto t0 = std::chrono::steady_clock::now();
+        auto elapsedMs = [&](std::chrono::steady_clock::time_point from) {
+            return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - from)
+                .count();
+        };
+        while (elapsedMs(t0) < settleMs)
+        {
+            for (int i = 0; i < 20; ++i)
+                pass();
+            require(sph_stream_sync(), "sph_stream_sync");
+        }
+        for (int i = 0; i < warmup; ++i)
+            pass();
+        require(sph_stream_sync(), "sph_stream_sync");
+        void *begin = nullptr, *end = nullptr;
+        require(sph_event_create(&begin), "sph_event_create");
+        require(sph_event_create(&end), "sph_event_create");
+        const auto w0 = std::chrono::steady_clock::now();
+        require(sph_event_record(begin), "sph_event_record");
+        for (int i = 0; i < steps; ++i)
+            pass();
+        require(sph_event_record(end), "sph_event_record");
+        require(sph_stream_sync(), "sph_stream_sync");
+        *wallMs = elapsedMs(w0) / steps;
+        float ms = 0;
+        require(sph_event_elapsed_ms(begin, end, &ms), "sph_event_elapsed_ms");
+        *eventMs = ms / static_cast<float>(steps);
+        sph_event_destroy(begin);
+        sph_event_destroy(end);
+        Util::ResourceManager::ClearAll();
     });
 }
 

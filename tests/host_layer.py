@@ -25,6 +25,12 @@ def lib():
                                      ctypes.POINTER(ctypes.c_longlong)]
         h.sphh_compute_gemm.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int, _fp, _ip,
                                         ctypes.c_int]
+        h.sphh_compute_gemm_fresh_y.argtypes = h.sphh_compute_gemm.argtypes
+        h.sphh_gemm_half.argtypes = [_fp, _ip, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                     ctypes.c_uint, ctypes.c_int]
+        h.sphh_bench_gemm_half_fresh_y.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                                   ctypes.c_int, ctypes.c_int, ctypes.c_double,
+                                                   _fp, ctypes.POINTER(ctypes.c_double)]
         h.sphh_transpose.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int]
         h.sphh_mlp_forward.argtypes = [_fp, ctypes.c_int, _ip, ctypes.c_int,
                                        ctypes.POINTER(_fp), ctypes.POINTER(_fp), _fp, ctypes.c_int]
@@ -103,6 +109,33 @@ def compute_gemm(y, a, b):
                                 _ints(a.shape), a.ndim, _f(np.ascontiguousarray(b)),
                                 _ints(b.shape), b.ndim))
     return out
+
+
+def compute_gemm_fresh_y(y_shape, a, b):
+    """Compute::Gemm(y, a, b) with y a NEW TensorData of y_shape (never filled by the caller)."""
+    out = np.full(y_shape, np.float32(-777.0))
+    _ok(lib().sphh_compute_gemm_fresh_y(_f(out), _ints(y_shape), len(y_shape),
+                                        _f(np.ascontiguousarray(a)), _ints(a.shape), a.ndim,
+                                        _f(np.ascontiguousarray(b)), _ints(b.shape), b.ndim))
+    return out
+
+
+def gemm_half(y, a_dev_ptr, b_dev_ptr, K, fresh_y):
+    """Compute::GemmHalf(y, a, b, K) on device arrays of binary16; y is a numpy array whose
+    contents are uploaded unless fresh_y (then y is a new TensorData of that shape)."""
+    out = np.ascontiguousarray(y.copy())
+    _ok(lib().sphh_gemm_half(_f(out), _ints(y.shape), y.ndim, a_dev_ptr, b_dev_ptr, K,
+                             1 if fresh_y else 0))
+    return out
+
+
+def bench_gemm_half_fresh_y(a_dev_ptr, b_dev_ptr, n, steps, warmup, settle_ms):
+    """(event ms, wall ms) per pass of: fresh y from the pool, Compute::GemmHalf, Clean()."""
+    ev = ctypes.c_float(0)
+    wall = ctypes.c_double(0)
+    _ok(lib().sphh_bench_gemm_half_fresh_y(a_dev_ptr, b_dev_ptr, n, steps, warmup, settle_ms,
+                                           ctypes.byref(ev), ctypes.byref(wall)))
+    return ev.value, wall.value
 
 
 def transpose(x, y_shape):

@@ -108,7 +108,8 @@ def test_overwrite_with_zero_k_stores_zeros_and_bad_flags_are_rejected(dev):
     kept = h.gpu_gemm_f32_ex(junk, one, one, 3, 4, 0, capi.SPH_GEMM_TRANS_A)
     assert np.array_equal(kept, junk)
     with pytest.raises(capi.SphError):
-        h.gpu_gemm_f32_ex(junk, one, one, 3, 4, 1, 64)
+        # operands of the stated size: the helper checks extents before every raw-pointer call
+        h.gpu_gemm_f32_ex(junk, np.zeros(3, np.float32), np.zeros(4, np.float32), 3, 4, 1, 64)
 
 
 def test_backward_shapes_of_the_mlp(dev):

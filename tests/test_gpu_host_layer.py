@@ -92,6 +92,75 @@ def test_repeated_outputs_accumulate_in_walk_order(dev):
     _assert_close_to_cpu(hl.compute_gemm(y0, a, b), y0, a, b, 1e-3)
 
 
+@pytest.mark.parametrize("shapes", [
+    ((64, 48), (64, 40), (40, 48)),                 # one product
+    ((5, 6, 8), (5, 6, 9), (5, 9, 8)),              # equal batches
+    ((5, 6, 8), (1, 6, 9), (5, 9, 8)),              # A shared by the batch
+    ((16, 70, 33), (16, 70, 20), (1, 20, 33)),      # B shared by the batch, ragged widths
+    ((300, 260), (300, 100), (100, 260)),           # tiled kernels
+    ((2, 4, 5), (6, 4, 2), (3, 2, 5)),              # outputs hit several times: must NOT overwrite
+    ((3,), (4,), (4, 3)),                           # 1-D operands
+])
+def test_fresh_y_is_stored_not_filled_and_read(dev, shapes):
+    """A new TensorData reads as zeros but its fill is deferred; Compute::Gemm into it stores the
+    product when the walk writes every element exactly once, and must give the bits of the
+    accumulating call on an explicitly zeroed y in every case."""
+    ys, as_, bs = shapes
+    h.announce("Compute::Gemm fresh y", ys, as_, bs)
+    a, b = synth.uniform(31, as_), synth.uniform(32, bs)
+    # a dirty block of y's size goes back to the pool first, so that the fresh y reuses it
+    hl.compute_gemm(np.full(ys, 9.0, np.float32), a, b)
+    got = hl.compute_gemm_fresh_y(ys, a, b)
+    on_zeros = hl.compute_gemm(np.zeros(ys, np.float32), a, b)
+    assert np.array_equal(got.view(np.uint32), on_zeros.view(np.uint32))
+    _assert_close_to_cpu(got, np.zeros(ys, np.float32), a, b, 1e-3)
+
+
+@pytest.mark.parametrize("shape", [(512, 512, 512, 1), (256, 264, 96, 3), (100, 40, 70, 1),
+                                   (4096, 4096, 4096, 1)])
+def test_gemm_half_operator_fresh_y_equals_accumulating_on_zeros(dev, shape):
+    """Compute::GemmHalf: the product stored into a fresh y has the bits of the product added
+    to a zero y, and both are within 1e-2 of the CPU loop on the widened operands."""
+    from sapphire_amd import capi
+    M, N, K, batch = shape
+    h.announce("Compute::GemmHalf fresh y", shape)
+    A = synth.normal(41, (batch, M, K), 1.0 / np.sqrt(K)).astype(np.float16)
+    B = synth.normal(42, (batch, K, N), 1.0 / np.sqrt(K)).astype(np.float16)
+    dA, dB = capi.DeviceBuffer.from_array(A), capi.DeviceBuffer.from_array(B)
+    assert dA.nbytes >= 2 * batch * M * K and dB.nbytes >= 2 * batch * K * N
+    ys = (batch, M, N) if batch > 1 else (M, N)
+    # leave a dirty block of y's size in the pool for the fresh y to pick up
+    hl.gemm_half(np.full(ys, 5.0, np.float32), dA.ptr, dB.ptr, K, fresh_y=False)
+    fresh = hl.gemm_half(np.full(ys, -3.0, np.float32), dA.ptr, dB.ptr, K, fresh_y=True)
+    on_zeros = hl.gemm_half(np.zeros(ys, np.float32), dA.ptr, dB.ptr, K, fresh_y=False)
+    dA.release()
+    dB.release()
+    assert np.array_equal(fresh.view(np.uint32), on_zeros.view(np.uint32))
+    rows = M if M <= 512 else 64      # the CPU loop on a row slice of the large case
+    for u in range(batch):
+        a32 = A[u, :rows].astype(np.float32)
+        b32 = B[u].astype(np.float32)
+        ref = po.gemm_rows(np.zeros((rows, N), np.float32), a32, b32, rows, N, K, threads=4)
+        got = fresh.reshape(batch, M, N)[u, :rows]
+        assert h.normalised_error(got, ref, np.abs(a32), np.abs(b32)) <= 1e-2
+
+
+def test_gemm_half_operator_accumulates_into_a_used_y(dev):
+    from sapphire_amd import capi
+    M, N, K = 130, 72, 64
+    h.announce("Compute::GemmHalf accumulate", M, N, K)
+    A = synth.normal(43, (M, K), 0.125).astype(np.float16)
+    B = synth.normal(44, (K, N), 0.125).astype(np.float16)
+    y0 = synth.uniform(45, (M, N))
+    dA, dB = capi.DeviceBuffer.from_array(A), capi.DeviceBuffer.from_array(B)
+    got = hl.gemm_half(y0, dA.ptr, dB.ptr, K, fresh_y=False)
+    dA.release()
+    dB.release()
+    a32, b32 = A.astype(np.float32), B.astype(np.float32)
+    ref = po.gemm_rows(y0.copy(), a32, b32, M, N, K, threads=2)
+    assert h.normalised_error(got, ref, np.abs(a32), np.abs(b32)) <= 1e-2
+
+
 def test_one_dimensional_operands(dev):
     h.announce("Compute::Gemm 1-D operands [4] x [4,3] -> [3]")
     a, b, y0 = synth.uniform(11, (4,)), synth.uniform(12, (4, 3)), synth.uniform(13, (3,))
