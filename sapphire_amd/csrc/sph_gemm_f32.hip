@@ -524,7 +524,11 @@ struct DmaTile
     static constexpr uint32_t kRowBytes = X * 4;          // k-major row
     static constexpr uint32_t kRowsPerCopyX = 1024 / kRowBytes;
     static constexpr uint32_t kBytesKContig = X * BK * 4;
-    static constexpr uint32_t kBytesXContig = X * BK * 4 + (BK / 4) * 128;
+    // X = 32: a copy (1 KiB, written lane-linear) holds 8 whole rows, so no padding can be put
+    // between rows 3 and 4; instead the copy fetches its rows in the order 0 4 1 5 2 6 3 7, which
+    // puts rows k and k + 4 (read together by the two lane halves) 128 bytes apart
+    static constexpr bool kPairedRows = X == 32;
+    static constexpr uint32_t kBytesXContig = kPairedRows ? X * BK * 4 : X * BK * 4 + (BK / 4) * 128;
 
     // position of chunk c of K-contiguous row x
     static __device__ __forceinline__ uint32_t Swizzle(uint32_t x)
@@ -534,11 +538,17 @@ struct DmaTile
     // LDS offset of copy j of a k-major slab (128 bytes of padding after every 4 rows)
     static __device__ __forceinline__ constexpr uint32_t CopyOffsetXContig(uint32_t j)
     {
-        return j * 1024u + ((j * kRowsPerCopyX) / 4u) * 128u;
+        return kPairedRows ? j * 1024u : j * 1024u + ((j * kRowsPerCopyX) / 4u) * 128u;
     }
     static __device__ __forceinline__ constexpr uint32_t RowOffsetXContig(uint32_t k)
     {
-        return k * kRowBytes + (k / 4u) * 128u;
+        return kPairedRows ? ((k & ~7u) + 2u * (k & 3u) + ((k >> 2) & 1u)) * kRowBytes
+                           : k * kRowBytes + (k / 4u) * 128u;
+    }
+    // k-major slab: the row of the slab that lies at row position p of the unpadded copy stream
+    static __device__ __forceinline__ constexpr uint32_t RowAtPosition(uint32_t p)
+    {
+        return kPairedRows ? (p & ~7u) + ((p & 7u) >> 1) + 4u * (p & 1u) : p;
     }
 };
 
@@ -557,13 +567,32 @@ struct DmaTile
 // 4 values that end at K - and the fragments are put right where they are used (zeros for
 // k >= K, for A and B alike), so the step adds what a zero-padded slab would: the same sum,
 // in the same order, as the register-staged kernel.
-template <int BM, int BN, int BK, int STAGES, bool TA, bool TB, bool WALK, bool TAIL = false>
-__global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args args)
+//
+// KSPLIT = 2: two groups of wavefronts share the tile; of the four 8-wide k blocks of a
+// 32-wide step group 0 multiplies the first two and group 1 the last two, each into a sum of
+// its own, and after the last step group 1 hands its sum to group 0 through LDS, which adds
+// it to its own (one fixed order: group 0's sum + group 1's) and stores.  A compute unit then
+// holds two wavefronts per SIMD with independent accumulators - one's wait for a barrier or
+// a fragment is covered by the other's matrix instructions - which is what a product with at
+// most one 64 x 64 tile per compute unit lacks.  With KSPLIT = 2 a 64 x 32 tile (two
+// wavefronts per group) gives products with fewer 64-tiles than compute units twice as many
+// workgroups.  The K products of an element are then summed in another order than with
+// KSPLIT = 1 (within the fp32 tolerance, not bit-identical to it).
+template <int BM, int BN, int BK, int STAGES, bool TA, bool TB, bool WALK, bool TAIL = false,
+          int KSPLIT = 1>
+__global__ __launch_bounds__(((BN >= 64) ? 4 : 2) * KSPLIT * 64) void GemmF32DmaKernel(
+    const GemmF32Args args)
 {
     static_assert(BK == 16 || BK == 32, "K step of 16 or 32");
     static_assert(!(WALK && TAIL), "a walk needs whole rings of steps");
-    constexpr int WM = BM / 2;
-    constexpr int WN = BN / 2;
+    static_assert(KSPLIT == 1 || (KSPLIT == 2 && BK == 32 && !WALK), "K split over two groups");
+    static_assert(BN >= 64 || KSPLIT == 2, "the 32-wide tile has two wavefronts per group");
+    constexpr int WAVES_M = 2;
+    constexpr int WAVES_N = BN >= 64 ? 2 : 1;
+    constexpr int GROUP_WAVES = WAVES_M * WAVES_N;      // wavefronts that cover the tile once
+    constexpr int NW = GROUP_WAVES * KSPLIT;            // wavefronts of the workgroup
+    constexpr int WM = BM / WAVES_M;
+    constexpr int WN = BN / WAVES_N;
     constexpr int TM = WM / 32;
     constexpr int TN = WN / 32;
     using TileA = DmaTile<BM, BK>;
@@ -571,10 +600,13 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     constexpr uint32_t kBytesA = TA ? TileA::kBytesXContig : TileA::kBytesKContig;
     constexpr uint32_t kBytesB = TB ? TileB::kBytesKContig : TileB::kBytesXContig;
     constexpr uint32_t kStageBytes = kBytesA + kBytesB;
-    constexpr uint32_t kCopiesPerWave = (TileA::kCopies + TileB::kCopies) / 4;  // per step
-    constexpr uint32_t kCopiesA = TileA::kCopies / 4;  // per wavefront
-    constexpr uint32_t kCopiesB = TileB::kCopies / 4;
-    constexpr uint32_t kBlocks = BK / 8;  // 8-wide k blocks (4 MFMAs each) per step
+    static_assert(TileA::kCopies % NW == 0 && TileB::kCopies % NW == 0,
+                  "every wavefront copies the same number of pieces");
+    constexpr uint32_t kCopiesPerWave = (TileA::kCopies + TileB::kCopies) / NW;  // per step
+    constexpr uint32_t kCopiesA = TileA::kCopies / NW;  // per wavefront
+    constexpr uint32_t kCopiesB = TileB::kCopies / NW;
+    constexpr uint32_t kBlocks = BK / 8 / KSPLIT;  // 8-wide k blocks (4 MFMAs each) per step
+                                                   // and wavefront
     constexpr int kQuads = TM * TN * 4;   // float4 of `out` per lane
 
     __shared__ __attribute__((aligned(1024))) char lds[STAGES * kStageBytes];
@@ -582,8 +614,9 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t waveM = wave >> 1;
-    const uint32_t waveN = wave & 1;
+    const uint32_t kgroup = wave / GROUP_WAVES;  // which k blocks of a step (0 without KSPLIT)
+    const uint32_t waveM = (wave % GROUP_WAVES) / WAVES_N;
+    const uint32_t waveN = (wave % GROUP_WAVES) % WAVES_N;
     const uint32_t l32 = lane & 31;
     const uint32_t khalf = lane >> 5;
 
@@ -601,7 +634,7 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     const uint32_t M = args.M, N = args.N, K = args.K;
 
     // Where a tile's operands and output start, and what this lane copies of it every step:
-    // copy j of an operand is taken by wavefront j % 4; lane offsets are bytes from the
+    // copy j of an operand is taken by wavefront j % NW; lane offsets are bytes from the
     // operand's base at step 0, the base advances by one K step per step.
     struct Place
     {
@@ -634,9 +667,9 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         return (gx * K + k4) * 4u - 16u + kTailBias;
     };
     auto laneOffsetXContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t pitch,
-                                 uint32_t rowBytes, uint32_t valid) {
+                                 uint32_t rowBytes, uint32_t valid, auto rowAtPosition) {
         const uint32_t b = j * 1024 + lane * 16;  // byte inside the unpadded slab
-        uint32_t k = b / rowBytes;
+        uint32_t k = rowAtPosition(b / rowBytes);
         if (k >= valid)
             k = 0;
         const uint32_t col = (b % rowBytes) / 4;
@@ -666,35 +699,35 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
 #pragma unroll
         for (uint32_t i = 0; i < kCopiesA; ++i)
         {
-            const uint32_t j = wave + 4 * i;
-            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, args.lda, TileA::kRowBytes, BK)
+            const uint32_t j = wave + NW * i;
+            p.aLane[i] = TA ? laneOffsetXContig(j, p.rowBase, M, args.lda, TileA::kRowBytes, BK, TileA::RowAtPosition)
                             : laneOffsetKContig(j, p.rowBase, M, BK);
             if constexpr (TAIL)
                 p.aTail[i] = TA ? laneOffsetXContig(j, p.rowBase, M, args.lda, TileA::kRowBytes,
-                                                    lastValid)
+                                                    lastValid, TileA::RowAtPosition)
                                 : laneOffsetKContig(j, p.rowBase, M, lastValid);
         }
 #pragma unroll
         for (uint32_t i = 0; i < kCopiesB; ++i)
         {
-            const uint32_t j = wave + 4 * i;
+            const uint32_t j = wave + NW * i;
             p.bLane[i] = TB ? laneOffsetKContig(j, p.colBase, N, BK)
-                            : laneOffsetXContig(j, p.colBase, N, args.ldb, TileB::kRowBytes, BK);
+                            : laneOffsetXContig(j, p.colBase, N, args.ldb, TileB::kRowBytes, BK, TileB::RowAtPosition);
             if constexpr (TAIL)
                 p.bTail[i] = TB ? laneOffsetKContig(j, p.colBase, N, lastValid)
                                 : laneOffsetXContig(j, p.colBase, N, args.ldb, TileB::kRowBytes,
-                                                    lastValid);
+                                                    lastValid, TileB::RowAtPosition);
         }
     };
     // LDS offsets of this wavefront's copies inside a stage
     uint32_t aDst[kCopiesA], bDst[kCopiesB];
 #pragma unroll
     for (uint32_t i = 0; i < kCopiesA; ++i)
-        aDst[i] = TA ? TileA::CopyOffsetXContig(wave + 4 * i) : (wave + 4 * i) * 1024;
+        aDst[i] = TA ? TileA::CopyOffsetXContig(wave + NW * i) : (wave + NW * i) * 1024;
 #pragma unroll
     for (uint32_t i = 0; i < kCopiesB; ++i)
         bDst[i] = kBytesA +
-                  (TB ? (wave + 4 * i) * 1024 : TileB::CopyOffsetXContig(wave + 4 * i));
+                  (TB ? (wave + NW * i) * 1024 : TileB::CopyOffsetXContig(wave + NW * i));
 
     Place cur, nxt;
     locate(logical, cur);
@@ -771,19 +804,26 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     // k-major operand: byte offset of this lane's column; the row offset is added per k.
     uint32_t aFrag[TM], bFrag[TN];
     uint32_t aSwz[TM], bSwz[TN];
+    // Group g of a K split takes k blocks kBlocks*g .. of every step: for a K-contiguous
+    // operand that is chunk 2*kBlocks*g + ..., folded into the swizzle (the bits do not overlap);
+    // for a k-major operand rows 8*kBlocks*g + ..., a constant added to the lane's offset.
+    const uint32_t groupChunk = kgroup * (2 * kBlocks);
+    const uint32_t groupRowsA = TileA::RowOffsetXContig(8 * kBlocks) * kgroup;
+    const uint32_t groupRowsB = TileB::RowOffsetXContig(8 * kBlocks) * kgroup;
+    static_assert(KSPLIT == 1 || (8 * kBlocks) % 4 == 0, "whole padding groups per k group");
 #pragma unroll
     for (int i = 0; i < TM; ++i)
     {
         const uint32_t x = waveM * WM + i * 32 + l32;
-        aFrag[i] = TA ? x * 4 : x * BK * 4;
-        aSwz[i] = TileA::Swizzle(x);
+        aFrag[i] = TA ? x * 4 + groupRowsA : x * BK * 4;
+        aSwz[i] = TileA::Swizzle(x) ^ groupChunk;
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j)
     {
         const uint32_t x = waveN * WN + j * 32 + l32;
-        bFrag[j] = kBytesA + (TB ? x * BK * 4 : x * 4);
-        bSwz[j] = TileB::Swizzle(x);
+        bFrag[j] = kBytesA + (TB ? x * BK * 4 : x * 4 + groupRowsB);
+        bSwz[j] = TileB::Swizzle(x) ^ groupChunk;
     }
 
     // fragments of k block q (k = 8q + 4*khalf + e, e = 0..3)
@@ -842,7 +882,8 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
     auto dropMissing = [&](float (&a)[TM][4], float (&b)[TN][4], uint32_t q, uint32_t valid) {
         if constexpr (TAIL)
         {
-            const uint32_t k0 = 8 * q + 4 * khalf;  // k of this lane's fragment element 0
+            // k of this lane's fragment element 0 (q counts this group's blocks)
+            const uint32_t k0 = 8 * (q + kgroup * kBlocks) + 4 * khalf;
             const uint32_t shift = (4 - valid % 4) % 4;
             const bool whole = k0 + 4 <= valid;
             const bool reaches = !whole && k0 < valid;
@@ -1129,6 +1170,43 @@ __global__ __launch_bounds__(kThreads) void GemmF32DmaKernel(const GemmF32Args a
         }
     }
     WaitVmem<0>();  // the surplus copies of the last steps still target LDS
+
+    if constexpr (KSPLIT == 2)
+    {
+        // group 1 hands its sums over: float4 v of block (i, j) of wavefront w of a group lies at
+        // ((i*TN + j)*4 + v) * GROUP_WAVES*64 + w*64 + lane, so a wavefront access is contiguous
+        static_assert(TM * TN * 16 * GROUP_WAVES * 64 * 4 <= STAGES * kStageBytes, "fits the ring");
+        __syncthreads();  // every wavefront has read its last fragments
+        floatx4* hand = reinterpret_cast<floatx4*>(lds) + (wave % GROUP_WAVES) * 64 + lane;
+        if (kgroup == 1)
+        {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        hand[((i * TN + j) * 4 + v) * (GROUP_WAVES * 64)] =
+                            floatx4{ acc[i][j][4 * v], acc[i][j][4 * v + 1], acc[i][j][4 * v + 2],
+                                     acc[i][j][4 * v + 3] };
+        }
+        __syncthreads();
+        if (kgroup == 1)
+            return;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                {
+                    const floatx4 other = hand[((i * TN + j) * 4 + v) * (GROUP_WAVES * 64)];
+                    acc[i][j][4 * v] += other[0];
+                    acc[i][j][4 * v + 1] += other[1];
+                    acc[i][j][4 * v + 2] += other[2];
+                    acc[i][j][4 * v + 3] += other[3];
+                }
+    }
 
     if constexpr (!WALK)
         StoreTile<TM, TN>(acc, cur.out, cur.rowBase + waveM * WM, cur.colBase + waveN * WN, M, N,
@@ -1534,11 +1612,22 @@ void LaunchSkinny(const GemmF32Args& args, dim3 grid, uint32_t tile, bool wide, 
 }
 
 // `walk`: 64-tiles only, each workgroup takes several tiles
+// `ksplit`: 0, or 2 = K split over two groups of wavefronts on 64 x 32 tiles
 template <bool TA, bool TB>
 void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dma, bool walk,
-                 hipStream_t stream)
+                 int ksplit, hipStream_t stream)
 {
     const dim3 block(kThreads);
+    if (dma && ksplit != 0)
+    {
+        if (args.K % 32 == 0)
+            hipLaunchKernelGGL((GemmF32DmaKernel<64, 32, 32, 4, TA, TB, false, false, 2>), grid,
+                               dim3(256), 0, stream, args);
+        else
+            hipLaunchKernelGGL((GemmF32DmaKernel<64, 32, 32, 4, TA, TB, false, true, 2>), grid,
+                               dim3(256), 0, stream, args);
+        return;
+    }
     if (dma)
     {
         if (big && args.K % 16 != 0)
@@ -1606,20 +1695,37 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // (not when the whole product goes to the few-tile kernel, which takes any N as it is)
     const uint64_t wholeTiles64 =
         static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
-    const bool wholeIsFewTiles =
-        wholeTiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) && args.K >= 64;
-    if (args.split == 0 && args.N % 4 != 0 && args.N > 4 && args.M > 1 && args.K >= kBK &&
+    // Between a quarter and a half as many 64-tiles as compute units the straight-to-LDS
+    // kernel on 64 x 32 tiles (K split over two groups of wavefronts) gives every compute
+    // unit a tile and beats the few-tile kernel, whose 32 x 32 tiles ask the caches for twice
+    // the operand bytes per flop (512 x 1024 x 1024: 17.0 us on the few-tile kernel).
+    const uint64_t cusAll = static_cast<uint64_t>(sph::ComputeUnits());
+    const bool midTiled = wholeTiles64 * 4 > cusAll && wholeTiles64 * 2 <= cusAll &&
+                          args.basesOk != 0 && args.K >= 64 && args.M >= 4 && args.N >= 4 &&
+                          // (an A stored K x M is copied 4 rows at a time and cut into two
+                          // launches from 68 rows up; asked of either storage, so that the
+                          // choice does not depend on the flags)
+                          (args.M % 4 == 0 || args.M >= 68) &&
+                          static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
+                          static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
+    const bool wholeIsFewTiles = wholeTiles64 * 2 <= cusAll && args.K >= 64 && !midTiled;
+    // decided once, on the whole product, and carried by its parts (bit 2: tiled kernels, bit 3:
+    // the K-split kernel on 64 x 32 tiles), so that a product's columns and rows are all summed
+    // in one order however it is cut up
+    if (args.split == 0 && !wholeIsFewTiles)
+        args.split = midTiled ? 12u : 4u;
+    if ((args.split & 3u) == 0 && args.N % 4 != 0 && args.N > 4 && args.M > 1 && args.K >= kBK &&
         !wholeIsFewTiles)
     {
         const uint32_t whole = args.N & ~3u;
         GemmF32Args left = args;
-        left.split = 1;
+        left.split |= 1u;
         left.N = whole;
         const int rc = Launch(left, units, allowVector, outOffsetsAligned, transA, transB, stream);
         if (rc != SPH_OK)
             return rc;
         GemmF32Args right = args;
-        right.split = 1;
+        right.split |= 1u;
         right.N = args.N - whole;
         right.B = args.B + (transB ? static_cast<size_t>(whole) * args.K : whole);
         right.out = args.out + whole;
@@ -1637,10 +1743,10 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // the whole product, so that its parts run the kernels the whole would)
     const uint64_t tiles64 =
         static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
-    const bool fewTiles = (args.split & 4u) == 0 &&
-                          ((tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) &&
-                            args.K >= 64) ||
-                           (part && args.N < 4));
+    const bool fewTiles = (part && args.N < 4) ||
+                          ((args.split & 4u) == 0 &&
+                           tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) &&
+                           args.K >= 64);
     if ((args.split & 2u) == 0 && transA && args.M % 4 != 0 && args.M >= 68 && dmaShape &&
         !fewTiles)
     {
@@ -1672,7 +1778,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
 
     // a single output row is a reduction over the rows of B, not a matrix-core job
     if (args.M == 1 && !transB && args.entries == nullptr && args.K >= 64 && units <= 65535 &&
-        args.split == 0)
+        (args.split & 3u) == 0)
     {
         hipLaunchKernelGGL(GemvRowKernel, dim3((args.N + 63) / 64, units), dim3(kGemvWaves * 64),
                            0, stream, args);
@@ -1737,9 +1843,15 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const uint64_t cost128 = rounds128 * 400 + (rounds128 == 1 ? 32 : 0);
     const uint64_t cost64 = ((tiles64 + cus - 1) / cus) * 107;
     const bool big = cost128 <= cost64;
+    // 64 x 32 tiles with K split over two groups of wavefronts (see the top of Launch).  The same
+    // split on 64 x 64 tiles with eight wavefronts was measured for products with one 64-tile
+    // per compute unit and does not pay (1024^3: 18.8 against 18.4 us): their loop already runs
+    // at the matrix pipe's rate and what is left is the fixed cost of a launch.
+    const int ksplit = ((args.split & 8u) != 0 && dma && !big && args.K >= 64) ? 2 : 0;
     const uint32_t bm = big ? 128 : 64;
+    const uint32_t bn = ksplit == 2 ? 32 : bm;
     args.tilesM = (args.M + bm - 1) / bm;
-    args.tilesN = (args.N + bm - 1) / bm;
+    args.tilesN = (args.N + bn - 1) / bn;
     const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
     if (blocks >= (1ull << 31) - 8)
         return sph::Fail(SPH_ERR_INVALID, "sph_gemm_f32 - too many tiles for one launch");
@@ -1765,18 +1877,18 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // kernel would need more than 256 registers for it and lose its second resident workgroup
     // (measured 4096^3: 921 -> 966 us), so it keeps one tile per workgroup.
     const uint32_t slotsPerXcd = static_cast<uint32_t>(cus / 8 * 2);
-    const bool walk = dma && !big &&
+    const bool walk = dma && !big && ksplit == 0 &&
                       args.M % 64 == 0 && args.N % 64 == 0 && args.K % 128 == 0 &&
                       (reinterpret_cast<uintptr_t>(args.bias) & 15u) == 0;
     const dim3 grid((walk ? std::min(slotsPerXcd, args.perXcd) : args.perXcd) * 8);
     if (transA && transB)
-        LaunchTiled<true, true>(args, grid, big, aligned, dma, walk, stream);
+        LaunchTiled<true, true>(args, grid, big, aligned, dma, walk, ksplit, stream);
     else if (transA)
-        LaunchTiled<true, false>(args, grid, big, aligned, dma, walk, stream);
+        LaunchTiled<true, false>(args, grid, big, aligned, dma, walk, ksplit, stream);
     else if (transB)
-        LaunchTiled<false, true>(args, grid, big, aligned, dma, walk, stream);
+        LaunchTiled<false, true>(args, grid, big, aligned, dma, walk, ksplit, stream);
     else
-        LaunchTiled<false, false>(args, grid, big, aligned, dma, walk, stream);
+        LaunchTiled<false, false>(args, grid, big, aligned, dma, walk, ksplit, stream);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }

@@ -137,6 +137,19 @@ def gpu_transpose(x, rows, cols, batch=1):
     return out
 
 
+# fp32: a product with more than a quarter and at most half as many 64 x 64 output tiles as the
+# chip has compute units (K >= 64) runs on 64 x 32 tiles with K split over two groups of
+# wavefronts when its operands allow the straight-to-LDS copies; the K products of an element
+# are then summed in another order than by the other fp32 kernels.
+F32_CUS = 256
+
+
+def f32_k_split_range(M, N, K, batch=1):
+    tiles64 = -(-M // 64) * -(-N // 64) * batch
+    return (4 * tiles64 > F32_CUS and 2 * tiles64 <= F32_CUS and K >= 64 and M >= 4 and N >= 4
+            and (M % 4 == 0 or M >= 68))
+
+
 # Small products run on the few-tile kernel: at most one 32 x 32 output tile per compute unit
 # (256 of them), or a matrix of at most 16 rows or columns with at most four 16 x 16 tiles per
 # compute unit.  The tests of the tiled kernels' edges use small matrices, so each of those shapes

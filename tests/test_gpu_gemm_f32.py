@@ -159,7 +159,13 @@ def test_partial_last_k_step(dev, dims, flags):
     other = dC.download(np.float32, (M * N + 1,))[1:].reshape(M, N)
     for d in (dA, dB, dC):
         d.release()
-    assert np.array_equal(got.view(np.uint32), other.view(np.uint32))
+    if h.f32_k_split_range(M, N, K):
+        # 65 .. 128 tiles of 64 x 64: aligned operands run the kernel that splits K over two groups
+        # of wavefronts, misaligned ones the few-tile kernel: two orders of the K products, both
+        # held to the tolerance
+        assert h.normalised_error(other[:256], ref, np.abs(A[:256]), np.abs(B)) <= TOL_F32
+    else:
+        assert np.array_equal(got.view(np.uint32), other.view(np.uint32))
 
 
 # N = 4 q + r, r != 0: the first 4 q columns on the tiled kernels with the
