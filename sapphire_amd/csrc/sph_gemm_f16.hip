@@ -257,26 +257,46 @@ constexpr int kStageHalfs = kT * kTK;
 // each.  To write (and, without CSP, read) whole 256-byte row segments instead, each
 // wavefront turns its 128 x 64 part round through a private 16 KiB piece of LDS, 64 rows at a
 // time: after that a lane holds 4 consecutive columns and 16 consecutive lanes cover one row.
-constexpr int CLoopSteps(int csp)
+constexpr int CLoopSteps(int csp, int rowBlocks = 8)
 {
-    return (8 * csp + 1 + 3) / 4 * 4;
+    return (rowBlocks * csp + 1 + 3) / 4 * 4;
 }
-template <bool RAGGED, int CSP, bool TA, bool TB, bool TAIL>
+//
+// NT = 128: the tile is 256 rows by 128 columns and the eight wavefronts are arranged 4 x 2, a
+// 64 x 64 part each (4 x 4 blocks, 64 accumulator registers), for products with too few
+// 256 x 256 tiles to fill the chip: against 128 x 128 tiles a compute unit moves three quarters
+// of the bytes per flop into LDS and a wavefront reads 8 fragments per 16 matrix instructions
+// instead of 4 per 4.  The B stage then has k-rows of 256 bytes (the same chunk swizzle) and a
+// wavefront makes two copies of A and one of B per step.
+template <bool RAGGED, int CSP, bool TA, bool TB, bool TAIL, int NT = 256>
 __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 {
+    static_assert(NT == 256 || NT == 128, "256 x 256 or 256 x 128 tiles");
     constexpr int WAVES = 8;
-    constexpr int ROUNDS = 2;               // copies per lane per operand per stage
-    constexpr int WAVE_LDS = ROUNDS * 1024;
-    constexpr int COPIES_PER_STAGE = 2 * ROUNDS;
+    constexpr int WN = NT / 64;               // wavefronts across the tile: 4 or 2
+    constexpr int WMROWS = kT / (WAVES / WN); // rows per wavefront: 128 or 64
+    constexpr int MB = WMROWS / 16;           // 16-row blocks per wavefront: 8 or 4
+    constexpr int ROUNDS_A = 2;               // 1 KiB copies per wavefront and stage: A 16 KiB,
+    constexpr int ROUNDS_B = NT / 128;        // B 64 * NT bytes
+    constexpr int COPIES_PER_STAGE = ROUNDS_A + ROUNDS_B;
+    constexpr int kBytesStageA = kStageBytes;
+    constexpr int kBytesStageB = NT * kTK * 2;
     constexpr uint32_t kBias = 4096;
     constexpr bool CLOOP = CSP != 0;
-    constexpr int kCLoopSteps = CLoopSteps(CSP);
+    constexpr int kCLoopSteps = CLoopSteps(CSP, MB);
     static_assert(!(CLOOP && RAGGED), "old values are added in the loop for whole tiles only");
 
-    __shared__ __attribute__((aligned(1024))) _Float16 Lds[2][kTStages][kStageHalfs];
+    // the ring of stages; the epilogue reuses it as eight private pieces of 16 KiB
+    constexpr int kRingBytes = kTStages * (kBytesStageA + kBytesStageB);
+    constexpr int kLdsBytes = kRingBytes > WAVES * 64 * 64 * 4 ? kRingBytes : WAVES * 64 * 64 * 4;
+    __shared__ __attribute__((aligned(1024))) char LdsRaw[kLdsBytes];
     __shared__ __attribute__((aligned(1024))) float CMail[CLOOP ? WAVES * 1024 : 4];
-    auto& As = Lds[0];
-    auto& Bs = Lds[1];
+    auto AStage = [&](int stage) {
+        return reinterpret_cast<_Float16*>(LdsRaw + stage * kBytesStageA);
+    };
+    auto BStage = [&](int stage) {
+        return reinterpret_cast<_Float16*>(LdsRaw + kTStages * kBytesStageA + stage * kBytesStageB);
+    };
 
     uint32_t unit, tm, tn;
     if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
@@ -285,12 +305,12 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = tid >> 6;
-    const uint32_t waveM = wave >> 2;  // 0..1 -> 128 rows each
-    const uint32_t waveN = wave & 3;   // 0..3 -> 64 columns each
+    const uint32_t waveM = wave / WN;  // WMROWS rows each
+    const uint32_t waveN = wave % WN;  // 64 columns each
 
     const uint32_t K = args.K, N = args.N;
     const uint32_t rowsLeft = RAGGED ? min(static_cast<uint32_t>(kT), args.M - tm * kT) : kT;
-    const uint32_t colsLeft = RAGGED ? min(static_cast<uint32_t>(kT), N - tn * kT) : kT;
+    const uint32_t colsLeft = RAGGED ? min(static_cast<uint32_t>(NT), N - tn * NT) : NT;
     // An operand is either K-contiguous (x-rows of K halves: A as given, B stored N x K with
     // TB) or k-major (k-rows of x halves: B as given, A stored K x M with TA); x is the row of A
     // or the column of B.  A K-contiguous operand takes the "A stage" layout and the 16-byte
@@ -302,47 +322,54 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     const _Float16* __restrict__ A = args.A + args.strideA * static_cast<int64_t>(unit) +
                                      static_cast<size_t>(tm) * kT * (TA ? 1u : pitchA);
     const _Float16* __restrict__ B = args.B + args.strideB * static_cast<int64_t>(unit) +
-                                     static_cast<size_t>(tn) * kT * (TB ? pitchB : 1u);
+                                     static_cast<size_t>(tn) * NT * (TB ? pitchB : 1u);
     float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit) +
-                              static_cast<size_t>(tm) * kT * ldc + static_cast<size_t>(tn) * kT;
+                              static_cast<size_t>(tm) * kT * ldc + static_cast<size_t>(tn) * NT;
 
     // ---- global -> LDS copy plan --------------------------------------------
-    // A copy instruction moves 1 KiB per wavefront.  Wavefront w fills the WAVE_LDS bytes
-    // at w*WAVE_LDS of a stage in ROUNDS copies; copy r puts lane i's 16 bytes at
-    // w*WAVE_LDS + r*1024 + i*16.
+    // A copy instruction moves 1 KiB per wavefront.  Wavefront w fills ROUNDS KiB at
+    // w*ROUNDS*1024 of an operand's stage in ROUNDS copies (ROUNDS_A, ROUNDS_B); copy r puts lane
+    // i's 16 bytes at w*ROUNDS*1024 + r*1024 + i*16.
     //   K-contiguous: that is LDS row R = w*8*ROUNDS + r*8 + i/8, physical chunk i%8, which
     //      must hold logical chunk L = (i%8) ^ ((R/2)%8): x = R (L < 4) or R+128 (L >= 4),
     //      k offset (L%4)*8.
-    //   k-major: k = w*2*ROUNDS + r*2 + i/32, physical 16-byte chunk i%32, 32-byte chunks
+    //   k-major (256 columns; twice the k-rows per copy for 128): k = w*2*ROUNDS + r*2 + i/32,
+    //      physical 16-byte chunk i%32, 32-byte chunks
     //      swizzled as described above.
     // The global address of a copy is a uniform base that advances with the K step plus a
     // per-lane byte offset that never changes.  The instruction offset r*1024 is added to
     // both the LDS and the global address, so the lane offsets subtract it again.  K steps
     // beyond the last are clamped to it: those copies land in buffers that are no longer
     // read, which keeps the number of copies in flight constant.
-    auto laneKContig = [&](int r, uint32_t xLeft, uint32_t pitch) {
-        const uint32_t R = wave * (8 * ROUNDS) + 8 * r + (lane >> 3);
+    // (an operand of X rows or columns, `rounds` copies per wavefront: the rows / k-rows are
+    // dealt to the wavefronts in order, X / 2 LDS rows or 32 k-rows in all)
+    auto laneKContig = [&](int r, uint32_t xLeft, uint32_t pitch, uint32_t X, uint32_t rounds) {
+        const uint32_t R = wave * (8 * rounds) + 8 * r + (lane >> 3);
         const uint32_t L = (lane & 7) ^ ((R >> 1) & 7);
-        const uint32_t x = R + ((L & 4) ? 128u : 0u);
+        const uint32_t x = R + ((L & 4) ? X / 2 : 0u);
         return (min(x, xLeft - 1) * pitch + (L & 3) * 8) * 2 + kBias - r * 1024;
     };
-    auto laneKMajor = [&](int r, uint32_t xLeft, uint32_t pitch) {
-        const uint32_t phys16 = lane & 31;
-        const uint32_t k = wave * (2 * ROUNDS) + r * 2 + (lane >> 5);
+    auto laneKMajor = [&](int r, uint32_t xLeft, uint32_t pitch, uint32_t X, uint32_t rounds) {
+        const uint32_t lanesPerRow = X / 8;          // 16-byte chunks of a k-row
+        const uint32_t rowsPerCopy = 64 / lanesPerRow;
+        const uint32_t phys16 = lane % lanesPerRow;
+        const uint32_t k = (wave * rounds + r) * rowsPerCopy + lane / lanesPerRow;
         const uint32_t swz = 2 * (k & 3) + ((k >> 3) & 1);
         const uint32_t logical16 = (((phys16 >> 1) ^ swz) << 1) | (phys16 & 1);
         return (k * pitch + min(logical16 * 8, xLeft - 8)) * 2 + kBias - r * 1024;
     };
-    uint32_t aLane[ROUNDS], bLane[ROUNDS];
+    uint32_t aLane[ROUNDS_A], bLane[ROUNDS_B];
 #pragma unroll
-    for (int r = 0; r < ROUNDS; ++r)
-    {
-        aLane[r] = TA ? laneKMajor(r, rowsLeft, pitchA) : laneKContig(r, rowsLeft, pitchA);
-        bLane[r] = TB ? laneKContig(r, colsLeft, pitchB) : laneKMajor(r, colsLeft, pitchB);
-    }
+    for (int r = 0; r < ROUNDS_A; ++r)
+        aLane[r] = TA ? laneKMajor(r, rowsLeft, pitchA, kT, ROUNDS_A)
+                      : laneKContig(r, rowsLeft, pitchA, kT, ROUNDS_A);
+#pragma unroll
+    for (int r = 0; r < ROUNDS_B; ++r)
+        bLane[r] = TB ? laneKContig(r, colsLeft, pitchB, NT, ROUNDS_B)
+                      : laneKMajor(r, colsLeft, pitchB, NT, ROUNDS_B);
     const uint32_t waveU = __builtin_amdgcn_readfirstlane(wave);
-    const uint32_t aLds = LdsAddress(&As[0][0]) + waveU * WAVE_LDS;
-    const uint32_t bLds = LdsAddress(&Bs[0][0]) + waveU * WAVE_LDS;
+    const uint32_t aLds = LdsAddress(AStage(0)) + waveU * (ROUNDS_A * 1024);
+    const uint32_t bLds = LdsAddress(BStage(0)) + waveU * (ROUNDS_B * 1024);
     const char* aGlobal = reinterpret_cast<const char*>(A) - kBias;
     const char* bGlobal = reinterpret_cast<const char*>(B) - kBias;
     const size_t aStepBytes = TA ? static_cast<size_t>(kTK) * pitchA * 2 : kTK * 2;
@@ -360,13 +387,13 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
         constexpr int r = decltype(round)::value;
         const uint32_t src = min(kt, steps - 1);
         const size_t start = (TAIL && src == steps - 1) ? aLastBytes : static_cast<size_t>(src) * aStepBytes;
-        DmaToLds16<r * 1024>(aLane[r], aGlobal + start, aLds + stage * kStageBytes);
+        DmaToLds16<r * 1024>(aLane[r], aGlobal + start, aLds + stage * kBytesStageA);
     };
     auto copyB = [&](uint32_t kt, int stage, auto round) {
         constexpr int r = decltype(round)::value;
         const uint32_t src = min(kt, steps - 1);
         const size_t start = (TAIL && src == steps - 1) ? bLastBytes : static_cast<size_t>(src) * bStepBytes;
-        DmaToLds16<r * 1024>(bLane[r], bGlobal + start, bLds + stage * kStageBytes);
+        DmaToLds16<r * 1024>(bLane[r], bGlobal + start, bLds + stage * kBytesStageB);
     };
 
     // ---- LDS -> fragment read plan ---------------------------------------------------
@@ -379,64 +406,73 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     //      of it: one offset per block.
     const uint32_t l16 = lane & 15;
     const uint32_t g = lane >> 4;
-    auto offKContig = [&](uint32_t x0) {
-        const uint32_t row = (x0 & 127u) + l16;
-        return row * 64 + ((((x0 >> 7) * 4 + g) ^ ((l16 >> 1) & 7)) * 8);  // + b*16*64
+    // (X = extent of the operand in the tile: 256 rows of A, NT columns of B)
+    auto offKContig = [&](uint32_t x0, uint32_t X) {
+        const uint32_t row = (x0 & (X / 2 - 1)) + l16;
+        return row * 64 + ((((x0 / (X / 2)) * 4 + g) ^ ((l16 >> 1) & 7)) * 8);  // + b*16*64
     };
-    auto offKMajor = [&](uint32_t x0, int b) {
+    auto offKMajor = [&](uint32_t x0, int b, uint32_t X) {
         const uint32_t kRow = 8 * g + (l16 >> 2);
         const uint32_t swz = 2 * ((l16 >> 2) & 3) + (g & 1);
-        return kRow * kT + (((x0 / 16 + b) ^ swz) * 16) + (l16 & 3) * 4;
+        return kRow * X + (((x0 / 16 + b) ^ swz) * 16) + (l16 & 3) * 4;
     };
-    constexpr int kOffA = TA ? 8 : 1, kOffB = TB ? 1 : 4;
+    constexpr int kOffA = TA ? MB : 1, kOffB = TB ? 1 : 4;
     uint32_t aOff[kOffA], bOff[kOffB];
 #pragma unroll
     for (int b = 0; b < kOffA; ++b)
-        aOff[b] = TA ? offKMajor(waveM * 128, b) : offKContig(waveM * 128);
+        aOff[b] = TA ? offKMajor(waveM * WMROWS, b, kT) : offKContig(waveM * WMROWS, kT);
 #pragma unroll
     for (int b = 0; b < kOffB; ++b)
-        bOff[b] = TB ? offKContig(waveN * 64) : offKMajor(waveN * 64, b);
+        bOff[b] = TB ? offKContig(waveN * 64, NT) : offKMajor(waveN * 64, b, NT);
     auto readKContig = [&](const _Float16* p) { return *reinterpret_cast<const halfx8*>(p); };
-    auto readKMajor = [&](const _Float16* p) { return Join(LdsReadTr(p), LdsReadTr(p + 4 * kT)); };
+    auto readKMajor = [&](const _Float16* p, int X) {
+        return Join(LdsReadTr(p), LdsReadTr(p + 4 * X));
+    };
     auto loadA = [&](int stage, int i) {
         if constexpr (TA)
-            return readKMajor(&As[stage][aOff[i]]);
+            return readKMajor(AStage(stage) + aOff[i], kT);
         else
-            return readKContig(&As[stage][aOff[0] + i * 16 * 64]);
+            return readKContig(AStage(stage) + aOff[0] + i * 16 * 64);
     };
     auto loadB = [&](int stage, int j) {
         if constexpr (TB)
-            return readKContig(&Bs[stage][bOff[0] + j * 16 * 64]);
+            return readKContig(BStage(stage) + bOff[0] + j * 16 * 64);
         else
-            return readKMajor(&Bs[stage][bOff[j]]);
+            return readKMajor(BStage(stage) + bOff[j], NT);
     };
 
-    floatx4 acc[8][4];
+    floatx4 acc[MB][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < MB; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             acc[i][j] = floatx4{ 0.f, 0.f, 0.f, 0.f };
 
 #define SPH_FENCE() __builtin_amdgcn_sched_barrier(0)
 
+    auto copyAllA = [&](uint32_t kt, int stage) {
+        copyA(kt, stage, std::integral_constant<int, 0>{});
+        copyA(kt, stage, std::integral_constant<int, 1>{});
+    };
+    auto copyAllB = [&](uint32_t kt, int stage) {
+        copyB(kt, stage, std::integral_constant<int, 0>{});
+        if constexpr (ROUNDS_B == 2)
+            copyB(kt, stage, std::integral_constant<int, 1>{});
+    };
 #pragma unroll
     for (int st = 0; st < 3; ++st)
     {
-        copyA(st, st, std::integral_constant<int, 0>{});
-        copyA(st, st, std::integral_constant<int, 1>{});
-        copyB(st, st, std::integral_constant<int, 0>{});
-        copyB(st, st, std::integral_constant<int, 1>{});
+        copyAllA(st, st);
+        copyAllB(st, st);
     }
-    copyA(3, 3, std::integral_constant<int, 0>{});
-    copyA(3, 3, std::integral_constant<int, 1>{});
-    // stage 0 is followed by 2.5 stages' worth of copies
-    WaitVmem<(5 * COPIES_PER_STAGE) / 2>();
+    copyAllA(3, 3);
+    // stage 0 is followed by the copies of stages 1 and 2 and of A's stage 3
+    WaitVmem<2 * COPIES_PER_STAGE + ROUNDS_A>();
     __syncthreads();
 
-    halfx8 af[8], bf0[4], bf1[4];
+    halfx8 af[MB], bf0[4], bf1[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MB / 2; ++i)
         af[i] = loadA(0, i);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -460,9 +496,10 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             mask(BF[j]);
-        // first half: rows 0-63, fetch this step's rows 64-127, request B of step kt+3
+        // first half: the upper half of the wavefront's row blocks, fetch this step's lower
+        // half, request B of step kt+3
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < MB / 2; ++i)
         {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -471,14 +508,17 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
                     mask(af[i]);
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(BF[j], af[i], acc[i][j], 0, 0, 0);
                 SPH_FENCE();
-                if (i < 2 && (j & 1) == 0)
-                    af[4 + 2 * i + j / 2] = loadA(cur, 4 + 2 * i + j / 2);
+                if (i < MB / 4 && (j & 1) == 0)
+                    af[MB / 2 + 2 * i + j / 2] = loadA(cur, MB / 2 + 2 * i + j / 2);
                 SPH_FENCE();
             }
             if (i == 1)
                 copyB(kt + 3, (cur + 3) % kTStages, std::integral_constant<int, 0>{});
-            if (i == 3)
-                copyB(kt + 3, (cur + 3) % kTStages, std::integral_constant<int, 1>{});
+            if constexpr (ROUNDS_B == 2)
+            {
+                if (i == 3)
+                    copyB(kt + 3, (cur + 3) % kTStages, std::integral_constant<int, 1>{});
+            }
             SPH_FENCE();
         }
         // step kt+1 has landed for every wavefront, and every wavefront is done reading
@@ -488,8 +528,9 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
         behindBarrier();
         // second half: rows 64-127, fetch the next step's rows 0-63 and B, request A of kt+4
 #pragma unroll
-        for (int i = 4; i < 8; ++i)
+        for (int i = MB / 2; i < MB; ++i)
         {
+            constexpr int kHalf = MB / 2;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
@@ -497,18 +538,19 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
                     mask(af[i]);
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(BF[j], af[i], acc[i][j], 0, 0, 0);
                 SPH_FENCE();
-                if (i < 6)
+                // the next step's first MB / 2 fragments of A and its 4 of B, one per slot
+                if ((j & 1) == 0)
                 {
-                    if ((j & 1) == 0)
-                        af[2 * (i - 4) + j / 2] = loadA(nxt, 2 * (i - 4) + j / 2);
-                    else
-                        BFN[2 * (i - 4) + j / 2] = loadB(nxt, 2 * (i - 4) + j / 2);
+                    if (i - kHalf < MB / 4)
+                        af[2 * (i - kHalf) + j / 2] = loadA(nxt, 2 * (i - kHalf) + j / 2);
                 }
+                else if (i - kHalf < 2)
+                    BFN[2 * (i - kHalf) + j / 2] = loadB(nxt, 2 * (i - kHalf) + j / 2);
                 SPH_FENCE();
             }
-            if (i == 5)
+            if (i == (MB == 8 ? 5 : 2))
                 copyA(kt + 4, cur, std::integral_constant<int, 0>{});
-            if (i == 7)
+            if (i == (MB == 8 ? 7 : 3))
                 copyA(kt + 4, cur, std::integral_constant<int, 1>{});
             SPH_FENCE();
         }
@@ -529,7 +571,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
         // instruction offset 64*j (added to both addresses) selects the block, so M0 takes it
         // off again.
         const uint32_t mail = LdsAddress(&CMail[0]) + waveU * 4096;
-        const uint32_t cLane0 = ((waveM * 128 + l16) * ldc + waveN * 64 + 4 * g) * 4;
+        const uint32_t cLane0 = ((waveM * WMROWS + l16) * ldc + waveN * 64 + 4 * g) * 4;
         const uint32_t cRowStep = 16 * ldc * 4;
         auto issueC = [&](auto bC) {
             constexpr int i = decltype(bC)::value;
@@ -563,7 +605,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
         // stage copies counted there plus the 4 block copies of step s-1 or s-2, if one of them
         // requested a block; ahead of the wait for block b in step CSP*(b+1) lie the stage
         // copies of the CSP steps since its request.
-        constexpr int kBlocks = 8;
+        constexpr int kBlocks = MB;
         static_assert(CSP >= 2, "at most one request among two consecutive steps");
         auto requestsAt = [](int st) { return st >= 0 && st % CSP == 0 && st / CSP < kBlocks; };
         auto cStep = [&](auto stageC, auto sC) {
@@ -635,12 +677,13 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     {
         // 64 rows x 64 floats per wavefront, 16-byte chunks XOR-swizzled with row % 16 so
         // that neither the column-wise writes nor the row-wise reads pile up on one bank
-        float* stage = reinterpret_cast<float*>(&Lds[0][0][0]) + wave * (64 * 64);
+        float* stage = reinterpret_cast<float*>(LdsRaw) + wave * (64 * 64);
         const uint32_t rdRow = lane >> 4;        // + 4*t
         const uint32_t rdChunk = lane & 15;
-        float* outBlock = out + static_cast<size_t>(waveM * 128 + rdRow) * ldc + waveN * 64 + rdChunk * 4;
+        float* outBlock =
+            out + static_cast<size_t>(waveM * WMROWS + rdRow) * ldc + waveN * 64 + rdChunk * 4;
         const size_t rowStep = static_cast<size_t>(4) * ldc;
-        const uint32_t rowFirst = waveM * 128 + rdRow;
+        const uint32_t rowFirst = waveM * WMROWS + rdRow;
         const bool colExists = !RAGGED || waveN * 64 + rdChunk * 4 < colsLeft;
         auto exists = [&](int half, int t) {
             return !RAGGED || (colExists && rowFirst + 4 * (half * 16 + t) < rowsLeft);
@@ -689,21 +732,28 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
         };
 
         float4 old[16];
+        // (64 rows at a time: twice for a wavefront part of 128 rows)
         if (CLOOP || args.overwrite)
         {
             stageHalf(0);
             storeHalf(0, old, std::false_type{});
-            stageHalf(1);
-            storeHalf(1, old, std::false_type{});
+            if constexpr (MB == 8)
+            {
+                stageHalf(1);
+                storeHalf(1, old, std::false_type{});
+            }
         }
         else
         {
             loadOld(0, old);
             stageHalf(0);
             storeHalf(0, old, std::true_type{});
-            loadOld(1, old);
-            stageHalf(1);
-            storeHalf(1, old, std::true_type{});
+            if constexpr (MB == 8)
+            {
+                loadOld(1, old);
+                stageHalf(1);
+                storeHalf(1, old, std::true_type{});
+            }
         }
     }
 }
@@ -1288,18 +1338,18 @@ typedef halfx8 halfx8a2 __attribute__((aligned(2)));
 
 // variant 0: whole tiles, out read in the epilogue; 1 / 2: out added inside the loop with
 // spacing 2 / 4; 3: ragged tiles
-template <bool TA, bool TB, bool TAIL>
+template <bool TA, bool TB, bool TAIL, int NT>
 void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16Args& args)
 {
     const dim3 g(grid), b(512);
     if (variant == 2)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 4, TA, TB, TAIL>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 4, TA, TB, TAIL, NT>), g, b, 0, stream, args);
     else if (variant == 1)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 2, TA, TB, TAIL>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 2, TA, TB, TAIL, NT>), g, b, 0, stream, args);
     else if (variant == 0)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 0, TA, TB, TAIL>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 0, TA, TB, TAIL, NT>), g, b, 0, stream, args);
     else
-        hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB, TAIL>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB, TAIL, NT>), g, b, 0, stream, args);
 }
 
 // ---------------------------------------------------------------------------
@@ -1541,7 +1591,7 @@ struct F16Layout
     bool transA, transB;
 };
 
-enum class F16Kernel { kTile256, kDma128, kGeneral };
+enum class F16Kernel { kTile256, kTile256x128, kDma128, kGeneral };
 
 // The kernel that would take M x N x K with these operands.  The straight-to-LDS copies take 16
 // bytes from any 2-byte-aligned address, so the rows of a K x N matrix B may start anywhere
@@ -1576,6 +1626,22 @@ F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16
                      (!transA || (M % 8 == 0 && M >= 8));
     if (dma && tiles256 >= minTiles && fills256 && offsetsFit)
         return F16Kernel::kTile256;
+    // Too few 256 x 256 tiles for the chip: 256 x 128 tiles while there are between 11/16 of a
+    // tile and one tile per compute unit.  All three tiled kernels are bound by what a compute
+    // unit's LDS moves per K step (fragment reads plus the copies' writes, about 128 bytes per
+    // clock: 64 KiB for a 128 x 128 step of 256 matrix-core clocks, 88 KiB for a 256 x 128 step of
+    // 512, 128 KiB for a 256 x 256 step of 1024), so the larger tile needs fewer LDS clocks per
+    // flop but only pays once it keeps most of the chip busy (measured, accumulating, 128-tiles
+    // against 256 x 128: 3072 x 2048 x 2048 42.2 / 35.3 us, 2048 x 4096 x 2048 47.3 / 42.0 us;
+    // 2048^3, 128 tiles on half of the compute units, 28.2 / 32.9 us).
+    const uint64_t tilesHalf =
+        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + 127) / 128) * batch;
+    const bool fillsHalf =
+        static_cast<uint64_t>(M) * N * 4 >=
+        static_cast<uint64_t>((M + kT - 1) / kT) * ((N + 127) / 128) * kT * 128 * 3;
+    const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
+    if (dma && tilesHalf * 16 >= cus * 11 && tilesHalf <= cus && fillsHalf && offsetsFit)
+        return F16Kernel::kTile256x128;
     if (dma && static_cast<uint64_t>(M) * (transA ? kTK : args.lda) < (1ull << 31) &&
         static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31) &&
         32ull * args.ldb < (1ull << 30))
@@ -1590,11 +1656,13 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     const uint32_t M = args.M, N = args.N, K = args.K;
     const bool transA = lay.transA, transB = lay.transB;
     const bool plain = !transA && !transB;
-    const bool whole256 = (M % kT == 0) && (N % kT == 0);
-    const bool tile256 = kind == F16Kernel::kTile256;
+    const bool half = kind == F16Kernel::kTile256x128;  // 256 x 128 tiles
+    const bool tile256 = kind == F16Kernel::kTile256 || half;
     const uint32_t edge = tile256 ? kT : kG;
+    const uint32_t edgeN = half ? 128u : edge;
+    const bool whole256 = (M % kT == 0) && (N % edgeN == 0);
     args.tilesM = (M + edge - 1) / edge;
-    args.tilesN = (N + edge - 1) / edge;
+    args.tilesN = (N + edgeN - 1) / edgeN;
     const uint64_t total = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
     SPH_REQUIRE(total < (1ull << 31) - 8, "too many tiles for one launch");
     args.totalTiles = static_cast<uint32_t>(total);
@@ -1605,16 +1673,23 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         // old contents of out added inside the loop: spacing 4 from 36 K steps, 2 from 20
         const bool cloop = whole256 && !args.overwrite;
         const uint32_t ksteps = (K + kTK - 1) / kTK;
-        const int variant = !whole256 ? 3 : (cloop && ksteps >= CLoopSteps(4)) ? 2
-                                          : (cloop && ksteps >= CLoopSteps(2)) ? 1 : 0;
+        const int rowBlocks = half ? 4 : 8;  // per wavefront
+        const int variant = !whole256 ? 3
+                            : (cloop && ksteps >= static_cast<uint32_t>(CLoopSteps(4, rowBlocks))) ? 2
+                            : (cloop && ksteps >= static_cast<uint32_t>(CLoopSteps(2, rowBlocks))) ? 1
+                                                                                                : 0;
         const bool tail = K % kTK != 0;
 #define SPH_TILE256(TA_, TB_)                                                                     \
     do                                                                                            \
     {                                                                                             \
-        if (tail)                                                                                 \
-            LaunchTile256<TA_, TB_, true>(variant, grid, stream, args);                           \
+        if (tail && half)                                                                         \
+            LaunchTile256<TA_, TB_, true, 128>(variant, grid, stream, args);                      \
+        else if (tail)                                                                            \
+            LaunchTile256<TA_, TB_, true, 256>(variant, grid, stream, args);                      \
+        else if (half)                                                                            \
+            LaunchTile256<TA_, TB_, false, 128>(variant, grid, stream, args);                     \
         else                                                                                      \
-            LaunchTile256<TA_, TB_, false>(variant, grid, stream, args);                          \
+            LaunchTile256<TA_, TB_, false, 256>(variant, grid, stream, args);                     \
     } while (0)
         if (transA && transB)
             SPH_TILE256(true, true);
