@@ -1076,6 +1076,281 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
 }
 
 // ---------------------------------------------------------------------------
+// 64 x 64 x 64 kernel with straight-to-LDS copies, ragged M and N
+// ---------------------------------------------------------------------------
+// For products with at most half as many 128 x 128 tiles as compute units.  The tiled kernels
+// are bound by what a compute unit's LDS moves per K step (the copies' writes plus the fragment
+// reads), so a product that gives only a quarter of the compute units a 128-tile uses a quarter
+// of the chip's LDS bandwidth; 64 x 64 tiles move half as many more bytes through LDS per flop
+// but spread them over four times as many compute units (1024^3: 10.8 us on 64 tiles of 128).
+// Four wavefronts (2 x 2), one 32 x 32 block of v_mfma_f32_32x32x16_f16 each; K advances 64 at
+// a time, so that a row of a K-contiguous operand is one whole 128-byte line per step; four
+// stages of 16 KiB, so two workgroups share a compute unit.
+// K-contiguous operand (A as given, B stored N x K): 64 rows of 128 bytes, 16-byte chunk c of
+// row x at position c ^ ((x >> 1) & 7): 16 consecutive rows reading one chunk touch every bank
+// once.  k-major operand (B as given, A stored K x M): 64 k-rows of 128 bytes, the two 64-byte
+// halves of k-row k swapped when (k >> 1) & 1, so that the four k-rows a transposing read
+// serves in one clock (64 bytes each) cover the 64 banks.
+// TAIL: K = 64 q + r, 0 < r < 64, K >= 64: a last step over the window [K - 64, K) whose slab has
+// the positions of the 64 - r values of k already multiplied cleared in LDS.
+constexpr int kS = 64;         // tile edge
+constexpr int kSK = 64;        // K step
+constexpr int kSStages = 4;
+constexpr int kSOperandBytes = kS * kSK * 2;        // 8 KiB
+constexpr int kSStageBytes = 2 * kSOperandBytes;    // A + B
+
+template <bool TA, bool TB, bool TAIL>
+__global__ __launch_bounds__(256) void GemmF16Dma64(const GemmF16Args args)
+{
+    constexpr int kCopiesPer = 2;            // 1 KiB copies per operand, step and wavefront
+    constexpr int kCopies = 2 * kCopiesPer;  // per step and wavefront
+    __shared__ __attribute__((aligned(1024))) char lds[kSStages * kSStageBytes];
+
+    uint32_t unit, tm, tn;
+    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
+        return;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t waveM = wave >> 1;
+    const uint32_t waveN = wave & 1;
+    const uint32_t M = args.M, N = args.N, K = args.K;
+
+    const _Float16* A = args.A + args.strideA * static_cast<int64_t>(unit);
+    const _Float16* B = args.B + args.strideB * static_cast<int64_t>(unit);
+    float* __restrict__ out = args.out + args.strideOut * static_cast<int64_t>(unit);
+    const uint32_t rowBase = tm * kS;
+    const uint32_t colBase = tn * kS;
+
+    // ---- copy plan: copy j of an operand (j = wave, wave + 4) covers LDS bytes j*1024 .. -----
+    // K-contiguous: 8 rows per copy; lane -> x = 8 j + lane / 8, physical chunk lane % 8.
+    auto laneKContig = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t pitch) {
+        const uint32_t x = j * 8 + (lane >> 3);
+        const uint32_t c = (lane & 7) ^ ((x >> 1) & 7);
+        const uint32_t gx = min(xBase + x, limit - 1);
+        return (gx * pitch + c * 8) * 2u;
+    };
+    // k-major: 8 k-rows per copy; lane -> k = 8 j + lane / 8, physical 16-byte chunk lane % 8 of
+    // which bit 2 (the 64-byte half) is swapped for k-rows with (k >> 1) & 1.
+    auto laneKMajor = [&](uint32_t j, uint32_t xBase, uint32_t limit, uint32_t pitch) {
+        const uint32_t k = j * 8 + (lane >> 3);
+        const uint32_t logical16 = (lane & 7) ^ (((k >> 1) & 1) << 2);
+        const uint32_t gx = min(xBase + logical16 * 8, limit - 8);
+        return (k * pitch + gx) * 2u;
+    };
+    const uint32_t pitchB = TB ? K : args.ldb;
+    uint32_t aLane[kCopiesPer], bLane[kCopiesPer], aDst[kCopiesPer], bDst[kCopiesPer];
+#pragma unroll
+    for (uint32_t i = 0; i < kCopiesPer; ++i)
+    {
+        const uint32_t j = wave + 4 * i;
+        aLane[i] = TA ? laneKMajor(j, rowBase, M, args.lda) : laneKContig(j, rowBase, M, args.lda);
+        bLane[i] = TB ? laneKContig(j, colBase, N, pitchB) : laneKMajor(j, colBase, N, pitchB);
+        aDst[i] = j * 1024;
+        bDst[i] = kSOperandBytes + j * 1024;
+    }
+    const size_t aStepBytes = TA ? static_cast<size_t>(kSK) * args.lda * 2 : kSK * 2;
+    const size_t bStepBytes = TB ? kSK * 2 : static_cast<size_t>(kSK) * pitchB * 2;
+    const uint32_t ldsBase = LdsAddress(lds);
+    const uint32_t steps = TAIL ? K / kSK + 1 : K / kSK;
+    // the last window starts K % 64 values of k after the one before it
+    const uint32_t kLast = K % kSK;
+    const size_t aLastBytes = TA ? static_cast<size_t>(kLast) * args.lda * 2 : kLast * 2;
+    const size_t bLastBytes = TB ? kLast * 2 : static_cast<size_t>(kLast) * pitchB * 2;
+    // Copy n (0, 1: A; 2, 3: B) of the next step to fetch, into stage `stage`.  Surplus steps
+    // re-fetch the last slab into a stage nobody reads any more, which keeps the number of
+    // outstanding copies the same in every step.
+    const char* aSrc = reinterpret_cast<const char*>(A);
+    const char* bSrc = reinterpret_cast<const char*>(B);
+    uint32_t stepsToAdvance = steps - 1;
+    auto issueOne = [&](uint32_t stage, uint32_t n) {
+        const uint32_t base = ldsBase + stage * kSStageBytes;
+        if (n < kCopiesPer)
+            DmaToLds16<0>(aLane[n], aSrc, base + aDst[n]);
+        else
+            DmaToLds16<0>(bLane[n - kCopiesPer], bSrc, base + bDst[n - kCopiesPer]);
+    };
+    auto advance = [&]() {
+        if (stepsToAdvance != 0)
+        {
+            size_t aBytes = aStepBytes, bBytes = bStepBytes;
+            if (TAIL && stepsToAdvance == 1)
+            {
+                aBytes = aLastBytes;
+                bBytes = bLastBytes;
+            }
+            aSrc += aBytes;
+            bSrc += bBytes;
+            --stepsToAdvance;
+        }
+    };
+
+    // ---- fragment plan: ks = 0..3, k = 16 ks + 8 khalf .. + 7 ---------------------------------
+    const uint32_t l32 = lane & 31;
+    const uint32_t khalf = lane >> 5;
+    const uint32_t g = lane >> 4;
+    const uint32_t s = lane & 15;
+    auto offKContig = [&](int ks, uint32_t x) {
+        return x * 128 + (((ks * 2 + khalf) ^ ((x >> 1) & 7)) << 4);
+    };
+    // 32 columns (or rows of a transposed A) from `half` * 32 on: lanes of g & 1 take the
+    // second 16 of them; the second read of a fragment is 4 k-rows further on
+    auto offKMajor = [&](int ks, uint32_t half) {
+        const uint32_t k = ks * 16 + 8 * (g >> 1) + (s >> 2);
+        return k * 128 + ((half ^ ((k >> 1) & 1)) << 6) + ((g & 1) << 5) + (s & 3) * 8;
+    };
+    uint32_t aOff[4], bOff[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+    {
+        aOff[ks] = TA ? offKMajor(ks, waveM) : offKContig(ks, waveM * 32 + l32);
+        bOff[ks] = kSOperandBytes + (TB ? offKContig(ks, waveN * 32 + l32) : offKMajor(ks, waveN));
+    }
+    auto readKContig = [&](const char* p) { return *reinterpret_cast<const halfx8*>(p); };
+    auto readKMajor = [&](const char* p) {
+        // the second read takes the k-rows 4 further on, whose halves are swapped alike
+        const _Float16* h = reinterpret_cast<const _Float16*>(p);
+        return Join(LdsReadTr(h), LdsReadTr(h + 4 * 64));
+    };
+    auto loadA = [&](const char* stage, int ks) {
+        if constexpr (TA)
+            return readKMajor(stage + aOff[ks]);
+        else
+            return readKContig(stage + aOff[ks]);
+    };
+    auto loadB = [&](const char* stage, int ks) {
+        if constexpr (TB)
+            return readKContig(stage + bOff[ks]);
+        else
+            return readKMajor(stage + bOff[ks]);
+    };
+
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+        acc[v] = 0.f;
+
+    // TAIL: the positions of the last slab whose k the step before has multiplied are cleared
+    // in LDS, by the lane that copied them, once the copies have landed and before the barrier
+    // that publishes the stage.
+    auto clearRepeated = [&](char* stage) {
+        const uint32_t repeated = kSK - K % kSK;
+#pragma unroll
+        for (uint32_t i = 0; i < kCopiesPer; ++i)
+        {
+            const uint32_t j = wave + 4 * i;
+            const uint32_t row = j * 8 + (lane >> 3);  // x of a K-contiguous slab, k of a k-major one
+            const uint32_t c = (lane & 7) ^ ((row >> 1) & 7);
+            const uintx4 contig = TailMask(c, repeated);
+            const uint32_t keepAll = row < repeated ? 0u : ~0u;
+            const uintx4 major = { keepAll, keepAll, keepAll, keepAll };
+            uintx4* a = reinterpret_cast<uintx4*>(stage + j * 1024 + lane * 16);
+            uintx4* b = reinterpret_cast<uintx4*>(stage + kSOperandBytes + j * 1024 + lane * 16);
+            *a = *a & (TA ? major : contig);
+            *b = *b & (TB ? contig : major);
+        }
+    };
+
+#pragma unroll
+    for (uint32_t p = 0; p < kSStages - 1; ++p)
+    {
+#pragma unroll
+        for (uint32_t n = 0; n < kCopies; ++n)
+            issueOne(p, n);
+        advance();
+    }
+    halfx8 af[2][4], bf[2][4];
+    WaitVmem<(kSStages - 2) * kCopies>();
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+    {
+        af[0][ks] = loadA(lds, ks);
+        bf[0][ks] = loadB(lds, ks);
+    }
+
+    // One step with the stage known at compile time: the fragments of step st are in set P;
+    // behind the first matrix instruction the wait for the copies of step st + 1 and the
+    // barrier, behind each one a copy of step st + 3; the fragments of step st + 1 are read
+    // into set Q from the stage the barrier has just published.
+    auto step = [&](auto uC, uint32_t st, halfx8 (&PA)[4], halfx8 (&PB)[4], halfx8 (&QA)[4],
+                    halfx8 (&QB)[4]) {
+        constexpr uint32_t u = decltype(uC)::value;
+        char* next = lds + ((u + 1) % kSStages) * kSStageBytes;
+        const uint32_t fill = (u + kSStages - 1) % kSStages;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+        {
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(PB[ks], PA[ks], acc, 0, 0, 0);
+            if (ks == 0)
+            {
+                WaitVmem<(kSStages - 3) * kCopies>();
+                if constexpr (TAIL)
+                {
+                    if (st + 2 == steps)
+                    {
+                        clearRepeated(next);
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    }
+                }
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
+            issueOne(fill, ks);
+            if (ks == 3)
+                advance();
+            __builtin_amdgcn_sched_barrier(0);
+            QA[ks] = loadA(next, ks);
+            QB[ks] = loadB(next, ks);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (uint32_t s0 = 0; s0 < steps; s0 += kSStages)
+    {
+        step(std::integral_constant<uint32_t, 0>{}, s0, af[0], bf[0], af[1], bf[1]);
+        if (s0 + 1 >= steps)
+            break;
+        step(std::integral_constant<uint32_t, 1>{}, s0 + 1, af[1], bf[1], af[0], bf[0]);
+        if (s0 + 2 >= steps)
+            break;
+        step(std::integral_constant<uint32_t, 2>{}, s0 + 2, af[0], bf[0], af[1], bf[1]);
+        if (s0 + 3 >= steps)
+            break;
+        step(std::integral_constant<uint32_t, 3>{}, s0 + 3, af[1], bf[1], af[0], bf[0]);
+    }
+    WaitVmem<0>();  // the surplus copies of the last steps still target LDS
+
+    // ---- epilogue: lane holds row l % 32 of its block, columns 8 q + 4 (l / 32) + 0..3 ----------
+    const bool accumulate = args.overwrite == 0;
+    const uint32_t r = rowBase + waveM * 32 + l32;
+    float4 old[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+    {
+        const uint32_t c = colBase + waveN * 32 + 8 * q + 4 * khalf;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (accumulate && r < M && c < N)  // N % 8 == 0: whole quads only
+            v = Load4(out + static_cast<size_t>(r) * args.ldc + c);
+        old[q] = v;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+    {
+        const uint32_t c = colBase + waveN * 32 + 8 * q + 4 * khalf;
+        if (r < M && c < N)
+        {
+            float4 v = old[q];
+            v.x += acc[4 * q + 0];
+            v.y += acc[4 * q + 1];
+            v.z += acc[4 * q + 2];
+            v.w += acc[4 * q + 3];
+            Store4(out + static_cast<size_t>(r) * args.ldc + c, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // general kernel: 128 x 128 x 32, any shape
 // ---------------------------------------------------------------------------
 constexpr int kG = 128;
@@ -1591,7 +1866,7 @@ struct F16Layout
     bool transA, transB;
 };
 
-enum class F16Kernel { kTile256, kTile256x128, kDma128, kGeneral };
+enum class F16Kernel { kTile256, kTile256x128, kDma64, kDma128, kGeneral };
 
 // The kernel that would take M x N x K with these operands.  The straight-to-LDS copies take 16
 // bytes from any 2-byte-aligned address, so the rows of a K x N matrix B may start anywhere
@@ -1642,9 +1917,15 @@ F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16
     const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
     if (dma && tilesHalf * 16 >= cus * 11 && tilesHalf <= cus && fillsHalf && offsetsFit)
         return F16Kernel::kTile256x128;
-    if (dma && static_cast<uint64_t>(M) * (transA ? kTK : args.lda) < (1ull << 31) &&
-        static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31) &&
-        32ull * args.ldb < (1ull << 30))
+    const bool offsets128Fit = static_cast<uint64_t>(M) * (transA ? kTK : args.lda) < (1ull << 31) &&
+                               static_cast<uint64_t>(N) * (transB ? K : kTK) < (1ull << 31) &&
+                               32ull * args.ldb < (1ull << 30);
+    // at most half as many 128-tiles as compute units: 64 x 64 tiles with K steps of 64
+    const uint64_t tiles128 =
+        static_cast<uint64_t>((M + kG - 1) / kG) * ((N + kG - 1) / kG) * batch;
+    if (dma && offsets128Fit && K >= kSK && tiles128 <= cus / 2)
+        return F16Kernel::kDma64;
+    if (dma && offsets128Fit)
         return F16Kernel::kDma128;
     return F16Kernel::kGeneral;
 }
@@ -1700,6 +1981,33 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         else
             SPH_TILE256(false, false);
 #undef SPH_TILE256
+    }
+    else if (kind == F16Kernel::kDma64)
+    {
+        args.tilesM = (M + kS - 1) / kS;
+        args.tilesN = (N + kS - 1) / kS;
+        const uint64_t tiles = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
+        SPH_REQUIRE(tiles < (1ull << 31) - 8, "too many tiles for one launch");
+        args.totalTiles = static_cast<uint32_t>(tiles);
+        const dim3 g(((args.totalTiles + 7) / 8) * 8), b(256);
+        const bool tail = K % kSK != 0;
+#define SPH_DMA64(TA_, TB_)                                                                       \
+    do                                                                                            \
+    {                                                                                             \
+        if (tail)                                                                                 \
+            hipLaunchKernelGGL((GemmF16Dma64<TA_, TB_, true>), g, b, 0, stream, args);            \
+        else                                                                                      \
+            hipLaunchKernelGGL((GemmF16Dma64<TA_, TB_, false>), g, b, 0, stream, args);           \
+    } while (0)
+        if (transA && transB)
+            SPH_DMA64(true, true);
+        else if (transA)
+            SPH_DMA64(true, false);
+        else if (transB)
+            SPH_DMA64(false, true);
+        else
+            SPH_DMA64(false, false);
+#undef SPH_DMA64
     }
     else if (kind == F16Kernel::kDma128)
     {
@@ -1866,18 +2174,25 @@ void LaunchFew(const GemmF16Args& args, uint32_t blocks, uint32_t tile, bool wid
 
 // Products with at most one 32 x 32 output tile per compute unit, and narrow ones (16 rows or
 // columns at most) with up to four 16 x 16 tiles per compute unit, run on the few-tile kernel,
-// whatever their storage flags and alignment: the decision looks at M, N and the batch only, so
-// one product always takes the same kernel and sums in the same order.  Measured against the
+// whatever their storage flags and alignment: the decision looks at M, N, K and the batch only,
+// so one product always takes the same kernel and sums in the same order.  Measured against the
 // 128-tile kernel (us, plain / A stored K x M / B stored N x K): 256 x 1024 x 1024 6.5 / 7.0 /
 // 7.3 against 10.6 / 11.7 / 10.3, 512^3 5.2 against 8.5, 100 x 1024 x 784 5.4 against 10.4,
 // 1024 x 10 x 1024 4.5 against 12.5, 16384 x 10 x 256 4.6 against 11.9; with two tiles per
 // compute unit (512 x 1024 x 1024) the two are level, with four the tiled kernel wins.
-bool TakesFewTiles(uint32_t M, uint32_t N, uint32_t batch)
+// A product that the 64 x 64-tile kernel takes whole whatever its storage flags (M and N multiples
+// of 8, K >= 64) goes there from half a 32-tile per compute unit up (measured, few-tile kernel
+// against 64-tiles: 256 x 1024 x 1024 6.5 / 5.8 us, 256 x 512 x 2048 8.9 / 7.6, 128 x 1024 x 1024
+// 6.4 / 5.7; below that the few-tile kernel wins: 256^3 3.6 / 4.2, 64 x 1024 x 1024 4.8 / 5.7,
+// 256 x 256 x 4096 11.0 / 11.4).
+bool TakesFewTiles(uint32_t M, uint32_t N, uint32_t K, uint32_t batch)
 {
     const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
     const uint64_t blocks32 = static_cast<uint64_t>((M + 31) / 32) * ((N + 31) / 32) * batch;
     const uint64_t blocks16 = static_cast<uint64_t>((M + 15) / 16) * ((N + 15) / 16) * batch;
-    return blocks32 <= cus || (std::min(M, N) <= 16 && blocks16 <= 4 * cus);
+    const bool tiles64Whole = M % 8 == 0 && N % 8 == 0 && K >= 64;
+    const uint64_t limit32 = tiles64Whole ? cus / 2 - 1 : cus;
+    return blocks32 <= limit32 || (std::min(M, N) <= 16 && blocks16 <= 4 * cus);
 }
 
 int LaunchFewTiles(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream)
@@ -1964,7 +2279,7 @@ int sph_gemm_f16f32(float* out, const sph_f16* A, const sph_f16* B, uint32_t M, 
     args.strideB = strideB;
     args.overwrite = (flags & SPH_GEMM_OVERWRITE) ? 1u : 0u;
 
-    if (TakesFewTiles(M, N, batch))
+    if (TakesFewTiles(M, N, K, batch))
         return LaunchFewTiles(args, batch, lay, stream);
     return LaunchF16(args, batch, lay, stream);
 }

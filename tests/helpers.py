@@ -158,10 +158,15 @@ def f32_k_split_range(M, N, K, batch=1):
 F16_FEW_TILE_CUS = 256
 
 
-def f16_few_tiles(M, N, batch):
+def f16_few_tiles(M, N, batch, K=None):
+    """Whether the few-tile kernel takes the product.  With K the exact rule; without it the
+    wider one (every product this says no to runs on the tiled kernels whatever its K)."""
     b32 = -(-M // 32) * -(-N // 32) * batch
     b16 = -(-M // 16) * -(-N // 16) * batch
-    return b32 <= F16_FEW_TILE_CUS or (min(M, N) <= 16 and b16 <= 4 * F16_FEW_TILE_CUS)
+    limit = F16_FEW_TILE_CUS
+    if K is not None and M % 8 == 0 and N % 8 == 0 and K >= 64:
+        limit = F16_FEW_TILE_CUS // 2 - 1     # the 64 x 64-tile kernel takes these from here up
+    return b32 <= limit or (min(M, N) <= 16 and b16 <= 4 * F16_FEW_TILE_CUS)
 
 
 def f16_both_kernel_families(shapes):

@@ -273,14 +273,15 @@ def test_transposed_a_with_ragged_rows_and_columns(dev, shape, flags):
 # order, with guard floats behind every unit of out.
 @pytest.mark.parametrize("flags", [0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B,
                                    capi.SPH_GEMM_TRANS_A | capi.SPH_GEMM_TRANS_B])
-@pytest.mark.parametrize("shape", [(256, 1024, 1024, 1), (100, 1024, 784, 1), (300, 300, 300, 1),
+@pytest.mark.parametrize("shape", [(252, 1020, 1024, 1), (100, 1024, 784, 1), (300, 300, 300, 1),
+                                   (500, 500, 300, 1), (96, 1024, 1024, 1),
                                    (128, 128, 4096, 1), (64, 64, 8203, 1), (33, 47, 5, 1),
                                    (17, 16, 31, 2), (1, 1000, 37, 1), (1000, 1, 1029, 1),
-                                   (255, 257, 1031, 1), (512, 512, 515, 1), (96, 80, 1040, 3),
+                                   (255, 257, 1031, 1), (508, 510, 515, 1), (96, 80, 1040, 3),
                                    (2048, 10, 300, 1), (16, 4000, 64, 1)])
 def test_few_tile_kernel_exact_on_integers(dev, shape, flags):
     M, N, K, batch = shape
-    assert h.f16_few_tiles(M, N, batch)
+    assert h.f16_few_tiles(M, N, batch, K)
     h.announce("sph_gemm_f16f32 few-tile kernel", shape, "flags", flags)
     A = synth.small_integers(91, (batch, M, K), span=3).astype(np.float16)
     B = synth.small_integers(92, (batch, K, N), span=3).astype(np.float16)
