@@ -65,8 +65,15 @@ def parse():
                    help="also time the neighbouring kernels (backward pass, conversions, CSR x "
                         "CSR, one-pass kernels; reported under 'others')")
     p.add_argument("--only", choices=["gemm", "gemm_operator", "spmm", "copy", "backward", "backward_reference", "gemm_f32",
-                                      "csr", "spgemm", "shapes", "mfma_ceiling"], default=None,
+                                      "csr", "spgemm", "shapes", "mfma_ceiling", "one"], default=None,
                    help="run a single kernel (for profiler runs); the JSON line is reduced")
+    p.add_argument("--dims", type=int, nargs=3, metavar=("M", "N", "K"), default=[1024, 1024, 1024],
+                   help="with --only one: the product to time")
+    p.add_argument("--f32", action="store_true",
+                   help="with --only one: sph_gemm_f32_ex instead of sph_gemm_f16f32")
+    p.add_argument("--flags", type=int, default=0,
+                   help="with --only one: SPH_GEMM_* flags of the call (1 overwrite, 2 A stored "
+                        "K x M, 4 B stored N x K)")
     p.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                    help="untimed run-up before each timed leg that lets the clock reach its "
                         "working frequency (0 = none)")
@@ -434,10 +441,12 @@ def bench_mlp_backward(capi, synth, steps, warmup, direct, graph=False, fused_up
 SMALL = [(256, 1024, 1024), (100, 1024, 784), (1024, 10, 1024), (128, 128, 4096), (512, 1024, 1024)]
 OFF_GRID_F16 = [(4096, 4096, 4096), (4096, 4096, 4080), (4096, 4096, 4095), (4096, 4100, 4096),
                 (4096, 4095, 4096), (4095, 4095, 4095), (2048, 2052, 2048), (1024, 1024, 1001),
-                (1024, 1024, 1024)] + SMALL
+                (1024, 1024, 1024), (1024, 1024, 4096), (2048, 2048, 2048), (3072, 2048, 2048),
+                (2048, 4096, 2048), (1025, 1025, 1025)] + SMALL
 OFF_GRID_F32 = [(1024, 1024, 1024), (1024, 1024, 1000), (1024, 1024, 1001), (1000, 1000, 1000),
                 (1001, 1001, 1001), (1024, 1026, 1024), (2048, 2048, 2047), (2048, 2050, 2048),
-                (4096, 4096, 4096), (4096, 4095, 4096), (4096, 4096, 4100)] + SMALL
+                (4096, 4096, 4096), (4096, 4095, 4096), (4096, 4096, 4100), (1025, 1025, 1025),
+                (8192, 65, 64), (384, 1024, 1024)] + SMALL
 
 
 def bench_off_grid(capi, synth, steps, warmup):
@@ -471,6 +480,30 @@ def bench_off_grid(capi, synth, steps, warmup):
         for flags in (0, capi.SPH_GEMM_TRANS_A, capi.SPH_GEMM_TRANS_B):
             one("sph_gemm_f32_ex", M, N, K, flags, A, B)
     return rows
+
+
+def bench_one(capi, synth, M, N, K, f32, flags, steps, warmup):
+    """One M x N x K product (operands as for --only shapes), for profiler runs of one kernel."""
+    entry = "sph_gemm_f32_ex" if f32 else "sph_gemm_f16f32"
+    if f32:
+        A, B = synth.uniform(1, (M, K)), synth.uniform(2, (K, N))
+    else:
+        A = synth.normal(1, (M, K), 1.0 / np.sqrt(K)).astype(np.float16)
+        B = synth.normal(2, (K, N), 1.0 / np.sqrt(K)).astype(np.float16)
+    C = np.zeros((M, N), np.float32)
+    dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (A, B, C))
+    capi.require_gemm_extents(dC, dA, dB, M, N, K, 1, M * N, M * K, K * N,
+                              operand_bytes=4 if f32 else 2)
+
+    def launch():
+        capi.call(entry, dC.ptr, dA.ptr, dB.ptr, M, N, K, 1, M * N, M * K, K * N, flags)
+
+    ms, _ = timed_launches(capi, launch, steps, warmup)
+    for d in (dA, dB, dC):
+        d.release()
+    tf = 2.0 * M * N * K / (ms * 1e-3) / 1e12
+    return {"entry_point": entry, "M": M, "N": N, "K": K, "flags": flags, "launch_ms": ms,
+            "tflops": tf, "frac_of_peak": tf / (PEAK_FP32_TFLOPS if f32 else PEAK_FP16_TFLOPS)}
 
 
 def bench_sgd_step(capi, steps, warmup, mib=64):
@@ -894,6 +927,11 @@ def main():
 
     if args.only == "shapes":
         result["off_grid_shapes"] = bench_off_grid(capi, synth, min(args.steps, 20), 3)
+
+    if args.only == "one":
+        M, N, K = args.dims
+        result["one"] = bench_one(capi, synth, M, N, K, args.f32, args.flags, args.steps,
+                                  args.warmup)
 
     if args.only == "csr":
         ms_csr, ms_one, ms_dense, dense_bytes, csr_bytes = bench_csr_conversion(
