@@ -80,6 +80,12 @@ int sph_free(void* ptr);                               /* Memory.cpp:38-44 */
 int sph_malloc_async(void** ptr, size_t bytes);
 int sph_free_async(void* ptr);
 int sph_mem_pool_trim(void);
+/* Number of device and pinned-host allocations the library has made in this
+ * process so far (hipMalloc, hipMallocAsync, hipHostMalloc: the caller's own
+ * sph_malloc* calls and the library's internal scratch blocks and tables).  No
+ * counterpart in the reference.  For callers that must show that a call
+ * allocates nothing: read it before and after. */
+int sph_allocation_count(uint64_t* count);
 int sph_memcpy_h2d(void* dev, const void* host, size_t bytes); /* :46-53 */
 int sph_memcpy_d2h(void* host, const void* dev, size_t bytes); /* :55-63 */
 int sph_memcpy_d2d(void* dst, const void* src, size_t bytes);  /* :65-72 */
@@ -102,7 +108,11 @@ int sph_stream_wait_stream(void* hipStream);
 /* The hipStream_t this thread's calls run on (created on first use). */
 int sph_get_stream(void** hipStream);
 /* Run this thread's later calls on a caller-owned hipStream_t; NULL returns
- * to the library's own stream. */
+ * to the library's own stream.  The stream must outlive every buffer that was
+ * used on it and is still held by a pool above this library (the C++ layer's
+ * ResourceManager remembers the stream a block was last used on and makes the
+ * next user wait for it): drain the stream and release or ClearAll() such
+ * pools before destroying it. */
 int sph_set_stream(void* hipStream);
 
 /* Events on this thread's stream, for timing launches from a host language

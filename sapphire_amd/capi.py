@@ -65,6 +65,7 @@ SIGNATURES = {
     "sph_malloc_async": [ctypes.POINTER(_vp), _sz],
     "sph_free_async": [_vp],
     "sph_mem_pool_trim": [],
+    "sph_allocation_count": [ctypes.POINTER(ctypes.c_uint64)],
     "sph_memcpy_h2d": [_vp, _vp, _sz],
     "sph_memcpy_d2h": [_vp, _vp, _sz],
     "sph_memcpy_d2d": [_vp, _vp, _sz],

@@ -631,6 +631,7 @@ int ExclusiveScanInPlace(uint32_t* data, uint32_t n, uint32_t* lastHost, hipStre
         // per-block totals: the caller's workspace, or a stream-ordered scratch allocation
         const bool own = sums == nullptr;
         if (own)
+            ::sph::CountAllocation();
             SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&sums),
                                        blocks * sizeof(uint32_t), stream));
         hipLaunchKernelGGL(ScanBlocksKernel, dim3(blocks), dim3(kScanThreads), 0, stream, data,
@@ -758,6 +759,7 @@ int sph_csr_from_dense_f32(float* V, uint32_t* COL, uint32_t* ROW, uint32_t capa
     const uint32_t stage = static_cast<uint32_t>(stage64);
     const size_t stageEntries = static_cast<size_t>(M) * stage;
     float* stageV = nullptr;
+    ::sph::CountAllocation();
     SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&stageV), stageEntries * 8, stream));
     uint32_t* stageCol = reinterpret_cast<uint32_t*>(stageV + stageEntries);
     const uint32_t rowsPerGroup = kStageWaves / wpr;
@@ -913,6 +915,7 @@ int sph_csr_validate_u32(const uint32_t* COL, const uint32_t* ROW, uint32_t M, u
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
     uint32_t* problems = nullptr;
+    ::sph::CountAllocation();
     SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&problems), sizeof(uint32_t), stream));
     SPH_HIP_TRY(hipMemsetAsync(problems, 0, sizeof(uint32_t), stream));
     const uint64_t items = std::max<uint64_t>(std::max<uint64_t>(M, nnz), 1);

@@ -1804,6 +1804,8 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         args.tilesM = (args.M + tile - 1) / tile;
         args.tilesN = (args.N + tile - 1) / tile;
         const uint64_t blocks = static_cast<uint64_t>(args.tilesM) * args.tilesN * units;
+        if (blocks >= (1ull << 31))
+            return sph::Fail(SPH_ERR_INVALID, "sph_gemm_f32 - too many tiles for one launch");
         const dim3 gridSkinny(static_cast<uint32_t>(blocks));
         const bool wide = tile == 16 && blocks <= static_cast<uint64_t>(sph::ComputeUnits()) &&
                           args.K >= 512;
@@ -1911,7 +1913,9 @@ int GrowTable(EntryTable& t, size_t count)
     size_t cap = 1024;
     while (cap < count)
         cap *= 2;
+    ::sph::CountAllocation();
     SPH_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&t.dev), cap * sizeof(SphGemmEntry)));
+    ::sph::CountAllocation();
     SPH_HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&t.staging), cap * sizeof(SphGemmEntry),
                               hipHostMallocDefault));
     if (t.uploaded == nullptr)

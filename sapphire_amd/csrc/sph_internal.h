@@ -41,6 +41,10 @@ bool ScanWaitsOrAllocates(uint32_t n, const uint32_t* lastHost);
 // sph_csr_row_offsets_noalloc_f32 on the calling thread's device.
 int ResolveCsrScratch(uint32_t** scratch);
 
+// Counts one device or pinned-host allocation made by the library (read back through
+// sph_allocation_count); called next to every hipMalloc / hipMallocAsync / hipHostMalloc.
+void CountAllocation();
+
 // True between sph_graph_begin_capture and sph_graph_end_capture on this thread.  Entry
 // points that must wait for the device or allocate refuse to run while it is set.
 bool Capturing();

@@ -8,6 +8,8 @@
 // ends, so no stream is destroyed while the runtime may be shutting down.
 #include "sph_internal.h"
 
+#include <atomic>
+
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -42,8 +44,18 @@ struct ThreadSlots
 thread_local ThreadSlots tlsSlots;
 }  // namespace
 
+namespace
+{
+std::atomic<uint64_t> gAllocations{0};
+}
+
 namespace sph
 {
+void CountAllocation()
+{
+    gAllocations.fetch_add(1, std::memory_order_relaxed);
+}
+
 int Fail(int status, const std::string& msg)
 {
     tlsLastError = msg;
@@ -183,6 +195,7 @@ int sph_malloc(void** ptr, size_t bytes)
     SPH_REFUSE_WHILE_CAPTURING();
     SPH_REQUIRE(ptr != nullptr, "ptr is null");
     SPH_HIP_TRY(hipSetDevice(tlsSlots.device));
+    ::sph::CountAllocation();
     SPH_HIP_TRY(hipMalloc(ptr, bytes));
     return SPH_OK;
 }
@@ -212,6 +225,7 @@ int sph_malloc_async(void** ptr, size_t bytes)
             gPoolRetains[d] = true;
         }
     }
+    ::sph::CountAllocation();
     SPH_HIP_TRY(hipMallocAsync(ptr, bytes != 0 ? bytes : 1, stream));
     return SPH_OK;
 }
@@ -223,6 +237,13 @@ int sph_free_async(void* ptr)
         return SPH_OK;
     SPH_STREAM_OR_FAIL(stream);
     SPH_HIP_TRY(hipFreeAsync(ptr, stream));
+    return SPH_OK;
+}
+
+int sph_allocation_count(uint64_t* count)
+{
+    SPH_REQUIRE(count != nullptr, "count is null");
+    *count = gAllocations.load(std::memory_order_relaxed);
     return SPH_OK;
 }
 
@@ -239,6 +260,7 @@ int sph_host_malloc(void** ptr, size_t bytes)
 {
     SPH_REFUSE_WHILE_CAPTURING();
     SPH_REQUIRE(ptr != nullptr, "ptr is null");
+    ::sph::CountAllocation();
     SPH_HIP_TRY(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
     return SPH_OK;
 }

@@ -837,6 +837,7 @@ int sph_spgemm_load_u32(uint32_t* load, const uint32_t* COLA, const uint32_t* RO
     unsigned long long* total = nullptr;
     if (productsHost != nullptr)
     {
+        ::sph::CountAllocation();
         SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&total), sizeof(*total), stream));
         hipLaunchKernelGGL(ClearTotalKernel, dim3(1), dim3(1), 0, stream, total);
     }
@@ -899,6 +900,7 @@ int sph_spgemm_f32(float* VC, uint32_t* COLC, uint32_t* ROWC, uint32_t capacity,
     float* stageV = nullptr;
     if (staged)
     {
+        ::sph::CountAllocation();
         SPH_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&stageV), slot * M * 8 + 4, stream));
         args.VC = stageV;
         args.COLC = reinterpret_cast<uint32_t*>(stageV + slot * M);

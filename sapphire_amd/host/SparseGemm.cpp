@@ -144,10 +144,30 @@ void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cu
     try
     {
         // The number of products of a pair bounds the entries of its result; with room for that
-        // many the products are computed once (the counting pass stages every row).  All
-        // products are enqueued before any entry count is read back, so the stream is drained
-        // once for the batch and not once per matrix.
+        // many the products are computed once (the counting pass stages every row).  Reading
+        // that bound back drains the stream once per matrix (a small kernel each); the products
+        // themselves are all enqueued before any entry count is read back, so they cost one
+        // more drain for the whole batch.  When the arrays for the bound (or the staging area
+        // behind sph_spgemm_f32, 8 bytes per bounded entry and more) cannot be had, the matrix
+        // falls back to the two passes: count, allocate exactly, fill.
         std::vector<uint32_t> capacity(count);
+        std::vector<bool> exact(count, false);
+        auto twoPasses = [&](uint32_t i) {
+            const SparseMatrix& a = cudaA[i];
+            const SparseMatrix& b = cudaB[i];
+            SparseMatrix& c = result[i];
+            uint32_t nnz = 0;
+            check(sph_spgemm_row_offsets_f32(c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m, a.N,
+                                             n, &nnz));
+            const std::size_t exactBytes = std::max<std::size_t>(nnz, 1) * 4;
+            c.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(exactBytes, true));
+            c.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(exactBytes, true));
+            check(sph_spgemm_fill_f32(c.V, c.COL, c.ROW, a.V, a.COL, a.ROW, b.V, b.COL, b.ROW, m,
+                                      a.N, n));
+            c.NNZ = nnz;
+            capacity[i] = nnz;
+            exact[i] = true;
+        };
         for (uint32_t i = 0; i < count; ++i)
         {
             const SparseMatrix& a = cudaA[i];
@@ -169,14 +189,34 @@ void Gemm(SparseMatrix** hostOutput, SparseMatrix** cudaOutput, SparseMatrix* cu
             c.ROW = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(
                 (static_cast<std::size_t>(m) + 1) * 4, true));
             const std::size_t bytes = std::max<std::size_t>(capacity[i], 1) * 4;
-            c.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
-            c.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
-            check(sph_spgemm_f32(c.V, c.COL, c.ROW, capacity[i], a.V, a.COL, a.ROW, b.V, b.COL,
-                                 b.ROW, m, a.N, n, nullptr));
+            bool oneCall = true;
+            try
+            {
+                c.V = static_cast<float*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
+                c.COL = static_cast<uint32_t*>(Util::ResourceManager::GetMemoryCuda(bytes, true));
+                oneCall = sph_spgemm_f32(c.V, c.COL, c.ROW, capacity[i], a.V, a.COL, a.ROW, b.V,
+                                         b.COL, b.ROW, m, a.N, n, nullptr) == SPH_OK;
+            }
+            catch (const std::runtime_error&)
+            {
+                oneCall = false;  // no memory for the bound
+            }
+            if (!oneCall)
+            {
+                if (c.V != nullptr)
+                    Util::ResourceManager::FreePreservedCuda(c.V);
+                if (c.COL != nullptr)
+                    Util::ResourceManager::FreePreservedCuda(c.COL);
+                c.V = nullptr;
+                c.COL = nullptr;
+                twoPasses(i);
+            }
         }
         for (uint32_t i = 0; i < count; ++i)
         {
             SparseMatrix& c = result[i];
+            if (exact[i])
+                continue;
             uint32_t nnz = 0;
             Compute::Cuda::CopyDeviceToHost(&nnz, c.ROW + m, sizeof(nnz));
             c.NNZ = nnz;
@@ -228,8 +268,12 @@ void SparseGemm(TensorUtil::TensorData& y, const TensorUtil::TensorData& a,
     if (static_cast<uint32_t>(b.Rows()) != m->N || static_cast<uint32_t>(y.Rows()) != m->M ||
         y.Cols() != b.Cols())
         throw std::invalid_argument("Compute::SparseGemm - shape mismatch");
-    Sparse::Cuda::Gemm(y.CudaMutableRawPtr(), m, b.CudaRawPtr(),
-                       static_cast<unsigned int>(b.Cols()), accumulate,
+    // every element of y is written; a fresh y (zero fill deferred) is stored into, not read
+    const bool whole = static_cast<std::size_t>(y.Size()) ==
+                       static_cast<std::size_t>(m->M) * static_cast<std::size_t>(b.Cols());
+    const bool store = whole && (!accumulate || y.TakeDeferredZero());
+    Sparse::Cuda::Gemm(store ? y.CudaOverwriteRawPtr() : y.CudaMutableRawPtr(), m, b.CudaRawPtr(),
+                       static_cast<unsigned int>(b.Cols()), store ? false : accumulate,
                        y.GetCudaDevice().GetID());
 }
 }  // namespace Sapphire::Compute

@@ -51,6 +51,35 @@ def test_two_calls_in_a_row_second_smaller(dev):
         assert np.array_equal(new, want)
 
 
+def _allocations():
+    count = ctypes.c_uint64(0)
+    capi.call("sph_allocation_count", ctypes.byref(count))
+    return count.value
+
+
+def test_the_call_makes_no_allocation(dev):
+    """The library counts every hipMalloc / hipMallocAsync / hipHostMalloc it makes.  Across the
+    no-allocation entry the count stays put, for a scan that needs the block totals (more than
+    65536 rows) and for one that does not; across the allocating entry on the same input it
+    moves, which shows that the counter sees the scratch block."""
+    M, N, ld = 200000, 12, 12
+    dense = sparse_dense(4400, (M, ld), 0.2)
+    dD = capi.DeviceBuffer.from_array(dense)
+    dRow = capi.DeviceBuffer(4 * (M + 1))
+    capi.sync()
+    h.announce("sph_csr_row_offsets_noalloc_f32 allocation count", (M, N, ld))
+    before = _allocations()
+    capi.call("sph_csr_row_offsets_noalloc_f32", dRow.ptr, dD.ptr, M, N, ld)
+    capi.call("sph_csr_row_offsets_noalloc_f32", dRow.ptr, dD.ptr, 5000, N, ld)
+    capi.sync()
+    assert _allocations() == before
+    capi.call("sph_csr_row_offsets_f32", dRow.ptr, dD.ptr, M, N, ld, None)
+    capi.sync()
+    assert _allocations() == before + 1
+    dD.release()
+    dRow.release()
+
+
 def test_rejects_more_rows_than_the_array_covers(dev):
     dRow = capi.DeviceBuffer(64)
     with pytest.raises(capi.SphError) as err:
