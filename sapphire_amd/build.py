@@ -110,7 +110,7 @@ HARNESS_LIB = os.path.join(HARNESS_DIR, "libhost_harness.so")
 def build_harness():
     """C entry points over the C++ layer for the Python parity tests."""
     flags = ["-O2", "-std=c++17", "-fPIC", "-x", "c++",
-             "-I" + os.path.join(ROOT, "include"), "-I" + HOST]
+             "-I" + os.path.join(ROOT, "include"), "-I" + HOST, "-I" + CSRC]
     objs = _compile_all(_sources(HARNESS_DIR, {".cpp"}), flags, "harness")
     _run([_hipcc(), "-shared", "-fPIC", "-o", HARNESS_LIB] + objs +
          ["-L" + PKG, "-lsapphire_host", "-lsapphire_hip", "-Wl,-rpath,$ORIGIN/../../sapphire_amd"])

@@ -48,6 +48,7 @@
 // anywhere; only a copy's 8 columns have to lie inside the row) and the last r columns to
 // GemmF16Few, as do the last M % 8 rows of an A stored K x M.
 #include "sph_internal.h"
+#include "sph_k_partition.h"
 
 #include <algorithm>
 #include <type_traits>
@@ -1672,10 +1673,8 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
     const uint32_t col = tn * TILE + lt;
 
     // this wavefront's K range, in groups of kGroupK
-    const uint32_t groups = (K + kGroupK - 1) / kGroupK;
-    const uint32_t perWave = (groups + WAVES - 1) / WAVES;
-    const uint32_t gBegin = min(wave * perWave, groups);
-    const uint32_t gEnd = min(gBegin + perWave, groups);
+    constexpr int kDepth = 4;  // groups in flight
+    const sph::KPartition part = sph::PartitionK(K, kGroupK, WAVES, wave, kDepth);
 
     Acc acc;
 #pragma unroll
@@ -1758,23 +1757,20 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(b, a, acc, 0, 0, 0);
     };
 
-    constexpr int kDepth = 4;  // groups in flight
-    const uint32_t whole = K / kGroupK;          // groups with every k below K
-    const uint32_t wholeEnd = min(gEnd, whole);  // this wavefront's whole groups end here
-    if (gBegin < wholeEnd)
+    const uint32_t whole = part.whole;
+    if (part.gBegin < part.wholeEnd)
     {
-        const uint32_t lastWhole = wholeEnd - 1;
-        const uint32_t roundsEnd = gBegin + (wholeEnd - gBegin) / kDepth * kDepth;
+        const uint32_t wholeEnd = part.wholeEnd, roundsEnd = part.roundsEnd;
         FragA fa[kDepth];
         FragB fb[kDepth];
 #pragma unroll
         for (int d = 0; d < kDepth; ++d)
         {
             // past the last whole group: that group once more, loaded and not used
-            fa[d] = loadA(min(gBegin + d, lastWhole));
-            fb[d] = loadB(min(gBegin + d, lastWhole));
+            fa[d] = loadA(sph::KPartitionFirst(part, d));
+            fb[d] = loadB(sph::KPartitionFirst(part, d));
         }
-        for (uint32_t g = gBegin; g < roundsEnd; g += kDepth)
+        for (uint32_t g = part.gBegin; g < roundsEnd; g += kDepth)
         {
 #pragma unroll
             for (int d = 0; d < kDepth; ++d)
@@ -1784,7 +1780,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
                 // at the end of each round); the fences keep that order
                 multiply(fa[d].get(), fb[d].get());
                 __builtin_amdgcn_sched_barrier(0);
-                const uint32_t next = min(g + kDepth + d, lastWhole);
+                const uint32_t next = sph::KPartitionNext(part, g, kDepth, d);
                 fa[d] = loadA(next);
                 fb[d] = loadB(next);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1796,7 +1792,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
             if (roundsEnd + d < wholeEnd)
                 multiply(fa[d].get(), fb[d].get());
     }
-    if (gBegin <= whole && whole < gEnd)
+    if (part.ownsPartial)
     {
         // at most one group, and only in the wavefront that holds the end of K
         const halfx8 a = TA ? loadPartial(aPtr, args.lda, whole) : loadPartial(aPtr, 1, whole);

@@ -30,6 +30,7 @@
 // (batch, stride) arithmetic -- stride 0 repeats an operand -- or from a table of element
 // offsets in device memory.
 #include "sph_internal.h"
+#include "sph_k_partition.h"
 
 #include <algorithm>
 #include <cstring>
@@ -1274,11 +1275,11 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
     const uint32_t row = tm * TILE + lt;
     const uint32_t col = tn * TILE + lt;
 
-    // this wavefront's K range, in groups of kGroupK (one float4 of A per lane)
-    const uint32_t groups = (K + kGroupK - 1) / kGroupK;
-    const uint32_t perWave = (groups + WAVES - 1) / WAVES;
-    const uint32_t gBegin = min(wave * perWave, groups);
-    const uint32_t gEnd = min(gBegin + perWave, groups);
+    // this wavefront's K range, in groups of kGroupK (one float4 of A per lane); groups in
+    // flight: 8, or twice the wavefronts per tile, are slower: the loop is bound by what the
+    // caches deliver, not by the latency of a load
+    constexpr int kDepth = 4;
+    const sph::KPartition part = sph::PartitionK(K, kGroupK, WAVES, wave, kDepth);
 
     const bool rowOk = row < M;
     const bool colOk = col < N;
@@ -1345,24 +1346,19 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
         multiply(b.w, a.w);
     };
 
-    // groups in flight; 8, or twice the wavefronts per tile, are slower: the loop is bound by
-    // what the caches deliver, not by the latency of a load
-    constexpr int kDepth = 4;
-    const uint32_t whole = K / kGroupK;        // groups with every k below K
-    const uint32_t wholeEnd = min(gEnd, whole);  // this wavefront's whole groups end here
-    if (gBegin < wholeEnd)
+    const uint32_t whole = part.whole;
+    if (part.gBegin < part.wholeEnd)
     {
-        const uint32_t lastWhole = wholeEnd - 1;
-        const uint32_t roundsEnd = gBegin + (wholeEnd - gBegin) / kDepth * kDepth;
+        const uint32_t wholeEnd = part.wholeEnd, roundsEnd = part.roundsEnd;
         float4 fa[kDepth], fb[kDepth];
 #pragma unroll
         for (int d = 0; d < kDepth; ++d)
         {
             // past the last whole group: that group once more, loaded and not used
-            fa[d] = loadA(min(gBegin + d, lastWhole));
-            fb[d] = loadB(min(gBegin + d, lastWhole));
+            fa[d] = loadA(sph::KPartitionFirst(part, d));
+            fb[d] = loadB(sph::KPartitionFirst(part, d));
         }
-        for (uint32_t g = gBegin; g < roundsEnd; g += kDepth)
+        for (uint32_t g = part.gBegin; g < roundsEnd; g += kDepth)
         {
 #pragma unroll
             for (int d = 0; d < kDepth; ++d)
@@ -1372,7 +1368,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
                 // at the end of each round); the fences keep that order
                 multiplyGroup(fa[d], fb[d]);
                 __builtin_amdgcn_sched_barrier(0);
-                const uint32_t next = min(g + kDepth + d, lastWhole);
+                const uint32_t next = sph::KPartitionNext(part, g, kDepth, d);
                 fa[d] = loadA(next);
                 fb[d] = loadB(next);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1384,7 +1380,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
             if (roundsEnd + d < wholeEnd)
                 multiplyGroup(fa[d], fb[d]);
     }
-    if (gBegin <= whole && whole < gEnd)
+    if (part.ownsPartial)
     {
         // at most one group, and only in the wavefront that holds the end of K
         const float4 a = TA ? loadPartial(aPtr, args.lda, whole) : loadPartial(aPtr, 1, whole);

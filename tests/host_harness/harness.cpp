@@ -17,6 +17,7 @@
 #include <Sapphire/util/ResourceManager.hpp>
 
 #include <sapphire_hip.h>
+#include <sph_k_partition.h>
 
 #include <algorithm>
 #include <chrono>
@@ -253,6 +254,32 @@ int sphh_compute_gemm(float* yData, const int* y, int yn, const float* aData, co
         Download(Out, yData);
         Util::ResourceManager::Clean();
     });
+}
+
+// The K partition of the few-tile GEMM kernels, computed by the code the kernels use
+// (sapphire_amd/csrc/sph_k_partition.h).  out: gBegin, gEnd, whole, wholeEnd, lastWhole,
+// roundsEnd, ownsPartial.  No device is touched.
+int sphh_k_partition(unsigned K, unsigned groupK, unsigned waves, unsigned wave, unsigned depth,
+                     unsigned* out)
+{
+    const sph::KPartition p = sph::PartitionK(K, groupK, waves, wave, depth);
+    out[0] = p.gBegin;
+    out[1] = p.gEnd;
+    out[2] = p.whole;
+    out[3] = p.wholeEnd;
+    out[4] = p.lastWhole;
+    out[5] = p.roundsEnd;
+    out[6] = p.ownsPartial ? 1u : 0u;
+    return 0;
+}
+
+// slot d of the load pipeline: the group it holds before the first round (g == 0xffffffff) or
+// the one loaded while round g .. g + depth - 1 is multiplied
+unsigned sphh_k_partition_slot(unsigned K, unsigned groupK, unsigned waves, unsigned wave,
+                               unsigned depth, unsigned g, unsigned d)
+{
+    const sph::KPartition p = sph::PartitionK(K, groupK, waves, wave, depth);
+    return g == 0xffffffffu ? sph::KPartitionFirst(p, d) : sph::KPartitionNext(p, g, depth, d);
 }
 
 // Compute::Gemm into a FRESH y (never filled, never read): the operator sees the deferred zero

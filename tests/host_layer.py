@@ -31,6 +31,9 @@ def lib():
         h.sphh_bench_gemm_half_fresh_y.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                    ctypes.c_int, ctypes.c_int, ctypes.c_double,
                                                    _fp, ctypes.POINTER(ctypes.c_double)]
+        h.sphh_k_partition.argtypes = [ctypes.c_uint] * 5 + [ctypes.POINTER(ctypes.c_uint)]
+        h.sphh_k_partition_slot.argtypes = [ctypes.c_uint] * 7
+        h.sphh_k_partition_slot.restype = ctypes.c_uint
         h.sphh_transpose.argtypes = [_fp, _ip, ctypes.c_int, _fp, _ip, ctypes.c_int]
         h.sphh_mlp_forward.argtypes = [_fp, ctypes.c_int, _ip, ctypes.c_int,
                                        ctypes.POINTER(_fp), ctypes.POINTER(_fp), _fp, ctypes.c_int]
@@ -136,6 +139,21 @@ def bench_gemm_half_fresh_y(a_dev_ptr, b_dev_ptr, n, steps, warmup, settle_ms):
     _ok(lib().sphh_bench_gemm_half_fresh_y(a_dev_ptr, b_dev_ptr, n, steps, warmup, settle_ms,
                                            ctypes.byref(ev), ctypes.byref(wall)))
     return ev.value, wall.value
+
+
+def k_partition(K, group_k, waves, wave, depth):
+    """The few-tile kernels' K partition for one wavefront, from the kernels' own header."""
+    out = (ctypes.c_uint * 7)()
+    lib().sphh_k_partition(K, group_k, waves, wave, depth, out)
+    keys = ("g_begin", "g_end", "whole", "whole_end", "last_whole", "rounds_end", "owns_partial")
+    return dict(zip(keys, [int(v) for v in out]))
+
+
+def k_partition_slot(K, group_k, waves, wave, depth, g, d):
+    """Group held by slot d of the load pipeline: before the first round (g None) or the one
+    loaded while the round that starts at group g is multiplied."""
+    return int(lib().sphh_k_partition_slot(K, group_k, waves, wave, depth,
+                                           0xffffffff if g is None else g, d))
 
 
 def transpose(x, y_shape):
