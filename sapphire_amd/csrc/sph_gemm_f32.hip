@@ -61,11 +61,10 @@ struct GemmF32Args
     // some of the columns of a wider matrix; likewise of an A stored K x M: M, unless a launch
     // covers some of the rows
     uint32_t ldb, ldc, lda;
-    // tiled kernels: rows of this launch's out below this one are computed but not stored (a
-    // launch over the last 4 rows of a product whose other rows another launch has written)
-    uint32_t rowStoreFrom;
     uint32_t split;      // launcher: 1 = a part of the columns, 2 = a part of the rows, 4 = the
-                         // tiled kernels have been chosen
+                         // tiled kernels have been chosen, 8 = the K-split kernel among them,
+                         // 16 = a thin strip of a wider product: the few-tile kernel, 16 x 16
+                         // tiles, four wavefronts
     uint32_t basesOk;    // launcher: the caller's A and B start on 16-byte boundaries
     uint32_t tilesM, tilesN;
     uint32_t tilesTotal;  // tilesM * tilesN * units
@@ -80,6 +79,19 @@ struct GemmF32Args
     uint32_t sgd;
     float sgdScale, sgdRate;
     int64_t strideOut, strideA, strideB;
+};
+
+// Thin strips of a product's last rows and columns that ride along with the launch of its body:
+// the first `padded` workgroups of the grid (a multiple of 8, so that the body's workgroups keep
+// their place among the 8 XCDs) run the few-tile kernel's code on part[0] (blocks[0] of them) and
+// part[1] (blocks[1]), the rest the body's tiles.  A strip's workgroups are short and sit beside
+// the body's on the same compute units, where a launch of their own would start after the
+// body's last tile has finished.
+struct GemmF32Strips
+{
+    GemmF32Args part[2];
+    uint32_t blocks[2];
+    uint32_t padded;
 };
 
 // Slab loaders.  An operand is stored either with K contiguous (A as given, B when it is
@@ -301,7 +313,7 @@ __device__ __forceinline__ void StoreTile(const floatx16 (&acc)[TM][TN], float* 
             {
                 const uint32_t r = rowBase + i * 32 + l32;
                 const uint32_t c = colBase + j * 32 + 8 * q + 4 * khalf;
-                if (r < M && c < N && r >= args.rowStoreFrom)
+                if (r < M && c < N)
                 {
                     float4 v = old[(i * TN + j) * 4 + q];
                     v.x = Combine(args, v.x, acc[i][j][4 * q + 0]);
@@ -579,10 +591,13 @@ struct DmaTile
 // wavefronts per group) gives products with fewer 64-tiles than compute units twice as many
 // workgroups.  The K products of an element are then summed in another order than with
 // KSPLIT = 1 (within the fp32 tolerance, not bit-identical to it).
+template <int TILE, bool TA, bool TB, int WAVES>
+__device__ __forceinline__ void GemmF32SkinnyBody(const GemmF32Args& args, uint32_t block);
+
 template <int BM, int BN, int BK, int STAGES, bool TA, bool TB, bool WALK, bool TAIL = false,
           int KSPLIT = 1>
 __global__ __launch_bounds__(((BN >= 64) ? 4 : 2) * KSPLIT * 64) void GemmF32DmaKernel(
-    const GemmF32Args args)
+    const GemmF32Args args, const GemmF32Strips strips)
 {
     static_assert(BK == 16 || BK == 32, "K step of 16 or 32");
     static_assert(!(WALK && TAIL), "a walk needs whole rings of steps");
@@ -612,6 +627,22 @@ __global__ __launch_bounds__(((BN >= 64) ? 4 : 2) * KSPLIT * 64) void GemmF32Dma
 
     __shared__ __attribute__((aligned(1024))) char lds[STAGES * kStageBytes];
 
+    // strips of the product's edge come first in the grid (a walk has none)
+    uint32_t block = blockIdx.x;
+    if constexpr (!WALK)
+    {
+        static_assert(NW == 4, "the strips' code runs on four wavefronts");
+        if (block < strips.padded)
+        {
+            if (block < strips.blocks[0])
+                GemmF32SkinnyBody<16, TA, TB, 4>(strips.part[0], block);
+            else if (block - strips.blocks[0] < strips.blocks[1])
+                GemmF32SkinnyBody<16, TA, TB, 4>(strips.part[1], block - strips.blocks[0]);
+            return;
+        }
+        block -= strips.padded;
+    }
+
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -622,12 +653,12 @@ __global__ __launch_bounds__(((BN >= 64) ? 4 : 2) * KSPLIT * 64) void GemmF32Dma
     const uint32_t khalf = lane >> 5;
 
     // ---- the tile(s) of this workgroup ------------------------------------------------------
-    uint32_t logical = (blockIdx.x & 7u) * args.perXcd + (blockIdx.x >> 3);
+    uint32_t logical = (block & 7u) * args.perXcd + (block >> 3);
     uint32_t logicalEnd = args.tilesTotal;
     uint32_t logicalStride = 0;
     if constexpr (WALK)
     {
-        logicalEnd = min((blockIdx.x & 7u) * args.perXcd + args.perXcd, args.tilesTotal);
+        logicalEnd = min((block & 7u) * args.perXcd + args.perXcd, args.tilesTotal);
         logicalStride = gridDim.x >> 3;
     }
     if (logical >= logicalEnd)
@@ -1233,7 +1264,7 @@ __global__ __launch_bounds__(((BN >= 64) ? 4 : 2) * KSPLIT * 64) void GemmF32Dma
 // many compute units, is preferred whenever its tiles still fit the chip.
 // ---------------------------------------------------------------------------
 template <int TILE, bool TA, bool TB, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32Args args)
+__device__ __forceinline__ void GemmF32SkinnyBody(const GemmF32Args& args, uint32_t block)
 {
     static_assert(TILE == 32 || TILE == 16, "MFMA shapes 32x32x2 and 16x16x4");
     constexpr uint32_t kLaneGroups = 64 / TILE;       // values of k per MFMA
@@ -1249,7 +1280,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
     const uint32_t lt = lane % TILE;   // row of A / column of B this lane feeds
     const uint32_t kh = lane / TILE;   // which k of an MFMA
 
-    uint32_t id = blockIdx.x;
+    uint32_t id = block;
     const uint32_t tn = id % args.tilesN;
     id /= args.tilesN;
     const uint32_t tm = id % args.tilesM;
@@ -1468,6 +1499,12 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32A
     }
 }
 
+template <int TILE, bool TA, bool TB, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void GemmF32SkinnyKernel(const GemmF32Args args)
+{
+    GemmF32SkinnyBody<TILE, TA, TB, WAVES>(args, blockIdx.x);
+}
+
 // ---------------------------------------------------------------------------
 // One output row (M = 1):  out[1 x N] (+)= a[1 x K] * B[K x N], e.g. the column sums
 // ones x dy of the bias gradient.  A matrix-core tile would use one of its 32 rows; this is a
@@ -1609,41 +1646,43 @@ void LaunchSkinny(const GemmF32Args& args, dim3 grid, uint32_t tile, bool wide, 
 
 // `walk`: 64-tiles only, each workgroup takes several tiles
 // `ksplit`: 0, or 2 = K split over two groups of wavefronts on 64 x 32 tiles
+// `strips`: edge strips that ride along; only the straight-to-LDS kernels that are no walk take
+// any
 template <bool TA, bool TB>
-void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dma, bool walk,
-                 int ksplit, hipStream_t stream)
+void LaunchTiled(const GemmF32Args& args, const GemmF32Strips& strips, dim3 grid, bool big,
+                 bool vec, bool dma, bool walk, int ksplit, hipStream_t stream)
 {
     const dim3 block(kThreads);
     if (dma && ksplit != 0)
     {
         if (args.K % 32 == 0)
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 32, 32, 4, TA, TB, false, false, 2>), grid,
-                               dim3(256), 0, stream, args);
+                               dim3(256), 0, stream, args, strips);
         else
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 32, 32, 4, TA, TB, false, true, 2>), grid,
-                               dim3(256), 0, stream, args);
+                               dim3(256), 0, stream, args, strips);
         return;
     }
     if (dma)
     {
         if (big && args.K % 16 != 0)
             hipLaunchKernelGGL((GemmF32DmaKernel<128, 128, 16, 4, TA, TB, false, true>), grid,
-                               block, 0, stream, args);
+                               block, 0, stream, args, strips);
         else if (big)
             hipLaunchKernelGGL((GemmF32DmaKernel<128, 128, 16, 4, TA, TB, false>), grid, block, 0,
-                               stream, args);
+                               stream, args, strips);
         else if (walk)
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB, true>), grid, block, 0,
-                               stream, args);
+                               stream, args, strips);
         else if (args.K % 32 == 0)
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB, false>), grid, block, 0,
-                               stream, args);
+                               stream, args, strips);
         else if (args.K % 16 == 0)
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 16, 6, TA, TB, false>), grid, block, 0,
-                               stream, args);
+                               stream, args, strips);
         else
             hipLaunchKernelGGL((GemmF32DmaKernel<64, 64, 32, 4, TA, TB, false, true>), grid,
-                               block, 0, stream, args);
+                               block, 0, stream, args, strips);
         return;
     }
     if (big)
@@ -1666,9 +1705,77 @@ void LaunchTiled(const GemmF32Args& args, dim3 grid, bool big, bool vec, bool dm
     }
 }
 
+// Tile edge: the matrix pipes bound the tiled kernels, so a launch lasts as long as the compute
+// unit with the most tiles needs.  A 128-tile costs four 64-tiles and moves half the operand
+// bytes per flop (measured 7 % faster at equal load), but a compute unit with a single 128-tile
+// has nothing to run beside that tile's first loads and epilogue, which four 64-tiles overlap
+// (measured 6 % slower then).  Returns the smaller cost of the busiest compute unit and which
+// edge has it.
+uint64_t TileCost(uint32_t M, uint32_t N, uint32_t units, bool* big)
+{
+    const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
+    const uint64_t tiles128 = static_cast<uint64_t>((M + 127) / 128) * ((N + 127) / 128) * units;
+    const uint64_t tiles64 = static_cast<uint64_t>((M + 63) / 64) * ((N + 63) / 64) * units;
+    const uint64_t rounds128 = (tiles128 + cus - 1) / cus;
+    const uint64_t cost128 = rounds128 * 400 + (rounds128 == 1 ? 32 : 0);
+    const uint64_t cost64 = ((tiles64 + cus - 1) / cus) * 107;
+    *big = cost128 <= cost64;
+    return std::min(cost128, cost64);
+}
+
+template <bool TA, bool TB>
+void LaunchStripAlone(const GemmF32Args& strip, uint32_t blocks, hipStream_t stream)
+{
+    hipLaunchKernelGGL((GemmF32SkinnyKernel<16, TA, TB, 4>), dim3(blocks), dim3(256), 0, stream,
+                       strip);
+}
+
+int LaunchStrip(const GemmF32Args& strip, uint32_t blocks, bool transA, bool transB,
+                hipStream_t stream)
+{
+    if (transA && transB)
+        LaunchStripAlone<true, true>(strip, blocks, stream);
+    else if (transA)
+        LaunchStripAlone<true, false>(strip, blocks, stream);
+    else if (transB)
+        LaunchStripAlone<false, true>(strip, blocks, stream);
+    else
+        LaunchStripAlone<false, false>(strip, blocks, stream);
+    SPH_CHECK_LAUNCH();
+    return SPH_OK;
+}
+
+// A thin strip of a product's last rows or columns: 16 x 16 tiles of the few-tile kernel on four
+// wavefronts, whether it then rides along with the body's launch (`pending` has room) or is
+// launched on its own, so that its bits do not depend on which.
+int AddStrip(GemmF32Args strip, uint32_t units, bool outOffsetsAligned, bool transA, bool transB,
+             GemmF32Strips* pending, hipStream_t stream)
+{
+    strip.tilesM = (strip.M + 15) / 16;
+    strip.tilesN = (strip.N + 15) / 16;
+    const uint64_t blocks = static_cast<uint64_t>(strip.tilesM) * strip.tilesN * units;
+    if (blocks >= (1ull << 30))
+        return sph::Fail(SPH_ERR_INVALID, "sph_gemm_f32 - too many tiles for one launch");
+    strip.outVec = (outOffsetsAligned && (strip.N % 4 == 0) && (strip.ldc % 4 == 0) &&
+                    (reinterpret_cast<uintptr_t>(strip.out) & 15u) == 0)
+                       ? 1u
+                       : 0u;
+    for (int i = 0; i < 2 && pending != nullptr; ++i)
+        if (pending->blocks[i] == 0)
+        {
+            pending->part[i] = strip;
+            pending->blocks[i] = static_cast<uint32_t>(blocks);
+            pending->padded = (pending->blocks[0] + pending->blocks[1] + 7u) & ~7u;
+            return SPH_OK;
+        }
+    return LaunchStrip(strip, static_cast<uint32_t>(blocks), transA, transB, stream);
+}
+
 // `transA`: A is stored K x M; `transB`: B is stored N x K.
-int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOffsetsAligned,
-           bool transA, bool transB, hipStream_t stream)
+// `pending`: strips waiting for a launch to ride along with; a launch that takes them empties
+// the list.
+int LaunchPart(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOffsetsAligned,
+               bool transA, bool transB, GemmF32Strips* pending, hipStream_t stream)
 {
     GemmF32Args args = base;
     if (args.split == 0)
@@ -1681,14 +1788,6 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
                 ? 1u
                 : 0u;
     }
-    const bool part = (args.split & 1u) != 0;  // some of the columns of a wider product
-    // N = 4 q + r, r != 0: the rows of a B stored K x N are copied 4 columns at a time, so the
-    // first 4 q columns go to the kernels below (row pitches stay N) and the last r to the
-    // kernel for narrow products; every output element is still computed by one kernel
-    // (measured 4096 x 4095 x 4096: 1615 us on the register-staged kernel's 4-byte loads).
-    // A B stored N x K would not need this; it is split all the same, so that a product does
-    // not depend on how its operands are stored.
-    // (not when the whole product goes to the few-tile kernel, which takes any N as it is)
     const uint64_t wholeTiles64 =
         static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
     // Between a quarter and a half as many 64-tiles as compute units the straight-to-LDS
@@ -1698,9 +1797,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const uint64_t cusAll = static_cast<uint64_t>(sph::ComputeUnits());
     const bool midTiled = wholeTiles64 * 4 > cusAll && wholeTiles64 * 2 <= cusAll &&
                           args.basesOk != 0 && args.K >= 64 && args.M >= 4 && args.N >= 4 &&
-                          // (an A stored K x M is copied 4 rows at a time and cut into two
-                          // launches from 68 rows up; asked of either storage, so that the
-                          // choice does not depend on the flags)
+                          // (rows past the last multiple of 4 are cut off from 68 rows up)
                           (args.M % 4 == 0 || args.M >= 68) &&
                           static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
                           static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
@@ -1708,58 +1805,112 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     // decided once, on the whole product, and carried by its parts (bit 2: tiled kernels, bit 3:
     // the K-split kernel on 64 x 32 tiles), so that a product's columns and rows are all summed
     // in one order however it is cut up
-    if (args.split == 0 && !wholeIsFewTiles)
+    const bool whole = args.split == 0;
+    if (whole && !wholeIsFewTiles)
         args.split = midTiled ? 12u : 4u;
-    if ((args.split & 3u) == 0 && args.N % 4 != 0 && args.N > 4 && args.M > 1 && args.K >= kBK &&
-        !wholeIsFewTiles)
+    // A product for the tiled kernels is cut into a body and up to two thin strips of its last
+    // rows and columns, which the few-tile kernel's code computes (it reads any rows and columns
+    // from anywhere); every output element is still computed once.  Cut off are
+    //  - the last N % 4 columns: the rows of a B stored K x N are copied 4 columns at a time
+    //    (measured 4096 x 4095 x 4096: 1615 us on the register-staged kernel's 4-byte loads);
+    //  - the last M % 4 rows, from 68 rows up: an A stored K x M is copied 4 rows at a time;
+    //  - up to 16 rows or columns past a multiple of the tile edge, when the compute unit with
+    //    the most tiles then has fewer of them (1025^3: 17 x 17 tiles of 64 are two per
+    //    compute unit somewhere, 16 x 16 one everywhere; measured 44.8 -> 23.4 us).
+    // The cut depends on M, N, K and the batch only, not on how the operands are stored or
+    // aligned, so a product's bits do not depend on that either.
+    if (whole && (args.split & 4u) != 0 && args.M > 1 && args.K >= kBK)
     {
-        const uint32_t whole = args.N & ~3u;
-        GemmF32Args left = args;
-        left.split |= 1u;
-        left.N = whole;
-        const int rc = Launch(left, units, allowVector, outOffsetsAligned, transA, transB, stream);
-        if (rc != SPH_OK)
-            return rc;
-        GemmF32Args right = args;
-        right.split |= 1u;
-        right.N = args.N - whole;
-        right.B = args.B + (transB ? static_cast<size_t>(whole) * args.K : whole);
-        right.out = args.out + whole;
-        if (args.bias != nullptr)
-            right.bias = args.bias + whole;
-        return Launch(right, units, allowVector, outOffsetsAligned, transA, transB, stream);
+        const uint32_t baseM = (args.M >= 68 && args.N >= 4) ? args.M % 4 : 0;
+        const uint32_t baseN = args.N > 4 ? args.N % 4 : 0;
+        uint32_t peelM = baseM, peelN = baseN;
+        if ((args.split & 8u) == 0)
+        {
+            auto candidates = [](uint32_t x, uint32_t base, bool allowed, uint32_t* list) {
+                int n = 0;
+                list[n++] = base;
+                for (uint32_t edge = 64; edge <= 128 && allowed; edge *= 2)
+                {
+                    const uint32_t r = x % edge;
+                    if (r != 0 && r <= 16 && r > base && x - r >= edge && r != list[n - 1])
+                        list[n++] = r;
+                }
+                return n;
+            };
+            uint32_t listM[3], listN[3];
+            const int countM = candidates(args.M, baseM, args.N >= 4, listM);
+            const int countN = candidates(args.N, baseN, true, listN);
+            // a strip's 16 x 16 tile: a sixteenth of a 64-tile's flops at about a quarter of
+            // its rate, beside the body's tiles
+            auto stripCost = [&](uint32_t rows, uint32_t cols) {
+                const uint64_t blocks =
+                    static_cast<uint64_t>((rows + 15) / 16) * ((cols + 15) / 16) * units;
+                return (blocks + cusAll - 1) / cusAll * 27;
+            };
+            uint64_t best = ~0ull;
+            for (int i = 0; i < countM; ++i)
+                for (int j = 0; j < countN; ++j)
+                {
+                    bool big;
+                    uint64_t cost = TileCost(args.M - listM[i], args.N - listN[j], units, &big);
+                    if (listM[i] > baseM)
+                        cost += stripCost(listM[i], args.N);
+                    if (listN[j] > baseN)
+                        cost += stripCost(args.M - listM[i], listN[j]);
+                    if (cost < best)
+                    {
+                        best = cost;
+                        peelM = listM[i];
+                        peelN = listN[j];
+                    }
+                }
+        }
+        if (peelM != 0 || peelN != 0)
+        {
+            GemmF32Args body = args;
+            body.split |= 3u;
+            body.M = args.M - peelM;
+            body.N = args.N - peelN;
+            if (peelM != 0)
+            {
+                // rows [M - peelM, M), every column
+                GemmF32Args bottom = args;
+                bottom.split |= 3u;
+                bottom.M = peelM;
+                bottom.A = args.A + (transA ? body.M : static_cast<size_t>(body.M) * args.K);
+                bottom.out = args.out + static_cast<size_t>(body.M) * args.ldc;
+                const int rc = AddStrip(bottom, units, outOffsetsAligned, transA, transB, pending,
+                                        stream);
+                if (rc != SPH_OK)
+                    return rc;
+            }
+            if (peelN != 0)
+            {
+                // rows [0, M - peelM), columns [N - peelN, N)
+                GemmF32Args right = args;
+                right.split |= 3u;
+                right.M = body.M;
+                right.N = peelN;
+                right.B = args.B + (transB ? static_cast<size_t>(body.N) * args.K : body.N);
+                right.out = args.out + body.N;
+                if (args.bias != nullptr)
+                    right.bias = args.bias + body.N;
+                const int rc = AddStrip(right, units, outOffsetsAligned, transA, transB, pending,
+                                        stream);
+                if (rc != SPH_OK)
+                    return rc;
+            }
+            return LaunchPart(body, units, allowVector, outOffsetsAligned, transA, transB, pending,
+                              stream);
+        }
     }
-    // M = 4 q + r, r != 0, with A stored K x M: its rows are copied 4 rows of the product at a
-    // time.  The first 4 q rows go to the kernels below; the last 4 rows are launched once more
-    // on their own and store only the r rows the first launch has not written.  Both launches
-    // run the same kernels as an A stored M x K would, so the storage does not change a bit.
-    const bool dmaShape = args.basesOk != 0 && args.K >= kBK && args.N >= 4 &&
-                          (transB || args.N % 4 == 0);
     // few 64 x 64 tiles and a long K: the kernel that splits K inside the workgroup (decided on
     // the whole product, so that its parts run the kernels the whole would)
     const uint64_t tiles64 =
         static_cast<uint64_t>((args.M + 63) / 64) * ((args.N + 63) / 64) * units;
-    const bool fewTiles = (part && args.N < 4) ||
-                          ((args.split & 4u) == 0 &&
-                           tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) &&
-                           args.K >= 64);
-    if ((args.split & 2u) == 0 && transA && args.M % 4 != 0 && args.M >= 68 && dmaShape &&
-        !fewTiles)
-    {
-        GemmF32Args top = args;
-        top.split |= 6u;
-        top.M = args.M & ~3u;
-        const int rc = Launch(top, units, allowVector, outOffsetsAligned, transA, transB, stream);
-        if (rc != SPH_OK)
-            return rc;
-        GemmF32Args bottom = args;
-        bottom.split |= 6u;
-        bottom.M = 4;
-        bottom.A = args.A + (args.M - 4);
-        bottom.out = args.out + static_cast<size_t>(args.M - 4) * args.ldc;
-        bottom.rowStoreFrom = 4 - args.M % 4;
-        return Launch(bottom, units, allowVector, outOffsetsAligned, transA, transB, stream);
-    }
+    const bool fewTiles = (args.split & 4u) == 0 &&
+                          tiles64 * 2 <= static_cast<uint64_t>(sph::ComputeUnits()) &&
+                          args.K >= 64;
     args.outVec = (outOffsetsAligned && (args.N % 4 == 0) && (args.ldc % 4 == 0) &&
                    (reinterpret_cast<uintptr_t>(args.out) & 15u) == 0)
                       ? 1u
@@ -1784,6 +1935,7 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
 
     if (fewTiles)
     {
+        // (a product's strips are planned by AddStrip: always 16 x 16 tiles on four wavefronts)
         // 16 x 16 tiles while there are at most two per compute unit, or for a matrix of at most
         // 16 rows or columns: a quarter of the matrix-core work per workgroup on four times as
         // many compute units and less of a tile outside a narrow matrix, but twice the operand
@@ -1817,12 +1969,6 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
         return SPH_OK;
     }
 
-    // Tile edge: the matrix pipes bound these kernels, so a launch lasts as long as the
-    // compute unit with the most tiles needs.  A 128-tile costs four 64-tiles and moves half
-    // the operand bytes per flop (measured 7 % faster at equal load), but a compute unit with
-    // a single 128-tile has nothing to run beside that tile's first loads and epilogue, which
-    // four 64-tiles overlap (measured 6 % slower then); pick the edge with the smaller cost of
-    // the busiest compute unit.
     const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
     // straight-to-LDS pipeline: whole K steps, 16-byte chunks everywhere, at least one chunk
     // per clamped edge, and lane offsets that fit 32 bits
@@ -1835,12 +1981,8 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const bool dma = dmaLayout && args.K >= kBK && args.M >= 4 && args.N >= 4 &&
                      static_cast<uint64_t>(args.M) * args.K < (1ull << 30) &&
                      static_cast<uint64_t>(args.K) * args.N < (1ull << 30);
-    const uint64_t tiles128 =
-        static_cast<uint64_t>((args.M + 127) / 128) * ((args.N + 127) / 128) * units;
-    const uint64_t rounds128 = (tiles128 + cus - 1) / cus;
-    const uint64_t cost128 = rounds128 * 400 + (rounds128 == 1 ? 32 : 0);
-    const uint64_t cost64 = ((tiles64 + cus - 1) / cus) * 107;
-    const bool big = cost128 <= cost64;
+    bool big;
+    (void)TileCost(args.M, args.N, units, &big);
     // 64 x 32 tiles with K split over two groups of wavefronts (see the top of Launch).  The same
     // split on 64 x 64 tiles with eight wavefronts was measured for products with one 64-tile
     // per compute unit and does not pay (1024^3: 18.8 against 18.4 us): their loop already runs
@@ -1878,17 +2020,38 @@ int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOf
     const bool walk = dma && !big && ksplit == 0 &&
                       args.M % 64 == 0 && args.N % 64 == 0 && args.K % 128 == 0 &&
                       (reinterpret_cast<uintptr_t>(args.bias) & 15u) == 0;
-    const dim3 grid((walk ? std::min(slotsPerXcd, args.perXcd) : args.perXcd) * 8);
+    // strips that wait ride along with a straight-to-LDS launch that is no walk
+    GemmF32Strips strips{};
+    if (pending != nullptr && dma && !walk && pending->padded != 0 &&
+        blocks + pending->padded < (1ull << 31) - 8)
+    {
+        strips = *pending;
+        *pending = GemmF32Strips{};
+    }
+    const dim3 grid((walk ? std::min(slotsPerXcd, args.perXcd) : args.perXcd) * 8 + strips.padded);
     if (transA && transB)
-        LaunchTiled<true, true>(args, grid, big, aligned, dma, walk, ksplit, stream);
+        LaunchTiled<true, true>(args, strips, grid, big, aligned, dma, walk, ksplit, stream);
     else if (transA)
-        LaunchTiled<true, false>(args, grid, big, aligned, dma, walk, ksplit, stream);
+        LaunchTiled<true, false>(args, strips, grid, big, aligned, dma, walk, ksplit, stream);
     else if (transB)
-        LaunchTiled<false, true>(args, grid, big, aligned, dma, walk, ksplit, stream);
+        LaunchTiled<false, true>(args, strips, grid, big, aligned, dma, walk, ksplit, stream);
     else
-        LaunchTiled<false, false>(args, grid, big, aligned, dma, walk, ksplit, stream);
+        LaunchTiled<false, false>(args, strips, grid, big, aligned, dma, walk, ksplit, stream);
     SPH_CHECK_LAUNCH();
     return SPH_OK;
+}
+
+int Launch(const GemmF32Args& base, uint32_t units, bool allowVector, bool outOffsetsAligned,
+           bool transA, bool transB, hipStream_t stream)
+{
+    GemmF32Strips pending{};
+    int rc = LaunchPart(base, units, allowVector, outOffsetsAligned, transA, transB, &pending,
+                        stream);
+    // strips no launch has taken along: each on its own
+    for (int i = 0; i < 2 && rc == SPH_OK; ++i)
+        if (pending.blocks[i] != 0)
+            rc = LaunchStrip(pending.part[i], pending.blocks[i], transA, transB, stream);
+    return rc;
 }
 
 int GrowTable(EntryTable& t, size_t count)
