@@ -59,6 +59,9 @@ typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+// eight halves that need only be 4-byte aligned: a 16-byte vector memory access asks for no more
+typedef halfx8 halfx8a4 __attribute__((aligned(4)));
 typedef __attribute__((address_space(3))) void* LdsPtr;
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) shortx4* LdsShortx4Ptr;
@@ -80,6 +83,81 @@ struct GemmF16Args
     uint32_t overwrite;
     uint32_t outVec;  // general kernel: out may be accessed 16 bytes at a time
 };
+
+// Eight consecutive halves from any 2-byte-aligned address, as aligned dwords: a 16-byte load from
+// an address that is no multiple of 4 is several times slower than one from a multiple of 4
+// (measured on the few-tile kernel, 128 x 128 x 4095 against x 4096: 24.4 / 10.5 us).  The five
+// dwords that hold the halves are loaded (four as one access, the fifth on its own) and, for an
+// odd half index, shifted down by 16 bits.  Every dword read holds at least one of the eight
+// halves, so nothing is read that does not share an aligned dword with the operand.  The
+// shift is applied by Get(), where the value is used, so that a load can stay in flight until
+// then.
+struct Halves8
+{
+    uintx4 w;
+    uint32_t extra;
+    __device__ __forceinline__ static Halves8 Load(const _Float16* p)
+    {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        const uint32_t odd = static_cast<uint32_t>(a >> 1) & 1u;
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(a - 2 * odd);
+        typedef uintx4 uintx4a4 __attribute__((aligned(4)));
+        Halves8 h;
+        h.w = *reinterpret_cast<const uintx4a4*>(q);
+        h.extra = q[3 + odd];  // even address: the fourth dword once more
+        return h;
+    }
+    // 16 for halves loaded from an address that is no multiple of 4, else 0
+    __device__ __forceinline__ static uint32_t Shift(const _Float16* p)
+    {
+        return (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)) & 2u) * 8u;
+    }
+    __device__ __forceinline__ halfx8 Get(uint32_t shift) const
+    {
+        uintx4 r;
+        r[0] = __builtin_amdgcn_alignbit(w[1], w[0], shift);
+        r[1] = __builtin_amdgcn_alignbit(w[2], w[1], shift);
+        r[2] = __builtin_amdgcn_alignbit(w[3], w[2], shift);
+        r[3] = __builtin_amdgcn_alignbit(extra, w[3], shift);
+        return __builtin_bit_cast(halfx8, r);
+    }
+};
+
+// Thin strips of a product's last rows and columns that ride along with the launch of its body:
+// the first `padded` workgroups of the grid (a multiple of 8, so that the body's workgroups keep
+// their place among the 8 XCDs) run the few-tile kernel's code, 16 x 16 tiles, on part[0]
+// (blocks[0] of them) and part[1] (blocks[1]), the rest the body's tiles.  A strip's workgroups
+// are short and sit beside the body's on the same compute units, where a launch of their own
+// would start after the body's last tile has finished.
+struct GemmF16Strips
+{
+    GemmF16Args part[2];
+    uint32_t blocks[2];
+    uint32_t padded;
+};
+
+template <int TILE, bool TA, bool TB, int WAVES, bool ODD>
+__device__ __forceinline__ void GemmF16FewBody(const GemmF16Args& args, uint32_t block,
+                                               float* partial);
+
+// The strip a workgroup of a body's launch computes, if it is one of the first `padded`: true,
+// and the workgroup is done.  Otherwise `block` becomes the workgroup's number among the body's.
+// `scratch`: (WAVES - 1) * 256 floats of LDS.
+template <bool TA, bool TB, int WAVES>
+__device__ __forceinline__ bool RunStrip(const GemmF16Strips& strips, uint32_t& block,
+                                         float* scratch)
+{
+    if (block >= strips.padded)
+    {
+        block -= strips.padded;
+        return false;
+    }
+    const uint32_t which = block < strips.blocks[0] ? 0u : 1u;
+    const uint32_t local = block - (which != 0 ? strips.blocks[0] : 0u);
+    if (local < strips.blocks[which])
+        GemmF16FewBody<16, TA, TB, WAVES, true>(strips.part[which], local, scratch);
+    return true;
+}
 
 // Transposing LDS read: within each group of 16 lanes, lane s supplies the
 // address of 4 halves (row s/4 of a 4-row block, columns 4*(s%4)..+3) and
@@ -155,7 +233,6 @@ __device__ __forceinline__ halfx8 Join(halfx4 lo, halfx4 hi)
 // positions (those of group `group`, 8 group .. 8 group + 7); TailMask gives the bits of the
 // ones that are new, KeepNew clears the others.  Both operands are cleared, so that a value
 // that lies in both windows counts once even when it is an infinity.
-typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uintx4 TailMask(uint32_t group, uint32_t repeated)
 {
     uintx4 m;
@@ -270,7 +347,8 @@ constexpr int CLoopSteps(int csp, int rowBlocks = 8)
 // instead of 4 per 4.  The B stage then has k-rows of 256 bytes (the same chunk swizzle) and a
 // wavefront makes two copies of A and one of B per step.
 template <bool RAGGED, int CSP, bool TA, bool TB, bool TAIL, int NT = 256>
-__global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
+__global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args,
+                                                      const GemmF16Strips strips)
 {
     static_assert(NT == 256 || NT == 128, "256 x 256 or 256 x 128 tiles");
     constexpr int WAVES = 8;
@@ -300,7 +378,10 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args)
     };
 
     uint32_t unit, tm, tn;
-    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
+    uint32_t block = blockIdx.x;
+    if (RunStrip<TA, TB, WAVES>(strips, block, reinterpret_cast<float*>(LdsRaw)))
+        return;
+    if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
         return;
 
     const uint32_t tid = threadIdx.x;
@@ -781,7 +862,8 @@ constexpr int kDStageBytes = 2 * kD * kTK * 2;  // A + B
 // TAIL: K = 32 q + r, 0 < r < 32: a last step over the window [K - 32, K) whose slab has the
 // positions of the 32 - r values of k already multiplied cleared in LDS.
 template <bool TA, bool TB, bool TAIL, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args args)
+__global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args args,
+                                                            const GemmF16Strips strips)
 {
     static_assert(WAVES == 4 || WAVES == 8, "2 x 2 or 2 x 4 wavefronts");
     constexpr int WN = WAVES / 2;          // wavefronts across the tile
@@ -792,7 +874,10 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
     constexpr uint32_t kBytesA = kD * kTK * 2;  // 8 KiB
 
     uint32_t unit, tm, tn;
-    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
+    uint32_t block = blockIdx.x;
+    if (RunStrip<TA, TB, WAVES>(strips, block, reinterpret_cast<float*>(lds)))
+        return;
+    if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
         return;
 
     const uint32_t tid = threadIdx.x;
@@ -1101,14 +1186,18 @@ constexpr int kSOperandBytes = kS * kSK * 2;        // 8 KiB
 constexpr int kSStageBytes = 2 * kSOperandBytes;    // A + B
 
 template <bool TA, bool TB, bool TAIL>
-__global__ __launch_bounds__(256) void GemmF16Dma64(const GemmF16Args args)
+__global__ __launch_bounds__(256) void GemmF16Dma64(const GemmF16Args args,
+                                                    const GemmF16Strips strips)
 {
     constexpr int kCopiesPer = 2;            // 1 KiB copies per operand, step and wavefront
     constexpr int kCopies = 2 * kCopiesPer;  // per step and wavefront
     __shared__ __attribute__((aligned(1024))) char lds[kSStages * kSStageBytes];
 
     uint32_t unit, tm, tn;
-    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
+    uint32_t block = blockIdx.x;
+    if (RunStrip<TA, TB, 4>(strips, block, reinterpret_cast<float*>(lds)))
+        return;
+    if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
         return;
 
     const uint32_t tid = threadIdx.x;
@@ -1360,19 +1449,26 @@ constexpr int kGThreads = 256;
 constexpr int kGLda = kGK + 8;   // halves per A row in LDS (80 B)
 constexpr int kGLdb = kG + 32;   // halves per B row in LDS (320 B)
 
-// VEC: halves per global load (8, 4, 2 or 1), the largest power of two that divides K, the row
-// stride of A, N and the alignment of the bases.
+// VEC = 8: K, the row strides, N and the bases are all multiples of 8 halves, so every 8-half
+// piece is 16-byte aligned and lies wholly inside or outside its row.  VEC = 2: multiples of 2
+// halves, VEC = 1: anything; a piece that lies inside its row is still read 16 bytes at a time
+// (one load from a 4-byte-aligned address, or aligned dwords that are shifted, see Halves8),
+// one that straddles the row's end half by half.
 // TA: A is stored K x M; TB: B is stored N x K.  A transposed operand is read along its
 // contiguous dimension like the other one and turned round on its way into LDS (8 two-byte
 // stores per chunk instead of one 16-byte store), so the MFMA side does not change.
 template <int VEC, bool TA, bool TB>
-__global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args args)
+__global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args args,
+                                                            const GemmF16Strips strips)
 {
     __shared__ __attribute__((aligned(16))) _Float16 As[2][kG * kGLda];
     __shared__ __attribute__((aligned(16))) _Float16 Bs[2][kGK * kGLdb];
 
     uint32_t unit, tm, tn;
-    if (!MapTile(blockIdx.x, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
+    uint32_t block = blockIdx.x;
+    if (RunStrip<TA, TB, 4>(strips, block, reinterpret_cast<float*>(&As[0][0])))
+        return;
+    if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
         return;
 
     const uint32_t tid = threadIdx.x;
@@ -1390,9 +1486,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
 
     halfx8 stageA[2], stageB[2];
 
-    // 8 consecutive halves starting at p, of which those with index + first < limit exist; read
-    // in pieces of VEC halves (the row stride and the base are multiples of VEC halves, so a
-    // piece is aligned and lies wholly inside or outside the row)
+    // 8 consecutive halves starting at p, of which those with index + first < limit exist
     auto load8 = [&](const _Float16* p, uint32_t first, uint32_t limit) {
         halfx8 v = { 0, 0, 0, 0, 0, 0, 0, 0 };
         if constexpr (VEC == 8)
@@ -1400,36 +1494,22 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
             if (first < limit)
                 v = *reinterpret_cast<const halfx8*>(p);
         }
-        else if constexpr (VEC == 4)
-        {
-#pragma unroll
-            for (int e = 0; e < 8; e += 4)
-                if (first + e < limit)
-                {
-                    const halfx4 w = *reinterpret_cast<const halfx4*>(p + e);
-                    v[e] = w[0];
-                    v[e + 1] = w[1];
-                    v[e + 2] = w[2];
-                    v[e + 3] = w[3];
-                }
-        }
-        else if constexpr (VEC == 2)
-        {
-#pragma unroll
-            for (int e = 0; e < 8; e += 2)
-                if (first + e < limit)
-                {
-                    const halfx2 w = *reinterpret_cast<const halfx2*>(p + e);
-                    v[e] = w[0];
-                    v[e + 1] = w[1];
-                }
-        }
         else
         {
+            if (first + 8 <= limit)
+            {
+                if constexpr (VEC >= 2)
+                    v = *reinterpret_cast<const halfx8a4*>(p);
+                else
+                    v = Halves8::Load(p).Get(Halves8::Shift(p));
+            }
+            else
+            {
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (first + e < limit)
-                    v[e] = p[e];
+                for (int e = 0; e < 8; ++e)
+                    if (first + e < limit)
+                        v[e] = p[e];
+            }
         }
         return v;
     };
@@ -1610,22 +1690,21 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
     }
 }
 
-typedef halfx8 halfx8a2 __attribute__((aligned(2)));
-
 // variant 0: whole tiles, out read in the epilogue; 1 / 2: out added inside the loop with
 // spacing 2 / 4; 3: ragged tiles
 template <bool TA, bool TB, bool TAIL, int NT>
-void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16Args& args)
+void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16Args& args,
+                   const GemmF16Strips& strips)
 {
     const dim3 g(grid), b(512);
     if (variant == 2)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 4, TA, TB, TAIL, NT>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 4, TA, TB, TAIL, NT>), g, b, 0, stream, args, strips);
     else if (variant == 1)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 2, TA, TB, TAIL, NT>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 2, TA, TB, TAIL, NT>), g, b, 0, stream, args, strips);
     else if (variant == 0)
-        hipLaunchKernelGGL((GemmF16Tile256<false, 0, TA, TB, TAIL, NT>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<false, 0, TA, TB, TAIL, NT>), g, b, 0, stream, args, strips);
     else
-        hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB, TAIL, NT>), g, b, 0, stream, args);
+        hipLaunchKernelGGL((GemmF16Tile256<true, 0, TA, TB, TAIL, NT>), g, b, 0, stream, args, strips);
 }
 
 // ---------------------------------------------------------------------------
@@ -1636,14 +1715,20 @@ void LaunchTile256(int variant, uint32_t grid, hipStream_t stream, const GemmF16
 // kernels, and each of their workgroups then waits out a memory latency per K step (128 x 1024
 // x 1024: 10.6 us on 8 compute units).  Here every wavefront reads its fragments straight from
 // global memory in MFMA layout - lane l holds row (column) l % TILE and the 8 values
-// k = kGroupK g + 8 (l / TILE) .. + 7 of group g: one 16-byte load from an operand stored with K
-// contiguous (any 2-byte-aligned address), eight 2-byte loads `ld` apart from one stored
-// k-major - keeps the loads of several groups in flight, and accumulates a private TILE x TILE
+// k = kGroupK g + 8 (l / TILE) .. + 7 of group g: 16 bytes from an operand stored with K
+// contiguous (any 2-byte-aligned address, see ODD below), eight 2-byte loads `ld` apart from one
+// stored k-major - keeps the loads of several groups in flight, and accumulates a private TILE x TILE
 // partial over its share of K.  The partials are added in wavefront order through LDS, so the
 // result does not depend on timing, and the k assignment is the same for every storage order,
 // so it does not depend on the flags either.  Any M, N, K, pitch and alignment.
-template <int TILE, bool TA, bool TB, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
+// ODD: rows of an operand stored with K contiguous may start at an odd half (any pitch, any
+// base): they are read as aligned dwords and shifted.  Otherwise they start at multiples of 4
+// bytes and a lane's 8 halves are one 16-byte load: two thirds of the loads (128 x 128 x 4096:
+// 10.5 us against 15.8).  A product's strips always take the first form.
+// `partial`: (WAVES - 1) * TILE * TILE floats of LDS
+template <int TILE, bool TA, bool TB, int WAVES, bool ODD>
+__device__ __forceinline__ void GemmF16FewBody(const GemmF16Args& args, uint32_t block,
+                                               float* partial)
 {
     static_assert(TILE == 32 || TILE == 16, "MFMA shapes 32x32x16 and 16x16x32");
     constexpr uint32_t kLaneGroups = 64 / TILE;     // groups of TILE lanes
@@ -1652,14 +1737,12 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
     constexpr int kQuads = kAcc / 4;
     using Acc = typename std::conditional<TILE == 32, floatx16, floatx4>::type;
 
-    __shared__ float partial[WAVES - 1][TILE * TILE];
-
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t lt = lane % TILE;  // row of A / column of B this lane feeds
     const uint32_t kh = lane / TILE;  // which 8 values of k of an MFMA
 
-    uint32_t id = blockIdx.x;
+    uint32_t id = block;
     const uint32_t tn = id % args.tilesN;
     id /= args.tilesN;
     const uint32_t tm = id % args.tilesM;
@@ -1689,15 +1772,21 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
     // operand stored k-major stay in a register each while they are in flight and are packed
     // where they are used: packed where they are loaded, every round would end with a wait for
     // its last load.
-    struct AlongK
+    struct AlongKOdd
+    {
+        Halves8 h;
+        __device__ __forceinline__ halfx8 get(uint32_t shift) const { return h.Get(shift); }
+    };
+    struct AlongKEven
     {
         halfx8 v;
-        __device__ __forceinline__ halfx8 get() const { return v; }
+        __device__ __forceinline__ halfx8 get(uint32_t) const { return v; }
     };
+    using AlongK = typename std::conditional<ODD, AlongKOdd, AlongKEven>::type;
     struct AcrossK
     {
         uint32_t r[8];
-        __device__ __forceinline__ halfx8 get() const
+        __device__ __forceinline__ halfx8 get(uint32_t) const
         {
             uintx4 w;
 #pragma unroll
@@ -1706,11 +1795,18 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
             return __builtin_bit_cast(halfx8, w);
         }
     };
+    // (a group is a whole number of dwords on from the operand's first one, so one shift serves
+    // every group of a lane)
+    const uint32_t aShift = Halves8::Shift(aPtr + kh * 8);
+    const uint32_t bShift = Halves8::Shift(bPtr + kh * 8);
     using FragA = typename std::conditional<TA, AcrossK, AlongK>::type;
     using FragB = typename std::conditional<TB, AlongK, AcrossK>::type;
     auto loadAlongK = [&](const _Float16* rowPtr, uint32_t g) {
         AlongK f;
-        f.v = *reinterpret_cast<const halfx8a2*>(rowPtr + (g * kGroupK + kh * 8));
+        if constexpr (ODD)
+            f.h = Halves8::Load(rowPtr + (g * kGroupK + kh * 8));
+        else
+            f.v = *reinterpret_cast<const halfx8a4*>(rowPtr + (g * kGroupK + kh * 8));
         return f;
     };
     auto loadAcrossK = [&](const _Float16* colPtr, size_t ld, uint32_t g) {
@@ -1778,7 +1874,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
                 // multiply, then load the group kDepth further on into the same registers
                 // (loading first needs a second set and a copy, behind a wait for every load,
                 // at the end of each round); the fences keep that order
-                multiply(fa[d].get(), fb[d].get());
+                multiply(fa[d].get(aShift), fb[d].get(bShift));
                 __builtin_amdgcn_sched_barrier(0);
                 const uint32_t next = sph::KPartitionNext(part, g, kDepth, d);
                 fa[d] = loadA(next);
@@ -1790,7 +1886,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
 #pragma unroll
         for (int d = 0; d < kDepth - 1; ++d)
             if (roundsEnd + d < wholeEnd)
-                multiply(fa[d].get(), fb[d].get());
+                multiply(fa[d].get(aShift), fb[d].get(bShift));
     }
     if (part.ownsPartial)
     {
@@ -1807,7 +1903,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
 #pragma unroll
         for (int q = 0; q < kQuads; ++q)
             *reinterpret_cast<float4*>(
-                &partial[wave - 1][lt * TILE + 4 * kLaneGroups * q + 4 * kh]) =
+                &partial[(wave - 1) * TILE * TILE + lt * TILE + 4 * kLaneGroups * q + 4 * kh]) =
                 make_float4(acc[4 * q + 0], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
     }
     __syncthreads();
@@ -1819,7 +1915,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
         for (int q = 0; q < kQuads; ++q)
         {
             const float4 p = *reinterpret_cast<const float4*>(
-                &partial[w][lt * TILE + 4 * kLaneGroups * q + 4 * kh]);
+                &partial[w * TILE * TILE + lt * TILE + 4 * kLaneGroups * q + 4 * kh]);
             acc[4 * q + 0] += p.x;
             acc[4 * q + 1] += p.y;
             acc[4 * q + 2] += p.z;
@@ -1854,6 +1950,14 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
                     p[e] = args.overwrite ? acc[4 * q + e] : p[e] + acc[4 * q + e];
         }
     }
+}
+
+template <int TILE, bool TA, bool TB, int WAVES, bool ODD>
+__global__ __launch_bounds__(WAVES * 64) void GemmF16Few(const GemmF16Args args)
+{
+    static_assert(!ODD || !TA || TB, "no operand with K contiguous: one form");
+    __shared__ __attribute__((aligned(16))) float partial[(WAVES - 1) * TILE * TILE];
+    GemmF16FewBody<TILE, TA, TB, WAVES, ODD>(args, blockIdx.x, partial);
 }
 
 // What one launch may assume about where its operands lie.
@@ -1926,9 +2030,10 @@ F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16
     return F16Kernel::kGeneral;
 }
 
-// One launch over all of args.N columns with the kernel `kind`.
+// One launch over all of args.N columns with the kernel `kind`; the workgroups of `strips` come
+// first in its grid.
 int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16Layout& lay,
-                    hipStream_t stream)
+                    const GemmF16Strips& strips, hipStream_t stream)
 {
     const uint32_t M = args.M, N = args.N, K = args.K;
     const bool transA = lay.transA, transB = lay.transB;
@@ -1943,7 +2048,7 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     const uint64_t total = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
     SPH_REQUIRE(total < (1ull << 31) - 8, "too many tiles for one launch");
     args.totalTiles = static_cast<uint32_t>(total);
-    const uint32_t grid = ((args.totalTiles + 7) / 8) * 8;
+    const uint32_t grid = ((args.totalTiles + 7) / 8) * 8 + strips.padded;
 
     if (tile256)
     {
@@ -1960,13 +2065,13 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     do                                                                                            \
     {                                                                                             \
         if (tail && half)                                                                         \
-            LaunchTile256<TA_, TB_, true, 128>(variant, grid, stream, args);                      \
+            LaunchTile256<TA_, TB_, true, 128>(variant, grid, stream, args, strips);                      \
         else if (tail)                                                                            \
-            LaunchTile256<TA_, TB_, true, 256>(variant, grid, stream, args);                      \
+            LaunchTile256<TA_, TB_, true, 256>(variant, grid, stream, args, strips);                      \
         else if (half)                                                                            \
-            LaunchTile256<TA_, TB_, false, 128>(variant, grid, stream, args);                     \
+            LaunchTile256<TA_, TB_, false, 128>(variant, grid, stream, args, strips);                     \
         else                                                                                      \
-            LaunchTile256<TA_, TB_, false, 256>(variant, grid, stream, args);                     \
+            LaunchTile256<TA_, TB_, false, 256>(variant, grid, stream, args, strips);                     \
     } while (0)
         if (transA && transB)
             SPH_TILE256(true, true);
@@ -1985,15 +2090,15 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         const uint64_t tiles = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
         SPH_REQUIRE(tiles < (1ull << 31) - 8, "too many tiles for one launch");
         args.totalTiles = static_cast<uint32_t>(tiles);
-        const dim3 g(((args.totalTiles + 7) / 8) * 8), b(256);
+        const dim3 g(((args.totalTiles + 7) / 8) * 8 + strips.padded), b(256);
         const bool tail = K % kSK != 0;
 #define SPH_DMA64(TA_, TB_)                                                                       \
     do                                                                                            \
     {                                                                                             \
         if (tail)                                                                                 \
-            hipLaunchKernelGGL((GemmF16Dma64<TA_, TB_, true>), g, b, 0, stream, args);            \
+            hipLaunchKernelGGL((GemmF16Dma64<TA_, TB_, true>), g, b, 0, stream, args, strips);            \
         else                                                                                      \
-            hipLaunchKernelGGL((GemmF16Dma64<TA_, TB_, false>), g, b, 0, stream, args);           \
+            hipLaunchKernelGGL((GemmF16Dma64<TA_, TB_, false>), g, b, 0, stream, args, strips);           \
     } while (0)
         if (transA && transB)
             SPH_DMA64(true, true);
@@ -2021,10 +2126,10 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     {                                                                                             \
         if (wide)                                                                                 \
             hipLaunchKernelGGL((GemmF16Dma128<TA_, TB_, TAIL_, 8>), g, dim3(512), 0, stream,      \
-                               args);                                                             \
+                               args, strips);                                                             \
         else                                                                                      \
             hipLaunchKernelGGL((GemmF16Dma128<TA_, TB_, TAIL_, 4>), g, dim3(256), 0, stream,      \
-                               args);                                                             \
+                               args, strips);                                                             \
     } while (0)
 #define SPH_DMA128(TA_, TB_)                                                                      \
     do                                                                                            \
@@ -2065,107 +2170,201 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         if (plain)
         {
             if (vec == 8)
-                hipLaunchKernelGGL((GemmF16General<8, false, false>), g, b, 0, stream, args);
-            else if (vec == 4)
-                hipLaunchKernelGGL((GemmF16General<4, false, false>), g, b, 0, stream, args);
-            else if (vec == 2)
-                hipLaunchKernelGGL((GemmF16General<2, false, false>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<8, false, false>), g, b, 0, stream, args,
+                                   strips);
+            else if (vec >= 2)
+                hipLaunchKernelGGL((GemmF16General<2, false, false>), g, b, 0, stream, args,
+                                   strips);
             else
-                hipLaunchKernelGGL((GemmF16General<1, false, false>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<1, false, false>), g, b, 0, stream, args,
+                                   strips);
         }
         else if (vec == 8)
         {
-            // transposed operands: 16-byte loads or single halves
             if (transA && transB)
-                hipLaunchKernelGGL((GemmF16General<8, true, true>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<8, true, true>), g, b, 0, stream, args, strips);
             else if (transA)
-                hipLaunchKernelGGL((GemmF16General<8, true, false>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<8, true, false>), g, b, 0, stream, args, strips);
             else
-                hipLaunchKernelGGL((GemmF16General<8, false, true>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<8, false, true>), g, b, 0, stream, args, strips);
         }
         else
         {
             if (transA && transB)
-                hipLaunchKernelGGL((GemmF16General<1, true, true>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<1, true, true>), g, b, 0, stream, args, strips);
             else if (transA)
-                hipLaunchKernelGGL((GemmF16General<1, true, false>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<1, true, false>), g, b, 0, stream, args, strips);
             else
-                hipLaunchKernelGGL((GemmF16General<1, false, true>), g, b, 0, stream, args);
+                hipLaunchKernelGGL((GemmF16General<1, false, true>), g, b, 0, stream, args, strips);
         }
     }
     SPH_CHECK_LAUNCH();
     return SPH_OK;
 }
 
-// Picks the kernels for one call.
-//
-// N = 8 q + r with r != 0 and a shape the straight-to-LDS kernels would take at N = 8 q: they
-// compute the first 8 q columns (row pitches of B and out stay N) and the few-tile kernel, which
-// reads any rows and columns from anywhere, the last r (measured 4096 x 4100 x 4096: 270 us on
-// the general kernel alone, 129 us this way).
-//
-// An A stored K x M is copied 8 rows of the product at a time, so with it M = 8 q + r is split
-// the same way: the first 8 q rows, then the few-tile kernel over the last r rows.  Every output
-// element is still computed by one kernel.
+// Picks the kernels for one call: a body for one of the kernels above and up to two thin strips
+// of the product's last rows and columns, which the few-tile kernel's code computes (it reads any
+// rows and columns from anywhere) on the first workgroups of the body's launch.  Every output
+// element is computed once.  Cut off are
+//  - the last N % 8 columns, when a straight-to-LDS kernel then takes the rest (its copies are 8
+//    columns wide; row pitches of B and out stay N; measured 4096 x 4100 x 4096: 270 us on the
+//    general kernel alone, 129 us with the strip in a launch of its own);
+//  - the last M % 8 rows of an A stored K x M, likewise (it is copied 8 rows of the product at a
+//    time);
+//  - up to 16 rows or columns past a multiple of the tile edge, when the compute unit with the
+//    most tiles then has fewer of them (1025^3: 17 x 17 tiles of 64 are two per compute unit
+//    somewhere, 16 x 16 one everywhere).
 int LaunchFewTiles(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream);
+
+// Tiles of the kernel `kind` over M x N and what one costs, in hundredths of the time a 64 x 64
+// tile takes on the 256-tile kernel (measured rates: the smaller the tile, the more LDS traffic
+// and fixed cost per flop).
+uint64_t F16Cost(F16Kernel kind, uint32_t M, uint32_t N, uint32_t batch)
+{
+    const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
+    uint32_t edgeM = kG, edgeN = kG;
+    uint64_t perTile = 1200;  // general kernel, 128 x 128
+    switch (kind)
+    {
+    case F16Kernel::kTile256: edgeM = edgeN = kT; perTile = 1600; break;
+    case F16Kernel::kTile256x128: edgeM = kT; edgeN = 128; perTile = 920; break;
+    case F16Kernel::kDma128: perTile = 760; break;
+    case F16Kernel::kDma64: edgeM = edgeN = kS; perTile = 220; break;
+    case F16Kernel::kGeneral: break;
+    }
+    const uint64_t tiles =
+        static_cast<uint64_t>((M + edgeM - 1) / edgeM) * ((N + edgeN - 1) / edgeN) * batch;
+    return (tiles + cus - 1) / cus * perTile;
+}
 
 int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_t stream)
 {
     const uint32_t M = args.M, N = args.N;
-    const F16Kernel whole = PickF16(args, N, batch, lay);
-    if (whole != F16Kernel::kGeneral)
-        return LaunchF16Kernel(args, batch, whole, lay, stream);
-
-    // A stored K x M with M = 8 q + r, r != 0: the first 8 q rows as a product of their own (if
-    // a straight-to-LDS kernel then takes them), the last r rows on the few-tile kernel, which
-    // reads any rows from anywhere
-    if (lay.transA && M % 8 != 0 && M >= 16 && (N & ~7u) >= 8)
-    {
-        GemmF16Args top = args;
-        top.M = M & ~7u;
-        if (PickF16(top, N & ~7u, batch, lay) != F16Kernel::kGeneral)
+    const uint64_t cus = static_cast<uint64_t>(sph::ComputeUnits());
+    // candidates for the rows (columns) cut off: none, the remainder the copies cannot take, and
+    // the remainders past a tile edge
+    auto candidates = [](uint32_t x, uint32_t unit, bool unitAllowed, uint32_t* list) {
+        int n = 0;
+        list[n++] = 0;
+        if (unitAllowed && x % unit != 0 && x > 2 * unit)
+            list[n++] = x % unit;
+        for (uint32_t edge = 64; edge <= 256; edge *= 2)
         {
-            GemmF16Args bottom = args;
-            bottom.M = M % 8;
-            bottom.A = args.A + top.M;
-            bottom.out = args.out + static_cast<size_t>(top.M) * args.ldc;
-            const int rc = LaunchF16(top, batch, lay, stream);
-            return rc != SPH_OK ? rc : LaunchFewTiles(bottom, batch, lay, stream);
+            const uint32_t r = x % edge;
+            bool seen = false;
+            for (int i = 0; i < n; ++i)
+                seen = seen || list[i] == r;
+            if (r != 0 && r <= 16 && x - r >= edge && !seen)
+                list[n++] = r;
         }
-    }
+        return n;
+    };
+    uint32_t listM[5], listN[5];
+    const int countM = candidates(M, 8, lay.transA, listM);
+    const int countN = candidates(N, 8, true, listN);
+    // a strip's 16 x 16 tile: a sixteenth of a 64-tile's flops at about a quarter of its rate
+    auto stripCost = [&](uint32_t rows, uint32_t cols) {
+        const uint64_t blocks =
+            static_cast<uint64_t>((rows + 15) / 16) * ((cols + 15) / 16) * batch;
+        return (blocks + cus - 1) / cus * 60;
+    };
+    uint64_t best = ~0ull;
+    uint32_t peelM = 0, peelN = 0;
+    F16Kernel kind = F16Kernel::kGeneral;
+    for (int i = 0; i < countM; ++i)
+        for (int j = 0; j < countN; ++j)
+        {
+            GemmF16Args body = args;
+            body.M = M - listM[i];
+            const uint32_t bodyN = N - listN[j];
+            const F16Kernel k = PickF16(body, bodyN, batch, lay);
+            uint64_t cost = F16Cost(k, body.M, bodyN, batch);
+            if (listM[i] != 0)
+                cost += stripCost(listM[i], N);
+            if (listN[j] != 0)
+                cost += stripCost(body.M, listN[j]);
+            if (cost < best)
+            {
+                best = cost;
+                peelM = listM[i];
+                peelN = listN[j];
+                kind = k;
+            }
+        }
 
-    const uint32_t wholeChunks = N & ~7u;
-    if (N % 8 == 0)
-        return LaunchF16Kernel(args, batch, whole, lay, stream);
-    // fewer than 8 columns, or no straight-to-LDS kernel for the first 8 q: one kernel for all
-    if (wholeChunks == 0)
-        return LaunchFewTiles(args, batch, lay, stream);
-    const F16Kernel most = PickF16(args, wholeChunks, batch, lay);
-    if (most == F16Kernel::kGeneral)
-        return LaunchF16Kernel(args, batch, whole, lay, stream);
-    GemmF16Args left = args;
-    left.N = wholeChunks;
-    const int rc = LaunchF16Kernel(left, batch, most, lay, stream);
-    if (rc != SPH_OK)
-        return rc;
-    GemmF16Args right = args;
-    right.N = N - wholeChunks;
-    right.out = args.out + wholeChunks;
-    right.B = args.B + (lay.transB ? static_cast<size_t>(wholeChunks) * args.K : wholeChunks);
-    return LaunchFewTiles(right, batch, lay, stream);
+    GemmF16Strips strips{};
+    int count = 0;
+    auto addStrip = [&](GemmF16Args strip) {
+        strip.tilesM = (strip.M + 15) / 16;
+        strip.tilesN = (strip.N + 15) / 16;
+        const uint64_t blocks = static_cast<uint64_t>(strip.tilesM) * strip.tilesN * batch;
+        if (blocks >= (1ull << 30))
+            return false;
+        strips.part[count] = strip;
+        strips.blocks[count] = static_cast<uint32_t>(blocks);
+        ++count;
+        strips.padded = (strips.blocks[0] + strips.blocks[1] + 7u) & ~7u;
+        return true;
+    };
+    GemmF16Args body = args;
+    body.M = M - peelM;
+    body.N = N - peelN;
+    if (peelM != 0)
+    {
+        // rows [M - peelM, M), every column
+        GemmF16Args bottom = args;
+        bottom.M = peelM;
+        bottom.A = args.A + (lay.transA ? body.M : static_cast<size_t>(body.M) * args.lda);
+        bottom.out = args.out + static_cast<size_t>(body.M) * args.ldc;
+        SPH_REQUIRE(addStrip(bottom), "too many tiles for one launch");
+    }
+    if (peelN != 0)
+    {
+        // rows [0, M - peelM), columns [N - peelN, N)
+        GemmF16Args right = args;
+        right.M = body.M;
+        right.N = peelN;
+        right.B = args.B + (lay.transB ? static_cast<size_t>(body.N) * args.K : body.N);
+        right.out = args.out + body.N;
+        SPH_REQUIRE(addStrip(right), "too many tiles for one launch");
+    }
+    return LaunchF16Kernel(body, batch, kind, lay, strips, stream);
+}
+
+template <bool TA, bool TB, bool ODD>
+void LaunchFewForm(const GemmF16Args& args, uint32_t blocks, uint32_t tile, bool wide,
+                   hipStream_t stream)
+{
+    const dim3 g(blocks);
+    if (tile == 16 && wide)
+        hipLaunchKernelGGL((GemmF16Few<16, TA, TB, 16, ODD>), g, dim3(1024), 0, stream, args);
+    else if (tile == 16)
+        hipLaunchKernelGGL((GemmF16Few<16, TA, TB, 4, ODD>), g, dim3(256), 0, stream, args);
+    else
+        hipLaunchKernelGGL((GemmF16Few<32, TA, TB, 4, ODD>), g, dim3(256), 0, stream, args);
 }
 
 template <bool TA, bool TB>
 void LaunchFew(const GemmF16Args& args, uint32_t blocks, uint32_t tile, bool wide,
                hipStream_t stream)
 {
-    const dim3 g(blocks);
-    if (tile == 16 && wide)
-        hipLaunchKernelGGL((GemmF16Few<16, TA, TB, 16>), g, dim3(1024), 0, stream, args);
-    else if (tile == 16)
-        hipLaunchKernelGGL((GemmF16Few<16, TA, TB, 4>), g, dim3(256), 0, stream, args);
-    else
-        hipLaunchKernelGGL((GemmF16Few<32, TA, TB, 4>), g, dim3(256), 0, stream, args);
+    // do the rows of an operand stored with K contiguous all start at multiples of 4 bytes?
+    uint64_t mix = 0;
+    if (!TA)
+        mix |= args.lda | static_cast<uint64_t>(args.strideA) |
+               (reinterpret_cast<uintptr_t>(args.A) / 2);
+    if (TB)
+        mix |= args.K | static_cast<uint64_t>(args.strideB) |
+               (reinterpret_cast<uintptr_t>(args.B) / 2);
+    if constexpr (!TA || TB)
+    {
+        if ((mix & 1u) != 0)
+        {
+            LaunchFewForm<TA, TB, true>(args, blocks, tile, wide, stream);
+            return;
+        }
+    }
+    LaunchFewForm<TA, TB, false>(args, blocks, tile, wide, stream);
 }
 
 // Products with at most one 32 x 32 output tile per compute unit, and narrow ones (16 rows or
