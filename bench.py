@@ -442,7 +442,8 @@ SMALL = [(256, 1024, 1024), (100, 1024, 784), (1024, 10, 1024), (128, 128, 4096)
 OFF_GRID_F16 = [(4096, 4096, 4096), (4096, 4096, 4080), (4096, 4096, 4095), (4096, 4100, 4096),
                 (4096, 4095, 4096), (4095, 4095, 4095), (2048, 2052, 2048), (1024, 1024, 1001),
                 (1024, 1024, 1024), (1024, 1024, 4096), (2048, 2048, 2048), (3072, 2048, 2048),
-                (2048, 4096, 2048), (1025, 1025, 1025)] + SMALL
+                (2048, 4096, 2048), (1025, 1025, 1025), (1001, 1001, 1001), (4097, 4097, 4097),
+                (128, 128, 4095)] + SMALL
 OFF_GRID_F32 = [(1024, 1024, 1024), (1024, 1024, 1000), (1024, 1024, 1001), (1000, 1000, 1000),
                 (1001, 1001, 1001), (1024, 1026, 1024), (2048, 2048, 2047), (2048, 2050, 2048),
                 (4096, 4096, 4096), (4096, 4095, 4096), (4096, 4096, 4100), (1025, 1025, 1025),

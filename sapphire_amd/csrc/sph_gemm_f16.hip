@@ -124,38 +124,40 @@ struct Halves8
 };
 
 // Thin strips of a product's last rows and columns that ride along with the launch of its body:
-// the first `padded` workgroups of the grid (a multiple of 8, so that the body's workgroups keep
-// their place among the 8 XCDs) run the few-tile kernel's code, 16 x 16 tiles, on part[0]
-// (blocks[0] of them) and part[1] (blocks[1]), the rest the body's tiles.  A strip's workgroups
-// are short and sit beside the body's on the same compute units, where a launch of their own
-// would start after the body's last tile has finished.
+// the workgroups from `first` on (the body's own come before, so they keep their numbers and with
+// them their place among the 8 XCDs) run the few-tile kernel's code, 16 x 16 tiles, on part[0]
+// (blocks[0] of them) and then part[1] (blocks[1]).  A strip's workgroups are short; coming last
+// they fill the places that the body's last tiles leave free, where a launch of their own would
+// start after the body's last tile has finished.
 struct GemmF16Strips
 {
     GemmF16Args part[2];
     uint32_t blocks[2];
-    uint32_t padded;
+    uint32_t first;  // launcher: the number of the body's workgroups
 };
 
 template <int TILE, bool TA, bool TB, int WAVES, bool ODD>
 __device__ __forceinline__ void GemmF16FewBody(const GemmF16Args& args, uint32_t block,
                                                float* partial);
 
-// The strip a workgroup of a body's launch computes, if it is one of the first `padded`: true,
-// and the workgroup is done.  Otherwise `block` becomes the workgroup's number among the body's.
-// `scratch`: (WAVES - 1) * 256 floats of LDS.
+// Tile edge of the strips.  (A kernel of eight wavefronts keeps one or two workgroups on a compute
+// unit and its strips' workgroups take such a place each; 32 x 32 tiles would halve their number
+// but load twice the rows each, and measured slower: 2048 x 2052 x 2048 31.6 -> 41.2 us,
+// 4096 x 4100 x 4096 129 -> 144 us.)
+constexpr uint32_t kStripTile = 16;
+
+// The strip a workgroup of a body's launch computes, if it is one of those from `first` on: true,
+// and the workgroup is done.  `scratch`: (WAVES - 1) * kStripTile^2 floats of LDS.
 template <bool TA, bool TB, int WAVES>
-__device__ __forceinline__ bool RunStrip(const GemmF16Strips& strips, uint32_t& block,
+__device__ __forceinline__ bool RunStrip(const GemmF16Strips& strips, uint32_t block,
                                          float* scratch)
 {
-    if (block >= strips.padded)
-    {
-        block -= strips.padded;
+    if (block < strips.first)
         return false;
-    }
-    const uint32_t which = block < strips.blocks[0] ? 0u : 1u;
-    const uint32_t local = block - (which != 0 ? strips.blocks[0] : 0u);
-    if (local < strips.blocks[which])
-        GemmF16FewBody<16, TA, TB, WAVES, true>(strips.part[which], local, scratch);
+    const uint32_t local = block - strips.first;
+    const uint32_t which = local < strips.blocks[0] ? 0u : 1u;
+    GemmF16FewBody<static_cast<int>(kStripTile), TA, TB, WAVES, true>(
+        strips.part[which], local - (which != 0 ? strips.blocks[0] : 0u), scratch);
     return true;
 }
 
@@ -378,7 +380,7 @@ __global__ __launch_bounds__(512) void GemmF16Tile256(const GemmF16Args args,
     };
 
     uint32_t unit, tm, tn;
-    uint32_t block = blockIdx.x;
+    const uint32_t block = blockIdx.x;
     if (RunStrip<TA, TB, WAVES>(strips, block, reinterpret_cast<float*>(LdsRaw)))
         return;
     if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
@@ -874,7 +876,7 @@ __global__ __launch_bounds__(WAVES * 64) void GemmF16Dma128(const GemmF16Args ar
     constexpr uint32_t kBytesA = kD * kTK * 2;  // 8 KiB
 
     uint32_t unit, tm, tn;
-    uint32_t block = blockIdx.x;
+    const uint32_t block = blockIdx.x;
     if (RunStrip<TA, TB, WAVES>(strips, block, reinterpret_cast<float*>(lds)))
         return;
     if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
@@ -1194,7 +1196,7 @@ __global__ __launch_bounds__(256) void GemmF16Dma64(const GemmF16Args args,
     __shared__ __attribute__((aligned(1024))) char lds[kSStages * kSStageBytes];
 
     uint32_t unit, tm, tn;
-    uint32_t block = blockIdx.x;
+    const uint32_t block = blockIdx.x;
     if (RunStrip<TA, TB, 4>(strips, block, reinterpret_cast<float*>(lds)))
         return;
     if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
@@ -1465,7 +1467,7 @@ __global__ __launch_bounds__(kGThreads) void GemmF16General(const GemmF16Args ar
     __shared__ __attribute__((aligned(16))) _Float16 Bs[2][kGK * kGLdb];
 
     uint32_t unit, tm, tn;
-    uint32_t block = blockIdx.x;
+    const uint32_t block = blockIdx.x;
     if (RunStrip<TA, TB, 4>(strips, block, reinterpret_cast<float*>(&As[0][0])))
         return;
     if (!MapTile(block, args.tilesM, args.tilesN, args.totalTiles, unit, tm, tn))
@@ -2030,10 +2032,10 @@ F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16
     return F16Kernel::kGeneral;
 }
 
-// One launch over all of args.N columns with the kernel `kind`; the workgroups of `strips` come
-// first in its grid.
+// One launch over all of args.N columns with the kernel `kind`; the workgroups of the strips
+// `ride` come last in its grid.
 int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16Layout& lay,
-                    const GemmF16Strips& strips, hipStream_t stream)
+                    const GemmF16Strips& ride, hipStream_t stream)
 {
     const uint32_t M = args.M, N = args.N, K = args.K;
     const bool transA = lay.transA, transB = lay.transB;
@@ -2048,7 +2050,9 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
     const uint64_t total = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
     SPH_REQUIRE(total < (1ull << 31) - 8, "too many tiles for one launch");
     args.totalTiles = static_cast<uint32_t>(total);
-    const uint32_t grid = ((args.totalTiles + 7) / 8) * 8 + strips.padded;
+    GemmF16Strips strips = ride;
+    strips.first = ((args.totalTiles + 7) / 8) * 8;
+    const uint32_t grid = strips.first + strips.blocks[0] + strips.blocks[1];
 
     if (tile256)
     {
@@ -2090,7 +2094,8 @@ int LaunchF16Kernel(GemmF16Args args, uint32_t batch, F16Kernel kind, const F16L
         const uint64_t tiles = static_cast<uint64_t>(args.tilesM) * args.tilesN * batch;
         SPH_REQUIRE(tiles < (1ull << 31) - 8, "too many tiles for one launch");
         args.totalTiles = static_cast<uint32_t>(tiles);
-        const dim3 g(((args.totalTiles + 7) / 8) * 8 + strips.padded), b(256);
+        strips.first = ((args.totalTiles + 7) / 8) * 8;
+        const dim3 g(strips.first + strips.blocks[0] + strips.blocks[1]), b(256);
         const bool tail = K % kSK != 0;
 #define SPH_DMA64(TA_, TB_)                                                                       \
     do                                                                                            \
@@ -2295,15 +2300,14 @@ int LaunchF16(GemmF16Args args, uint32_t batch, const F16Layout& lay, hipStream_
     GemmF16Strips strips{};
     int count = 0;
     auto addStrip = [&](GemmF16Args strip) {
-        strip.tilesM = (strip.M + 15) / 16;
-        strip.tilesN = (strip.N + 15) / 16;
+        strip.tilesM = (strip.M + kStripTile - 1) / kStripTile;
+        strip.tilesN = (strip.N + kStripTile - 1) / kStripTile;
         const uint64_t blocks = static_cast<uint64_t>(strip.tilesM) * strip.tilesN * batch;
         if (blocks >= (1ull << 30))
             return false;
         strips.part[count] = strip;
         strips.blocks[count] = static_cast<uint32_t>(blocks);
         ++count;
-        strips.padded = (strips.blocks[0] + strips.blocks[1] + 7u) & ~7u;
         return true;
     };
     GemmF16Args body = args;

@@ -82,16 +82,17 @@ struct GemmF32Args
 };
 
 // Thin strips of a product's last rows and columns that ride along with the launch of its body:
-// the first `padded` workgroups of the grid (a multiple of 8, so that the body's workgroups keep
-// their place among the 8 XCDs) run the few-tile kernel's code on part[0] (blocks[0] of them) and
-// part[1] (blocks[1]), the rest the body's tiles.  A strip's workgroups are short and sit beside
-// the body's on the same compute units, where a launch of their own would start after the
-// body's last tile has finished.
+// the workgroups from `first` on (the body's own come before, so they keep their numbers and with
+// them their place among the 8 XCDs) run the few-tile kernel's code on part[0] (blocks[0] of
+// them) and then part[1] (blocks[1]).  A strip's workgroups are short; coming last they fill the
+// places that the body's last tiles leave free, where a launch of their own would start after the
+// body's last tile has finished.  (Placed first they cost a large product a round of tiles on
+// some compute units: 4096 x 4095 x 4096 with B stored N x K 931 -> 1147 us.)
 struct GemmF32Strips
 {
     GemmF32Args part[2];
     uint32_t blocks[2];
-    uint32_t padded;
+    uint32_t first;  // launcher: the number of the body's workgroups
 };
 
 // Slab loaders.  An operand is stored either with K contiguous (A as given, B when it is
@@ -627,20 +628,20 @@ __global__ __launch_bounds__(((BN >= 64) ? 4 : 2) * KSPLIT * 64) void GemmF32Dma
 
     __shared__ __attribute__((aligned(1024))) char lds[STAGES * kStageBytes];
 
-    // strips of the product's edge come first in the grid (a walk has none)
-    uint32_t block = blockIdx.x;
+    // strips of the product's edge come last in the grid (a walk has none)
+    const uint32_t block = blockIdx.x;
     if constexpr (!WALK)
     {
         static_assert(NW == 4, "the strips' code runs on four wavefronts");
-        if (block < strips.padded)
+        if (block >= strips.first)
         {
-            if (block < strips.blocks[0])
-                GemmF32SkinnyBody<16, TA, TB, 4>(strips.part[0], block);
-            else if (block - strips.blocks[0] < strips.blocks[1])
-                GemmF32SkinnyBody<16, TA, TB, 4>(strips.part[1], block - strips.blocks[0]);
+            const uint32_t local = block - strips.first;
+            if (local < strips.blocks[0])
+                GemmF32SkinnyBody<16, TA, TB, 4>(strips.part[0], local);
+            else
+                GemmF32SkinnyBody<16, TA, TB, 4>(strips.part[1], local - strips.blocks[0]);
             return;
         }
-        block -= strips.padded;
     }
 
     const uint32_t tid = threadIdx.x;
@@ -1765,7 +1766,6 @@ int AddStrip(GemmF32Args strip, uint32_t units, bool outOffsetsAligned, bool tra
         {
             pending->part[i] = strip;
             pending->blocks[i] = static_cast<uint32_t>(blocks);
-            pending->padded = (pending->blocks[0] + pending->blocks[1] + 7u) & ~7u;
             return SPH_OK;
         }
     return LaunchStrip(strip, static_cast<uint32_t>(blocks), transA, transB, stream);
@@ -2022,13 +2022,14 @@ int LaunchPart(const GemmF32Args& base, uint32_t units, bool allowVector, bool o
                       (reinterpret_cast<uintptr_t>(args.bias) & 15u) == 0;
     // strips that wait ride along with a straight-to-LDS launch that is no walk
     GemmF32Strips strips{};
-    if (pending != nullptr && dma && !walk && pending->padded != 0 &&
-        blocks + pending->padded < (1ull << 31) - 8)
+    if (pending != nullptr && dma && !walk && pending->blocks[0] != 0 &&
+        blocks + pending->blocks[0] + pending->blocks[1] < (1ull << 31) - 8)
     {
         strips = *pending;
         *pending = GemmF32Strips{};
     }
-    const dim3 grid((walk ? std::min(slotsPerXcd, args.perXcd) : args.perXcd) * 8 + strips.padded);
+    strips.first = (walk ? std::min(slotsPerXcd, args.perXcd) : args.perXcd) * 8;
+    const dim3 grid(strips.first + strips.blocks[0] + strips.blocks[1]);
     if (transA && transB)
         LaunchTiled<true, true>(args, strips, grid, big, aligned, dma, walk, ksplit, stream);
     else if (transA)
