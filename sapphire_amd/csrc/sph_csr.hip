@@ -910,7 +910,7 @@ int sph_csr_validate_u32(const uint32_t* COL, const uint32_t* ROW, uint32_t M, u
     SPH_REQUIRE(ROW != nullptr, "ROW is null");
     SPH_REQUIRE(nnz == 0 || COL != nullptr, "COL is null");
     SPH_REQUIRE(M < 0xffffffffu, "too many rows");
-    SPH_REFUSE_WHILE_CAPTURING();  // reads the verdict back
+    SPH_REFUSE_WHILE_CAPTURING();  // reads the result back
     hipStream_t stream = sph::CurrentStream();
     if (stream == nullptr)
         return SPH_ERR_DEVICE;
