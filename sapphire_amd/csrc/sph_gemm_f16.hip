@@ -3,7 +3,7 @@
 // Includes/Sapphire/compute/dense/cuda/kernels/GemmKernel.cuh:14-50): half
 // inputs, fp32 accumulation, row-major operands, result added into out.
 //
-// Four kernels:
+// Six kernels:
 //
 //   GemmF16Few      products with at most one 32 x 32 output tile per compute unit (or at most 16
 //     rows or columns), whatever K, the storage flags and the alignment: one 32 x 32 or 16 x 16
@@ -32,21 +32,29 @@
 //     the 32 workgroups that land on one XCD (ids congruent mod 8) cover a compact
 //     8 x 4 block of tiles and share their A and B panels through that XCD's L2.
 //
+//   GemmF16Tile256<..., NT = 128>  the same kernel on 256 x 128 tiles, taken while there are
+//     between 11/16 of such a tile and one tile per compute unit.
+//
 //   GemmF16Dma128   the same conditions, any M: the
-//     same ingredients on 128 x 128 tiles with 4 wavefronts (v_mfma_f32_32x32x16_f16), for
+//     same ingredients on 128 x 128 tiles with 4 or 8 wavefronts (v_mfma_f32_32x32x16_f16), for
 //     shapes with too few 256-tiles to fill the chip.
 //
+//   GemmF16Dma64    at most half as many 128 x 128 tiles as compute units and K >= 64: 64 x 64
+//     tiles, K steps of 64, 4 wavefronts.
+//
 //   GemmF16General  everything else.  128 x 128 tile, 4 wavefronts, K step 32,
-//     global loads staged through registers, 16, 8, 4 or 2 bytes at a time (the
-//     widest that K, N, the strides and the bases allow), padded LDS rows.
+//     global loads staged through registers, 16 bytes at a time (aligned, from a 4-byte
+//     boundary, or as aligned dwords that are shifted when a row starts at an odd half), padded
+//     LDS rows.
 //
 // K = 32 q + r, r != 0, K >= 64 stays on the first two kernels: a last step over [K - 32, K) in
 // which the fragment positions whose k was multiplied already are cleared.
 //
 // N = 8 q + r, r != 0: the first 8 q columns go to the tiled straight-to-LDS kernels when they
 // would take that shape (the copies into LDS need no alignment, so rows of B and of out may start
-// anywhere; only a copy's 8 columns have to lie inside the row) and the last r columns to
-// GemmF16Few, as do the last M % 8 rows of an A stored K x M.
+// anywhere; only a copy's 8 columns have to lie inside the row) and the last r columns to the
+// code of GemmF16Few, as do the last M % 8 rows of an A stored K x M and up to 16 rows or columns
+// just past a tile edge: as strips on the last workgroups of the body's own launch (LaunchF16).
 #include "sph_internal.h"
 #include "sph_k_partition.h"
 

@@ -13,6 +13,9 @@
 //                        multiple of the step ends in a partial step);
 //                        with more 64-tiles than resident workgroups each workgroup walks
 //                        several tiles and the copy stream runs across the tile boundaries;
+//                        with 65 to 128 tiles of 64 x 64, 64 x 32 tiles whose K steps are
+//                        split over two groups of wavefronts (KSPLIT = 2: another order of
+//                        the K products, chosen for the whole product at once);
 //   GemmF32Kernel        any shape and alignment: register-staged double buffering, 16-byte
 //                        loads when possible, scalar predicated loads otherwise (small K,
 //                        misaligned bases, e.g. some of the reference's random test sizes,
@@ -20,8 +23,11 @@
 //   GemmF32SkinnyKernel  few output tiles: 16 x 16 or 32 x 32 tiles with K split over the
 //                        wavefronts of a workgroup;
 //   GemvRowKernel        a single output row.
-// An N that is no multiple of 4 is split by the launcher: the first 4 q columns to the kernels
-// above, the last ones to the few-tile kernel.
+// A product for the tiled kernels is cut by the launcher into a body and up to two thin strips:
+// the last N % 4 columns, the last M % 4 rows (from 68 rows up) and up to 16 rows or columns
+// just past a tile edge.  The strips are computed by the few-tile kernel's code on the last
+// workgroups of the body's own launch (GemmF32Strips), or by launches of their own beside a
+// register-staged body.
 // The first two share one decomposition: a workgroup (4 wavefronts, 2 x 2) owns a BM x BN tile
 // of one M x N unit, BM = BN = 128 or 64 (whichever loads the busiest compute unit less),
 // and they add the K products of an element in the same order, so which of them
