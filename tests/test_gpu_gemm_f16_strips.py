@@ -2,7 +2,7 @@
 last N % 8 columns (and, of an A stored K x M, the last M % 8 rows) that the straight-to-LDS
 copies cannot take, and up to 16 rows or columns past a multiple of the tile edge when that
 spares the busiest compute unit a tile.  The strips are computed by the few-tile kernel's code on
-the first workgroups of the body's launch, whichever of the tiled kernels the body takes.
+the last workgroups of the body's launch, whichever of the tiled kernels the body takes.
 
 Integer-valued operands make every product and partial sum exact, so body, strips and the seam
 between them are checked bit for bit against the CPU loop; N(0, 1/sqrt(K)) operands are held to
@@ -153,3 +153,35 @@ def test_operands_that_start_at_an_odd_half(dev):
     for d in (dA, dB, dC):
         d.release()
     assert np.array_equal(got, _oracle(C, A, np.ascontiguousarray(B.T), M, N, K))
+
+
+@pytest.mark.parametrize("block", range(6))
+def test_random_shapes_just_past_a_tile_grid(dev, block):
+    """Seeded shapes a few rows and columns past multiples of 64, 128 and 256 with about one tile
+    per compute unit, where the cut depends on both remainders; all flag combinations, integer
+    operands (bit for bit), guard words."""
+    rng = np.random.default_rng(9400 + block)
+    for it in range(8):
+        M = int(rng.choice([960, 1024, 1088, 2048, 4096])) + int(rng.integers(0, 19))
+        N = int(rng.choice([960, 1024, 1088, 2048, 4096])) + int(rng.integers(0, 19))
+        K = int(rng.choice([24, 33, 64, 65, 96, 130]))
+        flags = int(rng.integers(0, 8))
+        h.announce("sph_gemm_f16f32 random, past a tile grid", (M, N, K), "flags", flags)
+        seed = 940000 + 100 * block + 3 * it
+        A = synth.small_integers(seed, (M, K), span=3).astype(np.float16)
+        B = synth.small_integers(seed + 1, (K, N), span=3).astype(np.float16)
+        C = synth.small_integers(seed + 2, (M, N), span=100)
+        As, Bs = _stored(A, B, flags)
+        guard = np.full(64, np.float32(-777.25), np.float32)
+        padded = np.concatenate([guard, C.ravel(), guard]).astype(np.float32)
+        dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (As, Bs, padded))
+        assert dC.nbytes >= 4 * (128 + M * N) and dA.nbytes >= 2 * M * K and dB.nbytes >= 2 * K * N
+        capi.call("sph_gemm_f16f32", dC.at(4 * 64), dA.ptr, dB.ptr, M, N, K, 1, M * N, M * K,
+                  K * N, flags)
+        back = dC.download(np.float32, padded.shape)
+        for d in (dA, dB, dC):
+            d.release()
+        assert np.array_equal(back[:64], guard) and np.array_equal(back[-64:], guard)
+        ref = _oracle(C, A, B, M, N, K)
+        want = ref - C if flags & OW else ref
+        assert np.array_equal(back[64:-64].reshape(M, N), want), (M, N, K, flags)

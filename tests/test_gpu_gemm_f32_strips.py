@@ -168,3 +168,34 @@ def test_grouped_units_with_strips(dev):
         o = units - 1 - u
         ref = po.gemm_rows(C[o].copy(), A[u], B[u % 2], M, N, K)
         assert h.normalised_error(got[o], ref, np.abs(A[u]), np.abs(B[u % 2])) <= TOL_F32
+
+
+@pytest.mark.parametrize("block", range(6))
+def test_random_shapes_just_past_a_tile_grid(dev, block):
+    """Seeded shapes a few rows and columns past multiples of 64 and 128 with about one tile per
+    compute unit, where the cut depends on both remainders; all flag combinations, guard words."""
+    rng = np.random.default_rng(9300 + block)
+    for it in range(8):
+        M = int(rng.choice([960, 1024, 1088, 2048])) + int(rng.integers(0, 19))
+        N = int(rng.choice([960, 1024, 1088, 512])) + int(rng.integers(0, 19))
+        K = int(rng.choice([16, 24, 33, 64, 100]))
+        flags = int(rng.integers(0, 8))
+        h.announce("sph_gemm_f32_ex random, past a tile grid", (M, N, K), "flags", flags)
+        seed = 930000 + 100 * block + 3 * it
+        A, B = synth.uniform(seed, (M, K)), synth.uniform(seed + 1, (K, N))
+        C = synth.uniform(seed + 2, (M, N))
+        As, Bs = _stored(A, B, flags)
+        guard = np.full(64, np.float32(-777.25), np.float32)
+        padded = np.concatenate([guard, C.ravel(), guard])
+        dA, dB, dC = (capi.DeviceBuffer.from_array(x) for x in (As, Bs, padded))
+        assert dC.nbytes >= 4 * (128 + M * N) and dA.nbytes >= 4 * M * K and dB.nbytes >= 4 * K * N
+        capi.call("sph_gemm_f32_ex", dC.at(4 * 64), dA.ptr, dB.ptr, M, N, K, 1, M * N, M * K,
+                  K * N, flags)
+        back = dC.download(np.float32, padded.shape)
+        for d in (dA, dB, dC):
+            d.release()
+        assert np.array_equal(back[:64], guard) and np.array_equal(back[-64:], guard)
+        start = np.zeros_like(C) if flags & OW else C
+        ref = po.gemm_rows(start.copy(), A, B, M, N, K, threads=8)
+        err = h.normalised_error(back[64:-64].reshape(M, N), ref, np.abs(A), np.abs(B))
+        assert err <= TOL_F32, (M, N, K, flags, err)
