@@ -217,11 +217,6 @@ __device__ __forceinline__ float4 NtLoad4(const float* p)
     const floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4a4*>(p));
     return make_float4(v[0], v[1], v[2], v[3]);
 }
-__device__ __forceinline__ void NtStore4(float* p, float4 v)
-{
-    const floatx4 w = { v.x, v.y, v.z, v.w };
-    __builtin_nontemporal_store(w, reinterpret_cast<floatx4a4*>(p));
-}
 __device__ __forceinline__ float4 Load4(const float* p)
 {
     const floatx4 v = *reinterpret_cast<const floatx4a4*>(p);
@@ -291,7 +286,6 @@ constexpr int kT = 256;         // tile edge
 constexpr int kTK = 32;         // K step
 constexpr int kTStages = 4;
 constexpr int kStageBytes = kT * kTK * 2;  // per operand per stage (16 KiB)
-constexpr int kStageHalfs = kT * kTK;
 
 // ---------------------------------------------------------------------------
 // 256 x 256 tile kernel, v_mfma_f32_16x16x32_f16
@@ -1986,7 +1980,6 @@ F16Kernel PickF16(const GemmF16Args& args, uint32_t N, uint32_t batch, const F16
 {
     const uint32_t M = args.M, K = args.K;
     const bool transA = lay.transA, transB = lay.transB;
-    const bool plain = !transA && !transB;
     // the 256-tile kernel needs about one tile per compute unit; below three quarters of that
     // the 128-tile kernel keeps more of the chip busy (measured: 2048^3 44 -> 31 us)
     const uint64_t minTiles = static_cast<uint64_t>(sph::ComputeUnits()) * 3 / 4;

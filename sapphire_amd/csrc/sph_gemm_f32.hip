@@ -1320,7 +1320,6 @@ __device__ __forceinline__ void GemmF32SkinnyBody(const GemmF32Args& args, uint3
     const sph::KPartition part = sph::PartitionK(K, kGroupK, WAVES, wave, kDepth);
 
     const bool rowOk = row < M;
-    const bool colOk = col < N;
 
     Acc acc;
 #pragma unroll
