@@ -41,7 +41,9 @@ def _stored(A, B, flags):
 # general kernel (K below one step of the copies): 1025 x 1030 x 24.
 SHAPES = [(1025, 1025, 65, 1), (1025, 1025, 128, 1), (1000, 1004, 200, 1), (1032, 1027, 77, 1),
           (321, 323, 96, 6), (1100, 2052, 64, 1), (2049, 2056, 72, 1), (3073, 2050, 64, 1),
-          (4097, 4100, 64, 1), (4097, 4097, 96, 1), (1025, 1030, 24, 1)]
+          (4097, 4100, 64, 1), (4097, 4097, 96, 1), (1025, 1030, 24, 1),
+          # a batch on 256 x 256 tiles: 4 x (9 x 9) tiles cut to 4 x (8 x 8)
+          (2049, 2052, 64, 4)]
 
 
 @pytest.mark.parametrize("flags", [0, TA, TB, TA | TB])

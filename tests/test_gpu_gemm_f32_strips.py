@@ -37,7 +37,7 @@ def _stored(A, B, flags):
 SHAPES = [(1025, 1025, 40, 1), (1025, 1024, 70, 1), (1024, 1025, 33, 1), (1040, 1036, 48, 1),
           (1001, 1001, 36, 1), (1031, 1000, 64, 1), (2049, 2049, 32, 1), (8192, 65, 64, 1),
           (8192, 67, 17, 1), (513, 514, 24, 4), (321, 323, 50, 7), (1025, 1025, 16, 1),
-          (2061, 1030, 20, 1)]
+          (2061, 1030, 20, 1), (1025, 1026, 20, 3)]
 
 
 @pytest.mark.parametrize("flags", [0, TA, TB, TA | TB, OW, OW | TA | TB])
