@@ -10,9 +10,9 @@
 // single add into out.  Each output element is owned by exactly one lane which
 // walks the row front to back, so the result is bit-identical to that loop.
 //
-// Three mappings.
+// Two mappings.
 //
-// SpmmSlabVec4 (the first 4 * (N / 4) dense columns): the dense columns are cut
+// SpmmSlabVec4 (N >= 4): the dense columns are cut
 // into slabs of 64 (32 for narrow operands); all workgroups that run on one XCD (ids
 // congruent mod 8) work on the same slab, so the part of B an XCD gathers from (K x 64
 // floats, 2 MiB at K = 8192) stays resident in that XCD's L2 instead of being streamed
@@ -22,7 +22,9 @@
 // one 256-byte gather per row, eight of them in flight per lane.  The loop has no branches:
 // entries past the end of a row gather row 0 of B and a select keeps them out of the sum.
 //
-// SpmmNarrow (the last N % 4 columns): one lane per (row, column), eight gathers in flight.
+// With N = 4 q + r the one lane per row whose four columns would reach past N takes the last
+// four columns instead and stores only the r sums that are its own (a separate pass over the last
+// r columns, one lane per row and column, cost as much as three quarters of a 256-column product).
 //
 // SpmmRowScalar: one wavefront per sparse row, one column per lane (operands whose byte
 // offsets do not fit 32 bits, N < 4); the row's (COL, V) pairs are fetched 64 at a time and
@@ -126,9 +128,15 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
                                (threadIdx.x >> 6) * kRowsPerWave + lane / LPR;
     const uint32_t row = part * plan.rowsPerPart + rowInPart;
     const uint32_t N = args.N;
-    const uint32_t col = slab * kSlabCols + t * 4;
+    // A lane whose four columns reach past N (N = 4 q + r: one lane per row, in the last slab)
+    // takes columns N - 4 .. N - 1 instead and stores only the last r of its sums: the 16-byte
+    // accesses need no alignment beyond 4 bytes, and the other columns are another lane's.
+    const uint32_t colNatural = slab * kSlabCols + t * 4;
+    const bool ragged = colNatural < N && colNatural + 4 > N;
+    const uint32_t col = ragged ? N - 4 : colNatural;
+    const uint32_t storeFrom = ragged ? colNatural + 4 - N : 0;  // first component to store
     const bool rowOk = rowInPart < plan.rowsPerPart && row < args.M;
-    const bool active = rowOk && col < N;
+    const bool active = rowOk && colNatural < N;
 
     uint32_t p = 0, end = 0;
     if (rowOk)
@@ -137,12 +145,12 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
         end = args.ROW[row + 1];
     }
     // Every lane gathers from a valid address on every step, so the loop has no branches:
-    // lanes outside the matrix read the slab's first columns, entries past the end of a row
+    // lanes outside the matrix read the last four columns, entries past the end of a row
     // read row 0 of B (their COL is 0), and a select keeps such products out of the sum.
     // Byte offsets into B fit 32 bits (checked by the launcher) and are formed with a 24-bit
     // multiply-add.
     const char* __restrict__ Bbytes = reinterpret_cast<const char*>(args.B);
-    const uint32_t colBytes = (col < N ? col : slab * kSlabCols) * 4;
+    const uint32_t colBytes = (colNatural < N ? col : N - 4) * 4;
     const uint32_t rowBytes = args.ldB * 4;
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 
@@ -217,54 +225,23 @@ __global__ __launch_bounds__(kThreads) void SpmmSlabVec4(const SpmmArgs args, co
         }
         else if (args.accumulate)
         {
+            // (the ragged lane reads values another lane is about to replace or has replaced in
+            // the components it does not store; it uses only the ones it owns)
             const float4 old = Load4(dst);
             sum.x = old.x + sum.x;
             sum.y = old.y + sum.y;
             sum.z = old.z + sum.z;
             sum.w = old.w + sum.w;
         }
-        Store4(dst, sum);
-    }
-}
-
-// Up to 4 output columns (the last N % 4 of a wider operand): one lane per (row, column), 16
-// rows per wavefront; a lane walks its row front to back, eight gathers in flight.
-__global__ __launch_bounds__(kThreads) void SpmmNarrow(const SpmmArgs args)
-{
-    const uint32_t row = (blockIdx.x * kThreads + threadIdx.x) / 4;
-    const uint32_t col = threadIdx.x & 3;
-    if (row >= args.M || col >= args.N)
-        return;
-    const uint32_t begin = args.ROW[row];
-    const uint32_t end = args.ROW[row + 1];
-    const float* __restrict__ B = args.B + col;
-    const size_t ld = args.ldB;
-    float sum = 0.f;
-    uint32_t p = begin;
-    for (; p + 8 <= end; p += 8)
-    {
-        uint32_t c[8];
-        float v[8], b[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
+        if (!ragged)
+            Store4(dst, sum);
+        else
         {
-            c[j] = args.COL[p + j];
-            v[j] = args.V[p + j];
+            if (storeFrom <= 1) dst[1] = sum.y;
+            if (storeFrom <= 2) dst[2] = sum.z;
+            dst[3] = sum.w;
         }
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            b[j] = B[c[j] * ld];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            sum = sum + v[j] * b[j];
     }
-    for (; p < end; ++p)
-        sum = sum + args.V[p] * B[args.COL[p] * ld];
-    float* dst = args.out + static_cast<size_t>(row) * args.ldOut + col;
-    if (args.rowBias != nullptr)
-        *dst = (0.f + args.rowBias[row]) + sum;
-    else
-        *dst = args.accumulate ? (*dst + sum) : sum;
 }
 
 // one output column per lane; any N, any alignment
@@ -343,25 +320,26 @@ static int LaunchSpmm(float* out, const float* V, const uint32_t* COL, const uin
 
     // the slab kernel forms 32-bit byte offsets into B with a 24-bit multiply; larger operands
     // run on the scalar kernel, whose offsets are 64-bit.  Its 16-byte accesses need no
-    // alignment beyond 4 bytes, so N = 4 q + r is served by the slab kernel on the first 4 q
-    // columns (row pitches stay N) and by the narrow kernel on the last r: every output
-    // element is still summed by one lane in storage order
+    // alignment beyond 4 bytes, so any N >= 4 is served by the slab kernel: every output
+    // element is summed by one lane in storage order
     // (measured on the 8192 x 8192 matrix at 1 %: N = 255 134 us on the scalar kernel).
     const bool slabFits = static_cast<uint64_t>(Kdim) * N * 4 < (1ull << 32) &&
                           Kdim < (1u << 24) && N < (1u << 22);
-    const uint32_t whole = N & ~3u;
-    if (slabFits && whole != 0)
+    if (slabFits && N >= 4)
     {
-        SpmmArgs left = args;
-        left.N = whole;
         // 16 lanes per row (64-column slabs, 4 rows per wavefront) measured fastest from N = 64
         // up; narrower operands use 8 lanes per row so that fewer lanes idle
-        const int lanesPerRow = whole <= 32 ? 8 : 16;
+        const int lanesPerRow = N <= 32 ? 8 : 16;
         const uint32_t slabCols = 4u * static_cast<uint32_t>(lanesPerRow);
         const uint32_t rowsPerBlock = (64u / static_cast<uint32_t>(lanesPerRow)) * kWavesPerBlock;
         SlabPlan plan{};
-        plan.slabs = (whole + slabCols - 1) / slabCols;
-        plan.rowParts = plan.slabs >= 8 ? 1u : 8u / plan.slabs;
+        plan.slabs = (N + slabCols - 1) / slabCols;
+        // rows are cut into parts so that the (slab, part) work columns fill the 8 XCDs evenly:
+        // slabs * parts is the least common multiple of the slab count and 8
+        uint32_t common = 8;  // gcd(slabs, 8)
+        while (plan.slabs % common != 0)
+            common /= 2;
+        plan.rowParts = 8u / common;
         const uint32_t rowsPerPart = (M + plan.rowParts - 1) / plan.rowParts;
         plan.blocksPerColumn = (rowsPerPart + rowsPerBlock - 1) / rowsPerBlock;
         plan.rowsPerPart = plan.blocksPerColumn * rowsPerBlock;
@@ -370,22 +348,10 @@ static int LaunchSpmm(float* out, const float* V, const uint32_t* COL, const uin
         SPH_REQUIRE(grid < (1ull << 31), "too many workgroups for one launch");
         if (lanesPerRow == 16)
             hipLaunchKernelGGL(SpmmSlabVec4<16>, dim3(static_cast<uint32_t>(grid)),
-                               dim3(kThreads), 0, stream, left, plan);
+                               dim3(kThreads), 0, stream, args, plan);
         else
             hipLaunchKernelGGL(SpmmSlabVec4<8>, dim3(static_cast<uint32_t>(grid)), dim3(kThreads),
-                               0, stream, left, plan);
-        if (whole != N)
-        {
-            SPH_CHECK_LAUNCH();
-            SpmmArgs right = args;
-            right.N = N - whole;
-            right.B = B + whole;
-            right.out = out + whole;
-            const uint64_t lanes = static_cast<uint64_t>(M) * 4;
-            SPH_REQUIRE(lanes < (1ull << 31), "too many rows for one launch");
-            hipLaunchKernelGGL(SpmmNarrow, dim3(static_cast<uint32_t>((lanes + kThreads - 1) / kThreads)),
-                               dim3(kThreads), 0, stream, right);
-        }
+                               0, stream, args, plan);
     }
     else
     {
